@@ -1,0 +1,139 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused gated-attention operator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--no-cpu]
+
+A "step" is one kutacc_af2_gating_attention call on device-resident synthetic inputs of the chosen
+configuration (default: config 3, the N_res=384 triangle-attention shape the headline metric is
+quoted on).  Prints ONE JSON line: whole-call TFLOP/s from algorithmic flops
+(10*B*S*C^2 + 4*B*S^2*C), ms per call, the roofline of the dominant kernel (live hipEvent timing on
+the launch stream, read back through kutacc_hip_profile_*) and a CPU baseline (the bf16
+restatement of the reference algorithm in oracle/, timed on this host on a bounded batch sample).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(w, budget_s=15.0):
+    """Time oracle Rbf16 (reference rounding points, OpenMP on all host cores) on the first rows of the
+    batch; rows are independent, so throughput on the sample is throughput on the whole batch."""
+    import numpy as np
+    from oracle import oracle
+    from kutacc_amd.workloads import bf16_bits
+
+    def run(nrows):
+        sub = w.batch_slice(np.arange(nrows))
+        b = bf16_bits
+        args = (b(sub.x), b(sub.wq), b(sub.wk), b(sub.wv), b(sub.wg), sub.bg, b(sub.wo), sub.bo, b(sub.bias),
+                None if sub.nb is None else b(sub.nb), sub.H)
+        t0 = time.perf_counter()
+        oracle.gating_attention_bf16(*args, block_size=64, exp_mode=1)
+        return time.perf_counter() - t0, sub.flops()
+
+    probe = min(w.B, max(2, oracle.num_threads() // w.H + 1))
+    t_probe, _ = run(probe)
+    rows = int(min(w.B, max(probe, probe * budget_s / max(t_probe, 1e-3))))
+    t, fl = run(rows)
+    return {
+        "value": round(fl / t / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+        "sample": f"first {rows} of {w.B} batch rows of the same workload, one call, {t:.2f} s "
+                  f"(= {t / rows * w.B * 1e3:.0f} ms/call extrapolated to the full batch)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the operator shards over the batch axis with no "
+                 "exchange; multi-GPU runs are not part of it). Use --gpus 1.")
+
+    import torch
+    import helpers
+    from kutacc_amd import capi
+    from kutacc_amd.workloads import make_workload
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    w = make_workload(a.config)
+    op, ten, scratch = helpers.make_op(w, device="cuda:0")
+    stream = torch.cuda.current_stream()
+    capi.set_stream(stream.cuda_stream)
+    capi.set_blocking(False)
+    L = capi.lib()
+
+    for _ in range(a.warmup):
+        op.run()
+    assert not capi.error_flag()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        op.run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    assert not capi.error_flag()
+    ms = wall / a.steps * 1e3
+    tflops = w.flops() / (ms * 1e-3) / 1e12
+
+    # per-kernel durations: same K calls again with hipEvents recorded around each kernel on the stream
+    L.kutacc_hip_profile_enable(1)
+    for _ in range(a.steps):
+        op.run()
+    torch.cuda.synchronize()
+    L.kutacc_hip_profile_enable(0)
+    kernels = []
+    name = ctypes.create_string_buffer(128)
+    tot, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+    i = 0
+    while L.kutacc_hip_profile_read(i, name, 128, ctypes.byref(tot), ctypes.byref(cnt), ctypes.byref(fl)) == 0:
+        kernels.append(dict(name=name.value.decode(), avg_ms=tot.value / max(cnt.value, 1), launches=cnt.value,
+                            flops_per_launch=fl.value))
+        i += 1
+    dom = max(kernels, key=lambda k: k["avg_ms"] * k["launches"]) if kernels else None
+    roofline = None
+    if dom:
+        ach = dom["flops_per_launch"] / (dom["avg_ms"] * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                    "avg_kernel_ms": round(dom["avg_ms"], 5),
+                    "flops_per_launch": dom["flops_per_launch"]}
+
+    capi.set_blocking(True)
+    capi.set_stream(None)
+
+    rec = {
+        "metric": "gated-attention TFLOP/s + % bf16 MFMA peak; ms/call at N_res=384 tri-attn",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w.dtype, "data": "synthetic",
+        "config": {"workload": f"config {w.config} {w.name}: B={w.B} S={w.S} C={w.C} H={w.H} d={w.d}",
+                   "flops_per_call": w.flops(), "algorithmic_bytes_per_call": w.algorithmic_bytes(),
+                   "path": capi.last_path()},
+        "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        "kernels": [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in kk.items()} for kk in kernels],
+        "roofline": roofline,
+        "cpu_baseline": None if a.no_cpu else cpu_baseline(w),
+    }
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

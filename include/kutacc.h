@@ -1,0 +1,192 @@
+/*
+ * kutacc.h -- public interface of the MI355X (gfx950) build of the KuTACC gated-attention path.
+ *
+ * Interface contract: every name, argument order, struct layout and enum value below is the one a
+ * caller of the Kunpeng library already compiles against (reference include/kutacc.h), restricted
+ * to the entry points that feed or form the fused gated-attention operator.  A program built
+ * against the reference header links and runs against this library for those entry points; the
+ * remaining kutacc_af2_* / kutacc_comm_* symbols are exported as "not implemented on this
+ * backend" stubs (see kutacc_amd/csrc/unsupported.cpp) so that the shared object still resolves.
+ *
+ * Differences a caller can observe, all additive:
+ *   - DType gains kFP32 (value 2, after kBF16) so that fp32 tensors can be described.
+ *   - data pointers may be HIP device pointers (fast path) or host pointers (staged through the
+ *     device); the two kinds must not be mixed within one call.
+ *   - "prepacked" operands are plain row-major: the pack routines below are identity copies.
+ *
+ * Requires a compiler that knows the __bf16 type (ROCm clang++ / hipcc).
+ */
+#ifndef KUTACC_H
+#define KUTACC_H
+
+#include <cstddef>
+#include <cstdint>
+#include <vector>
+
+#define kutacc_export __attribute__((visibility("default")))
+
+/* Status codes; only kutacc_get_version returns one (reference include/kutacc.h:28-29). */
+#define KUTACC_OK 0
+#define KUTACC_ERROR (-1)
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Opaque tensor descriptor; produced by kutacc::TensorWrapper::get_tensor()
+ * (reference include/kutacc.h:49). */
+typedef void *kutacc_tensor_h;
+
+/* Version record, six C strings owned by the library (reference include/kutacc.h:32-39). */
+typedef struct kutacc_version {
+    const char *product_name;
+    const char *product_version;
+    const char *component_name;
+    const char *component_version;
+    const char *component_abi_version;
+    const char *component_appendinfo;
+} kutacc_version_t;
+
+/* Fills *version; returns KUTACC_ERROR for a null argument
+ * (reference include/kutacc.h:47, src/version/version.cpp:28-35). */
+kutacc_export int kutacc_get_version(kutacc_version_t *version);
+
+/* Rank bookkeeping of the reference's shared-memory collectives (reference include/kutacc.h:51-53).
+ * Exported for link compatibility; this single-GPU build never changes them. */
+kutacc_export extern int64_t world_size;
+kutacc_export extern int64_t rank;
+
+/* Weights of one gated-attention block (reference include/kutacc.h:77-89).
+ *   query_w/key_w/value_w/gating_w/output_w : [nchannels, nchannels], stored [out, in] row-major
+ *   gating_b/output_b                       : fp32 [nchannels]
+ *   nchannels == nheads * head_size */
+typedef struct kutacc_af2_attention_weights {
+    int64_t nchannels;
+    int64_t nheads;
+    int64_t head_size;
+
+    kutacc_tensor_h query_w;
+    kutacc_tensor_h key_w;
+    kutacc_tensor_h value_w;
+    kutacc_tensor_h gating_w;
+    kutacc_tensor_h gating_b;
+    kutacc_tensor_h output_w;
+    kutacc_tensor_h output_b;
+} kutacc_af2_attention_weights_t;
+
+/* Problem extent plus caller-owned scratch tensors (reference include/kutacc.h:95-104).
+ *   q, k, gate, avg : [batch, seq_len, nheads, head_size]
+ *   v               : [nheads, head_size, batch, seq_len]  (transposed, as the reference writes it,
+ *                     src/attention/gating_attention.cpp:57-61,123-127)
+ * The library may overwrite them; after a call `avg` holds the gated weighted average. */
+typedef struct kutacc_af2_attention_inputs {
+    int64_t batch;
+    int64_t seq_len;
+
+    kutacc_tensor_h q;
+    kutacc_tensor_h k;
+    kutacc_tensor_h v;
+    kutacc_tensor_h gate;
+    kutacc_tensor_h avg;
+} kutacc_af2_attention_inputs_t;
+
+/*
+ * Fused Evoformer gated attention with pair bias (reference include/kutacc.h:297-300,
+ * src/attention/gating_attention.cpp:33-200):
+ *
+ *   q,k,v = input.Wq^T, input.Wk^T, input.Wv^T         gate = input.Wg^T + gating_b
+ *   p     = softmax_k(q.k^T / sqrt(head_size) + bias[b,k] + nonbatched_bias[h,q,k])
+ *   out   = ((p.v) * sigmoid(gate)).Wo^T + output_b
+ *
+ *   input            [batch*seq_len, nchannels], already layer-normalised
+ *   bias             [batch, 1, 1, seq_len] mask bias (0 or -1e9), element (b,k) at b*strides[0]+k
+ *   nonbatched_bias  [nheads, seq_len, seq_len]; a tensor whose sizes[0]==0 means "absent"
+ *   out              [batch, seq_len, nchannels]
+ *   block_size       query tiling of the CPU implementation; validated (>0), otherwise advisory
+ *
+ * All six pointer arguments must be non-null.  Violations print one KUTACC_CHECK line on stderr,
+ * latch the process-wide error flag and return without touching `out`.
+ */
+kutacc_export void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inputs_t *q_based_ptr,
+                                               kutacc_tensor_h bias, kutacc_tensor_h nonbatched_bias,
+                                               kutacc_af2_attention_weights_t *weight_ptr, kutacc_tensor_h out,
+                                               int64_t block_size);
+
+/*
+ * LayerNorm of ONE row of `size` elements, bf16 in/out, fp32 gamma/beta
+ * (reference include/kutacc.h:334, src/normalization/layernorm_kernel.h:21-53).
+ * Raw pointers, not handles.  See kutacc_hip_layernorm_rows in kutacc_hip.h for the batched form.
+ */
+kutacc_export void kutacc_af2_layernorm(__bf16 *data, float *gamma, float *beta, int64_t size, float eps, __bf16 *out);
+
+/*
+ * result[m,n] = beta*result + act[m,k].weight[n,k]^T (+ bias_data[n]), bf16 operands and result
+ * (reference include/kutacc.h:399-400, src/linear/linear.cpp:21-50).  m = numel(act)/k,
+ * k = last dim of act, n = numel(weight)/k; result is written contiguously as [m,n].
+ */
+kutacc_export void kutacc_af2_linear(kutacc_tensor_h act, kutacc_tensor_h weight, float *bias_data,
+                                     kutacc_tensor_h result, int64_t beta);
+
+/*
+ * "Pre-pack" a [n,k] bf16 matrix with leading dimension ldb (reference include/kutacc.h:407-408,
+ * src/linear/mm.cpp:94-110).  On this backend the packed layout is dense row-major [n,k], so this
+ * is a strided copy; num_threads is accepted and ignored.
+ */
+kutacc_export void kutacc_af2_linear_weight_prepack(const __bf16 *weight, __bf16 *result, int64_t n, int64_t k,
+                                                    int64_t ldb, int64_t num_threads = 0);
+
+/*
+ * Element count of a packed operand: m*k for identifier 'A', k*n for 'B'
+ * (reference include/kutacc.h:418, src/utils/blas.cpp:93-98).
+ */
+kutacc_export size_t kutacc_af2_gemm_pack_get_size(char identifier, char transa, char transb, int m, int n, int k);
+
+#ifdef __cplusplus
+}
+#endif
+
+#ifdef __cplusplus
+namespace kutacc {
+
+/* Element type tag carried by a tensor descriptor (reference include/kutacc.h:467-471).
+ * kFP32 is new on this backend and sits after the reference's values. */
+typedef enum TensorDataType {
+    kInt64 = 0,
+    kBF16 = 1,
+    kFP32 = 2,
+    kNumTypes
+} DType;
+
+/* GEMM epilogue switches of the reference's BLAS shim (reference include/kutacc.h:474-482).
+ * Kept so that callers naming the type still compile; this backend reads none of it. */
+struct BlasExtendParams {
+    int64_t num_threads;
+    bool prepack_a;
+    bool prepack_b;
+    bool row_bias;
+    bool col_bias;
+    void *bias;
+    bool relu;
+};
+
+/* Owns one strided, non-owning view {data, sizes, strides (in elements), dim, dtype} and hands it
+ * out as a kutacc_tensor_h (reference include/kutacc.h:484-497, src/tensor/tensor.cpp:20-30,88-92).
+ * As in the reference, copying a TensorWrapper is not supported. */
+struct kutacc_export TensorWrapper {
+private:
+    kutacc_tensor_h tensor_;
+
+public:
+    TensorWrapper(void *data_ptr, std::vector<int64_t> &&sizes, std::vector<int64_t> &&strides, int64_t dim,
+                  DType dtype);
+    TensorWrapper();
+    kutacc_tensor_h get_tensor()
+    {
+        return tensor_;
+    }
+    ~TensorWrapper();
+};
+} // namespace kutacc
+#endif
+
+#endif /* KUTACC_H */

@@ -1,0 +1,159 @@
+/*
+ * kutacc_hip.h -- the C-ABI launch layer between the C++ host side of libkutacc and its HIP kernels.
+ *
+ * Everything here is extern "C" with plain pointers and sizes: no C++ types, no torch types, no
+ * tensor handles.  The handle-based entry points of kutacc.h unpack their arguments and call these;
+ * an FFI user (ctypes, cgo, JNI) can call them directly on device memory.
+ *
+ * Conventions
+ *   - every data pointer is a HIP DEVICE pointer on the current device unless stated otherwise;
+ *   - `dtype` is a kutacc::DType value: 1 = bf16 storage, 2 = fp32 storage;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the library stream, see
+ *     kutacc_hip_set_stream); launches are asynchronous, the caller synchronises;
+ *   - the return value is 0 on success, a hipError_t value if a HIP call failed, or a negative
+ *     KUTACC_HIP_E* code if the arguments were rejected before anything was launched.
+ *   - strides are in elements.
+ */
+#ifndef KUTACC_HIP_H
+#define KUTACC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifndef kutacc_export
+#define kutacc_export __attribute__((visibility("default")))
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KUTACC_HIP_EINVAL (-2)      /* bad shape / stride / dtype / null pointer          */
+#define KUTACC_HIP_EUNSUPPORTED (-3) /* request is valid but no kernel on this backend takes it */
+
+#define KUTACC_DTYPE_BF16 1
+#define KUTACC_DTYPE_FP32 2
+
+/* Kernel family selection for kutacc_hip_gating_attention. */
+#define KUTACC_HIP_PATH_AUTO 0    /* fused MFMA kernels when the shape allows, else generic      */
+#define KUTACC_HIP_PATH_GENERIC 1 /* shape-agnostic scalar kernels (any head_size, bf16 or fp32)  */
+#define KUTACC_HIP_PATH_FUSED 2   /* bf16 MFMA kernels only; EUNSUPPORTED if the shape is not covered */
+
+/*
+ * Flat argument block of the gated-attention operator.  Replaces, for the launch layer, the
+ * (Tensor&, ...) parameter list of kutacc::gating_attention_kernel
+ * (reference src/attention/gating_attention.cpp:33-37); field meaning follows that function.
+ */
+typedef struct kutacc_hip_attention_args {
+    int64_t batch;     /* B */
+    int64_t seq_len;   /* S */
+    int64_t nheads;    /* H */
+    int64_t head_size; /* d;  nchannels C = H*d */
+    int32_t dtype;     /* storage type of input, weights matrices, biases tensors, scratch and out */
+    int32_t path;      /* KUTACC_HIP_PATH_* */
+
+    const void *input;    /* [B*S, C], row stride input_ld                                   */
+    int64_t input_ld;
+    const void *query_w;  /* [C, C] stored [out, in], row stride C                           */
+    const void *key_w;
+    const void *value_w;
+    const void *gating_w;
+    const void *output_w;
+    const float *gating_b; /* fp32 [C]                                                       */
+    const float *output_b; /* fp32 [C]                                                       */
+
+    const void *bias;      /* mask bias, element (b,k) at bias[b*bias_stride_b + k]          */
+    int64_t bias_stride_b;
+    const void *nonbatched_bias; /* pair bias, element (h,q,k) at h*nb_stride_h + q*nb_stride_q + k; NULL = absent */
+    int64_t nb_stride_h;
+    int64_t nb_stride_q;
+
+    /* Caller scratch.  q/k/v/gate are written only by the generic path; avg (gated weighted
+     * average, [B,S,H,d]) is written by every path.  Element (b,s,h,e) of q,k,gate,avg lives at
+     * b*stride_b + s*stride_s + h*stride_h + e; v is [H,d,B,S]: (h,e,b,s) at
+     * h*v_stride_h + e*v_stride_e + b*v_stride_b + s. */
+    void *q, *k, *v, *gate, *avg;
+    int64_t q_stride_b, q_stride_s, q_stride_h;
+    int64_t k_stride_b, k_stride_s, k_stride_h;
+    int64_t gate_stride_b, gate_stride_s, gate_stride_h;
+    int64_t avg_stride_b, avg_stride_s, avg_stride_h;
+    int64_t v_stride_h, v_stride_e, v_stride_b;
+
+    void *out;          /* [B*S, C], row stride out_ld                                       */
+    int64_t out_ld;
+} kutacc_hip_attention_args_t;
+
+/* Enqueue the whole operator on `stream`.  Replaces kutacc::gating_attention_kernel
+ * (reference src/attention/gating_attention.cpp:33-158). */
+kutacc_export int kutacc_hip_gating_attention(const kutacc_hip_attention_args_t *args, void *stream);
+
+/* Name of the kernel family the last successful kutacc_hip_gating_attention call used on this
+ * thread: "fused_mfma" or "generic".  Static storage. */
+kutacc_export const char *kutacc_hip_last_path(void);
+
+/*
+ * LayerNorm over the last axis of `rows` rows (row r at x + r*ld_x, out + r*ld_out), fp32 gamma and
+ * beta of length `size`.  Batched form of kutacc_af2_layernorm (reference
+ * src/normalization/layernorm_kernel.h:21-53), which handles exactly one row per call.
+ */
+kutacc_export int kutacc_hip_layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta,
+                                            void *out, int64_t ld_out, int64_t rows, int64_t size, float eps,
+                                            int32_t dtype, void *stream);
+
+/*
+ * result[m,n] = beta*result[m,n] + sum_k act[m,k]*weight[n,k] (+ bias[n]); act row stride ld_act,
+ * weight row stride ld_w, result dense [m,n].  Replaces kutacc::linear_kernel
+ * (reference src/linear/linear.cpp:21-42).  bias may be NULL.
+ */
+kutacc_export int kutacc_hip_linear(const void *act, int64_t ld_act, const void *weight, int64_t ld_w,
+                                    const float *bias, void *result, int64_t m, int64_t n, int64_t k, float beta,
+                                    int32_t dtype, void *stream);
+
+/*
+ * Pair-bias producer: nb[h,i,j] = sum_c LN(z[i,j,:])[c] * w[h,c], written directly in the [H,S,S]
+ * layout kutacc_af2_gating_attention expects.  One pass over z ([rows_i, rows_j, c_z], dense).
+ * Fuses what a caller of the reference does with kutacc_af2_layernorm per row
+ * (reference src/normalization/layernorm.cpp:17-20), kutacc_af2_linear
+ * (reference src/linear/linear.cpp:45-50) and a [S,S,H]->[H,S,S] permute.  gamma/beta fp32 [c_z];
+ * w is [H, c_z] in `dtype`.  If `z_norm` is non-NULL the normalised rows are also written there
+ * (dense, same shape as z) so the attention input comes out of the same pass.
+ */
+kutacc_export int kutacc_hip_pair_bias(const void *z, const float *gamma, const float *beta, const void *w,
+                                       void *nb, void *z_norm, int64_t rows_i, int64_t rows_j, int64_t c_z,
+                                       int64_t nheads, float eps, int32_t dtype, void *stream);
+
+/* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
+
+/* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.
+ * Default: the HIP null stream. */
+kutacc_export void kutacc_hip_set_stream(void *stream);
+kutacc_export void *kutacc_hip_get_stream(void);
+
+/* 1 (default): the handle-based API blocks until the device work has finished, as the CPU library
+ * does.  0: it returns after enqueueing when all operands are device pointers. */
+kutacc_export void kutacc_hip_set_blocking(int blocking);
+
+/* Per-kernel timing for benchmarks.  While enabled, each kernel launched by this library is
+ * bracketed by hipEvents on its stream.  kutacc_hip_profile_read(i, ...) waits for the recorded
+ * events and returns entry i (0 on success, -1 past the last entry): kernel name, summed
+ * milliseconds, number of launches and the algorithmic flops of one launch.  Enabling clears the
+ * previous totals. */
+kutacc_export void kutacc_hip_profile_enable(int on);
+kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, double *total_ms, int64_t *launches,
+                                          double *flops_per_launch);
+
+/* The process-wide sticky error flag behind KUTACC_CHECK (reference src/utils/check.cpp:16 keeps it
+ * hidden and never resets it).  Reading/clearing it is an addition for tests and long-lived hosts. */
+kutacc_export int kutacc_hip_error_flag(void);
+kutacc_export void kutacc_hip_clear_error(void);
+
+/* Tensor descriptors for callers that cannot run the C++ TensorWrapper constructor
+ * (reference include/kutacc.h:484-497).  The returned handle is what get_tensor() returns. */
+kutacc_export void *kutacc_hip_tensor_create(void *data, const int64_t *sizes, const int64_t *strides, int64_t dim,
+                                             int32_t dtype);
+kutacc_export void kutacc_hip_tensor_destroy(void *handle);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KUTACC_HIP_H */

@@ -1,0 +1,236 @@
+"""ctypes binding of libkutacc.so: the handle-based operator API of include/kutacc.h and the
+pointer-level launch layer of include/kutacc_hip.h.
+
+The Python functions keep the C names and argument order (reference include/kutacc.h:297-300, :334,
+:399-400, :407-408, :418, :47) so that tests read like calls into the C library.  torch is used only
+to own device memory and streams; nothing here computes.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libkutacc.so")
+
+KUTACC_OK = 0
+KUTACC_ERROR = -1
+K_INT64, K_BF16, K_FP32 = 0, 1, 2
+PATH_AUTO, PATH_GENERIC, PATH_FUSED = 0, 1, 2
+EINVAL, EUNSUPPORTED = -2, -3
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_i32 = ctypes.c_int32
+_f32p = ctypes.POINTER(ctypes.c_float)
+
+
+class Version(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_char_p) for n in ("product_name", "product_version", "component_name",
+                                                "component_version", "component_abi_version",
+                                                "component_appendinfo")]
+
+
+class AttentionWeights(ctypes.Structure):
+    """kutacc_af2_attention_weights_t"""
+    _fields_ = [("nchannels", _i64), ("nheads", _i64), ("head_size", _i64), ("query_w", _vp), ("key_w", _vp),
+                ("value_w", _vp), ("gating_w", _vp), ("gating_b", _vp), ("output_w", _vp), ("output_b", _vp)]
+
+
+class AttentionInputs(ctypes.Structure):
+    """kutacc_af2_attention_inputs_t"""
+    _fields_ = [("batch", _i64), ("seq_len", _i64), ("q", _vp), ("k", _vp), ("v", _vp), ("gate", _vp), ("avg", _vp)]
+
+
+class HipAttentionArgs(ctypes.Structure):
+    """kutacc_hip_attention_args_t"""
+    _fields_ = [
+        ("batch", _i64), ("seq_len", _i64), ("nheads", _i64), ("head_size", _i64), ("dtype", _i32), ("path", _i32),
+        ("input", _vp), ("input_ld", _i64),
+        ("query_w", _vp), ("key_w", _vp), ("value_w", _vp), ("gating_w", _vp), ("output_w", _vp),
+        ("gating_b", _vp), ("output_b", _vp),
+        ("bias", _vp), ("bias_stride_b", _i64),
+        ("nonbatched_bias", _vp), ("nb_stride_h", _i64), ("nb_stride_q", _i64),
+        ("q", _vp), ("k", _vp), ("v", _vp), ("gate", _vp), ("avg", _vp),
+        ("q_stride_b", _i64), ("q_stride_s", _i64), ("q_stride_h", _i64),
+        ("k_stride_b", _i64), ("k_stride_s", _i64), ("k_stride_h", _i64),
+        ("gate_stride_b", _i64), ("gate_stride_s", _i64), ("gate_stride_h", _i64),
+        ("avg_stride_b", _i64), ("avg_stride_s", _i64), ("avg_stride_h", _i64),
+        ("v_stride_h", _i64), ("v_stride_e", _i64), ("v_stride_b", _i64),
+        ("out", _vp), ("out_ld", _i64),
+    ]
+
+
+# every symbol the two public headers declare; tests check that the library exports all of them
+DECLARED_SYMBOLS = [
+    "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_layernorm", "kutacc_af2_linear",
+    "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
+    "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
+    "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
+    "kutacc_hip_gating_attention", "kutacc_hip_last_path", "kutacc_hip_layernorm_rows", "kutacc_hip_linear",
+    "kutacc_hip_pair_bias", "kutacc_hip_set_stream", "kutacc_hip_get_stream", "kutacc_hip_set_blocking",
+    "kutacc_hip_error_flag", "kutacc_hip_clear_error", "kutacc_hip_tensor_create", "kutacc_hip_tensor_destroy",
+    "kutacc_hip_profile_enable", "kutacc_hip_profile_read",
+]
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the built library.  There is no fallback: a missing library is an error."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m kutacc_amd.build` "
+                           "(the HIP library is the only implementation; there is no CPU path)")
+    L = ctypes.CDLL(LIB_PATH)
+    L.kutacc_get_version.argtypes = [ctypes.POINTER(Version)]
+    L.kutacc_get_version.restype = ctypes.c_int
+    L.kutacc_af2_gating_attention.argtypes = [_vp, ctypes.POINTER(AttentionInputs), _vp, _vp,
+                                              ctypes.POINTER(AttentionWeights), _vp, _i64]
+    L.kutacc_af2_gating_attention.restype = None
+    L.kutacc_af2_layernorm.argtypes = [_vp, _vp, _vp, _i64, ctypes.c_float, _vp]
+    L.kutacc_af2_layernorm.restype = None
+    L.kutacc_af2_linear.argtypes = [_vp, _vp, _vp, _vp, _i64]
+    L.kutacc_af2_linear.restype = None
+    L.kutacc_af2_linear_weight_prepack.argtypes = [_vp, _vp, _i64, _i64, _i64, _i64]
+    L.kutacc_af2_linear_weight_prepack.restype = None
+    L.kutacc_af2_gemm_pack_get_size.argtypes = [ctypes.c_char, ctypes.c_char, ctypes.c_char, ctypes.c_int,
+                                                ctypes.c_int, ctypes.c_int]
+    L.kutacc_af2_gemm_pack_get_size.restype = ctypes.c_size_t
+    L.kutacc_hip_gating_attention.argtypes = [ctypes.POINTER(HipAttentionArgs), _vp]
+    L.kutacc_hip_gating_attention.restype = ctypes.c_int
+    L.kutacc_hip_last_path.restype = ctypes.c_char_p
+    L.kutacc_hip_layernorm_rows.argtypes = [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_float, _i32, _vp]
+    L.kutacc_hip_layernorm_rows.restype = ctypes.c_int
+    L.kutacc_hip_linear.argtypes = [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _i64, _i64, ctypes.c_float, _i32, _vp]
+    L.kutacc_hip_linear.restype = ctypes.c_int
+    L.kutacc_hip_pair_bias.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _i32, _vp]
+    L.kutacc_hip_pair_bias.restype = ctypes.c_int
+    L.kutacc_hip_set_stream.argtypes = [_vp]
+    L.kutacc_hip_get_stream.restype = _vp
+    L.kutacc_hip_set_blocking.argtypes = [ctypes.c_int]
+    L.kutacc_hip_error_flag.restype = ctypes.c_int
+    L.kutacc_hip_tensor_create.argtypes = [_vp, ctypes.POINTER(_i64), ctypes.POINTER(_i64), _i64, _i32]
+    L.kutacc_hip_tensor_create.restype = _vp
+    L.kutacc_hip_tensor_destroy.argtypes = [_vp]
+    L.kutacc_hip_profile_enable.argtypes = [ctypes.c_int]
+    L.kutacc_hip_profile_read.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                          ctypes.POINTER(_i64), ctypes.POINTER(ctypes.c_double)]
+    L.kutacc_hip_profile_read.restype = ctypes.c_int
+    _lib = L
+    return L
+
+
+def get_version() -> dict:
+    v = Version()
+    rc = lib().kutacc_get_version(ctypes.byref(v))
+    assert rc == KUTACC_OK
+    return {n: getattr(v, n).decode() for n, _ in Version._fields_}
+
+
+def error_flag() -> bool:
+    return bool(lib().kutacc_hip_error_flag())
+
+
+def clear_error() -> None:
+    lib().kutacc_hip_clear_error()
+
+
+def last_path() -> str:
+    return lib().kutacc_hip_last_path().decode()
+
+
+def set_stream(stream_ptr: int | None) -> None:
+    lib().kutacc_hip_set_stream(_vp(stream_ptr or 0))
+
+
+def set_blocking(blocking: bool) -> None:
+    lib().kutacc_hip_set_blocking(1 if blocking else 0)
+
+
+class TensorHandle:
+    """Owns one kutacc_tensor_h (the C++ side's TensorWrapper) and keeps the backing array alive."""
+
+    def __init__(self, data_ptr: int, sizes, strides, dtype: int, keepalive=None):
+        self.sizes = [int(s) for s in sizes]
+        self.strides = [int(s) for s in strides]
+        n = len(self.sizes)
+        arr = _i64 * max(n, 1)
+        self._h = lib().kutacc_hip_tensor_create(_vp(data_ptr), arr(*self.sizes), arr(*self.strides), n, dtype)
+        self._keep = keepalive
+        self.dtype = dtype
+
+    @property
+    def handle(self) -> int:
+        return self._h
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h and _lib is not None:
+            _lib.kutacc_hip_tensor_destroy(_vp(h))
+
+
+def _torch_dtype_code(t) -> int:
+    import torch
+    if t.dtype == torch.bfloat16:
+        return K_BF16
+    if t.dtype == torch.float32:
+        return K_FP32
+    if t.dtype == torch.int64:
+        return K_INT64
+    raise TypeError(f"unsupported tensor dtype {t.dtype}")
+
+
+def tensor(t, dtype: int | None = None) -> TensorHandle:
+    """Handle for a torch tensor (device or host memory) or a numpy array (host memory).
+    numpy uint16 arrays are taken as bf16 bit patterns."""
+    if isinstance(t, np.ndarray):
+        code = dtype if dtype is not None else {np.dtype(np.uint16): K_BF16, np.dtype(np.float32): K_FP32,
+                                                 np.dtype(np.int64): K_INT64}[t.dtype]
+        return TensorHandle(t.ctypes.data, t.shape, [s // t.itemsize for s in t.strides], code, keepalive=t)
+    code = dtype if dtype is not None else _torch_dtype_code(t)
+    return TensorHandle(t.data_ptr(), list(t.shape), list(t.stride()), code, keepalive=t)
+
+
+def empty_tensor(dtype: int = K_BF16) -> TensorHandle:
+    """A rank-1 tensor with sizes[0] == 0: how a caller says "no nonbatched_bias"
+    (reference src/attention/gating_attention.cpp:103)."""
+    return TensorHandle(0, [0], [1], dtype)
+
+
+def kutacc_af2_gating_attention(input, q_based: AttentionInputs, bias, nonbatched_bias, weights: AttentionWeights, out,
+                                block_size: int) -> None:
+    """Arguments as in the C API; tensor arguments are TensorHandle objects (or None for a null handle)."""
+    h = lambda t: _vp(t.handle) if t is not None else None  # noqa: E731
+    lib().kutacc_af2_gating_attention(h(input), ctypes.byref(q_based) if q_based is not None else None, h(bias),
+                                      h(nonbatched_bias), ctypes.byref(weights) if weights is not None else None,
+                                      h(out), block_size)
+
+
+class GatedAttention:
+    """Convenience owner of everything one kutacc_af2_gating_attention call needs, for tensors that
+    already live where the call should run (torch tensors on the GPU, or numpy arrays on the host).
+    Builds the handles once; `run()` is exactly one C call."""
+
+    def __init__(self, x, wq, wk, wv, wg, bg, wo, bo, bias, nb, nheads, out, scratch, block_size=64):
+        B, S, C = x.shape
+        self.keep = dict(x=x, wq=wq, wk=wk, wv=wv, wg=wg, bg=bg, wo=wo, bo=bo, bias=bias, nb=nb, out=out, **scratch)
+        dt = tensor(x).dtype
+        self.h = {k: tensor(v) for k, v in self.keep.items() if v is not None and k not in ("bg", "bo")}
+        self.h["bg"] = tensor(bg, K_FP32)
+        self.h["bo"] = tensor(bo, K_FP32)
+        self.h_nb = self.h["nb"] if nb is not None else empty_tensor(dt)
+        self.weights = AttentionWeights(C, nheads, C // nheads, self.h["wq"].handle, self.h["wk"].handle,
+                                        self.h["wv"].handle, self.h["wg"].handle, self.h["bg"].handle,
+                                        self.h["wo"].handle, self.h["bo"].handle)
+        self.inputs = AttentionInputs(B, S, self.h["q"].handle, self.h["k"].handle, self.h["v"].handle,
+                                      self.h["gate"].handle, self.h["avg"].handle)
+        self.block_size = block_size
+
+    def run(self) -> None:
+        kutacc_af2_gating_attention(self.h["x"], self.inputs, self.h["bias"], self.h_nb, self.weights, self.h["out"],
+                                    self.block_size)

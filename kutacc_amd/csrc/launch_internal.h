@@ -1,0 +1,30 @@
+// C++-side declarations of the per-translation-unit launchers behind the extern "C" layer of
+// kutacc_hip.h.  Each returns the same int convention as that layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kutacc_hip.h"
+
+// Turn a HIP status into the int the C ABI returns (0 = success, else the hipError_t value).
+static inline int kutacc_hip_status(hipError_t e) { return e == hipSuccess ? 0 : (int)e; }
+
+namespace kutacc_launch {
+
+// generic_kernels.hip
+int gating_attention_generic(const kutacc_hip_attention_args_t &args, hipStream_t stream);
+int gemm_nt(int32_t dtype, const void *a, int64_t lda, const void *w, int64_t ldw, const float *bias, void *c,
+            int64_t c_rs, int64_t c_cs, int64_t m, int64_t n, int64_t k, float beta, hipStream_t stream);
+
+// fused_attention.hip
+bool fused_attention_supports(const kutacc_hip_attention_args_t &args);
+int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream);
+
+// row_kernels.hip
+int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
+                   int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream);
+int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
+              int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype,
+              hipStream_t stream);
+
+} // namespace kutacc_launch

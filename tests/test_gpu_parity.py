@@ -1,0 +1,328 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI, on a real MI355X.
+
+Every test calls libkutacc.so (handle-based kutacc_af2_* entry points, or the pointer-level
+kutacc_hip_* layer where a kernel family is forced) on device memory and compares with
+oracle/ on the same seeded inputs.  Full-size configurations are run at their real shape on the
+GPU; the oracle evaluates a subset of batch rows (rows are independent in this operator), chosen to
+include masked rows where the configuration has them.
+
+Tolerances (stated by the task): fp32 storage within 1e-4 relative of the fp32 oracle; bf16 storage
+within 2e-2 absolute + 1e-2 relative of the fp32 oracle.
+"""
+import functools
+
+import numpy as np
+import pytest
+
+from kutacc_amd import capi
+from kutacc_amd.workloads import CONFIGS, Workload, bf16_bits, make_workload, round_to_bf16
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    capi.set_stream(None)
+    capi.set_blocking(True)
+    return torch
+
+
+@functools.lru_cache(maxsize=2)
+def full_workload(config: int) -> Workload:
+    """Full-size inputs are expensive to draw (config 5: 134M normals); tests must not modify them."""
+    return make_workload(config)
+
+
+def oracle_rows(w: Workload, rows):
+    sub = w.batch_slice(rows)
+    return helpers.oracle_out(sub, return_avg=True)
+
+
+def pick_rows(w: Workload, n=4):
+    rows = list(np.linspace(0, w.B - 1, n).astype(int))
+    if w.config == 5:
+        pad = w.extras.get("pad", 0)
+        if pad:
+            rows[-1] = w.B - 1  # fully masked row
+            rows[-2] = w.B - pad  # first fully masked row
+            rows[1] = w.B - pad - 1  # last row that still sees unmasked keys
+    return sorted(set(int(r) for r in rows))
+
+
+# ---- the five configurations, full shape, default kernel selection -------------------------------------
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+def test_config_full_shape_matches_oracle(torch_cuda, config):
+    w = full_workload(config)
+    print(f"config {config}: B={w.B} S={w.S} H={w.H} dtype={w.dtype}", flush=True)
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    assert not capi.error_flag()
+    if w.dtype == "bf16":
+        assert capi.last_path() == "fused_mfma", "bf16 benchmark shapes must run on the MFMA kernels"
+    rows = pick_rows(w)
+    ref_out, ref_avg = oracle_rows(w, rows)
+    out = helpers.to_numpy(ten["out"][rows])
+    avg = helpers.to_numpy(scratch["avg"][rows]).reshape(len(rows), w.S, w.C)
+    e_avg = helpers.check_close(avg, ref_avg, w.dtype, f"config {config} gated average")
+    e_out = helpers.check_close(out, ref_out, w.dtype, f"config {config} out")
+    print(f"config {config}: path={capi.last_path()} max|err| avg={e_avg:.3g} out={e_out:.3g}", flush=True)
+
+
+# ---- both kernel families on reduced shapes, every row checked ---------------------------------------------
+SMALL = [
+    # config, batch, seq_len
+    (1, 3, 64), (2, 4, 256), (3, 5, 384), (4, 3, 1024), (5, 3, 1024),
+    (2, 3, 70), (3, 2, 33), (2, 2, 1), (3, 2, 200), (4, 2, 97),
+]
+
+
+@pytest.mark.parametrize("config,batch,seq", SMALL)
+@pytest.mark.parametrize("path", [capi.PATH_GENERIC, capi.PATH_FUSED])
+def test_reduced_shapes_both_kernel_families(torch_cuda, config, batch, seq, path):
+    if path == capi.PATH_FUSED and CONFIGS[config]["dtype"] != "bf16":
+        pytest.skip("the MFMA kernels take bf16 storage only; fp32 runs on the generic kernels")
+    w = make_workload(config, batch=batch, seq_len=seq)
+    if config == 5:
+        w.bias[-1, :] = round_to_bf16(np.full(seq, -1e9, dtype=np.float32))  # a fully masked row
+    print(f"config {config} B={batch} S={seq} path={path}", flush=True)
+    ten, scratch = helpers.to_device(w)
+    rc = helpers.run_hip(w, ten, scratch, path)
+    assert rc == 0, rc
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, "gated average")
+    helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
+
+
+def test_fp32_storage_meets_fp32_tolerance(torch_cuda):
+    w = make_workload(1)
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    assert not capi.error_flag() and capi.last_path() == "generic"
+    ref = helpers.oracle_out(w)
+    got = helpers.to_numpy(ten["out"])
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+# ---- properties that hold at any size -----------------------------------------------------------------------
+def test_result_independent_of_block_size(torch_cuda):
+    """The reference computes full-row softmax whatever the query tiling (gating_attention.cpp:102-121)."""
+    w = make_workload(3, batch=6)
+    outs = []
+    for bs in (1, 64, 384, 1000):
+        op, ten, scratch = helpers.make_op(w, block_size=bs)
+        op.run()
+        assert not capi.error_flag()
+        outs.append(ten["out"].clone())
+    for o in outs[1:]:
+        assert torch_cuda.equal(o, outs[0])
+
+
+def test_batch_permutation_permutes_output(torch_cuda):
+    w = make_workload(2, batch=16)
+    op, ten, _ = helpers.make_op(w)
+    op.run()
+    perm = np.random.Generator(np.random.PCG64(9)).permutation(w.B)
+    w2 = w.batch_slice(perm)
+    op2, ten2, _ = helpers.make_op(w2)
+    op2.run()
+    assert torch_cuda.equal(ten2["out"], ten["out"][torch_cuda.from_numpy(perm).cuda()])
+
+
+def test_fully_masked_rows_average_values_uniformly_full_size(torch_cuda):
+    """Config 5 at full size: every query of a fully masked batch row gets the plain mean of V (times
+    its gate), because the -1e9 mask bias absorbs the logits in fp32."""
+    w = full_workload(5)
+    pad = w.extras["pad"]
+    assert pad > 0
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    assert not capi.error_flag()
+    rows = [w.B - pad, w.B - 1]
+    x = w.x[rows].astype(np.float64)
+    v = x @ w.wv.astype(np.float64).T
+    gate = 1 / (1 + np.exp(-(x @ w.wg.astype(np.float64).T + w.bg)))
+    expect = v.mean(axis=1, keepdims=True) * gate
+    got = helpers.to_numpy(scratch["avg"][rows]).reshape(2, w.S, w.C)
+    helpers.check_close(got, expect, "bf16", "uniform average of fully masked rows")
+
+
+def test_masked_keys_do_not_leak(torch_cuda):
+    """Changing the token behind a masked key must not change any other row, bit for bit."""
+    w = make_workload(2, batch=4)
+    masked = np.flatnonzero(w.bias[0] != 0)
+    assert masked.size > 0
+    op, ten, _ = helpers.make_op(w)
+    op.run()
+    w2 = w.batch_slice(np.arange(w.B))
+    w2.x[:, masked] = round_to_bf16(np.float32(3.0) * w2.x[:, masked] + np.float32(1.0))
+    op2, ten2, _ = helpers.make_op(w2)
+    op2.run()
+    keep = torch_cuda.from_numpy(np.flatnonzero(w.bias[0] == 0)).cuda()
+    assert torch_cuda.equal(ten["out"][:, keep], ten2["out"][:, keep])
+
+
+def test_absent_pair_bias_equals_zero_pair_bias(torch_cuda):
+    w = make_workload(4, batch=3, seq_len=256)
+    op, ten, _ = helpers.make_op(w)
+    op.run()
+    w2 = w.batch_slice(np.arange(w.B))
+    w2.nb = np.zeros((w.H, w.S, w.S), dtype=np.float32)
+    op2, ten2, _ = helpers.make_op(w2)
+    op2.run()
+    assert not capi.error_flag()
+    assert torch_cuda.equal(ten["out"], ten2["out"])
+
+
+# ---- boundary behaviour ------------------------------------------------------------------------------------
+def test_host_pointers_are_staged_and_match_device_pointers(torch_cuda):
+    w = make_workload(3, batch=3, seq_len=96)
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    hten, hscratch = helpers.host_arrays(w)
+    hop = capi.GatedAttention(hten["x"], hten["wq"], hten["wk"], hten["wv"], hten["wg"], hten["bg"], hten["wo"],
+                              hten["bo"], hten["bias"], hten["nb"], w.H, hten["out"], hscratch)
+    hop.run()
+    assert not capi.error_flag()
+    dev_bits = ten["out"].view(torch_cuda.int16).cpu().numpy().view(np.uint16)
+    np.testing.assert_array_equal(hten["out"], dev_bits)
+    avg_bits = scratch["avg"].view(torch_cuda.int16).cpu().numpy().view(np.uint16)
+    np.testing.assert_array_equal(hscratch["avg"], avg_bits)
+
+
+def test_mixed_host_and_device_pointers_are_rejected(torch_cuda):
+    w = make_workload(3, batch=2, seq_len=64)
+    ten, scratch = helpers.to_device(w)
+    ten["wq"] = ten["wq"].cpu()
+    op = capi.GatedAttention(ten["x"], ten["wq"], ten["wk"], ten["wv"], ten["wg"], ten["bg"], ten["wo"], ten["bo"],
+                             ten["bias"], ten["nb"], w.H, ten["out"], scratch)
+    op.run()
+    assert capi.error_flag()
+    assert not ten["out"].any()
+
+
+def test_error_flag_makes_later_gpu_calls_noops(torch_cuda):
+    w = make_workload(3, batch=2, seq_len=64)
+    op, ten, _ = helpers.make_op(w)
+    capi.lib().kutacc_af2_gating_attention(None, None, None, None, None, None, 1)
+    assert capi.error_flag()
+    op.run()
+    assert not ten["out"].any(), "latched error: the call must not touch out"
+    capi.clear_error()
+    op.run()
+    assert ten["out"].any()
+
+
+def test_non_blocking_mode_on_caller_stream(torch_cuda):
+    torch = torch_cuda
+    w = make_workload(3, batch=4, seq_len=128)
+    op, ten, _ = helpers.make_op(w)
+    op.run()
+    ref = ten["out"].clone()
+    ten["out"].zero_()
+    s = torch.cuda.Stream()
+    try:
+        capi.set_stream(s.cuda_stream)
+        capi.set_blocking(False)
+        with torch.cuda.stream(s):
+            op.run()
+        s.synchronize()
+    finally:
+        capi.set_stream(None)
+        capi.set_blocking(True)
+    assert torch.equal(ten["out"], ref)
+
+
+# ---- row operators in front of the path ----------------------------------------------------------------------
+@pytest.mark.parametrize("size", [128, 256, 100])
+def test_layernorm_rows_match_oracle(torch_cuda, size):
+    from oracle import oracle
+    torch = torch_cuda
+    rng = np.random.Generator(np.random.PCG64(41))
+    x = round_to_bf16(rng.standard_normal((300, size)).astype(np.float32) * 2 + 0.5)
+    gamma = rng.standard_normal(size).astype(np.float32)
+    beta = rng.standard_normal(size).astype(np.float32)
+    dx = torch.from_numpy(x).cuda().bfloat16()
+    dg, db = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    dout = torch.zeros_like(dx)
+    rc = capi.lib().kutacc_hip_layernorm_rows(dx.data_ptr(), size, dg.data_ptr(), db.data_ptr(), dout.data_ptr(), size,
+                                              300, size, 1e-5, capi.K_BF16, None)
+    torch.cuda.synchronize()
+    assert rc == 0
+    ref = oracle.from_bf16_bits(oracle.layernorm_rows_bf16(bf16_bits(x), gamma, beta, 1e-5))
+    got = helpers.to_numpy(dout)
+    # same formula, different summation order: at most one bf16 ulp apart
+    assert np.all(np.abs(got - ref) <= 2.0 ** -7 * np.abs(ref) + 1e-6)
+    assert np.mean(got == ref) > 0.98
+    # the single-row entry point of kutacc.h on device pointers
+    one = torch.zeros(size, device="cuda", dtype=torch.bfloat16)
+    capi.lib().kutacc_af2_layernorm(dx[7].data_ptr(), dg.data_ptr(), db.data_ptr(), size, 1e-5, one.data_ptr())
+    assert not capi.error_flag()
+    assert torch.equal(one, dout[7])
+    # ... and on host pointers (staged)
+    hx = bf16_bits(x[7])
+    hout = np.zeros(size, dtype=np.uint16)
+    capi.lib().kutacc_af2_layernorm(hx.ctypes.data, gamma.ctypes.data, beta.ctypes.data, size, 1e-5, hout.ctypes.data)
+    assert not capi.error_flag()
+    np.testing.assert_array_equal(hout, dout[7].view(torch.int16).cpu().numpy().view(np.uint16))
+
+
+def test_linear_matches_oracle(torch_cuda):
+    from oracle import oracle
+    torch = torch_cuda
+    rng = np.random.Generator(np.random.PCG64(42))
+    act = round_to_bf16(rng.standard_normal((5, 40, 128)).astype(np.float32))
+    wgt = round_to_bf16(rng.standard_normal((4, 128)).astype(np.float32) / 11)
+    bias = rng.standard_normal(4).astype(np.float32)
+    da, dw = torch.from_numpy(act).cuda().bfloat16(), torch.from_numpy(wgt).cuda().bfloat16()
+    dbias = torch.from_numpy(bias).cuda()
+    res = torch.zeros((200, 4), device="cuda", dtype=torch.bfloat16)
+    capi.lib().kutacc_af2_linear(capi.tensor(da).handle, capi.tensor(dw).handle, dbias.data_ptr(),
+                                 capi.tensor(res).handle, 0)
+    assert not capi.error_flag()
+    ref = oracle.from_bf16_bits(oracle.linear_bf16(bf16_bits(act), bf16_bits(wgt), bias))
+    got = helpers.to_numpy(res)
+    assert np.all(np.abs(got - ref) <= 2.0 ** -7 * np.abs(ref) + 1e-6)
+    # beta = 1 accumulates onto the previous result, no bias
+    capi.lib().kutacc_af2_linear(capi.tensor(da).handle, capi.tensor(dw).handle, None, capi.tensor(res).handle, 1)
+    ref2 = oracle.from_bf16_bits(oracle.linear_bf16(bf16_bits(act), bf16_bits(wgt), None, beta=1.0,
+                                                    result_bits=bf16_bits(got)))
+    assert np.all(np.abs(helpers.to_numpy(res) - ref2) <= 2.0 ** -7 * np.abs(ref2) + 1e-6)
+
+
+@pytest.mark.parametrize("config", [1, 3])
+def test_pair_bias_producer_matches_oracle(torch_cuda, config):
+    """LN(z) -> [H, c_z] linear -> [H, S, S], one pass; against oracle LayerNorm + Linear + permute."""
+    from oracle import oracle
+    torch = torch_cuda
+    w = make_workload(config, batch=2, keep_extras=True)
+    z, wb = w.extras["z"], w.extras["w_bias"]
+    S, cz, H = w.S, z.shape[-1], w.H
+    gamma = np.ones(cz, dtype=np.float32)
+    beta = np.zeros(cz, dtype=np.float32)
+    dt = torch.bfloat16 if w.dtype == "bf16" else torch.float32
+    code = capi.K_BF16 if w.dtype == "bf16" else capi.K_FP32
+    dz = torch.from_numpy(z).cuda().to(dt)
+    dw = torch.from_numpy(wb).cuda().to(dt)
+    dg, db = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    nb = torch.zeros((H, S, S), device="cuda", dtype=dt)
+    zn = torch.zeros_like(dz)
+    rc = capi.lib().kutacc_hip_pair_bias(dz.data_ptr(), dg.data_ptr(), db.data_ptr(), dw.data_ptr(), nb.data_ptr(),
+                                         zn.data_ptr(), S, S, cz, H, 1e-5, code, None)
+    torch.cuda.synchronize()
+    assert rc == 0
+    if w.dtype == "bf16":
+        zn_ref_bits = oracle.layernorm_rows_bf16(bf16_bits(z), gamma, beta, 1e-5)
+        nb_ref = oracle.from_bf16_bits(oracle.linear_bf16(zn_ref_bits.reshape(S * S, cz), bf16_bits(wb)))
+        zn_ref = oracle.from_bf16_bits(zn_ref_bits)
+        tol = lambda r: 2.0 ** -7 * np.abs(r) + 2e-3  # noqa: E731
+    else:
+        zn_ref = oracle.layernorm_rows_f32(z, gamma, beta, 1e-5)
+        nb_ref = oracle.linear_f32(zn_ref.reshape(S * S, cz), wb)
+        tol = lambda r: 1e-4 * np.abs(r) + 1e-5  # noqa: E731
+    nb_ref = nb_ref.reshape(S, S, H).transpose(2, 0, 1)
+    assert np.all(np.abs(helpers.to_numpy(zn) - zn_ref) <= tol(zn_ref))
+    assert np.all(np.abs(helpers.to_numpy(nb) - nb_ref) <= tol(nb_ref))

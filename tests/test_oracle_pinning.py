@@ -1,0 +1,331 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+The reference ships no numeric test, golden vector or fixture for the gated-attention operator (its
+tests only check that invalid arguments do not crash), and it cannot be built on this machine.  The
+oracle is therefore pinned by: library routines (torch matmul / scaled_dot_product_attention /
+layer_norm / linear), a pure-Python brute force on a tiny case, closed forms and invariants chosen so
+that a dropped term, a wrong index or a transposed operand fails at least one of them, and the
+committed float64 fixture.
+"""
+import itertools
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def make_case(seed, B, S, H, d, nb=True, bias_mode="zeros"):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    C = H * d
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
+    case = dict(x=f(B, S, C), wq=f(C, C) / math.sqrt(C), wk=f(C, C) / math.sqrt(C), wv=f(C, C) / math.sqrt(C),
+                wg=f(C, C) / math.sqrt(C), bg=f(C), wo=f(C, C) / math.sqrt(C), bo=f(C),
+                bias=np.zeros((B, S), dtype=np.float32), nb=f(H, S, S) if nb else None, nheads=H)
+    if bias_mode == "random_mask":
+        keep = rng.random((B, S)) > 0.3
+        keep[:, 0] = True
+        case["bias"] = (-1e9 * (1 - keep)).astype(np.float32)
+    return case
+
+
+def run_f32(case, **kw):
+    return oracle.gating_attention_f32(case["x"], case["wq"], case["wk"], case["wv"], case["wg"], case["bg"],
+                                       case["wo"], case["bo"], case["bias"], case["nb"], case["nheads"], **kw)
+
+
+def run_f64(case, **kw):
+    return oracle.gating_attention_f64_numpy(case["x"], case["wq"], case["wk"], case["wv"], case["wg"], case["bg"],
+                                             case["wo"], case["bo"], case["bias"], case["nb"], case["nheads"], **kw)
+
+
+# ---- library routines --------------------------------------------------------------------------------
+@pytest.mark.parametrize("nb,bias_mode", [(True, "zeros"), (False, "zeros"), (True, "random_mask")])
+def test_numpy_twin_matches_torch_sdpa(nb, bias_mode):
+    c = make_case(1, 3, 17, 2, 8, nb=nb, bias_mode=bias_mode)
+    B, S, C = c["x"].shape
+    H = c["nheads"]
+    d = C // H
+    t = lambda a: torch.from_numpy(np.asarray(a, dtype=np.float64))  # noqa: E731
+    x = t(c["x"])
+    q = (x @ t(c["wq"]).T).reshape(B, S, H, d).transpose(1, 2)
+    k = (x @ t(c["wk"]).T).reshape(B, S, H, d).transpose(1, 2)
+    v = (x @ t(c["wv"]).T).reshape(B, S, H, d).transpose(1, 2)
+    g = torch.sigmoid(x @ t(c["wg"]).T + t(c["bg"]))
+    # mask values are moderate here (-1e9 in float64 does not absorb; that case is tested separately)
+    mask = t(c["bias"])[:, None, None, :].expand(B, H, S, S).clone()
+    if nb:
+        mask = mask + t(c["nb"])[None]
+    o = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, scale=1.0 / math.sqrt(d))
+    o = o.transpose(1, 2).reshape(B, S, C) * g
+    ref = (o @ t(c["wo"]).T + t(c["bo"])).numpy()
+    got = run_f64(c)
+    if bias_mode == "random_mask":
+        # with -1e9 the fp32 bias add of the operator rounds the logit away; torch float64 keeps it.
+        # masked keys get weight 0 either way and rows always keep key 0, so results agree closely
+        np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
+    else:
+        np.testing.assert_allclose(got, ref, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 2, 4), (3, 33, 4, 32), (2, 64, 8, 32), (1, 70, 1, 48)])
+@pytest.mark.parametrize("nb,bias_mode", [(True, "zeros"), (False, "random_mask"), (True, "random_mask")])
+def test_c_oracle_matches_numpy_twin(shape, nb, bias_mode):
+    c = make_case(7, *shape, nb=nb, bias_mode=bias_mode)
+    out, avg = run_f32(c, return_avg=True)
+    ref, ref_avg = run_f64(c, return_avg=True)
+    np.testing.assert_allclose(out, ref, rtol=2e-6, atol=2e-6)
+    np.testing.assert_allclose(avg, ref_avg, rtol=2e-6, atol=2e-6)
+
+
+def test_c_oracle_matches_python_bruteforce():
+    """Every index written out by hand: catches transposed weights, head/channel mix-ups, wrong
+    softmax axis."""
+    c = make_case(3, 2, 5, 2, 4)
+    c["bias"][0, 3] = -1e9
+    B, S, C = c["x"].shape
+    H = c["nheads"]
+    d = C // H
+    x = c["x"].astype(np.float64)
+    out = np.zeros((B, S, C))
+    for b in range(B):
+        avg = np.zeros((S, C))
+        for h in range(H):
+            def proj(w, s, e, bvec=None):
+                o = h * d + e
+                acc = sum(x[b, s, i] * float(w[o, i]) for i in range(C))
+                return acc + (float(bvec[o]) if bvec is not None else 0.0)
+            for qi in range(S):
+                logits = []
+                for kj in range(S):
+                    s_ = sum(proj(c["wq"], qi, e) * proj(c["wk"], kj, e) for e in range(d)) / math.sqrt(d)
+                    xl = np.float32(np.float32(s_) + c["bias"][b, kj]) + c["nb"][h, qi, kj]
+                    logits.append(float(xl))
+                m = max(logits)
+                p = [math.exp(v - m) for v in logits]
+                z = sum(p)
+                for e in range(d):
+                    wavg = sum(p[kj] / z * proj(c["wv"], kj, e) for kj in range(S))
+                    gate = 1.0 / (1.0 + math.exp(-proj(c["wg"], qi, e, c["bg"])))
+                    avg[qi, h * d + e] = wavg * gate
+        for s in range(S):
+            for o in range(C):
+                out[b, s, o] = sum(avg[s, i] * float(c["wo"][o, i]) for i in range(C)) + float(c["bo"][o])
+    np.testing.assert_allclose(run_f32(c), out, rtol=2e-6, atol=2e-6)
+
+
+def test_c_oracle_matches_golden_fixture():
+    g = np.load(os.path.join(HERE, "golden", "gating_attention_tiny.npz"))
+    B, S, H, d = (int(v) for v in g["dims"])
+    for name in ("pair_bias", "no_pair_bias", "masked_key", "masked_row"):
+        nb = None if name == "no_pair_bias" else g["in.nb"]
+        out, avg = oracle.gating_attention_f32(g["in.x"], g["in.wq"], g["in.wk"], g["in.wv"], g["in.wg"], g["in.bg"],
+                                               g["in.wo"], g["in.bo"], g[f"{name}.bias"], nb, H, return_avg=True)
+        np.testing.assert_allclose(out, g[f"{name}.out"], rtol=2e-6, atol=2e-6, err_msg=name)
+        np.testing.assert_allclose(avg, g[f"{name}.avg"], rtol=2e-6, atol=2e-6, err_msg=name)
+
+
+# ---- closed forms and invariants --------------------------------------------------------------------
+def test_uniform_attention_when_query_weight_is_zero():
+    c = make_case(11, 2, 9, 2, 8, nb=False, bias_mode="random_mask")
+    c["wq"][:] = 0
+    _, avg = run_f32(c, return_avg=True)
+    B, S, C = c["x"].shape
+    v = c["x"].astype(np.float64) @ c["wv"].astype(np.float64).T
+    gate = 1 / (1 + np.exp(-(c["x"].astype(np.float64) @ c["wg"].astype(np.float64).T + c["bg"])))
+    for b in range(B):
+        keep = c["bias"][b] == 0
+        mean_v = v[b][keep].mean(axis=0)
+        np.testing.assert_allclose(avg[b], mean_v[None, :] * gate[b], rtol=1e-5, atol=1e-6)
+
+
+def test_gate_closed_forms():
+    c = make_case(12, 2, 7, 2, 8)
+    base = dict(c)
+    c0 = dict(base, wg=np.zeros_like(c["wg"]), bg=np.zeros_like(c["bg"]))
+    c1 = dict(base, wg=np.zeros_like(c["wg"]), bg=np.full_like(c["bg"], 30.0))
+    _, a0 = run_f32(c0, return_avg=True)
+    _, a1 = run_f32(c1, return_avg=True)
+    np.testing.assert_allclose(a0, 0.5 * a1, rtol=1e-6, atol=1e-7)  # sigmoid(0) = 1/2, sigmoid(30) = 1
+
+
+def test_zero_output_weight_gives_output_bias():
+    c = make_case(13, 2, 7, 2, 8)
+    c["wo"][:] = 0
+    out = run_f32(c)
+    np.testing.assert_array_equal(out, np.broadcast_to(c["bo"], out.shape))
+
+
+def test_constant_values_pass_through_softmax():
+    """Rows of P sum to one: if every key has the same value vector, avg equals it (times the gate)."""
+    c = make_case(14, 2, 9, 2, 8, bias_mode="random_mask")
+    c["x"][:] = c["x"][:, :1, :]  # identical tokens -> identical v for every key (q,k too, harmless)
+    _, avg = run_f32(c, return_avg=True)
+    x0 = c["x"][:, 0].astype(np.float64)
+    v0 = x0 @ c["wv"].astype(np.float64).T
+    gate = 1 / (1 + np.exp(-(x0 @ c["wg"].astype(np.float64).T + c["bg"])))
+    np.testing.assert_allclose(avg, np.broadcast_to((v0 * gate)[:, None, :], avg.shape), rtol=1e-5, atol=1e-6)
+
+
+def test_softmax_shift_invariance():
+    c = make_case(15, 2, 9, 2, 8)
+    out = run_f32(c)
+    c2 = dict(c, nb=c["nb"] + np.float32(3.0) * np.ones((1, 9, 1), dtype=np.float32),
+              bias=c["bias"] + np.float32(2.0))
+    np.testing.assert_allclose(run_f32(c2), out, rtol=1e-5, atol=1e-5)
+
+
+def test_key_permutation_and_batch_permutation():
+    c = make_case(16, 3, 8, 2, 8, bias_mode="random_mask")
+    out = run_f32(c)
+    # permuting the batch permutes the output
+    perm_b = np.array([2, 0, 1])
+    cb = dict(c, x=c["x"][perm_b], bias=c["bias"][perm_b])
+    np.testing.assert_allclose(run_f32(cb), out[perm_b], rtol=1e-6, atol=1e-6)
+    # permuting tokens (queries and keys together, with both biases) permutes the output rows
+    perm_s = np.random.Generator(np.random.PCG64(5)).permutation(8)
+    cs = dict(c, x=c["x"][:, perm_s], bias=c["bias"][:, perm_s], nb=c["nb"][:, perm_s][:, :, perm_s])
+    np.testing.assert_allclose(run_f32(cs), out[:, perm_s], rtol=1e-5, atol=1e-5)
+
+
+def test_masked_key_has_exactly_zero_weight():
+    c = make_case(17, 1, 6, 2, 8)
+    c["bias"][0, 2] = -1e9
+    _, avg = run_f32(c, return_avg=True)
+    # replace the masked token: its k and v change, every other row of avg must not move at all
+    c2 = dict(c, x=c["x"].copy())
+    c2["x"][0, 2] = 100.0
+    _, avg2 = run_f32(c2, return_avg=True)
+    rows = [0, 1, 3, 4, 5]
+    np.testing.assert_array_equal(avg[0, rows], avg2[0, rows])
+
+
+def test_fully_masked_row_attends_uniformly():
+    """-1e9 absorbs the logit and the pair bias in fp32, so all keys tie (reference
+    gating_attention.cpp:113-117 adds in fp32)."""
+    c = make_case(18, 2, 6, 2, 8)
+    c["bias"][1, :] = -1e9
+    _, avg = run_f32(c, return_avg=True)
+    x1 = c["x"][1].astype(np.float64)
+    v = x1 @ c["wv"].astype(np.float64).T
+    gate = 1 / (1 + np.exp(-(x1 @ c["wg"].astype(np.float64).T + c["bg"])))
+    np.testing.assert_allclose(avg[1], v.mean(axis=0)[None] * gate, rtol=1e-5, atol=1e-6)
+
+
+def test_absent_pair_bias_equals_zero_pair_bias():
+    c = make_case(19, 2, 7, 2, 8, nb=False)
+    out = run_f32(c)
+    c2 = dict(c, nb=np.zeros((2, 7, 7), dtype=np.float32))
+    np.testing.assert_array_equal(run_f32(c2), out)
+
+
+# ---- Rbf16 (reference rounding points) ---------------------------------------------------------------
+def to_bits_case(c):
+    b = oracle.to_bf16_bits
+    return dict(x=b(c["x"]), wq=b(c["wq"]), wk=b(c["wk"]), wv=b(c["wv"]), wg=b(c["wg"]), bg=c["bg"], wo=b(c["wo"]),
+                bo=c["bo"], bias=b(c["bias"]), nb=None if c["nb"] is None else b(c["nb"]), nheads=c["nheads"])
+
+
+def run_bf16(cb, **kw):
+    return oracle.gating_attention_bf16(cb["x"], cb["wq"], cb["wk"], cb["wv"], cb["wg"], cb["bg"], cb["wo"], cb["bo"],
+                                        cb["bias"], cb["nb"], cb["nheads"], **kw)
+
+
+@pytest.mark.parametrize("exp_mode", [0, 1])
+def test_bf16_restatement_close_to_fp32_oracle(exp_mode):
+    c = make_case(21, 3, 48, 4, 32, bias_mode="random_mask")
+    cb = to_bits_case(c)
+    # the fp32 oracle sees the same bf16-rounded inputs
+    cr = {k: (oracle.from_bf16_bits(v) if isinstance(v, np.ndarray) and v.dtype == np.uint16 else v)
+          for k, v in cb.items()}
+    ref = run_f32(cr)
+    got = oracle.from_bf16_bits(run_bf16(cb, exp_mode=exp_mode))
+    err = np.abs(got - ref)
+    assert np.all(err <= 2e-2 + 1e-2 * np.abs(ref)), float(err.max())
+
+
+def test_bf16_restatement_independent_of_block_size():
+    c = make_case(22, 2, 37, 2, 32)
+    cb = to_bits_case(c)
+    outs = [run_bf16(cb, block_size=bs) for bs in (1, 5, 16, 37, 64)]
+    for o in outs[1:]:
+        np.testing.assert_array_equal(o, outs[0])
+
+
+def test_bf16_restatement_scratch_layouts():
+    """q/k/gate/avg come back [B,S,H,d]; v comes back [H,d,B,S] (reference gating_attention.cpp:57-61)."""
+    c = make_case(23, 2, 9, 2, 32)
+    cb = to_bits_case(c)
+    _, s = run_bf16(cb, return_scratch=True)
+    x = oracle.from_bf16_bits(cb["x"]).astype(np.float64)
+    B, S, C = x.shape
+    v_ref = x @ oracle.from_bf16_bits(cb["wv"]).astype(np.float64).T  # [B,S,C]
+    v_got = oracle.from_bf16_bits(s["v"]).transpose(2, 3, 0, 1).reshape(B, S, C)
+    np.testing.assert_allclose(v_got, v_ref, rtol=1e-2, atol=1e-2)
+    q_ref = x @ oracle.from_bf16_bits(cb["wq"]).astype(np.float64).T
+    np.testing.assert_allclose(oracle.from_bf16_bits(s["q"]), q_ref, rtol=1e-2, atol=1e-2)
+
+
+# ---- row operators -----------------------------------------------------------------------------------
+def test_bf16_conversion_matches_torch():
+    rng = np.random.Generator(np.random.PCG64(31))
+    a = np.concatenate([rng.standard_normal(4096).astype(np.float32) * 100,
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf, 1e-40],
+                                 dtype=np.float32)])
+    bits = oracle.to_bf16_bits(a)
+    ref = torch.from_numpy(a).bfloat16().view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(bits, ref)
+    np.testing.assert_array_equal(oracle.from_bf16_bits(bits), torch.from_numpy(a).bfloat16().float().numpy())
+
+
+@pytest.mark.parametrize("size", [128, 256, 37])
+def test_layernorm_matches_torch(size):
+    rng = np.random.Generator(np.random.PCG64(32))
+    x = oracle.round_bf16(rng.standard_normal((50, size)).astype(np.float32) * 3 + 1)
+    gamma = rng.standard_normal(size).astype(np.float32)
+    beta = rng.standard_normal(size).astype(np.float32)
+    got = oracle.from_bf16_bits(oracle.layernorm_rows_bf16(oracle.to_bf16_bits(x), gamma, beta, 1e-5))
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x).double(), (size,), torch.from_numpy(gamma).double(),
+                                         torch.from_numpy(beta).double(), 1e-5).numpy()
+    # result is rounded to bf16: half an ulp (2^-9 relative) plus fp32 noise
+    assert np.all(np.abs(got - ref) <= 2.0 ** -8 * np.abs(ref) + 1e-6)
+    f32 = oracle.layernorm_rows_f32(x, gamma, beta, 1e-5)
+    np.testing.assert_allclose(f32, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_layernorm_constant_row_gives_beta_and_shift_invariance():
+    size = 128
+    gamma = np.linspace(0.5, 1.5, size).astype(np.float32)
+    beta = np.linspace(-1, 1, size).astype(np.float32)
+    const = np.full((1, size), 2.5, dtype=np.float32)
+    got = oracle.from_bf16_bits(oracle.layernorm_rows_bf16(oracle.to_bf16_bits(const), gamma, beta, 1e-5))
+    np.testing.assert_array_equal(got[0], oracle.round_bf16(beta))
+    rng = np.random.Generator(np.random.PCG64(33))
+    x = oracle.round_bf16(rng.integers(-8, 8, (4, size)).astype(np.float32) * 0.25)  # exactly representable
+    a = oracle.layernorm_rows_bf16(oracle.to_bf16_bits(x), gamma, beta, 1e-5)
+    b = oracle.layernorm_rows_bf16(oracle.to_bf16_bits(x + 16.0), gamma, beta, 1e-5)
+    diff = np.abs(oracle.from_bf16_bits(a) - oracle.from_bf16_bits(b))
+    assert np.all(diff <= 2.0 ** -7 * np.abs(oracle.from_bf16_bits(a)) + 1e-6)
+
+
+def test_linear_matches_torch():
+    rng = np.random.Generator(np.random.PCG64(34))
+    act = oracle.round_bf16(rng.standard_normal((37, 128)).astype(np.float32))
+    w = oracle.round_bf16(rng.standard_normal((4, 128)).astype(np.float32) / 11)
+    bias = rng.standard_normal(4).astype(np.float32)
+    ref = torch.nn.functional.linear(torch.from_numpy(act).double(), torch.from_numpy(w).double(),
+                                     torch.from_numpy(bias).double()).numpy()
+    got = oracle.from_bf16_bits(oracle.linear_bf16(oracle.to_bf16_bits(act), oracle.to_bf16_bits(w), bias))
+    assert np.all(np.abs(got - ref) <= 2.0 ** -8 * np.abs(ref) + 1e-6)
+    np.testing.assert_allclose(oracle.linear_f32(act, w, bias), ref, rtol=1e-6, atol=1e-6)
+    # beta accumulates into the existing result
+    prev = oracle.round_bf16(rng.standard_normal((37, 4)).astype(np.float32))
+    got2 = oracle.from_bf16_bits(oracle.linear_bf16(oracle.to_bf16_bits(act), oracle.to_bf16_bits(w), None, beta=1.0,
+                                                    result_bits=oracle.to_bf16_bits(prev)))
+    ref2 = ref - bias + prev
+    assert np.all(np.abs(got2 - ref2) <= 2.0 ** -8 * np.abs(ref2) + 1e-6)
