@@ -105,3 +105,24 @@ def check_close(got, ref, dtype: str, what=""):
         raise AssertionError(f"{what}: {int(bad.sum())} of {err.size} elements outside tolerance; worst at {i}: "
                              f"got {got[i]:.6g} ref {ref[i]:.6g} err {err[i]:.3g} tol {tol[i]:.3g}")
     return float(err.max())
+
+
+def assert_within(got, ref, tol, what=""):
+    """|got - ref| <= tol elementwise, with a short message naming the worst element on failure."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    tol = np.broadcast_to(np.asarray(tol, dtype=np.float64), ref.shape)
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    err = np.abs(got - ref)
+    bad = ~(err <= tol)
+    if bad.any():
+        i = np.unravel_index(np.argmax(np.where(bad, err - tol, -np.inf)), err.shape)
+        raise AssertionError(f"{what}: {int(bad.sum())} of {err.size} elements outside tolerance; worst at {i}: "
+                             f"got {got[i]:.6g} ref {ref[i]:.6g} err {err[i]:.3g} tol {tol[i]:.3g}")
+    return float(err.max())
+
+
+def same_bits(a, b) -> bool:
+    """Bitwise equality of two torch tensors, as a plain bool (keeps assertion messages short)."""
+    import torch
+    return bool(torch.equal(a, b))
