@@ -34,11 +34,12 @@ def hipcc() -> str:
 
 def build(verbose: bool = False) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
+    extra = os.environ.get("KUTACC_EXTRA_HIPFLAGS", "").split()  # e.g. -DKUTACC_TIMELINE for tuning builds
     objs = []
     procs = []
     for src in SOURCES:
         obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc(), *HIP_FLAGS, "-x", "hip", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
+        cmd = [hipcc(), *HIP_FLAGS, *extra, "-x", "hip", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
                os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)

@@ -1,13 +1,19 @@
 // Fused gated-attention kernels for gfx950 (CDNA4), bf16 storage, head_size 32.
 //
-// Kernel 1, fused_head_kernel: one workgroup per (batch row b, head h).  It reads the rows of
-// `input` once per staged weight group, projects K_h and V_h for the whole sequence into LDS, keeps
-// Q_h and sigmoid(gate_h) of each wave's own query blocks in registers, runs flash-style attention
-// with online softmax over 32-key tiles (logits never leave registers) and writes the gated weighted
-// average.  Everything that the reference materialises in memory between its GEMMs -- q, k, v, gate,
-// the [bs, S] logits block, the probabilities (reference src/attention/gating_attention.cpp:47-66,
-// 97-147) -- stays on chip.  Kernel 2, output_projection_kernel, is the final GEMM with fp32 bias
-// (reference :152-157).
+// Two kernels compute the gated weighted average avg = softmax(q.k^T/sqrt(d) + bias + pair_bias).v *
+// sigmoid(gate) for one (batch row b, head h) unit at a time; everything the reference materialises
+// in memory between its GEMMs -- q, k, v, gate, the [bs, S] logits block, the probabilities
+// (reference src/attention/gating_attention.cpp:47-66, 97-147) -- stays in LDS and registers:
+//
+//   persistent_head_kernel  seq_len <= 384 (C=128) / 256 (C=256).  One workgroup per CU keeps one head
+//       for its lifetime and walks batch rows.  Its waves are specialised: "projection" waves hold
+//       one weight matrix of the head in registers and produce K, V, Q, gate of the NEXT batch row
+//       into LDS (MFMA-bound) while the "attention" waves run the online softmax of the current one
+//       (VALU-bound); K/V are double-buffered, two workgroup barriers per batch row.
+//   fused_head_kernel       any seq_len <= 1024.  One workgroup per unit; projections first (weights
+//       staged through LDS in groups), then attention.
+//
+// A third kernel, output_projection_kernel, is the final GEMM with fp32 bias (reference :152-157).
 //
 // All contractions are v_mfma_f32_32x32x16_bf16 (fp32 accumulate).  Operand fragments use one
 // format throughout: a [32 rows x 16 k] slab, lane l holding row (l & 31), k-chunk (l >> 5)*8..+8,
@@ -23,28 +29,52 @@
 //     keys (pair-bias row loads become two 16-byte loads).
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
+#include <cstdlib>
+#include <type_traits>
+
 #include "device_util.h"
 #include "launch_internal.h"
 #include "profiler.h"
 
 using namespace kutacc_dev;
 
+// Phase timestamps for kernel tuning, compiled in only with -DKUTACC_TIMELINE (never in the shipped
+// library): wave leaders of every 256th workgroup record clock64() at the probes below, and
+// kutacc_debug_timeline() copies the table out.
+#ifdef KUTACC_TIMELINE
+__device__ unsigned long long g_timeline[8 * 16 * 12];
+#define TL(i)                                                                                 \
+    do {                                                                                      \
+        if ((blockIdx.x & 255) == 77 && (threadIdx.x & 63) == 0 && (blockIdx.x >> 8) < 8) {   \
+            g_timeline[((blockIdx.x >> 8) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = clock64(); \
+        }                                                                                     \
+    } while (0)
+extern "C" __attribute__((visibility("default"))) int kutacc_debug_timeline(unsigned long long *out, int n)
+{
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_timeline), (size_t)n * 8);
+}
+#else
+#define TL(i) ((void)0)
+#endif
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr float LOG2E = 1.44269504088896340736f;
-constexpr int HEAD = 32;          // head_size the MFMA kernels are written for
-constexpr int MAX_WAVES = 12;     // 768 threads: 3 waves per SIMD, 168 VGPRs each
+constexpr int HEAD = 32;            // head_size the MFMA kernels are written for
+constexpr int MAX_WAVES = 12;       // fused_head_kernel: 768 threads, 3 waves per SIMD, 168 VGPRs each
+constexpr float RESCALE_GAP = 5.5f; // running max may lag the true max by this much (natural log units, ~8 octaves)
 
-// Waves per workgroup a given instantiation may be launched with.  One query block per wave needs
-// about 150 VGPRs at C=128, which fits three waves per SIMD; the variants that hold more state
-// (more query blocks per wave, or 256 input channels in registers) get two waves per SIMD.
+// Waves per workgroup a given fused_head_kernel instantiation may be launched with.  One query block
+// per wave needs about 140 VGPRs at C=128, which fits three waves per SIMD; the variants that hold
+// more state (more query blocks per wave, or 256 input channels in registers) get two per SIMD.
 __host__ __device__ constexpr int max_waves(int C, int BPW) { return (C == 128 && BPW <= 2) ? MAX_WAVES : 8; }
-constexpr float RESCALE_GAP = 8.f; // running max may lag the true max by this many octaves
 
 enum Proj { PROJ_K = 0, PROJ_V = 1, PROJ_Q = 2, PROJ_G = 3 };
 
@@ -57,8 +87,9 @@ struct FusedParams {
     bf16_t *avg;
     int64_t x_ld, bias_sb, nb_sh, nb_sq, avg_sb, avg_ss, avg_sh;
     int B, S, H, NB, NW, GW;
-    int nb_vec; // pair-bias rows may be read with 16-byte loads
-    float qscale; // log2(e) / sqrt(head_size)
+    int nb_vec;   // pair-bias rows may be read with 16-byte loads
+    float qscale; // 1 / sqrt(head_size)
+    int ngrp;     // persistent kernel: batch-row groups per XCD
 };
 
 __device__ __forceinline__ int pi_row(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
@@ -66,6 +97,12 @@ __device__ __forceinline__ int pi_row(int r) { return 16 * ((r >> 2) & 1) + 4 * 
 __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f32x16 zero16()
+{
+    const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    return z;
 }
 
 __device__ __forceinline__ bf16x8 pack8(const f32x16 &v, int base)
@@ -110,12 +147,340 @@ __device__ __forceinline__ float half_swap_sum(float x)
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// 0/1 selection fragments that scatter the pair-bias words a lane loads (16 consecutive keys, 8 per
+// MFMA) onto the logits rows: row i of a tile is key pi(i); k-slot 8*g+e of the first MFMA carries
+// key 16*g+e, of the second key 16*g+8+e.
+__device__ __forceinline__ void make_selectors(int lane, bf16x8 &sel0, bf16x8 &sel1)
+{
+    const int r = lane & 31, g = lane >> 5;
+    const int gi = (r >> 2) & 1;          // which 16-key half row r belongs to
+    const int w = 4 * (r >> 3) + (r & 3); // position of row r's key inside that half
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        sel0[e] = (bf16_t)((gi == g && w == e) ? 1.0f : 0.0f);
+        sel1[e] = (bf16_t)((gi == g && w == e + 8) ? 1.0f : 0.0f);
+    }
+}
+
+// Mask bias of one batch row -> LDS as fp32 (keys past S get -inf), plus one flag bit per 32-key tile
+// saying "this tile needs the mask added" (non-zero bias or ragged tail).  Wave w covers keys
+// [64w, 64w+64); *flag_word must have been zeroed before, with a barrier in between.
+__device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *mask, uint32_t *flag_word, int S, int NB,
+                                                int wave, int lane)
+{
+    const int k = wave * 64 + lane;
+    if (wave * 64 < NB * 32) {
+        float mv = -INFINITY;
+        if (k < S) {
+            mv = to_f32(bias_row[k]);
+        }
+        if (k < NB * 32) {
+            mask[k] = mv;
+        }
+        const unsigned long long nz = __ballot(k < NB * 32 && mv != 0.f);
+        const uint32_t bits = (((uint32_t)nz != 0u ? 1u : 0u) | ((uint32_t)(nz >> 32) != 0u ? 2u : 0u)) << (2 * wave);
+        if (lane == 0 && bits != 0u) {
+            atomicOr(flag_word, bits);
+        }
+    }
+}
+
+// Wave-private staging panel in LDS: 32 rows x 128 bytes, in 16-byte slots.  A panel is filled with
+// four fully coalesced loads (each instruction reads 8 rows x 128 contiguous bytes = 8 whole cache
+// lines, lane l -> row 8i + l/8, slot l%8) and read back in MFMA fragment order (lane -> its own
+// row).  Loading fragments straight from global memory would touch 32 different cache lines per
+// instruction, four times the L1 tag traffic.  The slot index is XOR-swizzled by row so that both
+// access patterns are free of LDS bank conflicts.
+__device__ __forceinline__ int panel_slot(int row, int chunk)
+{
+    return row * 8 + (chunk ^ ((row & 7) ^ ((row >> 4) & 1)));
+}
+
+// issue the four coalesced loads of a panel: rows row0 .. row0+31 (clamped to last_row) of a
+// row-major bf16 matrix with leading dimension ld, 64 columns starting at col0
+struct PanelRegs {
+    uint4 r0, r1, r2, r3; // named members rather than an array, so that they always live in registers
+};
+
+__device__ __forceinline__ uint4 panel_load_one(const bf16_t *base, int64_t ld, int row, int last_row, int col0, int lane)
+{
+    row = row < last_row ? row : last_row;
+    return *reinterpret_cast<const uint4 *>(base + (int64_t)row * ld + col0 + (lane & 7) * 8);
+}
+
+__device__ __forceinline__ PanelRegs panel_load(const bf16_t *base, int64_t ld, int row0, int last_row, int col0, int lane)
+{
+    PanelRegs p;
+    const int row = row0 + (lane >> 3);
+    p.r0 = panel_load_one(base, ld, row, last_row, col0, lane);
+    p.r1 = panel_load_one(base, ld, row + 8, last_row, col0, lane);
+    p.r2 = panel_load_one(base, ld, row + 16, last_row, col0, lane);
+    p.r3 = panel_load_one(base, ld, row + 24, last_row, col0, lane);
+    return p;
+}
+
+__device__ __forceinline__ void panel_store(uint4 *panel, int lane, const PanelRegs &p)
+{
+    const int row = lane >> 3, chunk = lane & 7;
+    panel[panel_slot(row, chunk)] = p.r0;
+    panel[panel_slot(row + 8, chunk)] = p.r1;
+    panel[panel_slot(row + 16, chunk)] = p.r2;
+    panel[panel_slot(row + 24, chunk)] = p.r3;
+}
+
+// Flash-style attention of one 32-query block against all keys of the unit.
+//   lds_k / lds_v : K and V fragments of the unit, [tile][kstep][lane] in 16-byte units
+//   mask4         : fp32 mask bias in LDS, already offset by 16*g floats; flags: one bit per tile
+//   nb_head       : pair bias of this head, [S, S] with row stride nb_sq (HAS_NB only); q0row = first
+//                   query of the block
+//   panel         : wave-private 4 KB staging panel, or nullptr to load the pair bias directly
+//   q0, q1        : Q^T fragments scaled by 1/sqrt(d)
+// Returns the unnormalised O^T accumulator and the row sum (identical in both lane halves).
+// Per key tile: the logits accumulator starts at the mask bias (or 0); two MFMAs with the 0/1 selectors
+// add the pair bias straight from its bf16 words (exact), two add q.k; the running maximum is
+// refreshed only when some row's tile maximum exceeds it by RESCALE_GAP; probabilities go from the
+// accumulator registers into the B operand of the P.V MFMAs without touching LDS.  The logits of
+// tile t+1 are issued before the softmax of tile t so that the matrix core works under the VALU.
+// Pair bias arrives two key tiles (64 keys = one 128-byte line per query) at a time through the
+// staging panel, prefetched one pair ahead into registers; tiles of a ragged or unaligned tail are
+// read directly.
+template <bool HAS_NB>
+__device__ __forceinline__ void attend_block(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4, uint32_t flags,
+                                             const bf16_t *nb_head, int64_t nb_sq, int q0row, bool nb_vec, uint4 *panel,
+                                             bf16x8 q0, bf16x8 q1, bf16x8 sel0, bf16x8 sel1, int NB, int S, int lane,
+                                             f32x16 &o_out, float &l_out)
+{
+    const int r = lane & 31, g = lane >> 5;
+    const int prow = pi_row(r);
+    f32x16 o = zero16();
+    float m_run = -1e30f; // finite, so the first rescale factor is exp2(-huge) = 0, never NaN
+    float lsum = 0.f;     // this lane's share of the row sum; the two halves are added at the end
+    bf16x2 one2;
+    one2[0] = (bf16_t)1.0f, one2[1] = (bf16_t)1.0f;
+
+    const int qrow = q0row + prow < S ? q0row + prow : S - 1;
+    const bf16_t *nbrow = HAS_NB ? nb_head + (int64_t)qrow * nb_sq + 16 * g : nullptr;
+    // number of leading tile pairs that go through the staging panel
+    const int staged_pairs = (HAS_NB && panel != nullptr && nb_vec) ? S / 64 : 0;
+    PanelRegs pf; // the next staged pair, in flight from global memory
+    if (HAS_NB && staged_pairs > 0) {
+        pf = panel_load(nb_head, nb_sq, q0row, S - 1, 0, lane);
+    }
+
+    // pair-bias words of key tile t for this lane (16 consecutive keys): B operands of the selector MFMAs
+    auto nb_words = [&](int t, uint4 &w0, uint4 &w1) {
+        const int pair = t >> 1;
+        if (pair < staged_pairs) {
+            if ((t & 1) == 0) {
+                panel_store(panel, lane, pf); // the previous pair's reads were issued earlier in program order
+                if (pair + 1 < staged_pairs) {
+                    pf = panel_load(nb_head, nb_sq, q0row, S - 1, (pair + 1) * 64, lane);
+                }
+            }
+            const int c = 4 * (t & 1) + 2 * g;
+            w0 = panel[panel_slot(prow, c)];
+            w1 = panel[panel_slot(prow, c + 1)];
+        } else if (nb_vec && (t + 1) * 32 <= S) {
+            w0 = *reinterpret_cast<const uint4 *>(nbrow + t * 32);
+            w1 = *reinterpret_cast<const uint4 *>(nbrow + t * 32 + 8);
+        } else {
+            const uint16_t *s16 = reinterpret_cast<const uint16_t *>(nbrow + t * 32);
+            const int key0 = t * 32 + 16 * g;
+            uint32_t wds[8];
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const uint32_t a0 = key0 + 2 * v < S ? s16[2 * v] : 0u;
+                const uint32_t a1 = key0 + 2 * v + 1 < S ? s16[2 * v + 1] : 0u;
+                wds[v] = a0 | (a1 << 16);
+            }
+            w0.x = wds[0], w0.y = wds[1], w0.z = wds[2], w0.w = wds[3];
+            w1.x = wds[4], w1.y = wds[5], w1.z = wds[6], w1.w = wds[7];
+        }
+    };
+    // logits^T of key tile t (rows = keys, columns = this wave's 32 queries), natural-log units
+    auto logits = [&](int t, f32x16 &x) {
+        if ((flags >> t) & 1u) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 mv = mask4[t * 8 + a];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    x[4 * a + c] = mv[c];
+                }
+            }
+        } else {
+            x = zero16();
+        }
+        if (HAS_NB) {
+            uint4 w0, w1;
+            nb_words(t, w0, w1);
+            x = mfma(sel0, as_bf16x8(w0), x);
+            x = mfma(sel1, as_bf16x8(w1), x);
+        }
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
+    };
+    // online softmax of tile t held in xc, then O^T += V^T . P; before that, start tile t+1 into xn
+    auto step = [&](int t, f32x16 &xc, f32x16 &xn) {
+        if (t + 1 < NB) {
+            logits(t + 1, xn);
+        }
+        float mx = xc[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) {
+            mx = fmaxf(mx, xc[v]);
+        }
+        mx = half_swap_max(mx);
+        if (__any(mx > m_run + RESCALE_GAP)) {
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+            lsum *= alpha;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                o[v] *= alpha;
+            }
+            m_run = m_new;
+        }
+        const float ml = -m_run * LOG2E;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            xc[v] = __builtin_amdgcn_exp2f(fmaf(xc[v], LOG2E, ml));
+        }
+        // the row sum is taken over the bf16-rounded probabilities, two per dot2 instruction
+        const bf16x8 p0 = pack8(xc, 0), p1 = pack8(xc, 8);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            bf16x2 a, c;
+            a[0] = p0[2 * v], a[1] = p0[2 * v + 1];
+            c[0] = p1[2 * v], c[1] = p1[2 * v + 1];
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(a, one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(c, one2, lsum, false);
+        }
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 0) * 64 + lane]), p0, o);
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 1) * 64 + lane]), p1, o);
+    };
+
+    // softmax of a finished logits tile and its P.V accumulation (the part of `step` after the lookahead)
+    auto softmax_pv = [&](int t, f32x16 &xc) {
+        float mx = xc[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) {
+            mx = fmaxf(mx, xc[v]);
+        }
+        mx = half_swap_max(mx);
+        if (__any(mx > m_run + RESCALE_GAP)) {
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+            lsum *= alpha;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                o[v] *= alpha;
+            }
+            m_run = m_new;
+        }
+        const float ml = -m_run * LOG2E;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            xc[v] = __builtin_amdgcn_exp2f(fmaf(xc[v], LOG2E, ml));
+        }
+        const bf16x8 p0 = pack8(xc, 0), p1 = pack8(xc, 8);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            bf16x2 a, c;
+            a[0] = p0[2 * v], a[1] = p0[2 * v + 1];
+            c[0] = p1[2 * v], c[1] = p1[2 * v + 1];
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(a, one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(c, one2, lsum, false);
+        }
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 0) * 64 + lane]), p0, o);
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 1) * 64 + lane]), p1, o);
+    };
+    // logits of a tile whose pair bias sits in the staging panel; no branches, so that the scheduler
+    // can spread the LDS reads, MFMAs and the neighbouring softmax over each other
+    auto logits_staged = [&](int t, f32x16 &x, auto with_mask) {
+        if (decltype(with_mask)::value) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 mv = mask4[t * 8 + a];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    x[4 * a + c] = mv[c];
+                }
+            }
+        } else {
+            x = zero16();
+        }
+        const int c0 = 4 * (t & 1) + 2 * g;
+        x = mfma(sel0, as_bf16x8(panel[panel_slot(prow, c0)]), x);
+        x = mfma(sel1, as_bf16x8(panel[panel_slot(prow, c0 + 1)]), x);
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
+    };
+
+    f32x16 xa, xb;
+    logits(0, xa);
+    int t = 0;
+    // main loop: two key tiles per iteration while a further staged pair follows; straight-line body
+    auto main_loop = [&](auto with_mask) {
+        for (int pair = 0; pair + 1 < staged_pairs; ++pair) {
+            const int t0 = 2 * pair;
+            logits_staged(t0 + 1, xb, with_mask);
+            softmax_pv(t0, xa);
+            panel_store(panel, lane, pf); // pair+1; the reads of this pair were issued above
+            // prefetch pair+2 (clamped to the last staged pair: a harmless re-read instead of a branch)
+            const int nxt = pair + 2 < staged_pairs ? pair + 2 : staged_pairs - 1;
+            pf = panel_load(nb_head, nb_sq, q0row, S - 1, nxt * 64, lane);
+            logits_staged(t0 + 2, xa, with_mask);
+            softmax_pv(t0 + 1, xb);
+        }
+    };
+    if (HAS_NB && staged_pairs > 1) {
+        if (flags != 0u) {
+            main_loop(std::true_type{});
+        } else {
+            main_loop(std::false_type{});
+        }
+        t = 2 * (staged_pairs - 1);
+    }
+    // remaining tiles (last staged pair, unstaged or ragged tail, or everything when nothing is staged)
+    for (; t < NB; t += 2) {
+        step(t, xa, xb);
+        if (t + 1 < NB) {
+            step(t + 1, xb, xa);
+        }
+    }
+    o_out = o;
+    l_out = half_swap_sum(lsum);
+}
+
+// avg[b, q, h, :] = O / l * gate for the 32 queries of one block; gate values in accumulator order
+__device__ __forceinline__ void store_gated(bf16_t *dst, const f32x16 &o, float inv, const f32x16 &gate)
+{
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        bf16x4 ov;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            ov[c] = (bf16_t)(o[4 * a + c] * inv * gate[4 * a + c]);
+        }
+        *reinterpret_cast<bf16x4 *>(dst + 8 * a) = ov;
+    }
+}
+
+__device__ __forceinline__ float sigmoid_fast(float x)
+{
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
+}
+
+// ------------------------------------------------------------------------------------------------
+// fused_head_kernel: one workgroup per (b, h) unit
 // LDS carve-up, in 16-byte units unless noted:
 //   [0, GW*CK*64)               staged weight fragments  [slot][kstep][lane]
 //   [.., +NB*2*64)              K fragments              [tile][kstep][lane]
 //   [.., +NB*2*64)              V fragments              [tile][kstep][lane]
-//   then floats: mask[NB*32] (log2-scaled, -inf past S), then ints: tile_flag[NB]
-template <int C, int BPW>
+//   then floats: mask[NB*32] (-inf past S), then one uint32 of tile flags
+// ------------------------------------------------------------------------------------------------
+template <int C, int BPW, bool HAS_NB>
 __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(FusedParams p)
 {
     constexpr int CK = C / 16;
@@ -132,6 +497,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         return;
     }
     const int tid = threadIdx.x;
+    TL(0);
     const int nthreads = p.NW * 64;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
@@ -141,30 +507,25 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     uint4 *lds_k = lds_w + GW * CK * 64;
     uint4 *lds_v = lds_k + NB * 2 * 64;
     float *mask = reinterpret_cast<float *>(lds_v + NB * 2 * 64);
-    int *tile_flag = reinterpret_cast<int *>(mask + NB * 32);
+    uint32_t *flag_word = reinterpret_cast<uint32_t *>(mask + NB * 32);
 
-    // ---- mask bias -> LDS, pre-multiplied by log2(e); keys past S get -inf ----
-    for (int t = tid; t < NB; t += nthreads) {
-        tile_flag[t] = ((t + 1) * 32 > S) ? 1 : 0; // ragged last tile always takes the masked path
+    if (tid == 0) {
+        *flag_word = 0;
     }
     __syncthreads();
-    for (int k = tid; k < NB * 32; k += nthreads) {
-        float mv = -INFINITY;
-        if (k < S) {
-            mv = to_f32(p.bias[(int64_t)b * p.bias_sb + k]) * LOG2E;
-            if (mv != 0.f) {
-                atomicOr(&tile_flag[k >> 5], 1);
-            }
-        }
-        mask[k] = mv;
+    for (int part = wave; part * 64 < NB * 32; part += NW) {
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, part, lane);
     }
 
     // ---- projections, in groups of GW weight matrices staged through LDS ----
-    bf16x8 qf[BPW][2];   // Q^T fragments (B operand of the logits MFMA), scaled by log2(e)/sqrt(d)
+    bf16x8 qf[BPW][2];   // Q^T fragments (B operand of the logits MFMA), scaled by 1/sqrt(d)
     bf16x8 gate[BPW][2]; // sigmoid(gate) in accumulator order, packed
     const int npass = 4 / GW;
     for (int pass = 0; pass < npass; ++pass) {
         __syncthreads(); // previous group's fragments are no longer being read
+        if (pass == 0) {
+            TL(1);
+        }
         for (int idx = tid; idx < GW * CK * 64; idx += nthreads) {
             const int mm = idx / (CK * 64);
             const int ks = (idx >> 6) % CK;
@@ -173,6 +534,9 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             lds_w[idx] = *reinterpret_cast<const uint4 *>(src);
         }
         __syncthreads();
+        if (pass == 0) {
+            TL(2);
+        }
 #pragma unroll
         for (int i = 0; i < BPW; ++i) {
             const int j = wave + i * NW;
@@ -190,7 +554,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             for (int mm = 0; mm < GW; ++mm) {
                 const int m = pass * GW + mm;
                 const uint4 *wsrc = lds_w + mm * CK * 64 + lane;
-                f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                f32x16 acc = zero16();
                 if (m == PROJ_V) {
                     // V[s][d]: rows = sequence positions, so a lane ends up with 16 keys of one head-dim
 #pragma unroll
@@ -222,8 +586,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
                             const f32x4 bv = *reinterpret_cast<const f32x4 *>(bgp + 8 * a);
 #pragma unroll
                             for (int c = 0; c < 4; ++c) {
-                                const float gv = acc[4 * a + c] + bv[c];
-                                acc[4 * a + c] = 1.0f / (1.0f + __builtin_amdgcn_exp2f(-gv * LOG2E));
+                                acc[4 * a + c] = sigmoid_fast(acc[4 * a + c] + bv[c]);
                             }
                         }
                         gate[i][0] = pack8(acc, 0);
@@ -233,9 +596,16 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             }
         }
     }
+    TL(3);
     __syncthreads(); // K and V of the whole sequence are in LDS
+    TL(4);
 
     // ---- attention: each wave walks the key tiles for its own query blocks ----
+    const uint32_t flags = *flag_word;
+    const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
+    bf16x8 sel0, sel1;
+    make_selectors(lane, sel0, sel1);
+
 #pragma unroll
     for (int i = 0; i < BPW; ++i) {
         const int j = wave + i * NW;
@@ -243,91 +613,199 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             continue;
         }
         const int qpos = j * 32 + pi_row(r);
-        const int qrow = qpos < S ? qpos : S - 1;
-        const bf16_t *nbrow = p.nb ? p.nb + (int64_t)h * p.nb_sh + (int64_t)qrow * p.nb_sq + 16 * g : nullptr;
-        f32x16 o = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        float m_run = -1e30f; // finite, so the first rescale factor is exp2(-huge) = 0, never NaN
-        float lsum = 0.f;     // this lane's share of the row sum; the two halves are added at the end
-        for (int t = 0; t < NB; ++t) {
-            f32x16 x;
-            const bool ragged = (t + 1) * 32 > S;
-            if (nbrow != nullptr) {
-                if (p.nb_vec && !ragged) {
-                    const uint4 lo = *reinterpret_cast<const uint4 *>(nbrow + t * 32);
-                    const uint4 hi = *reinterpret_cast<const uint4 *>(nbrow + t * 32 + 8);
-                    const uint32_t wds[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        f32x16 o;
+        float l;
+        attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr, p.nb_sq, j * 32,
+                             p.nb_vec != 0, nullptr, qf[i][0], qf[i][1], sel0, sel1, NB, S, lane, o, l);
+        TL(5);
+        if (qpos < S) {
+            f32x16 gv;
 #pragma unroll
-                    for (int v = 0; v < 8; ++v) {
-                        x[2 * v] = __uint_as_float(wds[v] << 16) * LOG2E;
-                        x[2 * v + 1] = __uint_as_float(wds[v] & 0xffff0000u) * LOG2E;
-                    }
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int key = t * 32 + 16 * g + v;
-                        x[v] = key < S ? to_f32(nbrow[t * 32 + v]) * LOG2E : 0.f;
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    x[v] = 0.f;
-                }
+            for (int v = 0; v < 16; ++v) {
+                gv[v] = to_f32(gate[i][v >> 3][v & 7]);
             }
-            if (tile_flag[t]) {
-                const f32x4 *mp = reinterpret_cast<const f32x4 *>(mask + t * 32 + 16 * g);
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const f32x4 mv = mp[a];
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        x[4 * a + c] += mv[c];
-                    }
-                }
-            }
-            // logits^T tile: rows = keys of tile t, columns = this wave's 32 queries
-            x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), qf[i][0], x);
-            x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), qf[i][1], x);
+            store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * g, o,
+                        __builtin_amdgcn_rcpf(l), gv);
+        }
+    }
+}
 
-            float mx = x[0];
+// ------------------------------------------------------------------------------------------------
+// persistent_head_kernel: one workgroup per CU keeps one head for its lifetime and walks batch rows;
+// wave j owns sequence block j (its K/V projection and its 32 queries).  Compared with one workgroup
+// per (b, h) unit this stages the head's weights once, pays no workgroup launch per unit, and moves
+// the two big streams -- input rows and pair bias -- through wave-private staging panels with fully
+// coalesced loads.
+// LDS, 16-byte units: W[4][CK][64]  K[NB][2][64]  V[NB][2][64]  panel[NB waves][256]  gate[NB waves][2][64];
+// then floats mask[NB*32]; then one uint32 of tile flags.
+// Per batch row: project (K, V -> LDS; Q, gate -> registers), barrier, attend, barrier.
+// ------------------------------------------------------------------------------------------------
+template <int C, bool HAS_NB>
+__global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(FusedParams p)
+{
+    constexpr int CK = C / 16;
+    constexpr int NP = CK / 4; // staging panels (64 channels each) per input row block
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int S = p.S, NB = p.NB;
+    const int nthreads = NB * 64;
+    const int prow = pi_row(r);
+
+    // workgroup -> (XCD, head, batch-row group): the H workgroups that share a batch-row sequence sit
+    // on the same XCD (ids 8 apart) and walk it in step, so x[b] is read from HBM once per XCD
+    const int w = blockIdx.x;
+    const int xcd = w & 7;
+    const int slot = w >> 3;
+    const int h = slot % p.H;
+    const int grp = slot / p.H;
+    const int b0 = xcd + 8 * grp;
+    const int bstep = 8 * p.ngrp;
+    const int nrows = b0 < p.B ? (p.B - b0 + bstep - 1) / bstep : 0;
+
+    uint4 *lds_w = lds;
+    uint4 *lds_k = lds_w + 4 * CK * 64;
+    uint4 *lds_v = lds_k + NB * 2 * 64;
+    uint4 *panel = lds_v + NB * 2 * 64 + wave * 256;
+    uint4 *gate_park = lds_v + NB * 2 * 64 + NB * 256 + wave * 128 + lane; // sigmoid(gate) waits here during attention
+    float *mask = reinterpret_cast<float *>(lds_v + NB * 2 * 64 + NB * 256 + NB * 128);
+    uint32_t *flag_word = reinterpret_cast<uint32_t *>(mask + NB * 32);
+
+    // the head's rows of the four weight matrices, in fragment order, for the whole kernel
+    for (int idx = tid; idx < 4 * CK * 64; idx += nthreads) {
+        const int mm = idx / (CK * 64);
+        const int ks = (idx >> 6) % CK;
+        const int ln = idx & 63;
+        const bf16_t *src = p.w[mm] + (int64_t)(h * HEAD + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8;
+        lds_w[idx] = *reinterpret_cast<const uint4 *>(src);
+    }
+    if (tid == 0) {
+        *flag_word = 0;
+    }
+    bf16x8 sel0, sel1;
+    make_selectors(lane, sel0, sel1);
+    __syncthreads();
+
+    const int j = wave; // this wave's sequence block
+    const int qpos = j * 32 + prow;
+    for (int n = 0; n < nrows; ++n) {
+        const int b = b0 + n * bstep;
+        if (n == 2) {
+            TL(0);
+        }
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, wave, lane);
+
+        // ---- input rows of the block -> fragments, 64 channels per staging panel ----
+        const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
+        bf16x8 xf[CK];
+        {
+            PanelRegs ta, tb;
+            ta = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane);
 #pragma unroll
-            for (int v = 1; v < 16; ++v) {
-                mx = fmaxf(mx, x[v]);
-            }
-            mx = half_swap_max(mx);
-            if (__any(mx > m_run + RESCALE_GAP)) {
-                const float m_new = fmaxf(m_run, mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                lsum *= alpha;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    o[v] *= alpha;
+            for (int c = 0; c < NP; c += 2) {
+                if (c + 1 < NP) {
+                    tb = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 1) * 64, lane);
                 }
-                m_run = m_new;
+                panel_store(panel, lane, ta);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    xf[4 * c + k] = as_bf16x8(panel[panel_slot(prow, 2 * k + g)]);
+                }
+                if (c + 1 < NP) {
+                    if (c + 2 < NP) {
+                        ta = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 2) * 64, lane);
+                    }
+                    panel_store(panel, lane, tb);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        xf[4 * (c + 1) + k] = as_bf16x8(panel[panel_slot(prow, 2 * k + g)]);
+                    }
+                }
+            }
+        }
+        if (n == 2) {
+            TL(1);
+        }
+        // ---- four projections of the block ----
+        bf16x8 q0, q1;
+        {
+            const uint4 *wsrc = lds_w + lane;
+            f32x16 acc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                acc = mfma(as_bf16x8(wsrc[(PROJ_K * CK + ks) * 64]), xf[ks], acc);
+            }
+            lds_k[(j * 2 + 0) * 64 + lane] = as_uint4(pack8(acc, 0));
+            lds_k[(j * 2 + 1) * 64 + lane] = as_uint4(pack8(acc, 8));
+            acc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                acc = mfma(xf[ks], as_bf16x8(wsrc[(PROJ_V * CK + ks) * 64]), acc);
+            }
+            lds_v[(j * 2 + 0) * 64 + lane] = as_uint4(pack8(acc, 0));
+            lds_v[(j * 2 + 1) * 64 + lane] = as_uint4(pack8(acc, 8));
+            acc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                acc = mfma(as_bf16x8(wsrc[(PROJ_Q * CK + ks) * 64]), xf[ks], acc);
             }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                x[v] = __builtin_amdgcn_exp2f(x[v] - m_run);
-                lsum += x[v];
+                acc[v] *= p.qscale;
             }
-            // weighted sum: O^T[d][q] += V^T[d][keys] . P[keys][q]; P goes straight from registers
-            o = mfma(as_bf16x8(lds_v[(t * 2 + 0) * 64 + lane]), pack8(x, 0), o);
-            o = mfma(as_bf16x8(lds_v[(t * 2 + 1) * 64 + lane]), pack8(x, 8), o);
-        }
-        const float inv = 1.0f / half_swap_sum(lsum);
-        if (qpos < S) {
-            bf16_t *dst = p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * g;
+            q0 = pack8(acc, 0);
+            q1 = pack8(acc, 8);
+            acc = zero16();
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                acc = mfma(as_bf16x8(wsrc[(PROJ_G * CK + ks) * 64]), xf[ks], acc);
+            }
+            const float *bgp = p.bg + h * HEAD + 4 * g;
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                bf16x4 ov;
+                const f32x4 bv = *reinterpret_cast<const f32x4 *>(bgp + 8 * a);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const int v = 4 * a + c;
-                    const float gv = to_f32(gate[i][v >> 3][v & 7]);
-                    ov[c] = (bf16_t)(o[v] * inv * gv);
+                    acc[4 * a + c] = sigmoid_fast(acc[4 * a + c] + bv[c]);
                 }
-                *reinterpret_cast<bf16x4 *>(dst + 8 * a) = ov;
             }
+            gate_park[0] = as_uint4(pack8(acc, 0));
+            gate_park[64] = as_uint4(pack8(acc, 8));
+        }
+        if (n == 2) {
+            TL(2);
+        }
+        __syncthreads(); // K, V and the mask of this batch row are complete
+        if (n == 2) {
+            TL(3);
+        }
+
+        const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
+        f32x16 o;
+        float l;
+        attend_block<HAS_NB>(lds_k, lds_v, mask4, *flag_word, HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr, p.nb_sq,
+                             j * 32, p.nb_vec != 0, panel, q0, q1, sel0, sel1, NB, S, lane, o, l);
+        if (qpos < S) {
+            const bf16x8 gate0 = as_bf16x8(gate_park[0]), gate1 = as_bf16x8(gate_park[64]);
+            f32x16 gv;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                gv[v] = to_f32(gate0[v]);
+                gv[8 + v] = to_f32(gate1[v]);
+            }
+            store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * g, o,
+                        __builtin_amdgcn_rcpf(l), gv);
+        }
+        if (n == 2) {
+            TL(4);
+        }
+        __syncthreads(); // every wave is done with this row's K/V and mask
+        if (n == 2) {
+            TL(5);
+        }
+        if (tid == 0) {
+            *flag_word = 0;
         }
     }
 }
@@ -368,10 +846,7 @@ __global__ __launch_bounds__(256) void output_projection_kernel(const bf16_t *__
         f32x16 acc[4];
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                acc[n][v] = 0.f;
-            }
+            acc[n] = zero16();
         }
 #pragma unroll
         for (int ks = 0; ks < CK; ++ks) {
@@ -402,28 +877,44 @@ __global__ __launch_bounds__(256) void output_projection_kernel(const bf16_t *__
 }
 
 struct Plan {
+    bool persistent;
     int NB, NW, BPW, GW;
     size_t lds_bytes;
 };
 
+int device_attribute(hipDeviceAttribute_t attr, int fallback)
+{
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, attr, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return fallback;
+    }
+    return v;
+}
+
 int max_lds_bytes()
 {
-    static int cached = -1;
-    if (cached < 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) {
-            (void)hipGetLastError();
-            v = 64 * 1024;
-        }
-        cached = v;
-    }
+    static const int cached = device_attribute(hipDeviceAttributeMaxSharedMemoryPerBlock, 64 * 1024);
+    return cached;
+}
+
+int num_cus()
+{
+    static const int cached = device_attribute(hipDeviceAttributeMultiprocessorCount, 256);
     return cached;
 }
 
 size_t head_kernel_lds(int C, int NB, int GW)
 {
-    return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NB * 2 * 64 * 16 * 2 + (size_t)NB * 32 * 4 + (size_t)NB * 4;
+    return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NB * 2 * 64 * 16 * 2 + (size_t)NB * 32 * 4 + 16;
+}
+
+size_t persistent_kernel_lds(int C, int NB)
+{
+    // all four weight matrices of the head, K and V of one batch row, per wave one 4 KB panel and 2 KB of
+    // parked gate fragments, mask, flags
+    return (size_t)4 * (C / 16) * 64 * 16 + (size_t)NB * 2 * 64 * 16 * 2 + (size_t)NB * (4096 + 2048) +
+           (size_t)NB * 32 * 4 + 16;
 }
 
 bool make_plan(int64_t S, int C, Plan &pl)
@@ -433,6 +924,26 @@ bool make_plan(int64_t S, int C, Plan &pl)
         return false;
     }
     pl.NB = (int)NB;
+    pl.persistent = false;
+    const size_t cap = (size_t)max_lds_bytes();
+    const char *env = getenv("KUTACC_HIP_PLAN"); // experiment hook: "p" | "bpw,gw"
+    // persistent kernel: one wave per sequence block, everything of one head resident in LDS
+    const bool fits_persistent = NB <= max_waves(C, 1) && persistent_kernel_lds(C, (int)NB) <= cap;
+    if (fits_persistent && !(env && env[0] != 'p')) {
+        pl.persistent = true;
+        pl.NW = (int)NB, pl.BPW = 1, pl.GW = 4, pl.lds_bytes = persistent_kernel_lds(C, (int)NB);
+        return true;
+    }
+    if (env && env[0] != 'p') {
+        int bpw = 0, gw = 0;
+        if (sscanf(env, "%d,%d", &bpw, &gw) == 2 && bpw >= 1 && bpw <= 4 && (gw == 1 || gw == 2 || gw == 4)) {
+            const int nw = (int)((NB + bpw - 1) / bpw);
+            if (nw <= max_waves(C, bpw) && head_kernel_lds(C, pl.NB, gw) <= cap) {
+                pl.BPW = bpw, pl.NW = nw, pl.GW = gw, pl.lds_bytes = head_kernel_lds(C, pl.NB, gw);
+                return true;
+            }
+        }
+    }
     // fewest idle wave slots first, then fewest blocks per wave (more waves to overlap MFMA and VALU)
     int best_idle = 1 << 30;
     pl.BPW = 0;
@@ -449,7 +960,6 @@ bool make_plan(int64_t S, int C, Plan &pl)
     if (pl.BPW == 0) {
         return false;
     }
-    const size_t cap = (size_t)max_lds_bytes();
     for (int gw = 4; gw >= 1; gw >>= 1) {
         const size_t need = head_kernel_lds(C, pl.NB, gw);
         if (need <= cap) {
@@ -462,32 +972,64 @@ bool make_plan(int64_t S, int C, Plan &pl)
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-template <int C, int BPW>
-int launch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t stream)
+template <typename K>
+int opt_in_lds(K kern, size_t bytes, size_t &configured)
 {
-    auto kern = fused_head_kernel<C, BPW>;
-    static size_t configured = 0; // per instantiation: largest dynamic LDS size opted into so far
-    if (pl.lds_bytes > configured) {
+    if (bytes > configured) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (e != hipSuccess) {
             return (int)e;
         }
-        configured = pl.lds_bytes;
+        configured = bytes;
+    }
+    return 0;
+}
+
+template <int C, int BPW, bool HAS_NB>
+int launch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t stream)
+{
+    auto kern = fused_head_kernel<C, BPW, HAS_NB>;
+    static size_t configured = 0; // per instantiation: largest dynamic LDS size opted into so far
+    if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
+        return rc;
     }
     const int64_t units = ((int64_t)(p.B + 7) / 8) * 8 * p.H;
     kern<<<dim3((unsigned)units), dim3((unsigned)(pl.NW * 64)), pl.lds_bytes, stream>>>(p);
     return kutacc_hip_status(hipGetLastError());
 }
 
+template <int C, bool HAS_NB>
+int launch_persistent_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
+{
+    auto kern = persistent_head_kernel<C, HAS_NB>;
+    static size_t configured = 0;
+    if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
+        return rc;
+    }
+    // one workgroup per CU at most; groups of 8*H workgroups share batch-row sequences across the XCDs
+    const int per_ring = 8 * p.H;
+    int ngrp = num_cus() / per_ring;
+    const int need = (p.B + 7) / 8;
+    ngrp = ngrp < 1 ? 1 : ngrp;
+    ngrp = ngrp > need ? need : ngrp;
+    p.ngrp = ngrp;
+    kern<<<dim3((unsigned)(per_ring * ngrp)), dim3((unsigned)(pl.NW * 64)), pl.lds_bytes, stream>>>(p);
+    return kutacc_hip_status(hipGetLastError());
+}
+
 template <int C>
 int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t stream)
 {
+    const bool nb = p.nb != nullptr;
+    if (pl.persistent) {
+        return nb ? launch_persistent_kernel<C, true>(p, pl, stream) : launch_persistent_kernel<C, false>(p, pl, stream);
+    }
     switch (pl.BPW) {
-        case 1: return launch_head_kernel<C, 1>(p, pl, stream);
-        case 2: return launch_head_kernel<C, 2>(p, pl, stream);
-        case 3: return launch_head_kernel<C, 3>(p, pl, stream);
-        case 4: return launch_head_kernel<C, 4>(p, pl, stream);
+        case 1: return nb ? launch_head_kernel<C, 1, true>(p, pl, stream) : launch_head_kernel<C, 1, false>(p, pl, stream);
+        case 2: return nb ? launch_head_kernel<C, 2, true>(p, pl, stream) : launch_head_kernel<C, 2, false>(p, pl, stream);
+        case 3: return nb ? launch_head_kernel<C, 3, true>(p, pl, stream) : launch_head_kernel<C, 3, false>(p, pl, stream);
+        case 4: return nb ? launch_head_kernel<C, 4, true>(p, pl, stream) : launch_head_kernel<C, 4, false>(p, pl, stream);
         default: return KUTACC_HIP_EUNSUPPORTED;
     }
 }
@@ -497,18 +1039,13 @@ int launch_output_projection(const kutacc_hip_attention_args_t &a, hipStream_t s
 {
     auto kern = output_projection_kernel<C>;
     const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16;
-    static bool configured = false;
-    if (!configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) {
-            return (int)e;
-        }
-        configured = true;
+    static size_t configured = 0;
+    if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
+        return rc;
     }
     const int64_t M = a.batch * a.seq_len;
     const int64_t tiles = (M + 31) / 32;
-    const int tiles_per_wg = 16;
+    const int tiles_per_wg = 4;
     const int64_t gx = (tiles + tiles_per_wg - 1) / tiles_per_wg;
     kern<<<dim3((unsigned)gx, (unsigned)(C / 128)), 256, lds_bytes, stream>>>(
         (const bf16_t *)a.avg, a.avg_stride_s, (const bf16_t *)a.output_w, a.output_b, (bf16_t *)a.out, a.out_ld, M,
@@ -565,13 +1102,19 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     p.avg_sb = a.avg_stride_b, p.avg_ss = a.avg_stride_s, p.avg_sh = a.avg_stride_h;
     p.B = (int)a.batch, p.S = (int)a.seq_len, p.H = (int)a.nheads, p.NB = pl.NB, p.NW = pl.NW, p.GW = pl.GW;
     p.nb_vec = (p.nb != nullptr && aligned(p.nb, 16) && a.nb_stride_h % 8 == 0 && a.nb_stride_q % 8 == 0) ? 1 : 0;
-    // (float)(1/sqrt(head_size)) as the reference forms it (gating_attention.cpp:68), times log2(e)
-    p.qscale = (float)(1.0 / sqrt((double)a.head_size)) * LOG2E;
+    // (float)(1/sqrt(head_size)) as the reference forms it (gating_attention.cpp:68)
+    p.qscale = (float)(1.0 / sqrt((double)a.head_size));
+    p.ngrp = 1;
 
+    if (getenv("KUTACC_HIP_DEBUG")) {
+        fprintf(stderr, "[kutacc] fused plan: persistent=%d C=%d NB=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d\n",
+                (int)pl.persistent, C, pl.NB, pl.NW, pl.BPW, pl.GW, pl.lds_bytes, max_lds_bytes(), num_cus());
+    }
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
     {
-        kutacc_prof::KernelTimer t("fused_head_kernel", 8.0 * BS * C * C + 4.0 * BS * (double)a.seq_len * C, stream);
+        kutacc_prof::KernelTimer t(pl.persistent ? "persistent_head_kernel" : "fused_head_kernel",
+                                   8.0 * BS * C * C + 4.0 * BS * (double)a.seq_len * C, stream);
         rc = (C == 128) ? dispatch_head_kernel<128>(p, pl, stream) : dispatch_head_kernel<256>(p, pl, stream);
         if (rc != 0) {
             return rc;
