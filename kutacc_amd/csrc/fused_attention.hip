@@ -453,6 +453,125 @@ __device__ __forceinline__ void attend_block(const uint4 *lds_k, const uint4 *ld
     l_out = half_swap_sum(lsum);
 }
 
+// The same attention of one 32-query block for kernels without a staging panel (long sequences, where
+// K and V fill the LDS): every lane reads the pair bias of its own query row directly, 16 consecutive
+// keys per tile, prefetched one tile ahead into registers.
+template <bool HAS_NB>
+__device__ __forceinline__ void attend_block_direct(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4,
+                                                    uint32_t flags, const bf16_t *nbrow, bool nb_vec, bf16x8 q0,
+                                                    bf16x8 q1, bf16x8 sel0, bf16x8 sel1, int NB, int S, int lane,
+                                                    f32x16 &o_out, float &l_out)
+{
+    const int g = lane >> 5;
+    f32x16 o = zero16();
+    float m_run = -1e30f; // finite, so the first rescale factor is exp2(-huge) = 0, never NaN
+    float lsum = 0.f;     // this lane's share of the row sum; the two halves are added at the end
+    uint32_t nbw[8];      // pair-bias words of the NEXT tile to be turned into logits (prefetched)
+    bf16x2 one2;
+    one2[0] = (bf16_t)1.0f, one2[1] = (bf16_t)1.0f;
+
+    // raw pair-bias of key tile t for this lane: 16 consecutive keys, two bf16 per word
+    auto fetch_nb = [&](int t) {
+        if (!HAS_NB) {
+            return;
+        }
+        const bf16_t *src = nbrow + t * 32;
+        if (nb_vec && (t + 1) * 32 <= S) {
+            const uint4 lo = *reinterpret_cast<const uint4 *>(src);
+            const uint4 hi = *reinterpret_cast<const uint4 *>(src + 8);
+            nbw[0] = lo.x, nbw[1] = lo.y, nbw[2] = lo.z, nbw[3] = lo.w;
+            nbw[4] = hi.x, nbw[5] = hi.y, nbw[6] = hi.z, nbw[7] = hi.w;
+        } else {
+            const uint16_t *s16 = reinterpret_cast<const uint16_t *>(src);
+            const int key0 = t * 32 + 16 * g;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const uint32_t a0 = key0 + 2 * v < S ? s16[2 * v] : 0u;
+                const uint32_t a1 = key0 + 2 * v + 1 < S ? s16[2 * v + 1] : 0u;
+                nbw[v] = a0 | (a1 << 16);
+            }
+        }
+    };
+    // logits^T of key tile t (rows = keys, columns = this wave's 32 queries), natural-log units
+    auto logits = [&](int t, f32x16 &x) {
+        if ((flags >> t) & 1u) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 mv = mask4[t * 8 + a];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    x[4 * a + c] = mv[c];
+                }
+            }
+        } else {
+            x = zero16();
+        }
+        if (HAS_NB) {
+            uint4 w0, w1;
+            w0.x = nbw[0], w0.y = nbw[1], w0.z = nbw[2], w0.w = nbw[3];
+            w1.x = nbw[4], w1.y = nbw[5], w1.z = nbw[6], w1.w = nbw[7];
+            x = mfma(sel0, as_bf16x8(w0), x);
+            x = mfma(sel1, as_bf16x8(w1), x);
+            if (t + 1 < NB) {
+                fetch_nb(t + 1); // in flight while this tile's MFMAs and the previous tile's softmax run
+            }
+        }
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
+    };
+    // online softmax of tile t held in xc, then O^T += V^T . P; before that, start tile t+1 into xn
+    auto step = [&](int t, f32x16 &xc, f32x16 &xn) {
+        if (t + 1 < NB) {
+            logits(t + 1, xn);
+        }
+        float mx = xc[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) {
+            mx = fmaxf(mx, xc[v]);
+        }
+        mx = half_swap_max(mx);
+        if (__any(mx > m_run + RESCALE_GAP)) {
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+            lsum *= alpha;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                o[v] *= alpha;
+            }
+            m_run = m_new;
+        }
+        const float ml = -m_run * LOG2E;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            xc[v] = __builtin_amdgcn_exp2f(fmaf(xc[v], LOG2E, ml));
+        }
+        // the row sum is taken over the bf16-rounded probabilities, two per dot2 instruction
+        const bf16x8 p0 = pack8(xc, 0), p1 = pack8(xc, 8);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            bf16x2 a, c;
+            a[0] = p0[2 * v], a[1] = p0[2 * v + 1];
+            c[0] = p1[2 * v], c[1] = p1[2 * v + 1];
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(a, one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(c, one2, lsum, false);
+        }
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 0) * 64 + lane]), p0, o);
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 1) * 64 + lane]), p1, o);
+    };
+
+    f32x16 xa, xb;
+    fetch_nb(0);
+    logits(0, xa);
+    for (int t = 0; t < NB; t += 2) {
+        step(t, xa, xb);
+        if (t + 1 < NB) {
+            step(t + 1, xb, xa);
+        }
+    }
+    o_out = o;
+    l_out = half_swap_sum(lsum);
+}
+
 // avg[b, q, h, :] = O / l * gate for the 32 queries of one block; gate values in accumulator order
 __device__ __forceinline__ void store_gated(bf16_t *dst, const f32x16 &o, float inv, const f32x16 &gate)
 {
@@ -613,10 +732,12 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             continue;
         }
         const int qpos = j * 32 + pi_row(r);
+        const int qrow = qpos < S ? qpos : S - 1;
+        const bf16_t *nbrow = HAS_NB ? p.nb + (int64_t)h * p.nb_sh + (int64_t)qrow * p.nb_sq + 16 * g : nullptr;
         f32x16 o;
         float l;
-        attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr, p.nb_sq, j * 32,
-                             p.nb_vec != 0, nullptr, qf[i][0], qf[i][1], sel0, sel1, NB, S, lane, o, l);
+        attend_block_direct<HAS_NB>(lds_k, lds_v, mask4, flags, nbrow, p.nb_vec != 0, qf[i][0], qf[i][1], sel0, sel1, NB,
+                                    S, lane, o, l);
         TL(5);
         if (qpos < S) {
             f32x16 gv;
@@ -810,21 +931,24 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     }
 }
 
-// out[t][o] = sum_c avg[t][c] * Wo[o][c] + bo[o].  Computed transposed (rows = output features,
-// columns = tokens) so that each lane owns one token row and stores 4 consecutive features at a time.
-// One workgroup stages the fragments of a 128-feature slab of Wo in LDS and walks row tiles.
+// out[t][o] = sum_c avg[t][c] * Wo[o][c] + bo[o]  (reference src/attention/gating_attention.cpp:152-157).
+// HBM-bound: each row of avg is read once and each row of out written once, both as whole cache
+// lines through the wave-private staging panel.  A workgroup stages the fragments of a 128-feature
+// slab of Wo once and its four waves walk 32-row tiles.  The product is formed transposed
+// (rows = output features, columns = tokens), which leaves every lane with 4 consecutive features
+// of its own token per accumulator group -- an 8-byte panel write.
 template <int C>
-__global__ __launch_bounds__(256) void output_projection_kernel(const bf16_t *__restrict__ avg, int64_t avg_ld,
-                                                                const bf16_t *__restrict__ wo,
-                                                                const float *__restrict__ bo, bf16_t *__restrict__ out,
-                                                                int64_t out_ld, int64_t M, int tiles_per_wg)
+__global__ __launch_bounds__(256, C == 128 ? 3 : 2) void output_projection_kernel(
+    const bf16_t *__restrict__ avg, int64_t avg_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M)
 {
     constexpr int CK = C / 16;
-    constexpr int NSLAB = 128;
-    extern __shared__ uint4 lds[]; // [4 row blocks of 32 features][CK][64 lanes]
+    constexpr int NP = CK / 4;
+    extern __shared__ uint4 lds[]; // W slab [4 feature blocks][CK][64 lanes], then 4 panels of 256
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
-    const int n0 = blockIdx.y * NSLAB;
+    const int n0 = blockIdx.y * 128;
+    uint4 *panel = lds + 4 * CK * 64 + wave * 256;
     for (int idx = tid; idx < 4 * CK * 64; idx += 256) {
         const int nb_ = idx / (CK * 64);
         const int ks = (idx >> 6) % CK;
@@ -833,43 +957,70 @@ __global__ __launch_bounds__(256) void output_projection_kernel(const bf16_t *__
         lds[idx] = *reinterpret_cast<const uint4 *>(src);
     }
     __syncthreads();
-    const int64_t tile0 = (int64_t)blockIdx.x * tiles_per_wg;
-    for (int tt = wave; tt < tiles_per_wg; tt += 4) {
-        const int64_t row0 = (tile0 + tt) * 32;
-        if (row0 >= M) {
-            break;
-        }
-        int64_t row = row0 + r;
-        const bool live = row < M;
-        row = live ? row : M - 1;
-        const bf16_t *arow = avg + row * avg_ld + g * 8;
-        f32x16 acc[4];
+    const float *bias = bo + n0 + 4 * g; // read per use: 16 cached loads per tile instead of 64 live registers
+    const int64_t tiles = (M + 31) / 32;
+    const int last_row = (int)((M - 1) & 0x7fffffff);
+    for (int64_t tile = (int64_t)blockIdx.x * 4 + wave; tile < tiles; tile += (int64_t)gridDim.x * 4) {
+        const int row0 = (int)(tile * 32);
+        bf16x8 af[CK];
+        {
+            PanelRegs ta, tb;
+            ta = panel_load(avg, avg_ld, row0, last_row, 0, lane);
 #pragma unroll
-        for (int n = 0; n < 4; ++n) {
-            acc[n] = zero16();
-        }
+            for (int c = 0; c < NP; c += 2) {
+                if (c + 1 < NP) {
+                    tb = panel_load(avg, avg_ld, row0, last_row, (c + 1) * 64, lane);
+                }
+                panel_store(panel, lane, ta);
 #pragma unroll
-        for (int ks = 0; ks < CK; ++ks) {
-            const bf16x8 af = as_bf16x8(*reinterpret_cast<const uint4 *>(arow + ks * 16));
+                for (int k = 0; k < 4; ++k) {
+                    af[4 * c + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+                }
+                if (c + 1 < NP) {
+                    if (c + 2 < NP) {
+                        ta = panel_load(avg, avg_ld, row0, last_row, (c + 2) * 64, lane);
+                    }
+                    panel_store(panel, lane, tb);
 #pragma unroll
-            for (int n = 0; n < 4; ++n) {
-                acc[n] = mfma(as_bf16x8(lds[(n * CK + ks) * 64 + lane]), af, acc[n]);
+                    for (int k = 0; k < 4; ++k) {
+                        af[4 * (c + 1) + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+                    }
+                }
             }
         }
-        if (live) {
-            bf16_t *orow = out + row * out_ld + n0 + 4 * g;
-            const float *brow = bo + n0 + 4 * g;
 #pragma unroll
-            for (int n = 0; n < 4; ++n) {
+        for (int half = 0; half < 2; ++half) { // 64 output features per panel
+            f32x16 acc[2];
+            acc[0] = zero16(), acc[1] = zero16();
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+#pragma unroll
+                for (int n = 0; n < 2; ++n) {
+                    acc[n] = mfma(as_bf16x8(lds[((2 * half + n) * CK + ks) * 64 + lane]), af[ks], acc[n]);
+                }
+            }
+            // accumulators -> panel as bf16 [row][64 features], then whole-line stores
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
 #pragma unroll
                 for (int a = 0; a < 4; ++a) {
-                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(brow + n * 32 + 8 * a);
+                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(bias + (2 * half + n) * 32 + 8 * a);
                     bf16x4 ov;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         ov[c] = (bf16_t)(acc[n][4 * a + c] + bv[c]);
                     }
-                    *reinterpret_cast<bf16x4 *>(orow + n * 32 + 8 * a) = ov;
+                    bf16x4 *dst = reinterpret_cast<bf16x4 *>(panel + panel_slot(r, n * 4 + a)) + g;
+                    *dst = ov;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int prow_ = 8 * i + (lane >> 3);
+                const uint4 v = panel[panel_slot(prow_, lane & 7)];
+                const int64_t row = (int64_t)row0 + prow_;
+                if (row < M) {
+                    *reinterpret_cast<uint4 *>(out + row * out_ld + n0 + half * 64 + (lane & 7) * 8) = v;
                 }
             }
         }
@@ -1038,18 +1189,19 @@ template <int C>
 int launch_output_projection(const kutacc_hip_attention_args_t &a, hipStream_t stream)
 {
     auto kern = output_projection_kernel<C>;
-    const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16;
+    const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16 + 4 * 4096;
     static size_t configured = 0;
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
         return rc;
     }
     const int64_t M = a.batch * a.seq_len;
     const int64_t tiles = (M + 31) / 32;
-    const int tiles_per_wg = 4;
-    const int64_t gx = (tiles + tiles_per_wg - 1) / tiles_per_wg;
+    // enough workgroups to fill the chip twice over, each walking several tiles with its staged weights
+    int64_t gx = (tiles + 3) / 4;
+    const int64_t cap = (int64_t)num_cus() * (C == 128 ? 3 : 2);
+    gx = gx > cap ? cap : gx;
     kern<<<dim3((unsigned)gx, (unsigned)(C / 128)), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a.avg, a.avg_stride_s, (const bf16_t *)a.output_w, a.output_b, (bf16_t *)a.out, a.out_ld, M,
-        tiles_per_wg);
+        (const bf16_t *)a.avg, a.avg_stride_s, (const bf16_t *)a.output_w, a.output_b, (bf16_t *)a.out, a.out_ld, M);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -1076,7 +1228,7 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
         return false;
     }
     if (a.avg_stride_h != HEAD || a.avg_stride_s % 8 != 0 || a.avg_stride_b != a.seq_len * a.avg_stride_s ||
-        !aligned(a.avg, 16) || a.out_ld % 4 != 0 || !aligned(a.out, 8)) {
+        !aligned(a.avg, 16) || a.out_ld % 8 != 0 || !aligned(a.out, 16)) {
         return false;
     }
     Plan pl;
