@@ -758,7 +758,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
 // the two big streams -- input rows and pair bias -- through wave-private staging panels with fully
 // coalesced loads.
 // LDS, 16-byte units: W[4][CK][64]  K[NB][2][64]  V[NB][2][64]  panel[NB waves][256]  gate[NB waves][2][64];
-// then floats mask[NB*32]; then one uint32 of tile flags.
+// then floats mask[NB*32]; then two uint32 of tile flags (alternating by batch row).
 // Per batch row: project (K, V -> LDS; Q, gate -> registers), barrier, attend, barrier.
 // ------------------------------------------------------------------------------------------------
 template <int C, bool HAS_NB>
@@ -791,7 +791,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     uint4 *panel = lds_v + NB * 2 * 64 + wave * 256;
     uint4 *gate_park = lds_v + NB * 2 * 64 + NB * 256 + wave * 128 + lane; // sigmoid(gate) waits here during attention
     float *mask = reinterpret_cast<float *>(lds_v + NB * 2 * 64 + NB * 256 + NB * 128);
-    uint32_t *flag_word = reinterpret_cast<uint32_t *>(mask + NB * 32);
+    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask + NB * 32); // two, alternating by batch row
 
     // the head's rows of the four weight matrices, in fragment order, for the whole kernel
     for (int idx = tid; idx < 4 * CK * 64; idx += nthreads) {
@@ -802,7 +802,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         lds_w[idx] = *reinterpret_cast<const uint4 *>(src);
     }
     if (tid == 0) {
-        *flag_word = 0;
+        flag_words[0] = 0;
+        flag_words[1] = 0;
     }
     bf16x8 sel0, sel1;
     make_selectors(lane, sel0, sel1);
@@ -812,6 +813,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     const int qpos = j * 32 + prow;
     for (int n = 0; n < nrows; ++n) {
         const int b = b0 + n * bstep;
+        uint32_t *flag_word = flag_words + (n & 1);
         if (n == 2) {
             TL(0);
         }
@@ -926,7 +928,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             TL(5);
         }
         if (tid == 0) {
-            *flag_word = 0;
+            *flag_word = 0; // clean again for the row after next; the next row ORs into the other word
         }
     }
 }
