@@ -26,6 +26,13 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (two runs, scaled against a 256 MiB copy: FETCH x2.000, WRITE x1.000; see
+# profiles/gating_attention_cfg3_hbm_traffic.txt).  Not re-measured live; configurations without an entry report null.
+MEASURED_TRAFFIC_BYTES = {
+    (3, "persistent_head_kernel"): int((27116.1 * 2.0 + 46848.0) * 1024),
+}
+
 
 def cpu_baseline(w, budget_s=15.0):
     """Time oracle Rbf16 (reference rounding points, OpenMP on all host cores) on the first rows of the
@@ -61,6 +68,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy: a kernel of known traffic to scale the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run against")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the operator shards over the batch axis with no "
@@ -80,6 +90,12 @@ def main():
     capi.set_blocking(False)
     L = capi.lib()
 
+    if a.calibrate_copy:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(a.warmup):
         op.run()
     assert not capi.error_flag()
@@ -112,7 +128,8 @@ def main():
     if dom:
         ach = dom["flops_per_launch"] / (dom["avg_ms"] * 1e-3) / 1e12
         roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                    "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.config, dom["name"])),
                     "avg_kernel_ms": round(dom["avg_ms"], 5),
                     "flops_per_launch": dom["flops_per_launch"]}
 
