@@ -68,8 +68,10 @@ typedef struct kutacc_hip_attention_args {
     int64_t nb_stride_h;
     int64_t nb_stride_q;
 
-    /* Caller scratch.  q/k/v/gate are written only by the generic path; avg (gated weighted
-     * average, [B,S,H,d]) is written by every path.  Element (b,s,h,e) of q,k,gate,avg lives at
+    /* Caller scratch.  k/v/gate are written only by the generic path; q is written by the generic
+     * path and may be used as workspace by the fused path (a fragment-major copy of the pair bias), so
+     * its contents are unspecified after any call; avg (gated weighted average, [B,S,H,d]) is
+     * written by every path.  Element (b,s,h,e) of q,k,gate,avg lives at
      * b*stride_b + s*stride_s + h*stride_h + e; v is [H,d,B,S]: (h,e,b,s) at
      * h*v_stride_h + e*v_stride_e + b*v_stride_b + s. */
     void *q, *k, *v, *gate, *avg;

@@ -54,8 +54,15 @@ extern "C" __attribute__((visibility("default"))) int kutacc_debug_timeline(unsi
 {
     return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_timeline), (size_t)n * 8);
 }
+#define TLV(i, val)                                                                           \
+    do {                                                                                      \
+        if ((blockIdx.x & 255) == 77 && (threadIdx.x & 63) == 0 && (blockIdx.x >> 8) < 8) {   \
+            g_timeline[((blockIdx.x >> 8) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = (val);     \
+        }                                                                                     \
+    } while (0)
 #else
 #define TL(i) ((void)0)
+#define TLV(i, val) ((void)0)
 #endif
 
 namespace {
@@ -90,6 +97,8 @@ struct FusedParams {
     int nb_vec;   // pair-bias rows may be read with 16-byte loads
     float qscale; // 1 / sqrt(head_size)
     int ngrp;     // persistent kernel: batch-row groups per XCD
+    const uint4 *nbf; // pair bias * log2(e) in fragment-major order (pair_bias_fragments_kernel), or nullptr
+    int l2mode;       // persistent kernel: logits in log2 units (attend_block_l2); needs nbf when there is a pair bias
 };
 
 __device__ __forceinline__ int pi_row(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
@@ -166,13 +175,13 @@ __device__ __forceinline__ void make_selectors(int lane, bf16x8 &sel0, bf16x8 &s
 // saying "this tile needs the mask added" (non-zero bias or ragged tail).  Wave w covers keys
 // [64w, 64w+64); *flag_word must have been zeroed before, with a barrier in between.
 __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *mask, uint32_t *flag_word, int S, int NB,
-                                                int wave, int lane)
+                                                int wave, int lane, float scale = 1.0f)
 {
     const int k = wave * 64 + lane;
     if (wave * 64 < NB * 32) {
         float mv = -INFINITY;
         if (k < S) {
-            mv = to_f32(bias_row[k]);
+            mv = to_f32(bias_row[k]) * scale;
         }
         if (k < NB * 32) {
             mask[k] = mv;
@@ -451,6 +460,211 @@ __device__ __forceinline__ void attend_block(const uint4 *lds_k, const uint4 *ld
     }
     o_out = o;
     l_out = half_swap_sum(lsum);
+}
+
+// ---- attention of one 32-query block in log2 units (the mode the persistent kernel runs in whenever
+// it can) ----
+// All inputs of the logits are pre-scaled by log2(e): the Q fragments by the kernel, the pair bias by
+// pair_bias_fragments_kernel, the mask bias when it is staged.  The accumulator of the logits MFMAs is
+// then the exponent itself, and the softmax of a tile is 16 v_exp_f32 and 8 packed converts -- the
+// vector ALU no longer bounds the loop.  What the VALU used to do is done by the matrix core:
+//  * no running maximum: the probabilities are 2^logit, unshifted.  Softmax is shift invariant and
+//    fp32 and bf16 both carry 8 exponent bits, so this is exact in the same sense as the shifted form
+//    as long as nothing overflows or the whole row underflows; the caller checks the row sum for
+//    that (1e-30 < l < 1e30) and repeats the block with SHIFT = true and the true row maximum
+//    (row_max_l2) when the check fails.  SHIFT costs one subtract per logit.
+//  * the row sums come from a 16x16x32 MFMA whose A operand adds up the keys of each query
+//    (rowsum_selector), fed with the same bf16 probabilities as the P.V product.
+// Every operand of a tile is fetched ahead into registers that the loop carries: K and V fragments
+// from LDS one tile ahead, pair-bias fragments from global memory two tiles ahead (two contiguous 1 KB
+// loads per tile and wave).  The 8 MFMAs of a tile sit, fenced, between the exp/convert pieces of the
+// neighbouring tile's softmax.  The loop runs one extra (clamped) logits computation at the end
+// instead of a peeled epilogue.  Requires an even number of key tiles.
+//   nbf : this wave's fragment-major pair bias, already offset by the lane: tile t at nbf[(2t+m)*64]
+//   returns the row sum of every lane's query in l_out
+
+// A operand of the row-sum MFMA (16x16x32: lane -> row lane&15, k-chunk lane>>4).  The B operand is a
+// probability fragment of the 32x32x16 layout (lane -> query lane&31, 8 keys of half lane>>5), which the
+// 16x16x32 shape reads as column lane&15, k-chunk lane>>4: chunks 0 and 2 belong to query n, chunks 1 and
+// 3 to query n+16.  Row 0 of A therefore sums chunks 0 and 2, row 1 chunks 1 and 3; the sums of
+// queries n and n+16 end up in lane n, accumulator registers 0 and 1.
+__device__ __forceinline__ bf16x8 rowsum_selector(int lane)
+{
+    const int i = lane & 15, c = lane >> 4;
+    const float v = ((i == 0 && (c & 1) == 0) || (i == 1 && (c & 1) == 1)) ? 1.0f : 0.0f;
+    bf16x8 a;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (bf16_t)v;
+    }
+    return a;
+}
+
+__device__ __forceinline__ float rowsum_fetch(const f32x4 &lacc, int lane)
+{
+    const int q = lane & 31;
+    const int src = (q & 15) * 4;
+    const float a0 = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(lacc[0])));
+    const float a1 = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(lacc[1])));
+    return (q >> 4) ? a1 : a0;
+}
+
+template <bool HAS_NB, bool WITH_MASK, bool SHIFT>
+__device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4,
+                                                const uint4 *nbf, bf16x8 q0, bf16x8 q1, bf16x8 sel0, bf16x8 sel1,
+                                                bf16x8 sumsel, int NB, int lane, float shift, f32x16 &o_out, float &l_out)
+{
+    const int npairs = NB >> 1;
+    const uint4 *kp = lds_k + lane;
+    const uint4 *vp = lds_v + lane;
+
+    auto init = [&](int t) {
+        f32x16 x;
+        if (WITH_MASK) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 mv = mask4[t * 8 + a];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    x[4 * a + c] = mv[c];
+                }
+            }
+        } else {
+            x = zero16();
+        }
+        return x;
+    };
+    auto clampt = [&](int t) { return t < NB ? t : NB - 1; };
+
+    // pair-bias words: wa* belong to even tiles, wb* to odd tiles
+    uint4 wa0 = {}, wa1 = {}, wb0 = {}, wb1 = {}, k0, k1, v0, v1;
+    if (HAS_NB) {
+        wa0 = nbf[0], wa1 = nbf[64];
+        wb0 = nbf[2 * 64], wb1 = nbf[3 * 64];
+    }
+    k0 = kp[0], k1 = kp[64];
+    f32x16 xa = init(0), xb;
+    if (HAS_NB) {
+        xa = mfma(sel0, as_bf16x8(wa0), xa);
+        xa = mfma(sel1, as_bf16x8(wa1), xa);
+        wa0 = nbf[clampt(2) * 128], wa1 = nbf[clampt(2) * 128 + 64];
+    }
+    xa = mfma(as_bf16x8(k0), q0, xa);
+    xa = mfma(as_bf16x8(k1), q1, xa);
+    k0 = kp[2 * 64], k1 = kp[3 * 64];
+    v0 = vp[0], v1 = vp[64];
+
+    f32x16 o = zero16();
+    f32x4 lacc = {0.f, 0.f, 0.f, 0.f};
+
+    auto exp4 = [&](f32x16 &x, int base) {
+#pragma unroll
+        for (int v = base; v < base + 4; ++v) {
+#ifdef KUTACC_EXP_NOEXP
+            x[v] = SHIFT ? x[v] - shift : x[v] * 1.0001f;
+#else
+            x[v] = __builtin_amdgcn_exp2f(SHIFT ? x[v] - shift : x[v]);
+#endif
+        }
+    };
+    auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+    // One half step: the softmax and P.V of the finished tile `xc`, with the logits MFMAs of the
+    // following tile `xn` (pair-bias words w0, w1) spread between its pieces; t_w is the tile whose
+    // pair-bias words replace w0, w1 once consumed, t_k the tile whose K fragments replace k0, k1.
+    auto half_step = [&](f32x16 &xc, f32x16 &xn, int t_next, uint4 &w0, uint4 &w1, int t_w, int t_k) {
+        bf16x8 p0, p1;
+        xn = init(t_next);
+        if (HAS_NB) {
+#ifndef KUTACC_EXP_NOSEL
+            xn = mfma(sel0, as_bf16x8(w0), xn);
+#endif
+            exp4(xc, 0);
+            fence();
+#ifndef KUTACC_EXP_NOSEL
+            xn = mfma(sel1, as_bf16x8(w1), xn);
+#endif
+#ifndef KUTACC_EXP_NOW
+            w0 = nbf[t_w * 128], w1 = nbf[t_w * 128 + 64];
+#endif
+            exp4(xc, 4);
+            p0 = pack8(xc, 0);
+            fence();
+        } else {
+            exp4(xc, 0);
+            exp4(xc, 4);
+            p0 = pack8(xc, 0);
+            fence();
+        }
+        xn = mfma(as_bf16x8(k0), q0, xn);
+        o = mfma(as_bf16x8(v0), p0, o);
+        exp4(xc, 8);
+        fence();
+        xn = mfma(as_bf16x8(k1), q1, xn);
+#ifndef KUTACC_EXP_NOSUM
+        lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sumsel, p0, lacc, 0, 0, 0);
+#endif
+#ifndef KUTACC_EXP_NOKV
+        k0 = kp[(t_k * 2 + 0) * 64], k1 = kp[(t_k * 2 + 1) * 64];
+#endif
+        exp4(xc, 12);
+        p1 = pack8(xc, 8);
+        fence();
+        o = mfma(as_bf16x8(v1), p1, o);
+#ifndef KUTACC_EXP_NOSUM
+        lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sumsel, p1, lacc, 0, 0, 0);
+#endif
+    };
+
+    for (int pair = 0; pair < npairs; ++pair) {
+        const int t1 = 2 * pair + 1;
+        const int tn = pair + 1 < npairs ? 2 * pair + 2 : 2 * pair; // next pair's first tile, clamped
+        // ---- odd tile's logits under the even tile's softmax ----
+        half_step(xa, xb, t1, wb0, wb1, clampt(t1 + 2), tn);
+#ifndef KUTACC_EXP_NOKV
+        v0 = vp[(t1 * 2 + 0) * 64], v1 = vp[(t1 * 2 + 1) * 64];
+#endif
+        fence();
+        // ---- next pair's even tile under the odd tile's softmax ----
+        half_step(xb, xa, tn, wa0, wa1, clampt(tn + 2), tn + 1);
+#ifndef KUTACC_EXP_NOKV
+        v0 = vp[(tn * 2 + 0) * 64], v1 = vp[(tn * 2 + 1) * 64];
+#endif
+        fence();
+    }
+    o_out = o;
+    l_out = rowsum_fetch(lacc, lane);
+}
+
+// Row maxima of the logits (log2 units) of one 32-query block over all key tiles: the shift for the
+// repeat of attend_block_l2 after an overflow or underflow.  Not a hot path: operands are loaded at use.
+template <bool HAS_NB>
+__device__ __forceinline__ float row_max_l2(const uint4 *lds_k, const f32x4 *mask4, const uint4 *nbf, bf16x8 q0, bf16x8 q1,
+                                            bf16x8 sel0, bf16x8 sel1, int NB, int lane)
+{
+    float mx = -INFINITY;
+    for (int t = 0; t < NB; ++t) {
+        f32x16 x;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const f32x4 mv = mask4[t * 8 + a];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                x[4 * a + c] = mv[c];
+            }
+        }
+        if (HAS_NB) {
+            x = mfma(sel0, as_bf16x8(nbf[t * 128]), x);
+            x = mfma(sel1, as_bf16x8(nbf[t * 128 + 64]), x);
+        }
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            mx = fmaxf(mx, x[v]);
+        }
+    }
+    mx = half_swap_max(mx);
+    return mx; // finite: a fully masked row has -1e9*log2(e) everywhere
 }
 
 // The same attention of one 32-query block for kernels without a staging panel (long sequences, where
@@ -810,6 +1024,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     __syncthreads();
 
     const int j = wave; // this wave's sequence block
+    const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
+    const bf16x8 sumsel = rowsum_selector(lane);
     const int qpos = j * 32 + prow;
     for (int n = 0; n < nrows; ++n) {
         const int b = b0 + n * bstep;
@@ -817,7 +1033,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == 2) {
             TL(0);
         }
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, wave, lane);
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, wave, lane, p.l2mode ? LOG2E : 1.0f);
 
         // ---- input rows of the block -> fragments, 64 channels per staging panel ----
         const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
@@ -847,6 +1063,17 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                 }
             }
         }
+#ifdef KUTACC_OPT_TOUCH
+        // pull the next batch row's input block towards the L2 (one line per lane) while this row is
+        // projected; the value is only there to be waited for
+        uint32_t touch = 0;
+        if (n + 1 < nrows) {
+            const bf16_t *xn_ = p.x + (int64_t)(b + bstep) * S * p.x_ld;
+            int trow = j * 32 + (lane >> 1);
+            trow = trow < S ? trow : S - 1;
+            touch = *reinterpret_cast<const uint32_t *>(xn_ + (int64_t)trow * p.x_ld + (lane & 1) * 64);
+        }
+#endif
         if (n == 2) {
             TL(1);
         }
@@ -875,7 +1102,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                acc[v] *= p.qscale;
+                acc[v] *= qmul;
             }
             q0 = pack8(acc, 0);
             q1 = pack8(acc, 8);
@@ -899,6 +1126,9 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == 2) {
             TL(2);
         }
+#ifdef KUTACC_OPT_TOUCH
+        asm volatile("" ::"v"(touch));
+#endif
         __syncthreads(); // K, V and the mask of this batch row are complete
         if (n == 2) {
             TL(3);
@@ -907,8 +1137,30 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
         f32x16 o;
         float l;
-        attend_block<HAS_NB>(lds_k, lds_v, mask4, *flag_word, HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr, p.nb_sq,
-                             j * 32, p.nb_vec != 0, panel, q0, q1, sel0, sel1, NB, S, lane, o, l);
+        const uint32_t flags = *flag_word;
+        const bf16_t *nb_head = HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr;
+        if (p.l2mode) {
+            const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NB * 2) * 64 + lane : nullptr;
+            if (flags == 0u) {
+                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NB, lane, 0.f, o,
+                                                      l);
+            } else {
+                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NB, lane, 0.f, o,
+                                                     l);
+            }
+            const bool ok = !__any(!(l > 1e-30f && l < 1e30f));
+            if (n == 2) {
+                TLV(6, ok ? 1 : 0);
+            }
+            if (!ok) {
+                // some probability overflowed or a whole row underflowed: shift by the true row maxima
+                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, q0, q1, sel0, sel1, NB, lane);
+                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NB, lane, m, o, l);
+            }
+        } else {
+            attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, nb_head, p.nb_sq, j * 32, p.nb_vec != 0, panel, q0, q1, sel0,
+                                 sel1, NB, S, lane, o, l);
+        }
         if (qpos < S) {
             const bf16x8 gate0 = as_bf16x8(gate_park[0]), gate1 = as_bf16x8(gate_park[64]);
             f32x16 gv;
@@ -1027,6 +1279,52 @@ __global__ __launch_bounds__(256, C == 128 ? 3 : 2) void output_projection_kerne
             }
         }
     }
+}
+
+// Pair bias [H, S, S] -> fragment-major order: for head h, query block j and key tile t the two B
+// operands of the selector MFMAs, [h][j][t][2][64 lanes] x 16 bytes, so that a wave of the attention
+// kernels fetches the pair bias of a tile with two contiguous 1 KB loads straight into registers.
+// Lane (r, g) holds 16 consecutive keys 32t+16g.. of query row 32j+pi(r); queries past S repeat row
+// S-1 and keys past S read as zero (their mask bias is -inf).  The pair bias is shared by every batch
+// row, so this pass moves 2*H*S*S bytes once per call, against B times that in the attention kernel.
+__global__ __launch_bounds__(64) void pair_bias_fragments_kernel(const bf16_t *__restrict__ nb, int64_t nb_sh,
+                                                                 int64_t nb_sq, int S, int NB, int vec,
+                                                                 uint4 *__restrict__ out)
+{
+    const int lane = threadIdx.x;
+    const int r = lane & 31, g = lane >> 5;
+    const int t = blockIdx.x % NB, j = blockIdx.x / NB, h = blockIdx.y;
+    int q = 32 * j + pi_row(r);
+    q = q < S ? q : S - 1;
+    const int key0 = 32 * t + 16 * g;
+    const bf16_t *src = nb + (int64_t)h * nb_sh + (int64_t)q * nb_sq + key0;
+    uint4 w0, w1;
+    if (vec && key0 + 16 <= S) {
+        w0 = *reinterpret_cast<const uint4 *>(src);
+        w1 = *reinterpret_cast<const uint4 *>(src + 8);
+    } else {
+        const uint16_t *s16 = reinterpret_cast<const uint16_t *>(src);
+        uint32_t wds[8];
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            const uint32_t a0 = key0 + 2 * v < S ? s16[2 * v] : 0u;
+            const uint32_t a1 = key0 + 2 * v + 1 < S ? s16[2 * v + 1] : 0u;
+            wds[v] = a0 | (a1 << 16);
+        }
+        w0.x = wds[0], w0.y = wds[1], w0.z = wds[2], w0.w = wds[3];
+        w1.x = wds[4], w1.y = wds[5], w1.z = wds[6], w1.w = wds[7];
+    }
+    // into log2 units, rounded to bf16 again (the logits MFMAs of attend_block_l2 accumulate exponents of 2)
+    const bf16x8 s0 = as_bf16x8(w0), s1 = as_bf16x8(w1);
+    bf16x8 d0, d1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        d0[e] = (bf16_t)(to_f32(s0[e]) * LOG2E);
+        d1[e] = (bf16_t)(to_f32(s1[e]) * LOG2E);
+    }
+    uint4 *dst = out + ((((int64_t)h * NB + j) * NB + t) * 2) * 64 + lane;
+    dst[0] = as_uint4(d0);
+    dst[64] = as_uint4(d1);
 }
 
 struct Plan {
@@ -1259,6 +1557,17 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     // (float)(1/sqrt(head_size)) as the reference forms it (gating_attention.cpp:68)
     p.qscale = (float)(1.0 / sqrt((double)a.head_size));
     p.ngrp = 1;
+    p.nbf = nullptr;
+    p.l2mode = 0;
+    // Fragment-major copy of the pair bias for the fast attention loop.  It lives in the caller's q
+    // scratch tensor (which this path does not otherwise use; its contents are unspecified after any
+    // call) when that is dense, aligned and large enough; otherwise the kernels read the pair bias in
+    // place through the staging panels.
+    const int64_t nbf_bytes = (int64_t)a.nheads * pl.NB * pl.NB * 2048;
+    const bool q_dense = a.q != nullptr && aligned(a.q, 16) && a.q_stride_h == a.head_size && a.q_stride_s == C &&
+                         a.q_stride_b == a.seq_len * C;
+    const bool want_fragments = p.nb != nullptr && pl.persistent && a.seq_len % 64 == 0 && q_dense &&
+                                nbf_bytes <= a.batch * a.seq_len * C * 2 && !getenv("KUTACC_HIP_NO_FRAGMENTS");
 
     if (getenv("KUTACC_HIP_DEBUG")) {
         fprintf(stderr, "[kutacc] fused plan: persistent=%d C=%d NB=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d\n",
@@ -1266,6 +1575,20 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     }
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
+    if (want_fragments) {
+        kutacc_prof::KernelTimer t("pair_bias_fragments_kernel", 0.0, stream);
+        pair_bias_fragments_kernel<<<dim3((unsigned)(pl.NB * pl.NB), (unsigned)a.nheads), 64, 0, stream>>>(
+            p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.nb_vec, (uint4 *)a.q);
+        rc = kutacc_hip_status(hipGetLastError());
+        if (rc != 0) {
+            return rc;
+        }
+        p.nbf = (const uint4 *)a.q;
+    }
+    p.l2mode = (pl.persistent && a.seq_len % 64 == 0 && (p.nb == nullptr || p.nbf != nullptr) &&
+                !getenv("KUTACC_HIP_NO_FRAGMENTS"))
+                   ? 1
+                   : 0;
     {
         kutacc_prof::KernelTimer t(pl.persistent ? "persistent_head_kernel" : "fused_head_kernel",
                                    8.0 * BS * C * C + 4.0 * BS * (double)a.seq_len * C, stream);
