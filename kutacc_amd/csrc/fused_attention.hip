@@ -98,7 +98,7 @@ struct FusedParams {
     float qscale; // 1 / sqrt(head_size)
     int ngrp;     // persistent kernel: batch-row groups per XCD
     const uint4 *nbf; // pair bias * log2(e) in fragment-major order (pair_bias_fragments_kernel), or nullptr
-    int l2mode;       // persistent kernel: logits in log2 units (attend_block_l2); needs nbf when there is a pair bias
+    int l2mode;       // logits in log2 units (attend_block_l2); needs nbf when there is a pair bias
 };
 
 __device__ __forceinline__ int pi_row(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
@@ -847,9 +847,10 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     }
     __syncthreads();
     for (int part = wave; part * 64 < NB * 32; part += NW) {
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, part, lane);
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, part, lane, p.l2mode ? LOG2E : 1.0f);
     }
 
+    const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
     // ---- projections, in groups of GW weight matrices staged through LDS ----
     bf16x8 qf[BPW][2];   // Q^T fragments (B operand of the logits MFMA), scaled by 1/sqrt(d)
     bf16x8 gate[BPW][2]; // sigmoid(gate) in accumulator order, packed
@@ -908,7 +909,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
                     } else if (m == PROJ_Q) {
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            acc[v] *= p.qscale;
+                            acc[v] *= qmul;
                         }
                         qf[i][0] = pack8(acc, 0);
                         qf[i][1] = pack8(acc, 8);
@@ -938,6 +939,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
     bf16x8 sel0, sel1;
     make_selectors(lane, sel0, sel1);
+    const bf16x8 sumsel = rowsum_selector(lane);
 
 #pragma unroll
     for (int i = 0; i < BPW; ++i) {
@@ -947,11 +949,28 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         }
         const int qpos = j * 32 + pi_row(r);
         const int qrow = qpos < S ? qpos : S - 1;
-        const bf16_t *nbrow = HAS_NB ? p.nb + (int64_t)h * p.nb_sh + (int64_t)qrow * p.nb_sq + 16 * g : nullptr;
         f32x16 o;
         float l;
-        attend_block_direct<HAS_NB>(lds_k, lds_v, mask4, flags, nbrow, p.nb_vec != 0, qf[i][0], qf[i][1], sel0, sel1, NB,
-                                    S, lane, o, l);
+        if (p.l2mode) {
+            const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NB * 2) * 64 + lane : nullptr;
+            if (flags == 0u) {
+                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NB,
+                                                      lane, 0.f, o, l);
+            } else {
+                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NB,
+                                                     lane, 0.f, o, l);
+            }
+            if (__any(!(l > 1e-30f && l < 1e30f))) {
+                // some probability overflowed or a whole row underflowed: shift by the true row maxima
+                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, NB, lane);
+                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NB,
+                                                    lane, m, o, l);
+            }
+        } else {
+            const bf16_t *nbrow = HAS_NB ? p.nb + (int64_t)h * p.nb_sh + (int64_t)qrow * p.nb_sq + 16 * g : nullptr;
+            attend_block_direct<HAS_NB>(lds_k, lds_v, mask4, flags, nbrow, p.nb_vec != 0, qf[i][0], qf[i][1], sel0, sel1, NB,
+                                        S, lane, o, l);
+        }
         TL(5);
         if (qpos < S) {
             f32x16 gv;
@@ -981,6 +1000,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     constexpr int CK = C / 16;
     constexpr int NP = CK / 4; // staging panels (64 channels each) per input row block
     extern __shared__ uint4 lds[];
+    TL(7);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
@@ -1023,6 +1043,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     make_selectors(lane, sel0, sel1);
     __syncthreads();
 
+    TL(8);
     const int j = wave; // this wave's sequence block
     const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
     const bf16x8 sumsel = rowsum_selector(lane);
@@ -1032,6 +1053,12 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         uint32_t *flag_word = flag_words + (n & 1);
         if (n == 2) {
             TL(0);
+        }
+        if (n == 1) {
+            TL(9);
+        }
+        if (n == nrows - 1) {
+            TL(10);
         }
         stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, wave, lane, p.l2mode ? LOG2E : 1.0f);
 
@@ -1183,6 +1210,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             *flag_word = 0; // clean again for the row after next; the next row ORs into the other word
         }
     }
+    TL(11);
 }
 
 // out[t][o] = sum_c avg[t][c] * Wo[o][c] + bo[o]  (reference src/attention/gating_attention.cpp:152-157).
@@ -1566,7 +1594,7 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     const int64_t nbf_bytes = (int64_t)a.nheads * pl.NB * pl.NB * 2048;
     const bool q_dense = a.q != nullptr && aligned(a.q, 16) && a.q_stride_h == a.head_size && a.q_stride_s == C &&
                          a.q_stride_b == a.seq_len * C;
-    const bool want_fragments = p.nb != nullptr && pl.persistent && a.seq_len % 64 == 0 && q_dense &&
+    const bool want_fragments = p.nb != nullptr && a.seq_len % 64 == 0 && q_dense &&
                                 nbf_bytes <= a.batch * a.seq_len * C * 2 && !getenv("KUTACC_HIP_NO_FRAGMENTS");
 
     if (getenv("KUTACC_HIP_DEBUG")) {
@@ -1585,7 +1613,7 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
         }
         p.nbf = (const uint4 *)a.q;
     }
-    p.l2mode = (pl.persistent && a.seq_len % 64 == 0 && (p.nb == nullptr || p.nbf != nullptr) &&
+    p.l2mode = (a.seq_len % 64 == 0 && (p.nb == nullptr || p.nbf != nullptr) &&
                 !getenv("KUTACC_HIP_NO_FRAGMENTS"))
                    ? 1
                    : 0;
