@@ -1220,9 +1220,9 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 // (rows = output features, columns = tokens), which leaves every lane with 4 consecutive features
 // of its own token per accumulator group -- an 8-byte panel write.
 template <int C>
-__global__ __launch_bounds__(256, C == 128 ? 3 : 2) void output_projection_kernel(
+__global__ __launch_bounds__(256, 2) void output_projection_kernel(
     const bf16_t *__restrict__ avg, int64_t avg_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
-    bf16_t *__restrict__ out, int64_t out_ld, int64_t M)
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave)
 {
     constexpr int CK = C / 16;
     constexpr int NP = CK / 4;
@@ -1231,44 +1231,64 @@ __global__ __launch_bounds__(256, C == 128 ? 3 : 2) void output_projection_kerne
     const int r = lane & 31, g = lane >> 5;
     const int n0 = blockIdx.y * 128;
     uint4 *panel = lds + 4 * CK * 64 + wave * 256;
-    for (int idx = tid; idx < 4 * CK * 64; idx += 256) {
-        const int nb_ = idx / (CK * 64);
-        const int ks = (idx >> 6) % CK;
-        const int ln = idx & 63;
-        const bf16_t *src = wo + (int64_t)(n0 + nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8;
-        lds[idx] = *reinterpret_cast<const uint4 *>(src);
+    const float *bias = bo + n0 + 4 * g; // read per use: 16 cached loads per tile instead of 64 live registers
+    // Every wave owns a contiguous range of rows_per_wave rows (a multiple of 8), walked 32 rows at a
+    // time; the last step of a range may be partial.  Equal ranges rather than whole 32-row tiles dealt
+    // round robin: the kernel is short, and a wave with one tile more than its neighbours would set its
+    // duration.  The first two panels of a step are fetched while the previous step is multiplied and
+    // stored; those of the first step while the weight slab is staged.
+    const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
+    const int64_t stop = start + rows_per_wave < M ? start + rows_per_wave : M;
+    const int last_row = (int)(stop - 1);
+    PanelRegs ta, tb;
+    if (start < stop) {
+        ta = panel_load(avg, avg_ld, (int)start, last_row, 0, lane);
+        tb = panel_load(avg, avg_ld, (int)start, last_row, 64, lane);
+    }
+    {
+        constexpr int PER = 4 * CK * 64 / 256; // weight fragments per thread, all loads issued before the first store
+        uint4 wreg[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = tid + i * 256;
+            const int nb_ = idx / (CK * 64);
+            const int ks = (idx >> 6) % CK;
+            const int ln = idx & 63;
+            wreg[i] = *reinterpret_cast<const uint4 *>(wo + (int64_t)(n0 + nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            lds[tid + i * 256] = wreg[i];
+        }
     }
     __syncthreads();
-    const float *bias = bo + n0 + 4 * g; // read per use: 16 cached loads per tile instead of 64 live registers
-    const int64_t tiles = (M + 31) / 32;
-    const int last_row = (int)((M - 1) & 0x7fffffff);
-    for (int64_t tile = (int64_t)blockIdx.x * 4 + wave; tile < tiles; tile += (int64_t)gridDim.x * 4) {
-        const int row0 = (int)(tile * 32);
+    for (int64_t rbase = start; rbase < stop; rbase += 32) {
+        const int row0 = (int)rbase;
         bf16x8 af[CK];
-        {
-            PanelRegs ta, tb;
-            ta = panel_load(avg, avg_ld, row0, last_row, 0, lane);
+        panel_store(panel, lane, ta);
 #pragma unroll
-            for (int c = 0; c < NP; c += 2) {
-                if (c + 1 < NP) {
-                    tb = panel_load(avg, avg_ld, row0, last_row, (c + 1) * 64, lane);
-                }
-                panel_store(panel, lane, ta);
+        for (int k = 0; k < 4; ++k) {
+            af[k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+        }
+        panel_store(panel, lane, tb);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    af[4 * c + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
-                }
-                if (c + 1 < NP) {
-                    if (c + 2 < NP) {
-                        ta = panel_load(avg, avg_ld, row0, last_row, (c + 2) * 64, lane);
-                    }
-                    panel_store(panel, lane, tb);
+        for (int k = 0; k < 4; ++k) {
+            af[4 + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+        }
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        af[4 * (c + 1) + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
-                    }
-                }
+        for (int c = 2; c < NP; ++c) {
+            ta = panel_load(avg, avg_ld, row0, last_row, c * 64, lane);
+            panel_store(panel, lane, ta);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                af[4 * c + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
             }
+        }
+        {
+            // clamped to the last step instead of a branch: one harmless re-read at the end
+            const int rnext = rbase + 32 < stop ? row0 + 32 : row0;
+            ta = panel_load(avg, avg_ld, rnext, last_row, 0, lane);
+            tb = panel_load(avg, avg_ld, rnext, last_row, 64, lane);
         }
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
@@ -1301,7 +1321,7 @@ __global__ __launch_bounds__(256, C == 128 ? 3 : 2) void output_projection_kerne
                 const int prow_ = 8 * i + (lane >> 3);
                 const uint4 v = panel[panel_slot(prow_, lane & 7)];
                 const int64_t row = (int64_t)row0 + prow_;
-                if (row < M) {
+                if (row < stop) {
                     *reinterpret_cast<uint4 *>(out + row * out_ld + n0 + half * 64 + (lane & 7) * 8) = v;
                 }
             }
@@ -1524,12 +1544,14 @@ int launch_output_projection(const kutacc_hip_attention_args_t &a, hipStream_t s
     }
     const int64_t M = a.batch * a.seq_len;
     const int64_t tiles = (M + 31) / 32;
-    // enough workgroups to fill the chip twice over, each walking several tiles with its staged weights
+    // two resident workgroups per CU, each wave with an equal share of the rows
     int64_t gx = (tiles + 3) / 4;
-    const int64_t cap = (int64_t)num_cus() * (C == 128 ? 3 : 2);
+    const int64_t cap = (int64_t)num_cus() * 2;
     gx = gx > cap ? cap : gx;
+    const int64_t rpw = ((M + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
     kern<<<dim3((unsigned)gx, (unsigned)(C / 128)), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a.avg, a.avg_stride_s, (const bf16_t *)a.output_w, a.output_b, (bf16_t *)a.out, a.out_ld, M);
+        (const bf16_t *)a.avg, a.avg_stride_s, (const bf16_t *)a.output_w, a.output_b, (bf16_t *)a.out, a.out_ld, M,
+        (int)rpw);
     return kutacc_hip_status(hipGetLastError());
 }
 
