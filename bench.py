@@ -61,6 +61,58 @@ def cpu_baseline(w, budget_s=15.0):
     }
 
 
+def producer_rates(config, reps=50):
+    """Achieved HBM rates of the two row kernels in front of the operator, at this configuration's pair
+    tensor z [S, S, 128]: LayerNorm over all rows, and the fused LN -> [H, c_z] projection -> [H, S, S] pair
+    bias (with and without writing the normalised z).  Algorithmic bytes: rows*c_z*2 read, plus what is
+    written (rows*c_z*2 for LN / z_norm, rows*H*2 for the pair bias)."""
+    import numpy as np
+    import torch
+    from kutacc_amd import capi
+    from kutacc_amd.workloads import make_workload
+
+    w = make_workload(config, batch=2, keep_extras=True)
+    if "z" not in w.extras:
+        return None
+    z, wb = w.extras["z"], w.extras["w_bias"]
+    S, cz, H = z.shape[0], z.shape[-1], wb.shape[0]
+    dz = torch.from_numpy(z).cuda().to(torch.bfloat16)
+    dw = torch.from_numpy(wb).cuda().to(torch.bfloat16)
+    dg = torch.ones(cz, device="cuda", dtype=torch.float32)
+    db = torch.zeros(cz, device="cuda", dtype=torch.float32)
+    nb = torch.empty((H, S, S), device="cuda", dtype=torch.bfloat16)
+    zn = torch.empty_like(dz)
+    L = capi.lib()
+    rows = S * S
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    t_ln = timed(lambda: L.kutacc_hip_layernorm_rows(dz.data_ptr(), cz, dg.data_ptr(), db.data_ptr(), zn.data_ptr(), cz,
+                                                     rows, cz, 1e-5, capi.K_BF16, stream))
+    t_pb = timed(lambda: L.kutacc_hip_pair_bias(dz.data_ptr(), dg.data_ptr(), db.data_ptr(), dw.data_ptr(), nb.data_ptr(),
+                                                None, S, S, cz, H, 1e-5, capi.K_BF16, stream))
+    t_pbz = timed(lambda: L.kutacc_hip_pair_bias(dz.data_ptr(), dg.data_ptr(), db.data_ptr(), dw.data_ptr(), nb.data_ptr(),
+                                                 zn.data_ptr(), S, S, cz, H, 1e-5, capi.K_BF16, stream))
+    zb = rows * cz * 2
+    return {
+        "shape": f"z [{S},{S},{cz}] bf16, H={H}",
+        "layernorm_rows": {"us": round(t_ln * 1e6, 2), "GB/s": round(2 * zb / t_ln / 1e9, 1)},
+        "pair_bias": {"us": round(t_pb * 1e6, 2), "GB/s": round((zb + rows * H * 2) / t_pb / 1e9, 1)},
+        "pair_bias_with_z_norm": {"us": round(t_pbz * 1e6, 2), "GB/s": round((2 * zb + rows * H * 2) / t_pbz / 1e9, 1)},
+        "hbm_peak_GB/s": HBM_PEAK_GBS,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -71,6 +123,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy: a kernel of known traffic to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run against")
+    ap.add_argument("--producers", action="store_true",
+                    help="also time the LayerNorm and pair-bias producer kernels at this configuration's pair tensor "
+                         "and report their HBM rates in a \"producers\" object")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the operator shards over the batch axis with no "
@@ -149,6 +204,8 @@ def main():
         "roofline": roofline,
         "cpu_baseline": None if a.no_cpu else cpu_baseline(w),
     }
+    if a.producers:
+        rec["producers"] = producer_rates(a.config)
     print(json.dumps(rec))
 
 

@@ -105,10 +105,218 @@ __global__ __launch_bounds__(64 * ROW_WAVES) void pair_bias_kernel(const T *__re
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// bf16 fast paths (row length a multiple of 8 with row_len/8 in {8, 16, 32, 64} lanes per row, rows
+// and tensors 16-byte aligned).  A row is spread over LPR = row_len/8 lanes, 16 bytes each, so every
+// load and store instruction moves whole cache lines and 64/LPR rows; sums run over the LPR lanes
+// with DPP adds (no LDS traffic) up to 16 lanes and lane shuffles above.  Same arithmetic as the
+// generic kernels: shift by the row's first element, fp32 sums, clamped variance.
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(moved);
+}
+
+// sum over the LPR lanes that hold one row; every lane of the group gets the total
+template <int LPR>
+__device__ __forceinline__ float group_sum(float v)
+{
+    v = dpp_add<0xB1>(v);  // quad_perm [1,0,3,2]: lane ^ 1
+    v = dpp_add<0x4E>(v);  // quad_perm [2,3,0,1]: lane ^ 2
+    v = dpp_add<0x141>(v); // row_half_mirror: pairs the two quads of 8 lanes
+    if (LPR >= 16) {
+        v = dpp_add<0x140>(v); // row_mirror: pairs the two halves of 16 lanes
+    }
+    if (LPR >= 32) {
+        v += __shfl_xor(v, 16, 64);
+    }
+    if (LPR >= 64) {
+        v += __shfl_xor(v, 32, 64);
+    }
+    return v;
+}
+
+union Pack16 {
+    uint4 u;
+    bf16x8 b;
+    bf16x2 p[4];
+};
+
+// statistics of one row held as 8 values per lane; x0 = first element of the row
+template <int LPR>
+__device__ __forceinline__ void group_stats(const float (&x)[8], float x0, float n, float eps, float &rstd, float &shift)
+{
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float v = x[e] - x0;
+        s1 += v;
+        s2 = fmaf(v, v, s2);
+    }
+    s1 = group_sum<LPR>(s1);
+    s2 = group_sum<LPR>(s2);
+    const float mean = s1 / n + x0;
+    const float var = fmaxf((s2 - s1 * s1 / n) / n, 0.f);
+    rstd = 1.0f / sqrtf(var + eps);
+    shift = -rstd * mean;
+}
+
+template <int LPR>
+__global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *__restrict__ x, int64_t ld_x,
+                                                                  const float *__restrict__ gamma,
+                                                                  const float *__restrict__ beta, bf16_t *__restrict__ out,
+                                                                  int64_t ld_out, int64_t rows, float eps)
+{
+    constexpr int RPS = 64 / LPR; // rows per step of a wave
+    constexpr int U = 4;          // steps in flight
+    const int lane = threadIdx.x & 63;
+    const int sub = lane % LPR, grp = lane / LPR;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    float gm[8], bt[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        gm[e] = gamma[sub * 8 + e];
+        bt[e] = beta[sub * 8 + e];
+    }
+    const int64_t r0 = wave * (RPS * U);
+    Pack16 in[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        int64_t r = r0 + u * RPS + grp;
+        r = r < rows ? r : rows - 1;
+        in[u].u = *reinterpret_cast<const uint4 *>(x + r * ld_x + sub * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t r = r0 + u * RPS + grp;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[e] = (float)in[u].b[e];
+        }
+        const float x0 = __shfl(v[0], grp * LPR, 64);
+        float rstd, shift;
+        group_stats<LPR>(v, x0, (float)(LPR * 8), eps, rstd, shift);
+        Pack16 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            o.b[e] = (bf16_t)fmaf(fmaf(v[e], rstd, shift), gm[e], bt[e]);
+        }
+        if (r < rows) {
+            *reinterpret_cast<uint4 *>(out + r * ld_out + sub * 8) = o.u;
+        }
+    }
+}
+
+// Pair-bias producer, bf16, c_z = 128 (16 lanes per row), H <= 8.  A wave owns 64 consecutive rows of
+// z; its four 16-lane groups walk 16 rows each (all 16 loads of a lane are issued up front: 16 KB in
+// flight per wave).  The normalised row is rounded to bf16, as a caller of the reference would hand it
+// to kutacc_af2_linear, and dotted with the H weight rows by packed bf16 dot products with fp32
+// accumulation.  Lane 16q+s keeps the results of the row that group q handled in step s, so that at the end
+// lane L holds the H results of row r0+L and every head's 64 values leave as one 128-byte store.
+template <int H>
+__global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__restrict__ z, const float *__restrict__ gamma,
+                                                             const float *__restrict__ beta, const bf16_t *__restrict__ w,
+                                                             bf16_t *__restrict__ nb, bf16_t *__restrict__ z_norm,
+                                                             int64_t rows, float eps)
+{
+    constexpr int LPR = 16, CZ = 128;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & 15, grp = lane >> 4;
+    const int64_t r0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;
+    if (r0 >= rows) {
+        return;
+    }
+    Pack16 in[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        int64_t r = r0 + grp * 16 + s;
+        r = r < rows ? r : rows - 1;
+        in[s].u = *reinterpret_cast<const uint4 *>(z + r * CZ + sub * 8);
+    }
+    float gm[8], bt[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        gm[e] = gamma[sub * 8 + e];
+        bt[e] = beta[sub * 8 + e];
+    }
+    Pack16 wv[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+        wv[h].u = *reinterpret_cast<const uint4 *>(w + h * CZ + sub * 8);
+    }
+    float keep[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+        keep[h] = 0.f;
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        const int64_t r = r0 + grp * 16 + s;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[e] = (float)in[s].b[e];
+        }
+        const float x0 = __shfl(v[0], grp * 16, 64);
+        float rstd, shift;
+        group_stats<LPR>(v, x0, (float)CZ, eps, rstd, shift);
+        Pack16 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            o.b[e] = (bf16_t)fmaf(fmaf(v[e], rstd, shift), gm[e], bt[e]);
+        }
+        if (z_norm != nullptr && r < rows) {
+            *reinterpret_cast<uint4 *>(z_norm + r * CZ + sub * 8) = o.u;
+        }
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                acc = __builtin_amdgcn_fdot2_f32_bf16(o.p[k], wv[h].p[k], acc, false);
+            }
+            acc = group_sum<LPR>(acc);
+            keep[h] = sub == s ? acc : keep[h];
+        }
+    }
+    const int64_t r = r0 + lane;
+    if (r < rows) {
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            nb[(int64_t)h * rows + r] = (bf16_t)keep[h];
+        }
+    }
+}
+
 template <typename T>
 int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                      int64_t rows, int64_t size, float eps, hipStream_t stream)
 {
+    if (sizeof(T) == 2 && (size == 64 || size == 128 || size == 256 || size == 512) && ld_x % 8 == 0 && ld_out % 8 == 0 &&
+        (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % 16 == 0) {
+        const int lpr = (int)(size / 8);
+        const int64_t rows_per_block = 4 * 4 * (64 / lpr);
+        const int64_t nblk = (rows + rows_per_block - 1) / rows_per_block;
+        if (nblk > INT32_MAX) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        const bf16_t *xi = (const bf16_t *)x;
+        bf16_t *oi = (bf16_t *)out;
+        switch (lpr) {
+            case 8: layernorm_rows_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
+            case 16: layernorm_rows_bf16_kernel<16><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
+            case 32: layernorm_rows_bf16_kernel<32><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
+            default: layernorm_rows_bf16_kernel<64><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
+        }
+        return kutacc_hip_status(hipGetLastError());
+    }
     const int64_t blocks = (rows + ROW_WAVES - 1) / ROW_WAVES;
     if (blocks > INT32_MAX) {
         return KUTACC_HIP_EUNSUPPORTED;
@@ -123,6 +331,21 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
                      int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, hipStream_t stream)
 {
     const int64_t rows = rows_i * rows_j;
+    if (sizeof(T) == 2 && c_z == 128 && (nheads == 4 || nheads == 8) &&
+        (reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(z_norm)) % 16 == 0) {
+        const int64_t nblk = (rows + 255) / 256;
+        if (nblk > INT32_MAX) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        if (nheads == 4) {
+            pair_bias_bf16_kernel<4><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
+                                                                        (bf16_t *)nb, (bf16_t *)z_norm, rows, eps);
+        } else {
+            pair_bias_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
+                                                                        (bf16_t *)nb, (bf16_t *)z_norm, rows, eps);
+        }
+        return kutacc_hip_status(hipGetLastError());
+    }
     const int64_t blocks = (rows + ROW_WAVES - 1) / ROW_WAVES;
     if (blocks > INT32_MAX) {
         return KUTACC_HIP_EUNSUPPORTED;
