@@ -991,8 +991,11 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
 // the two big streams -- input rows and pair bias -- through wave-private staging panels with fully
 // coalesced loads.
 // LDS, 16-byte units: W[4][CK][64]  K[NB][2][64]  V[NB][2][64]  panel[NB waves][256]  gate[NB waves][2][64];
-// then floats mask[NB*32]; then two uint32 of tile flags (alternating by batch row).
-// Per batch row: project (K, V -> LDS; Q, gate -> registers), barrier, attend, barrier.
+// then floats mask[2][NB*32] and two uint32 of tile flags (both alternating by batch row).
+// Per batch row: load and project (K, V, Q -> registers; gate -> LDS), barrier (previous row's attention
+// is over everywhere), K and V -> LDS, barrier, attend.  A wave that finishes its attention early starts
+// on the next row's loads and projections while the slower waves of its SIMD still attend, so the
+// latency- and MFMA-bound projection phase overlaps the VALU-heavy attention phase.
 // ------------------------------------------------------------------------------------------------
 template <int C, bool HAS_NB>
 __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(FusedParams p)
@@ -1024,8 +1027,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     uint4 *lds_v = lds_k + NB * 2 * 64;
     uint4 *panel = lds_v + NB * 2 * 64 + wave * 256;
     uint4 *gate_park = lds_v + NB * 2 * 64 + NB * 256 + wave * 128 + lane; // sigmoid(gate) waits here during attention
-    float *mask = reinterpret_cast<float *>(lds_v + NB * 2 * 64 + NB * 256 + NB * 128);
-    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask + NB * 32); // two, alternating by batch row
+    float *mask_base = reinterpret_cast<float *>(lds_v + NB * 2 * 64 + NB * 256 + NB * 128); // two buffers of NB*32
+    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 2 * NB * 32);            // two, alternating by batch row
 
     // the head's rows of the four weight matrices, in fragment order, for the whole kernel
     for (int idx = tid; idx < 4 * CK * 64; idx += nthreads) {
@@ -1051,6 +1054,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     for (int n = 0; n < nrows; ++n) {
         const int b = b0 + n * bstep;
         uint32_t *flag_word = flag_words + (n & 1);
+        float *mask = mask_base + (n & 1) * NB * 32;
         if (n == 2) {
             TL(0);
         }
@@ -1106,6 +1110,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         }
         // ---- four projections of the block ----
         bf16x8 q0, q1;
+        uint4 kfrag0, kfrag1, vfrag0, vfrag1; // this block's K and V fragments, parked until the LDS arrays are free
         {
             const uint4 *wsrc = lds_w + lane;
             f32x16 acc = zero16();
@@ -1113,15 +1118,15 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             for (int ks = 0; ks < CK; ++ks) {
                 acc = mfma(as_bf16x8(wsrc[(PROJ_K * CK + ks) * 64]), xf[ks], acc);
             }
-            lds_k[(j * 2 + 0) * 64 + lane] = as_uint4(pack8(acc, 0));
-            lds_k[(j * 2 + 1) * 64 + lane] = as_uint4(pack8(acc, 8));
+            kfrag0 = as_uint4(pack8(acc, 0));
+            kfrag1 = as_uint4(pack8(acc, 8));
             acc = zero16();
 #pragma unroll
             for (int ks = 0; ks < CK; ++ks) {
                 acc = mfma(xf[ks], as_bf16x8(wsrc[(PROJ_V * CK + ks) * 64]), acc);
             }
-            lds_v[(j * 2 + 0) * 64 + lane] = as_uint4(pack8(acc, 0));
-            lds_v[(j * 2 + 1) * 64 + lane] = as_uint4(pack8(acc, 8));
+            vfrag0 = as_uint4(pack8(acc, 0));
+            vfrag1 = as_uint4(pack8(acc, 8));
             acc = zero16();
 #pragma unroll
             for (int ks = 0; ks < CK; ++ks) {
@@ -1156,6 +1161,14 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 #ifdef KUTACC_OPT_TOUCH
         asm volatile("" ::"v"(touch));
 #endif
+        __syncthreads(); // every wave is done with the previous row's attention: the K and V arrays are free
+        lds_k[(j * 2 + 0) * 64 + lane] = kfrag0;
+        lds_k[(j * 2 + 1) * 64 + lane] = kfrag1;
+        lds_v[(j * 2 + 0) * 64 + lane] = vfrag0;
+        lds_v[(j * 2 + 1) * 64 + lane] = vfrag1;
+        if (tid == 0) {
+            flag_words[(n + 1) & 1] = 0; // its readers (previous row) are done, its writers (next row) start after the next barrier
+        }
         __syncthreads(); // K, V and the mask of this batch row are complete
         if (n == 2) {
             TL(3);
@@ -1202,12 +1215,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == 2) {
             TL(4);
         }
-        __syncthreads(); // every wave is done with this row's K/V and mask
         if (n == 2) {
             TL(5);
-        }
-        if (tid == 0) {
-            *flag_word = 0; // clean again for the row after next; the next row ORs into the other word
         }
     }
     TL(11);
@@ -1411,9 +1420,9 @@ size_t head_kernel_lds(int C, int NB, int GW)
 size_t persistent_kernel_lds(int C, int NB)
 {
     // all four weight matrices of the head, K and V of one batch row, per wave one 4 KB panel and 2 KB of
-    // parked gate fragments, mask, flags
+    // parked gate fragments, two mask buffers, flags
     return (size_t)4 * (C / 16) * 64 * 16 + (size_t)NB * 2 * 64 * 16 * 2 + (size_t)NB * (4096 + 2048) +
-           (size_t)NB * 32 * 4 + 16;
+           (size_t)2 * NB * 32 * 4 + 16;
 }
 
 bool make_plan(int64_t S, int C, Plan &pl)
