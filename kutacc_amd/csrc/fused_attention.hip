@@ -98,6 +98,8 @@ struct FusedParams {
     float qscale; // 1 / sqrt(head_size)
     int ngrp;     // persistent kernel: batch-row groups per XCD
     const uint4 *nbf; // pair bias * log2(e) in fragment-major order (pair_bias_fragments_kernel), or nullptr
+    int NT;           // key tiles the LDS arrays are laid out for: NB rounded up to an even number (the log2-unit
+                      // loop walks tile pairs; a phantom tile is all zeros behind a -inf mask)
     int l2mode;       // logits in log2 units (attend_block_l2); needs nbf when there is a pair bias
 };
 
@@ -834,20 +836,27 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     const int nthreads = p.NW * 64;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
-    const int S = p.S, NB = p.NB, NW = p.NW, GW = p.GW;
+    const int S = p.S, NB = p.NB, NT = p.NT, NW = p.NW, GW = p.GW;
 
     uint4 *lds_w = lds;
     uint4 *lds_k = lds_w + GW * CK * 64;
-    uint4 *lds_v = lds_k + NB * 2 * 64;
-    float *mask = reinterpret_cast<float *>(lds_v + NB * 2 * 64);
-    uint32_t *flag_word = reinterpret_cast<uint32_t *>(mask + NB * 32);
+    uint4 *lds_v = lds_k + NT * 2 * 64;
+    float *mask = reinterpret_cast<float *>(lds_v + NT * 2 * 64);
+    uint32_t *flag_word = reinterpret_cast<uint32_t *>(mask + NT * 32);
 
     if (tid == 0) {
         *flag_word = 0;
     }
+    if (NT > NB) { // phantom key tile: zero K and V fragments
+        const uint4 z4 = {0u, 0u, 0u, 0u};
+        for (int idx = tid; idx < 128; idx += nthreads) {
+            lds_k[NB * 2 * 64 + idx] = z4;
+            lds_v[NB * 2 * 64 + idx] = z4;
+        }
+    }
     __syncthreads();
-    for (int part = wave; part * 64 < NB * 32; part += NW) {
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, part, lane, p.l2mode ? LOG2E : 1.0f);
+    for (int part = wave; part * 64 < NT * 32; part += NW) {
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, part, lane, p.l2mode ? LOG2E : 1.0f);
     }
 
     const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
@@ -952,18 +961,18 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         f32x16 o;
         float l;
         if (p.l2mode) {
-            const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NB * 2) * 64 + lane : nullptr;
+            const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NT * 2) * 64 + lane : nullptr;
             if (flags == 0u) {
-                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NB,
+                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
                                                       lane, 0.f, o, l);
             } else {
-                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NB,
+                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
                                                      lane, 0.f, o, l);
             }
             if (__any(!(l > 1e-30f && l < 1e30f))) {
                 // some probability overflowed or a whole row underflowed: shift by the true row maxima
-                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, NB, lane);
-                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NB,
+                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, NT, lane);
+                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
                                                     lane, m, o, l);
             }
         } else {
@@ -1007,7 +1016,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
-    const int S = p.S, NB = p.NB;
+    const int S = p.S, NB = p.NB, NT = p.NT;
     const int nthreads = NB * 64;
     const int prow = pi_row(r);
 
@@ -1024,11 +1033,11 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 
     uint4 *lds_w = lds;
     uint4 *lds_k = lds_w + 4 * CK * 64;
-    uint4 *lds_v = lds_k + NB * 2 * 64;
-    uint4 *panel = lds_v + NB * 2 * 64 + wave * 256;
-    uint4 *gate_park = lds_v + NB * 2 * 64 + NB * 256 + wave * 128 + lane; // sigmoid(gate) waits here during attention
-    float *mask_base = reinterpret_cast<float *>(lds_v + NB * 2 * 64 + NB * 256 + NB * 128); // two buffers of NB*32
-    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 2 * NB * 32);            // two, alternating by batch row
+    uint4 *lds_v = lds_k + NT * 2 * 64;
+    uint4 *panel = lds_v + NT * 2 * 64 + wave * 256;
+    uint4 *gate_park = lds_v + NT * 2 * 64 + NB * 256 + wave * 128 + lane; // sigmoid(gate) waits here during attention
+    float *mask_base = reinterpret_cast<float *>(lds_v + NT * 2 * 64 + NB * 256 + NB * 128); // two buffers of NT*32
+    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 2 * NT * 32);            // two, alternating by batch row
 
     // the head's rows of the four weight matrices, in fragment order, for the whole kernel
     for (int idx = tid; idx < 4 * CK * 64; idx += nthreads) {
@@ -1042,6 +1051,13 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         flag_words[0] = 0;
         flag_words[1] = 0;
     }
+    if (NT > NB) { // phantom key tile: zero K and V fragments, never written again
+        const uint4 z4 = {0u, 0u, 0u, 0u};
+        for (int idx = tid; idx < 128; idx += nthreads) {
+            lds_k[NB * 2 * 64 + idx] = z4;
+            lds_v[NB * 2 * 64 + idx] = z4;
+        }
+    }
     bf16x8 sel0, sel1;
     make_selectors(lane, sel0, sel1);
     __syncthreads();
@@ -1054,7 +1070,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     for (int n = 0; n < nrows; ++n) {
         const int b = b0 + n * bstep;
         uint32_t *flag_word = flag_words + (n & 1);
-        float *mask = mask_base + (n & 1) * NB * 32;
+        float *mask = mask_base + (n & 1) * NT * 32;
         if (n == 2) {
             TL(0);
         }
@@ -1064,7 +1080,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == nrows - 1) {
             TL(10);
         }
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NB, wave, lane, p.l2mode ? LOG2E : 1.0f);
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane, p.l2mode ? LOG2E : 1.0f);
 
         // ---- input rows of the block -> fragments, 64 channels per staging panel ----
         const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
@@ -1180,12 +1196,12 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         const uint32_t flags = *flag_word;
         const bf16_t *nb_head = HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr;
         if (p.l2mode) {
-            const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NB * 2) * 64 + lane : nullptr;
+            const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NT * 2) * 64 + lane : nullptr;
             if (flags == 0u) {
-                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NB, lane, 0.f, o,
+                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o,
                                                       l);
             } else {
-                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NB, lane, 0.f, o,
+                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o,
                                                      l);
             }
             const bool ok = !__any(!(l > 1e-30f && l < 1e30f));
@@ -1194,8 +1210,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             }
             if (!ok) {
                 // some probability overflowed or a whole row underflowed: shift by the true row maxima
-                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, q0, q1, sel0, sel1, NB, lane);
-                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NB, lane, m, o, l);
+                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, q0, q1, sel0, sel1, NT, lane);
+                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, m, o, l);
             }
         } else {
             attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, nb_head, p.nb_sq, j * 32, p.nb_vec != 0, panel, q0, q1, sel0,
@@ -1345,12 +1361,12 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
 // S-1 and keys past S read as zero (their mask bias is -inf).  The pair bias is shared by every batch
 // row, so this pass moves 2*H*S*S bytes once per call, against B times that in the attention kernel.
 __global__ __launch_bounds__(64) void pair_bias_fragments_kernel(const bf16_t *__restrict__ nb, int64_t nb_sh,
-                                                                 int64_t nb_sq, int S, int NB, int vec,
+                                                                 int64_t nb_sq, int S, int NB, int NT, int vec,
                                                                  uint4 *__restrict__ out)
 {
     const int lane = threadIdx.x;
     const int r = lane & 31, g = lane >> 5;
-    const int t = blockIdx.x % NB, j = blockIdx.x / NB, h = blockIdx.y;
+    const int t = blockIdx.x % NT, j = blockIdx.x / NT, h = blockIdx.y;
     int q = 32 * j + pi_row(r);
     q = q < S ? q : S - 1;
     const int key0 = 32 * t + 16 * g;
@@ -1379,7 +1395,7 @@ __global__ __launch_bounds__(64) void pair_bias_fragments_kernel(const bf16_t *_
         d0[e] = (bf16_t)(to_f32(s0[e]) * LOG2E);
         d1[e] = (bf16_t)(to_f32(s1[e]) * LOG2E);
     }
-    uint4 *dst = out + ((((int64_t)h * NB + j) * NB + t) * 2) * 64 + lane;
+    uint4 *dst = out + ((((int64_t)h * NB + j) * NT + t) * 2) * 64 + lane;
     dst[0] = as_uint4(d0);
     dst[64] = as_uint4(d1);
 }
@@ -1414,15 +1430,17 @@ int num_cus()
 
 size_t head_kernel_lds(int C, int NB, int GW)
 {
-    return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NB * 2 * 64 * 16 * 2 + (size_t)NB * 32 * 4 + 16;
+    const int NT = (NB + 1) & ~1; // key tiles, padded to a pair
+    return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NT * 2 * 64 * 16 * 2 + (size_t)NT * 32 * 4 + 16;
 }
 
 size_t persistent_kernel_lds(int C, int NB)
 {
     // all four weight matrices of the head, K and V of one batch row, per wave one 4 KB panel and 2 KB of
     // parked gate fragments, two mask buffers, flags
-    return (size_t)4 * (C / 16) * 64 * 16 + (size_t)NB * 2 * 64 * 16 * 2 + (size_t)NB * (4096 + 2048) +
-           (size_t)2 * NB * 32 * 4 + 16;
+    const int NT = (NB + 1) & ~1; // key tiles, padded to a pair
+    return (size_t)4 * (C / 16) * 64 * 16 + (size_t)NT * 2 * 64 * 16 * 2 + (size_t)NB * (4096 + 2048) +
+           (size_t)2 * NT * 32 * 4 + 16;
 }
 
 bool make_plan(int64_t S, int C, Plan &pl)
@@ -1612,6 +1630,7 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     p.x_ld = a.input_ld, p.bias_sb = a.bias_stride_b, p.nb_sh = a.nb_stride_h, p.nb_sq = a.nb_stride_q;
     p.avg_sb = a.avg_stride_b, p.avg_ss = a.avg_stride_s, p.avg_sh = a.avg_stride_h;
     p.B = (int)a.batch, p.S = (int)a.seq_len, p.H = (int)a.nheads, p.NB = pl.NB, p.NW = pl.NW, p.GW = pl.GW;
+    p.NT = (pl.NB + 1) & ~1;
     p.nb_vec = (p.nb != nullptr && aligned(p.nb, 16) && a.nb_stride_h % 8 == 0 && a.nb_stride_q % 8 == 0) ? 1 : 0;
     // (float)(1/sqrt(head_size)) as the reference forms it (gating_attention.cpp:68)
     p.qscale = (float)(1.0 / sqrt((double)a.head_size));
@@ -1622,32 +1641,35 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     // scratch tensor (which this path does not otherwise use; its contents are unspecified after any
     // call) when that is dense, aligned and large enough; otherwise the kernels read the pair bias in
     // place through the staging panels.
-    const int64_t nbf_bytes = (int64_t)a.nheads * pl.NB * pl.NB * 2048;
+    const int64_t nbf_bytes = (int64_t)a.nheads * pl.NB * p.NT * 2048;
     const bool q_dense = a.q != nullptr && aligned(a.q, 16) && a.q_stride_h == a.head_size && a.q_stride_s == C &&
                          a.q_stride_b == a.seq_len * C;
-    const bool want_fragments = p.nb != nullptr && a.seq_len % 64 == 0 && q_dense &&
+    const bool want_fragments = p.nb != nullptr && q_dense &&
                                 nbf_bytes <= a.batch * a.seq_len * C * 2 && !getenv("KUTACC_HIP_NO_FRAGMENTS");
 
-    if (getenv("KUTACC_HIP_DEBUG")) {
-        fprintf(stderr, "[kutacc] fused plan: persistent=%d C=%d NB=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d\n",
-                (int)pl.persistent, C, pl.NB, pl.NW, pl.BPW, pl.GW, pl.lds_bytes, max_lds_bytes(), num_cus());
-    }
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
     if (want_fragments) {
         kutacc_prof::KernelTimer t("pair_bias_fragments_kernel", 0.0, stream);
-        pair_bias_fragments_kernel<<<dim3((unsigned)(pl.NB * pl.NB), (unsigned)a.nheads), 64, 0, stream>>>(
-            p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.nb_vec, (uint4 *)a.q);
+        pair_bias_fragments_kernel<<<dim3((unsigned)(pl.NB * p.NT), (unsigned)a.nheads), 64, 0, stream>>>(
+            p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.NT, p.nb_vec, (uint4 *)a.q);
         rc = kutacc_hip_status(hipGetLastError());
         if (rc != 0) {
             return rc;
         }
         p.nbf = (const uint4 *)a.q;
     }
-    p.l2mode = (a.seq_len % 64 == 0 && (p.nb == nullptr || p.nbf != nullptr) &&
+    p.l2mode = ((p.nb == nullptr || p.nbf != nullptr) &&
                 !getenv("KUTACC_HIP_NO_FRAGMENTS"))
                    ? 1
                    : 0;
+    if (getenv("KUTACC_HIP_DEBUG")) {
+        fprintf(stderr,
+                "[kutacc] fused plan: persistent=%d C=%d NB=%d NT=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d log2_units=%d "
+                "fragments=%d\n",
+                (int)pl.persistent, C, pl.NB, p.NT, pl.NW, pl.BPW, pl.GW, pl.lds_bytes, max_lds_bytes(), num_cus(), p.l2mode,
+                p.nbf != nullptr ? 1 : 0);
+    }
     {
         kutacc_prof::KernelTimer t(pl.persistent ? "persistent_head_kernel" : "fused_head_kernel",
                                    8.0 * BS * C * C + 4.0 * BS * (double)a.seq_len * C, stream);

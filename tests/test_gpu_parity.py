@@ -77,6 +77,8 @@ SMALL = [
     # config, batch, seq_len
     (1, 3, 64), (2, 4, 256), (3, 5, 384), (4, 3, 1024), (5, 3, 1024),
     (2, 3, 70), (3, 2, 33), (2, 2, 1), (3, 2, 200), (4, 2, 97),
+    # ragged lengths with enough batch rows for the fragment-major pair-bias copy to fit the q scratch tensor
+    (3, 24, 200), (2, 16, 70), (3, 8, 33), (5, 12, 321),
 ]
 
 
