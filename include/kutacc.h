@@ -112,6 +112,23 @@ kutacc_export void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2
                                                kutacc_af2_attention_weights_t *weight_ptr, kutacc_tensor_h out,
                                                int64_t block_size);
 
+/**
+ * @brief global (extra-MSA column) attention: one query per batch row and head (the masked mean of the row),
+ *        one key/value head shared by all heads.  Reference include/kutacc.h:292-307 (declaration),
+ *        src/attention/global_attention.cpp:167-205 (entry), :30-164 (kernel).
+ * @param [in] q_based_ptr batch, seq_len and the scratch tensors q [batch, nchannels], k [batch*seq_len, head_size],
+ *             v [head_size, batch*seq_len], gate [batch, seq_len, nchannels], avg = q_avg [batch, nchannels];
+ *             this backend writes only avg (the masked mean) and leaves q, k, v, gate untouched
+ * @param [in] q_data shape [batch, seq_len, nchannels], bf16
+ * @param [in] q_mask shape [batch, seq_len, 1], bf16
+ * @param [in] weight_ptr nchannels must be 64; query_w, gating_w, output_w [64, 64], key_w, value_w [head_size, 64],
+ *             all stored [out, in]; gating_b, output_b fp32 [64]
+ * @param [out] out shape [batch, seq_len, nchannels], bf16
+ */
+kutacc_export void kutacc_af2_global_attention(kutacc_af2_attention_inputs_t *q_based_ptr, kutacc_tensor_h q_data,
+                                               kutacc_tensor_h q_mask, kutacc_af2_attention_weights_t *weight_ptr,
+                                               kutacc_tensor_h out);
+
 /*
  * LayerNorm of ONE row of `size` elements, bf16 in/out, fp32 gamma/beta
  * (reference include/kutacc.h:334, src/normalization/layernorm_kernel.h:21-53).

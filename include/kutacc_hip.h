@@ -89,6 +89,41 @@ typedef struct kutacc_hip_attention_args {
  * (reference src/attention/gating_attention.cpp:33-158). */
 kutacc_export int kutacc_hip_gating_attention(const kutacc_hip_attention_args_t *args, void *stream);
 
+/* Global (extra-MSA column) attention, reference src/attention/global_attention.cpp:30-164 (kernel) and
+ * :167-205 (entry).  One query per batch row and head (the masked mean of the row), one key/value head
+ * shared by all heads.  bf16 storage, nheads*head_size == 64 (the reference hard-wires nchannels == 64,
+ * :172), nheads <= 32, head_size <= 32.  The reference's scratch tensors q, k, v, gate are not needed and
+ * not touched; q_avg ([B, 64], may be NULL) receives the masked mean as the reference leaves it in `avg`. */
+typedef struct kutacc_hip_global_attention_args {
+    int64_t batch;     /* B */
+    int64_t seq_len;   /* S */
+    int64_t nheads;    /* H */
+    int64_t head_size; /* d;  H*d == 64 */
+    int32_t dtype;     /* KUTACC_DTYPE_BF16 */
+    int32_t reserved;
+
+    const void *q_data;       /* element (b,s,c) at b*q_data_stride_b + s*q_data_stride_s + c */
+    int64_t q_data_stride_b;
+    int64_t q_data_stride_s;
+    const void *q_mask;       /* element (b,s) at b*q_mask_stride_b + s */
+    int64_t q_mask_stride_b;
+    const void *query_w;      /* [64, 64] stored [out, in] */
+    const void *key_w;        /* [d, 64]  stored [out, in] */
+    const void *value_w;      /* [d, 64]  stored [out, in] */
+    const void *gating_w;     /* [64, 64] stored [out, in] */
+    const void *output_w;     /* [64, 64] stored [out, in] */
+    const float *gating_b;    /* fp32 [64] */
+    const float *output_b;    /* fp32 [64] */
+
+    void *q_avg;              /* [B, 64], row stride q_avg_stride_b; NULL = not wanted */
+    int64_t q_avg_stride_b;
+    void *out;                /* element (b,s,c) at b*out_stride_b + s*out_stride_s + c */
+    int64_t out_stride_b;
+    int64_t out_stride_s;
+} kutacc_hip_global_attention_args_t;
+
+kutacc_export int kutacc_hip_global_attention(const kutacc_hip_global_attention_args_t *args, void *stream);
+
 /* Name of the kernel family the last successful kutacc_hip_gating_attention call used on this
  * thread: "fused_mfma" or "generic".  Static storage. */
 kutacc_export const char *kutacc_hip_last_path(void);

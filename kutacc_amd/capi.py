@@ -63,13 +63,27 @@ class HipAttentionArgs(ctypes.Structure):
     ]
 
 
+class HipGlobalAttentionArgs(ctypes.Structure):
+    """kutacc_hip_global_attention_args_t"""
+    _fields_ = [
+        ("batch", _i64), ("seq_len", _i64), ("nheads", _i64), ("head_size", _i64), ("dtype", _i32), ("reserved", _i32),
+        ("q_data", _vp), ("q_data_stride_b", _i64), ("q_data_stride_s", _i64),
+        ("q_mask", _vp), ("q_mask_stride_b", _i64),
+        ("query_w", _vp), ("key_w", _vp), ("value_w", _vp), ("gating_w", _vp), ("output_w", _vp),
+        ("gating_b", _vp), ("output_b", _vp),
+        ("q_avg", _vp), ("q_avg_stride_b", _i64),
+        ("out", _vp), ("out_stride_b", _i64), ("out_stride_s", _i64),
+    ]
+
+
 # every symbol the two public headers declare; tests check that the library exports all of them
 DECLARED_SYMBOLS = [
-    "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_layernorm", "kutacc_af2_linear",
+    "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_global_attention", "kutacc_af2_layernorm",
+    "kutacc_af2_linear",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
-    "kutacc_hip_gating_attention", "kutacc_hip_last_path", "kutacc_hip_layernorm_rows", "kutacc_hip_linear",
+    "kutacc_hip_gating_attention", "kutacc_hip_global_attention", "kutacc_hip_last_path", "kutacc_hip_layernorm_rows", "kutacc_hip_linear",
     "kutacc_hip_pair_bias", "kutacc_hip_set_stream", "kutacc_hip_get_stream", "kutacc_hip_set_blocking",
     "kutacc_hip_error_flag", "kutacc_hip_clear_error", "kutacc_hip_tensor_create", "kutacc_hip_tensor_destroy",
     "kutacc_hip_profile_enable", "kutacc_hip_profile_read",
@@ -92,6 +106,11 @@ def lib() -> ctypes.CDLL:
     L.kutacc_af2_gating_attention.argtypes = [_vp, ctypes.POINTER(AttentionInputs), _vp, _vp,
                                               ctypes.POINTER(AttentionWeights), _vp, _i64]
     L.kutacc_af2_gating_attention.restype = None
+    L.kutacc_af2_global_attention.argtypes = [ctypes.POINTER(AttentionInputs), _vp, _vp, ctypes.POINTER(AttentionWeights),
+                                              _vp]
+    L.kutacc_af2_global_attention.restype = None
+    L.kutacc_hip_global_attention.argtypes = [ctypes.POINTER(HipGlobalAttentionArgs), _vp]
+    L.kutacc_hip_global_attention.restype = ctypes.c_int
     L.kutacc_af2_layernorm.argtypes = [_vp, _vp, _vp, _i64, ctypes.c_float, _vp]
     L.kutacc_af2_layernorm.restype = None
     L.kutacc_af2_linear.argtypes = [_vp, _vp, _vp, _vp, _i64]
@@ -234,3 +253,31 @@ class GatedAttention:
     def run(self) -> None:
         kutacc_af2_gating_attention(self.h["x"], self.inputs, self.h["bias"], self.h_nb, self.weights, self.h["out"],
                                     self.block_size)
+
+
+def kutacc_af2_global_attention(q_based: AttentionInputs, q_data, q_mask, weights: AttentionWeights, out) -> None:
+    """Arguments as in the C API; tensor arguments are TensorHandle objects (or None for a null handle)."""
+    h = lambda t: _vp(t.handle) if t is not None else None  # noqa: E731
+    lib().kutacc_af2_global_attention(ctypes.byref(q_based) if q_based is not None else None, h(q_data), h(q_mask),
+                                      ctypes.byref(weights) if weights is not None else None, h(out))
+
+
+class GlobalAttention:
+    """Owner of everything one kutacc_af2_global_attention call needs (torch tensors on the GPU or numpy arrays
+    on the host).  x [B,S,64]; mask [B,S,1]; wq, wg, wo [64,64]; wk, wv [d,64]; bg, bo fp32 [64]; out [B,S,64];
+    scratch: dict with q [B,64], k [B*S,d], v [d,B*S], gate [B,S,64], avg [B,64]."""
+
+    def __init__(self, x, mask, wq, wk, wv, wg, bg, wo, bo, nheads, out, scratch):
+        B, S, C = x.shape
+        self.keep = dict(x=x, mask=mask, wq=wq, wk=wk, wv=wv, wg=wg, bg=bg, wo=wo, bo=bo, out=out, **scratch)
+        self.h = {k: tensor(v) for k, v in self.keep.items() if k not in ("bg", "bo")}
+        self.h["bg"] = tensor(bg, K_FP32)
+        self.h["bo"] = tensor(bo, K_FP32)
+        self.weights = AttentionWeights(C, nheads, C // nheads, self.h["wq"].handle, self.h["wk"].handle,
+                                        self.h["wv"].handle, self.h["wg"].handle, self.h["bg"].handle,
+                                        self.h["wo"].handle, self.h["bo"].handle)
+        self.inputs = AttentionInputs(B, S, self.h["q"].handle, self.h["k"].handle, self.h["v"].handle,
+                                      self.h["gate"].handle, self.h["avg"].handle)
+
+    def run(self) -> None:
+        kutacc_af2_global_attention(self.inputs, self.h["x"], self.h["mask"], self.weights, self.h["out"])

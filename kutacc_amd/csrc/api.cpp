@@ -404,6 +404,119 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
                  rc > 0 ? std::string(" (") + hipGetErrorString((hipError_t)rc) + ")" : std::string());
 }
 
+int kutacc_hip_global_attention(const kutacc_hip_global_attention_args_t *a, void *stream)
+{
+    if (!a) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int rc = kutacc_launch::global_attention(*a, pick_stream(stream));
+    if (rc == 0) {
+        t_last_path = "global_mfma";
+    }
+    return rc;
+}
+
+void kutacc_af2_global_attention(kutacc_af2_attention_inputs_t *q_based_ptr, kutacc_tensor_h q_data, kutacc_tensor_h q_mask,
+                                 kutacc_af2_attention_weights_t *weight_ptr, kutacc_tensor_h out)
+{
+    // same first check as the reference, including the hard-wired channel count (global_attention.cpp:171-173)
+    KUTACC_CHECK(q_based_ptr != nullptr && q_data != nullptr && q_mask != nullptr && weight_ptr != nullptr &&
+                     out != nullptr && weight_ptr->nchannels == 64,
+                 "kutacc_af2_gating_attention: input args nullptr error or invalid int value error");
+    if (KUTACC_FAILED()) {
+        return;
+    }
+    const int64_t batch = q_based_ptr->batch, seq_len = q_based_ptr->seq_len;
+    const int64_t head_size = weight_ptr->head_size, nheads = weight_ptr->nheads, nchannels = weight_ptr->nchannels;
+    // scalar checks before any handle is looked into (global_attention.cpp:37-44)
+    KUTACC_CHECK(batch > 0 && seq_len > 0 && nchannels > 0 && nheads > 0 && head_size > 0 && batch <= INT32_MAX / seq_len &&
+                     seq_len <= INT32_MAX && nchannels <= INT32_MAX && head_size <= INT32_MAX &&
+                     nheads <= INT64_MAX / seq_len && nheads <= INT64_MAX / head_size,
+                 "input param <= 0 or overflow");
+    if (KUTACC_FAILED()) {
+        return;
+    }
+    KUTACC_CHECK(nchannels == nheads * head_size, "nchannels != nheads * head_size: ", nchannels, " vs ", nheads, "*",
+                 head_size);
+    kutacc_tensor_h handles[] = {q_based_ptr->avg,     weight_ptr->query_w,  weight_ptr->key_w,    weight_ptr->value_w,
+                                 weight_ptr->gating_w, weight_ptr->gating_b, weight_ptr->output_w, weight_ptr->output_b};
+    for (kutacc_tensor_h h : handles) {
+        KUTACC_CHECK(h != nullptr, "kutacc_af2_global_attention: tensor handle inside argument struct is null");
+    }
+    if (KUTACC_FAILED()) {
+        return;
+    }
+    TensorView &x = *kutacc::as_view(q_data), &mk = *kutacc::as_view(q_mask), &ot = *kutacc::as_view(out),
+               &qa = *kutacc::as_view(q_based_ptr->avg);
+    TensorView &wq = *kutacc::as_view(weight_ptr->query_w), &wk = *kutacc::as_view(weight_ptr->key_w),
+               &wv = *kutacc::as_view(weight_ptr->value_w), &wg = *kutacc::as_view(weight_ptr->gating_w),
+               &bg = *kutacc::as_view(weight_ptr->gating_b), &wo = *kutacc::as_view(weight_ptr->output_w),
+               &bo = *kutacc::as_view(weight_ptr->output_b);
+    KUTACC_CHECK(x.dtype == kutacc::kBF16 && mk.dtype == kutacc::kBF16 && ot.dtype == kutacc::kBF16 &&
+                     qa.dtype == kutacc::kBF16 && wq.dtype == kutacc::kBF16 && wk.dtype == kutacc::kBF16 &&
+                     wv.dtype == kutacc::kBF16 && wg.dtype == kutacc::kBF16 && wo.dtype == kutacc::kBF16,
+                 "addmm dtype invalid, a: [", (int)x.dtype, "]");
+    KUTACC_CHECK(x.data && mk.data && ot.data && qa.data && wq.data && wk.data && wv.data && wg.data && bg.data &&
+                     wo.data && bo.data,
+                 "addmm input invalid");
+    KUTACC_CHECK(ot.dim >= 2 && mk.dim >= 1 && qa.dim >= 1, "kutacc_af2_global_attention: out needs rank >= 2, q_mask and avg rank >= 1");
+    if (KUTACC_FAILED()) {
+        return;
+    }
+
+    kutacc_hip_global_attention_args_t a;
+    std::memset(&a, 0, sizeof(a));
+    a.batch = batch, a.seq_len = seq_len, a.nheads = nheads, a.head_size = head_size;
+    a.dtype = KUTACC_DTYPE_BF16;
+    // q_data is read as a dense [batch, seq_len, nchannels] array, as the reference does (:53, :81)
+    a.q_data = x.data, a.q_data_stride_b = seq_len * nchannels, a.q_data_stride_s = nchannels;
+    a.q_mask = mk.data, a.q_mask_stride_b = mk.stride(0);
+    a.query_w = wq.data, a.key_w = wk.data, a.value_w = wv.data, a.gating_w = wg.data, a.output_w = wo.data;
+    a.gating_b = (const float *)bg.data, a.output_b = (const float *)bo.data;
+    a.q_avg = qa.data, a.q_avg_stride_b = nchannels;
+    a.out = ot.data, a.out_stride_s = ot.stride(ot.dim >= 3 ? 1 : 0), a.out_stride_b = seq_len * a.out_stride_s;
+
+    hipStream_t s = g_stream;
+    const Space sp = space_of(x.data);
+    const void *all_ptrs[] = {mk.data, ot.data, qa.data, wq.data, wk.data, wv.data, wg.data, bg.data, wo.data, bo.data};
+    for (const void *ptr : all_ptrs) {
+        KUTACC_CHECK(space_of(ptr) == sp, "kutacc_af2_global_attention: host and device pointers mixed in one call");
+    }
+    if (KUTACC_FAILED()) {
+        return;
+    }
+    int rc;
+    if (sp == Space::Device) {
+        rc = finish_device_call(kutacc_hip_global_attention(&a, s), s);
+    } else {
+        // Staged path: mirror every operand on the device, run, copy out and q_avg back.
+        const size_t e = 2;
+        const int64_t M = batch * seq_len, C = nchannels;
+        Stager st(s);
+        a.q_data = st.in(x.data, (size_t)(M * C) * e);
+        a.q_mask = st.in(mk.data, span2(batch, a.q_mask_stride_b, seq_len) * e);
+        a.query_w = st.in(wq.data, (size_t)(C * C) * e);
+        a.key_w = st.in(wk.data, (size_t)(head_size * C) * e);
+        a.value_w = st.in(wv.data, (size_t)(head_size * C) * e);
+        a.gating_w = st.in(wg.data, (size_t)(C * C) * e);
+        a.output_w = st.in(wo.data, (size_t)(C * C) * e);
+        a.gating_b = (const float *)st.in(bg.data, (size_t)C * sizeof(float));
+        a.output_b = (const float *)st.in(bo.data, (size_t)C * sizeof(float));
+        a.q_avg = st.out(qa.data, (size_t)(batch * C) * e, false);
+        a.out = st.out(ot.data, span2(M, a.out_stride_s, C) * e, a.out_stride_s != C);
+        rc = st.rc;
+        if (rc == 0) {
+            rc = kutacc_hip_global_attention(&a, s);
+        }
+        const int rc2 = st.finish();
+        if (rc == 0) {
+            rc = rc2;
+        }
+    }
+    KUTACC_CHECK(rc == 0, "kutacc_af2_global_attention: launch layer returned ", rc,
+                 rc > 0 ? std::string(" (") + hipGetErrorString((hipError_t)rc) + ")" : std::string());
+}
+
 void kutacc_af2_layernorm(__bf16 *data, float *gamma, float *beta, int64_t size, float eps, __bf16 *out)
 {
     // The reference dereferences unconditionally (src/normalization/layernorm.cpp:17-20); a device

@@ -35,6 +35,7 @@
 
 #include "device_util.h"
 #include "launch_internal.h"
+#include "mfma_tiles.h"
 #include "profiler.h"
 
 using namespace kutacc_dev;
@@ -67,13 +68,6 @@ extern "C" __attribute__((visibility("default"))) int kutacc_debug_timeline(unsi
 
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-
-constexpr float LOG2E = 1.44269504088896340736f;
 constexpr int HEAD = 32;            // head_size the MFMA kernels are written for
 constexpr int MAX_WAVES = 12;       // fused_head_kernel: 768 threads, 3 waves per SIMD, 168 VGPRs each
 constexpr float RESCALE_GAP = 5.5f; // running max may lag the true max by this much (natural log units, ~8 octaves)
@@ -102,61 +96,6 @@ struct FusedParams {
                       // loop walks tile pairs; a phantom tile is all zeros behind a -inf mask)
     int l2mode;       // logits in log2 units (attend_block_l2); needs nbf when there is a pair bias
 };
-
-__device__ __forceinline__ int pi_row(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
-
-__device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c)
-{
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-
-__device__ __forceinline__ f32x16 zero16()
-{
-    const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    return z;
-}
-
-__device__ __forceinline__ bf16x8 pack8(const f32x16 &v, int base)
-{
-    bf16x8 r;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        r[i] = (bf16_t)v[base + i];
-    }
-    return r;
-}
-
-__device__ __forceinline__ bf16x8 as_bf16x8(uint4 u)
-{
-    union {
-        uint4 u;
-        bf16x8 b;
-    } c;
-    c.u = u;
-    return c.b;
-}
-
-__device__ __forceinline__ uint4 as_uint4(bf16x8 b)
-{
-    union {
-        uint4 u;
-        bf16x8 b;
-    } c;
-    c.b = b;
-    return c.u;
-}
-
-// combine the two 32-lane halves of a wave: returns op(x[lane], x[lane ^ 32]) in every lane
-__device__ __forceinline__ float half_swap_max(float x)
-{
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float half_swap_sum(float x)
-{
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
 
 // 0/1 selection fragments that scatter the pair-bias words a lane loads (16 consecutive keys, 8 per
 // MFMA) onto the logits rows: row i of a tile is key pi(i); k-slot 8*g+e of the first MFMA carries
@@ -194,49 +133,6 @@ __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *m
             atomicOr(flag_word, bits);
         }
     }
-}
-
-// Wave-private staging panel in LDS: 32 rows x 128 bytes, in 16-byte slots.  A panel is filled with
-// four fully coalesced loads (each instruction reads 8 rows x 128 contiguous bytes = 8 whole cache
-// lines, lane l -> row 8i + l/8, slot l%8) and read back in MFMA fragment order (lane -> its own
-// row).  Loading fragments straight from global memory would touch 32 different cache lines per
-// instruction, four times the L1 tag traffic.  The slot index is XOR-swizzled by row so that both
-// access patterns are free of LDS bank conflicts.
-__device__ __forceinline__ int panel_slot(int row, int chunk)
-{
-    return row * 8 + (chunk ^ ((row & 7) ^ ((row >> 4) & 1)));
-}
-
-// issue the four coalesced loads of a panel: rows row0 .. row0+31 (clamped to last_row) of a
-// row-major bf16 matrix with leading dimension ld, 64 columns starting at col0
-struct PanelRegs {
-    uint4 r0, r1, r2, r3; // named members rather than an array, so that they always live in registers
-};
-
-__device__ __forceinline__ uint4 panel_load_one(const bf16_t *base, int64_t ld, int row, int last_row, int col0, int lane)
-{
-    row = row < last_row ? row : last_row;
-    return *reinterpret_cast<const uint4 *>(base + (int64_t)row * ld + col0 + (lane & 7) * 8);
-}
-
-__device__ __forceinline__ PanelRegs panel_load(const bf16_t *base, int64_t ld, int row0, int last_row, int col0, int lane)
-{
-    PanelRegs p;
-    const int row = row0 + (lane >> 3);
-    p.r0 = panel_load_one(base, ld, row, last_row, col0, lane);
-    p.r1 = panel_load_one(base, ld, row + 8, last_row, col0, lane);
-    p.r2 = panel_load_one(base, ld, row + 16, last_row, col0, lane);
-    p.r3 = panel_load_one(base, ld, row + 24, last_row, col0, lane);
-    return p;
-}
-
-__device__ __forceinline__ void panel_store(uint4 *panel, int lane, const PanelRegs &p)
-{
-    const int row = lane >> 3, chunk = lane & 7;
-    panel[panel_slot(row, chunk)] = p.r0;
-    panel[panel_slot(row + 8, chunk)] = p.r1;
-    panel[panel_slot(row + 16, chunk)] = p.r2;
-    panel[panel_slot(row + 24, chunk)] = p.r3;
 }
 
 // Flash-style attention of one 32-query block against all keys of the unit.
@@ -800,11 +696,6 @@ __device__ __forceinline__ void store_gated(bf16_t *dst, const f32x16 &o, float 
         }
         *reinterpret_cast<bf16x4 *>(dst + 8 * a) = ov;
     }
-}
-
-__device__ __forceinline__ float sigmoid_fast(float x)
-{
-    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -1,0 +1,395 @@
+// Global (extra-MSA column) attention for gfx950, bf16 storage, 64 channels
+// (reference src/attention/global_attention.cpp:30-164; nchannels == 64 is hard-wired there, :172).
+//
+// Per batch row b there is ONE query per head, the masked mean of the row's tokens, and ONE key/value
+// head shared by all heads:
+//   q_avg = sum_s mask[s] x[s,:] / (sum_s mask[s] + 1e-10);  q = q_avg.Wq^T  viewed [H, d]
+//   logit[h,s] = q[h].(Wk x[s]) / sqrt(d) + (mask[s]*1e9 - 1e9);  p = softmax_s
+//   wavg[h,:] = sum_s p[h,s] (Wv x[s]);  out[s,:] = (sigmoid(x[s].Wg^T + bg) * wavg).Wo^T + bo
+// One workgroup (four waves) owns a batch row and walks it three times in 32-token tiles, each tile
+// fetched with whole-cache-line loads through the wave's LDS staging panel: (A) masked mean, (B)
+// logits, online softmax and weighted average, (C) gate, gating and output projection.  Nothing but
+// q_avg and out is written to memory.  All contractions are v_mfma_f32_32x32x16_bf16:
+//   B: logits^T[s, h] = X[s, :] . QK^T with QK[h, :] = q[h].Wk / sqrt(d) folded per batch row (heads are the
+//      columns, 8 of 32 used for H = 8); V[s, e] = X . Wv^T; O^T[e, h] += V^T . P^T -- the accumulators
+//      of the first two products are directly the operands of the third, as in the gated attention
+//      kernels (rows of a tile are the contraction index of the third product on both sides).
+//   C: G^T[c, s] = Wg . X^T with the rows of Wg ordered so that a lane's accumulators are the k-slots of
+//      the next product's B operand; OUT^T[o, s] = Wo . gated^T with the rows of Wo ordered so that a lane
+//      holds 16 consecutive output features of its token (two 16-byte stores).
+// The -1e9 mask bias is the accumulator's initial value and absorbs the logit in fp32, so a row whose mask
+// is all zero attends uniformly, as in the reference.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "device_util.h"
+#include "launch_internal.h"
+#include "mfma_tiles.h"
+#include "profiler.h"
+
+using namespace kutacc_dev;
+
+namespace {
+
+constexpr int GC = 64;        // channels
+constexpr int MERGE_LD = 18;  // floats per lane in the cross-wave merge area: m, l, 16 accumulators
+
+struct GlobalParams {
+    const bf16_t *x, *mask, *wq, *wk, *wv, *wg, *wo;
+    const float *bg, *bo;
+    bf16_t *q_avg, *out;
+    int64_t x_sb, x_ss, mask_sb, qavg_sb, out_sb, out_ss;
+    int B, S, H, d, NT;
+    float scale;
+};
+
+// channel that accumulator register v of lane half g holds in row block rb of the gate product
+__device__ __forceinline__ int gate_channel(int rb, int v, int g)
+{
+    const int idx = rb * 16 + v;
+    return 16 * (idx >> 3) + 8 * g + (idx & 7);
+}
+
+__device__ __forceinline__ void load_tile(const bf16_t *xb, int64_t ld, int t, int S, uint4 *panel, int lane, bf16x8 (&xf)[4])
+{
+    const int r = lane & 31, g = lane >> 5;
+    const PanelRegs pr = panel_load(xb, ld, t * 32, S - 1, 0, lane);
+    panel_store(panel, lane, pr);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
+    }
+}
+
+__global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p)
+{
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int b = blockIdx.x;
+    const int S = p.S, NT = p.NT, H = p.H, d = p.d;
+    const int spad = NT * 32;
+
+    uint4 *qk_frag = lds;            // [4 k-steps][64 lanes]
+    uint4 *wv_frag = qk_frag + 256;  // [4][64]
+    uint4 *wg_frag = wv_frag + 256;  // [2 row blocks][4][64]
+    uint4 *wo_frag = wg_frag + 512;  // [2 row blocks][4][64]
+    uint4 *panel = wo_frag + 512 + wave * 256;
+    float *maskb = reinterpret_cast<float *>(wo_frag + 512 + 4 * 256); // mask bias per token, -inf past S
+    float *mask01 = maskb + spad;                                       // mask value per token, 0 past S
+    float *part = mask01 + spad;                                        // [4 waves][68]: channel sums, mask sum
+    float *qavg = part + 4 * 68;                                        // [64]
+    float *qv = qavg + GC;                                              // [64] q, bf16-rounded
+    float *wavg = qv + GC;                                              // [64]
+    float *merge = wavg + GC;                                           // [4 waves][64 lanes][MERGE_LD]
+
+    const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
+
+    // ---- weights of phases B and C as MFMA fragments; mask ----
+    for (int idx = tid; idx < 256; idx += 256) {
+        const int ks = idx >> 6, l = idx & 63, e = l & 31, gg = l >> 5;
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (e < d) {
+            v = *reinterpret_cast<const uint4 *>(p.wv + e * GC + ks * 16 + gg * 8);
+        }
+        wv_frag[idx] = v;
+    }
+    for (int idx = tid; idx < 512; idx += 256) {
+        const int rb = idx >> 8, ks = (idx >> 6) & 3, l = idx & 63, i = l & 31, gg = l >> 5;
+        const int ch = gate_channel(rb, 4 * (i >> 3) + (i & 3), (i >> 2) & 1);
+        wg_frag[idx] = *reinterpret_cast<const uint4 *>(p.wg + ch * GC + ks * 16 + gg * 8);
+        const int o = 32 * rb + pi_row(i);
+        wo_frag[idx] = *reinterpret_cast<const uint4 *>(p.wo + o * GC + ks * 16 + gg * 8);
+    }
+    for (int s = tid; s < spad; s += 256) {
+        float m = 0.f, mb = -INFINITY;
+        if (s < S) {
+            m = to_f32(p.mask[(int64_t)b * p.mask_sb + s]);
+            mb = fmaf(m, 1e9f, -1e9f); // reference :120-121
+        }
+        mask01[s] = m;
+        maskb[s] = mb;
+    }
+    __syncthreads();
+
+    // ---- phase A: masked mean of the row, q, and the folded query-key matrix ----
+    {
+        float acc[4][8];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                acc[ks][e] = 0.f;
+            }
+        }
+        float msum = 0.f;
+        for (int t = wave; t < NT; t += 4) {
+            bf16x8 xf[4];
+            load_tile(xb, p.x_ss, t, S, panel, lane, xf);
+            const float m = mask01[t * 32 + r];
+            msum += g == 0 ? m : 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    acc[ks][e] = fmaf(m, to_f32(xf[ks][e]), acc[ks][e]);
+                }
+            }
+        }
+        // sum over the 32 lanes of each half (they hold different tokens of the same channels)
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) {
+            msum += __shfl_xor(msum, off, 64);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    acc[ks][e] += __shfl_xor(acc[ks][e], off, 64);
+                }
+            }
+        }
+        if (r == 0) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    part[wave * 68 + ks * 16 + g * 8 + e] = acc[ks][e];
+                }
+            }
+            if (g == 0) {
+                part[wave * 68 + 64] = msum;
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < GC) {
+        const float tot = part[tid] + part[68 + tid] + part[2 * 68 + tid] + part[3 * 68 + tid];
+        const float ms = part[64] + part[68 + 64] + part[2 * 68 + 64] + part[3 * 68 + 64];
+        const bf16_t qa = (bf16_t)(tot * (1.0f / (ms + 1e-10f))); // reference :66-74
+        qavg[tid] = to_f32(qa);
+        if (p.q_avg != nullptr) {
+            p.q_avg[(int64_t)b * p.qavg_sb + tid] = qa;
+        }
+    }
+    __syncthreads();
+    if (tid < GC) {
+        const bf16_t *wrow = p.wq + tid * GC;
+        float a = 0.f;
+#pragma unroll
+        for (int c8 = 0; c8 < 8; ++c8) {
+            const bf16x8 w8 = as_bf16x8(*reinterpret_cast<const uint4 *>(wrow + c8 * 8));
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                a = fmaf(qavg[c8 * 8 + e], to_f32(w8[e]), a);
+            }
+        }
+        qv[tid] = to_f32((bf16_t)a); // the reference stores q as bf16 (:76-80)
+    }
+    __syncthreads();
+    {
+        // B operand of the logits product: column h (zero for h >= H), 8 channels per lane and k-step
+        const int ks = tid >> 6, h = r;
+        bf16x8 f;
+#pragma unroll
+        for (int e8 = 0; e8 < 8; ++e8) {
+            const int c = ks * 16 + g * 8 + e8;
+            float a = 0.f;
+            if (h < H) {
+                for (int e = 0; e < d; ++e) {
+                    a = fmaf(qv[h * d + e], to_f32(p.wk[e * GC + c]), a);
+                }
+            }
+            f[e8] = (bf16_t)(a * p.scale);
+        }
+        qk_frag[ks * 64 + lane] = as_uint4(f);
+    }
+    __syncthreads();
+
+    // ---- phase B: logits, online softmax, weighted average of V; one (m, l, O^T) state per wave ----
+    {
+        f32x16 o = zero16();
+        float m_run = -1e30f, lsum = 0.f;
+        for (int t = wave; t < NT; t += 4) {
+            bf16x8 xf[4];
+            load_tile(xb, p.x_ss, t, S, panel, lane, xf);
+            f32x16 x1, vv = zero16();
+            const f32x4 *mb4 = reinterpret_cast<const f32x4 *>(maskb + t * 32 + 4 * g);
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 mv = mb4[2 * a];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    x1[4 * a + c] = mv[c];
+                }
+            }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                x1 = mfma(xf[ks], as_bf16x8(qk_frag[ks * 64 + lane]), x1);
+                vv = mfma(xf[ks], as_bf16x8(wv_frag[ks * 64 + lane]), vv);
+            }
+            float mx = x1[0];
+#pragma unroll
+            for (int v = 1; v < 16; ++v) {
+                mx = fmaxf(mx, x1[v]);
+            }
+            mx = half_swap_max(mx);
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+            lsum *= alpha;
+            const float ml = -m_new * LOG2E;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                o[v] *= alpha;
+                x1[v] = __builtin_amdgcn_exp2f(fmaf(x1[v], LOG2E, ml));
+            }
+            m_run = m_new;
+            const bf16x8 p0 = pack8(x1, 0), p1 = pack8(x1, 8);
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                lsum += to_f32(p0[v]) + to_f32(p1[v]);
+            }
+            o = mfma(pack8(vv, 0), p0, o);
+            o = mfma(pack8(vv, 8), p1, o);
+        }
+        float *mine = merge + (wave * 64 + lane) * MERGE_LD;
+        mine[0] = m_run;
+        mine[1] = half_swap_sum(lsum);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            mine[2 + v] = o[v];
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float mw[4], lw[4];
+        float M = -1e30f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            mw[w] = merge[(w * 64 + lane) * MERGE_LD];
+            lw[w] = merge[(w * 64 + lane) * MERGE_LD + 1];
+            M = fmaxf(M, mw[w]);
+        }
+        float L = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            mw[w] = __builtin_amdgcn_exp2f((mw[w] - M) * LOG2E);
+            L = fmaf(lw[w], mw[w], L);
+        }
+        const float inv = 1.0f / L;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float a = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                a = fmaf(merge[(w * 64 + lane) * MERGE_LD + 2 + v], mw[w], a);
+            }
+            const int e = 8 * (v >> 2) + 4 * g + (v & 3);
+            if (r < H && e < d) {
+                wavg[r * d + e] = to_f32((bf16_t)(a * inv)); // the reference stores the weighted average as bf16 (:126-130)
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- phase C: gate, gating, output projection ----
+    {
+        float bgv[32], wv_[32], bov[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int ch = gate_channel(i >> 4, i & 15, g);
+            bgv[i] = p.bg[ch];
+            wv_[i] = wavg[ch];
+            bov[i] = p.bo[32 * (i >> 4) + 16 * g + (i & 15)];
+        }
+        for (int t = wave; t < NT; t += 4) {
+            bf16x8 xf[4];
+            load_tile(xb, p.x_ss, t, S, panel, lane, xf);
+            bf16x8 gf[4];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                f32x16 ga = zero16();
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    ga = mfma(as_bf16x8(wg_frag[(rb * 4 + ks) * 64 + lane]), xf[ks], ga);
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    ga[v] = wv_[rb * 16 + v] * sigmoid_fast(ga[v] + bgv[rb * 16 + v]);
+                }
+                gf[2 * rb] = pack8(ga, 0);
+                gf[2 * rb + 1] = pack8(ga, 8);
+            }
+            const int s = t * 32 + r;
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob) {
+                f32x16 oa = zero16();
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    oa = mfma(as_bf16x8(wo_frag[(ob * 4 + kk) * 64 + lane]), gf[kk], oa);
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    oa[v] += bov[ob * 16 + v];
+                }
+                if (s < S) {
+                    bf16_t *dst = p.out + (int64_t)b * p.out_sb + (int64_t)s * p.out_ss + 32 * ob + 16 * g;
+                    *reinterpret_cast<uint4 *>(dst) = as_uint4(pack8(oa, 0));
+                    *reinterpret_cast<uint4 *>(dst + 8) = as_uint4(pack8(oa, 8));
+                }
+            }
+        }
+    }
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+} // namespace
+
+namespace kutacc_launch {
+
+int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t stream)
+{
+    if (a.batch <= 0 || a.seq_len <= 0 || a.nheads <= 0 || a.head_size <= 0 || !a.q_data || !a.q_mask || !a.query_w ||
+        !a.key_w || !a.value_w || !a.gating_w || !a.output_w || !a.gating_b || !a.output_b || !a.out) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (a.dtype != KUTACC_DTYPE_BF16 || a.nheads * a.head_size != GC || a.nheads > 32 || a.head_size > 32 ||
+        a.batch > INT32_MAX || a.seq_len > 16384) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    // 16-byte row loads of x and the weights, 16-byte stores of out rows
+    if (a.q_data_stride_s % 8 != 0 || a.q_data_stride_b % 8 != 0 || a.out_stride_s % 8 != 0 || a.out_stride_b % 8 != 0 ||
+        !aligned16(a.q_data) || !aligned16(a.out) || !aligned16(a.query_w) || !aligned16(a.key_w) ||
+        !aligned16(a.value_w) || !aligned16(a.gating_w) || !aligned16(a.output_w)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    GlobalParams p;
+    p.x = (const bf16_t *)a.q_data, p.mask = (const bf16_t *)a.q_mask;
+    p.wq = (const bf16_t *)a.query_w, p.wk = (const bf16_t *)a.key_w, p.wv = (const bf16_t *)a.value_w;
+    p.wg = (const bf16_t *)a.gating_w, p.wo = (const bf16_t *)a.output_w;
+    p.bg = a.gating_b, p.bo = a.output_b;
+    p.q_avg = (bf16_t *)a.q_avg, p.out = (bf16_t *)a.out;
+    p.x_sb = a.q_data_stride_b, p.x_ss = a.q_data_stride_s, p.mask_sb = a.q_mask_stride_b;
+    p.qavg_sb = a.q_avg_stride_b, p.out_sb = a.out_stride_b, p.out_ss = a.out_stride_s;
+    p.B = (int)a.batch, p.S = (int)a.seq_len, p.H = (int)a.nheads, p.d = (int)a.head_size;
+    p.NT = (int)((a.seq_len + 31) / 32);
+    p.scale = (float)(1.0 / sqrt((double)a.head_size)); // reference :98
+    const size_t lds_bytes = (size_t)(256 + 256 + 512 + 512 + 4 * 256) * 16 +
+                             (size_t)(2 * p.NT * 32 + 4 * 68 + 3 * GC + 4 * 64 * MERGE_LD) * 4;
+    static size_t configured = 0;
+    if (lds_bytes > configured) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(global_attention_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) {
+            return (int)e;
+        }
+        configured = lds_bytes;
+    }
+    const double BS = (double)a.batch * (double)a.seq_len;
+    kutacc_prof::KernelTimer t("global_attention_kernel", BS * (4.0 * GC * a.head_size + 4.0 * GC * GC + 4.0 * GC), stream);
+    global_attention_kernel<<<dim3((unsigned)a.batch), 256, lds_bytes, stream>>>(p);
+    return kutacc_hip_status(hipGetLastError());
+}
+
+} // namespace kutacc_launch

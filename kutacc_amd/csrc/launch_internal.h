@@ -20,6 +20,9 @@ int gemm_nt(int32_t dtype, const void *a, int64_t lda, const void *w, int64_t ld
 bool fused_attention_supports(const kutacc_hip_attention_args_t &args);
 int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream);
 
+// global_attention.hip
+int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);
+
 // row_kernels.hip
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                    int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream);

@@ -1,0 +1,127 @@
+// MFMA tile helpers shared by the attention kernels (gfx950, bf16 operands, fp32 accumulation).
+//
+// Operand fragments use one format throughout: a [32 rows x 16 k] slab, lane l holding row (l & 31),
+// k-chunk (l >> 5)*8..+8, i.e. 16 contiguous bytes of a row-major bf16 matrix.  Results of
+// v_mfma_f32_32x32x16_bf16 come out as D[i][j] with j = l & 31 and i = 8*(v/4) + 4*(l>>5) + (v&3) for
+// accumulator register v.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_util.h"
+
+namespace kutacc_dev {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+
+constexpr float LOG2E = 1.44269504088896340736f;
+
+__device__ __forceinline__ int pi_row(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
+
+__device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f32x16 zero16()
+{
+    const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    return z;
+}
+
+__device__ __forceinline__ bf16x8 pack8(const f32x16 &v, int base)
+{
+    bf16x8 r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        r[i] = (bf16_t)v[base + i];
+    }
+    return r;
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 u)
+{
+    union {
+        uint4 u;
+        bf16x8 b;
+    } c;
+    c.u = u;
+    return c.b;
+}
+
+__device__ __forceinline__ uint4 as_uint4(bf16x8 b)
+{
+    union {
+        uint4 u;
+        bf16x8 b;
+    } c;
+    c.b = b;
+    return c.u;
+}
+
+// combine the two 32-lane halves of a wave: returns op(x[lane], x[lane ^ 32]) in every lane
+__device__ __forceinline__ float half_swap_max(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Wave-private staging panel in LDS: 32 rows x 128 bytes, in 16-byte slots.  A panel is filled with
+// four fully coalesced loads (each instruction reads 8 rows x 128 contiguous bytes = 8 whole cache
+// lines, lane l -> row 8i + l/8, slot l%8) and read back in MFMA fragment order (lane -> its own
+// row).  Loading fragments straight from global memory would touch 32 different cache lines per
+// instruction, four times the L1 tag traffic.  The slot index is XOR-swizzled by row so that both
+// access patterns are free of LDS bank conflicts.
+__device__ __forceinline__ int panel_slot(int row, int chunk)
+{
+    return row * 8 + (chunk ^ ((row & 7) ^ ((row >> 4) & 1)));
+}
+
+// issue the four coalesced loads of a panel: rows row0 .. row0+31 (clamped to last_row) of a
+// row-major bf16 matrix with leading dimension ld, 64 columns starting at col0
+struct PanelRegs {
+    uint4 r0, r1, r2, r3; // named members rather than an array, so that they always live in registers
+};
+
+__device__ __forceinline__ uint4 panel_load_one(const bf16_t *base, int64_t ld, int row, int last_row, int col0, int lane)
+{
+    row = row < last_row ? row : last_row;
+    return *reinterpret_cast<const uint4 *>(base + (int64_t)row * ld + col0 + (lane & 7) * 8);
+}
+
+__device__ __forceinline__ PanelRegs panel_load(const bf16_t *base, int64_t ld, int row0, int last_row, int col0, int lane)
+{
+    PanelRegs p;
+    const int row = row0 + (lane >> 3);
+    p.r0 = panel_load_one(base, ld, row, last_row, col0, lane);
+    p.r1 = panel_load_one(base, ld, row + 8, last_row, col0, lane);
+    p.r2 = panel_load_one(base, ld, row + 16, last_row, col0, lane);
+    p.r3 = panel_load_one(base, ld, row + 24, last_row, col0, lane);
+    return p;
+}
+
+__device__ __forceinline__ void panel_store(uint4 *panel, int lane, const PanelRegs &p)
+{
+    const int row = lane >> 3, chunk = lane & 7;
+    panel[panel_slot(row, chunk)] = p.r0;
+    panel[panel_slot(row + 8, chunk)] = p.r1;
+    panel[panel_slot(row + 16, chunk)] = p.r2;
+    panel[panel_slot(row + 24, chunk)] = p.r3;
+}
+
+__device__ __forceinline__ float sigmoid_fast(float x)
+{
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
+}
+
+} // namespace kutacc_dev

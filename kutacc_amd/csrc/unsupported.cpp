@@ -19,7 +19,6 @@ KUTACC_UNSUPPORTED(kutacc_af2_transpose)
 KUTACC_UNSUPPORTED(kutacc_af2_all_gather)
 KUTACC_UNSUPPORTED(kutacc_af2_outer_product_mean_calc_left_and_right_mul)
 KUTACC_UNSUPPORTED(kutacc_af2_outer_product_mean_chunk)
-KUTACC_UNSUPPORTED(kutacc_af2_global_attention)
 KUTACC_UNSUPPORTED(kutacc_af2_transition)
 KUTACC_UNSUPPORTED(kutacc_af2_invariant_point)
 KUTACC_UNSUPPORTED(kutacc_af2_rigid_rot_vec_mul)

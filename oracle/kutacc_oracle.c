@@ -14,10 +14,11 @@
  *                                 buffers, OpenMP.  This is the timed CPU baseline, and measures how
  *                                 far the reference itself sits from R32.
  *
- * plus the two row operators in front of the path (LayerNorm, Linear).
+ * plus the two row operators in front of the path (LayerNorm, Linear) and an R32 restatement of the
+ * global (extra-MSA column) attention, reference src/attention/global_attention.cpp:30-164.
  *
  * Pinning status (the reference ships no numeric test for any of this):
- *   - R32, layernorm, linear: pinned by tests/test_oracle_pinning.py against library routines
+ *   - R32 (both attentions), layernorm, linear: pinned by tests/test_oracle_pinning.py against library routines
  *     (torch matmul / scaled_dot_product_attention / layer_norm / linear), a pure-Python brute
  *     force on tiny shapes, and closed-form invariants.
  *   - Rbf16 rounding points: pinned only relative to R32 (must agree within bf16 tolerances);
@@ -174,6 +175,114 @@ void oracle_gating_attention_f32(const float *input, const float *wq, const floa
         }
     }
     free(q), free(k), free(v), free(g), free(avg);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Global (extra-MSA column) attention, reference src/attention/global_attention.cpp:30-164.
+ * One query per batch row and head, one key/value head shared by all heads:
+ *   q_avg[b,:] = sum_s mask[b,s] x[b,s,:] / (sum_s mask[b,s] + 1e-10)                (:47-74)
+ *   q[b] = q_avg[b].Wq^T viewed [H, d];  k[b,s] = Wk.x[b,s] (d);  v[b,s] = Wv.x[b,s] (d)   (:76-92)
+ *   gate[b,s,:] = x[b,s,:].Wg^T + bg                                               (:93-97)
+ *   logit[h,s] = (q[b,h].k[b,s]) * 1/sqrt(d) + (mask[b,s]*1e9 - 1e9)   fp32 adds      (:112-124)
+ *   p = softmax_s(logit);  wavg[h,:] = sum_s p[h,s] v[b,s,:]                        (:126-132)
+ *   gated[b,s,:] = sigmoid(gate[b,s,:]) * wavg (wavg flattened [H*d] = C)           (:133-153)
+ *   out = gated.Wo^T + bo                                                           (:157-161)
+ * Wq, Wg, Wo are [C, C] stored [out, in]; Wk, Wv are [d, C].  mask is [B, S].
+ * R32: fp32 operands, double accumulation; the mask bias is formed and added in fp32 as the
+ * reference does, so an all-zero mask row gives uniform attention.
+ * ---------------------------------------------------------------------------------------------- */
+void oracle_global_attention_f32(const float *x, const float *mask, const float *wq, const float *wk, const float *wv,
+                                 const float *wg, const float *bg, const float *wo, const float *bo, int64_t B,
+                                 int64_t S, int64_t H, int64_t d, float *out, float *q_avg_out)
+{
+    const int64_t C = H * d;
+    const double scale = (double)(float)(1.0 / sqrt((double)d));
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < B; ++b) {
+        double *qa = malloc(sizeof(double) * C), *q = malloc(sizeof(double) * C);
+        double *k = malloc(sizeof(double) * S * d), *v = malloc(sizeof(double) * S * d);
+        double *p = malloc(sizeof(double) * S), *wavg = malloc(sizeof(double) * C);
+        double *gated = malloc(sizeof(double) * C);
+        const float *xb = x + b * S * C;
+        double msum = 0.0;
+        for (int64_t c = 0; c < C; ++c) {
+            qa[c] = 0.0;
+        }
+        for (int64_t s = 0; s < S; ++s) {
+            msum += (double)mask[b * S + s];
+            for (int64_t c = 0; c < C; ++c) {
+                qa[c] += (double)mask[b * S + s] * (double)xb[s * C + c];
+            }
+        }
+        for (int64_t c = 0; c < C; ++c) {
+            qa[c] /= (msum + 1e-10);
+            if (q_avg_out) {
+                q_avg_out[b * C + c] = (float)qa[c];
+            }
+        }
+        for (int64_t o = 0; o < C; ++o) {
+            double acc = 0.0;
+            for (int64_t c = 0; c < C; ++c) {
+                acc += qa[c] * (double)wq[o * C + c];
+            }
+            q[o] = acc;
+        }
+        for (int64_t s = 0; s < S; ++s) {
+            for (int64_t e = 0; e < d; ++e) {
+                double ak = 0.0, av = 0.0;
+                for (int64_t c = 0; c < C; ++c) {
+                    ak += (double)xb[s * C + c] * (double)wk[e * C + c];
+                    av += (double)xb[s * C + c] * (double)wv[e * C + c];
+                }
+                k[s * d + e] = ak;
+                v[s * d + e] = av;
+            }
+        }
+        for (int64_t h = 0; h < H; ++h) {
+            double m = -INFINITY;
+            for (int64_t s = 0; s < S; ++s) {
+                double dot = 0.0;
+                for (int64_t e = 0; e < d; ++e) {
+                    dot += q[h * d + e] * k[s * d + e];
+                }
+                const float biasf = fmaf(mask[b * S + s], 1e9f, -1e9f);
+                const float xf = (float)(dot * scale) + biasf;
+                p[s] = (double)xf;
+                if (p[s] > m) {
+                    m = p[s];
+                }
+            }
+            double sum = 0.0;
+            for (int64_t s = 0; s < S; ++s) {
+                p[s] = exp(p[s] - m);
+                sum += p[s];
+            }
+            for (int64_t e = 0; e < d; ++e) {
+                double acc = 0.0;
+                for (int64_t s = 0; s < S; ++s) {
+                    acc += p[s] * v[s * d + e];
+                }
+                wavg[h * d + e] = acc / sum;
+            }
+        }
+        for (int64_t s = 0; s < S; ++s) {
+            for (int64_t o = 0; o < C; ++o) {
+                double acc = (double)bg[o];
+                for (int64_t c = 0; c < C; ++c) {
+                    acc += (double)xb[s * C + c] * (double)wg[o * C + c];
+                }
+                gated[o] = wavg[o] / (1.0 + exp(-acc));
+            }
+            for (int64_t o = 0; o < C; ++o) {
+                double acc = (double)bo[o];
+                for (int64_t c = 0; c < C; ++c) {
+                    acc += gated[c] * (double)wo[o * C + c];
+                }
+                out[(b * S + s) * C + o] = (float)acc;
+            }
+        }
+        free(qa), free(q), free(k), free(v), free(p), free(wavg), free(gated);
+    }
 }
 
 /* ------------------------------------------------------------------------------------------------

@@ -161,6 +161,44 @@ def linear_f32(act, w, bias=None, beta=0.0, result=None):
     return res
 
 
+# ---- global (extra-MSA column) attention ------------------------------------------------------------
+def global_attention_f32(x, mask, wq, wk, wv, wg, bg, wo, bo, nheads, return_q_avg=False):
+    """x [B,S,C]; mask [B,S]; wq, wg, wo [C,C] stored [out,in]; wk, wv [d,C]; bg, bo [C] -> out [B,S,C]."""
+    x = _f32(x)
+    B, S, C = x.shape
+    d = C // nheads
+    args = [_f32(a) for a in (mask, wq, wk, wv, wg, bg, wo, bo)]
+    out = np.empty((B, S, C), dtype=np.float32)
+    qa = np.empty((B, C), dtype=np.float32) if return_q_avg else None
+    lib().oracle_global_attention_f32(_ptr(x, _f32p), *[_ptr(a, _f32p) for a in args], _i64(B), _i64(S), _i64(nheads),
+                                      _i64(d), _ptr(out, _f32p), _ptr(qa, _f32p))
+    return (out, qa) if return_q_avg else out
+
+
+def global_attention_f64_numpy(x, mask, wq, wk, wv, wg, bg, wo, bo, nheads):
+    """Textbook float64 formulation of reference src/attention/global_attention.cpp:30-164; the mask bias
+    mask*1e9 - 1e9 is formed and added in fp32 (:120-123)."""
+    f = lambda a: np.asarray(a, dtype=np.float64)  # noqa: E731
+    x, mask = f(x), f(mask)
+    B, S, C = x.shape
+    H, d = nheads, C // nheads
+    q_avg = (mask[:, :, None] * x).sum(axis=1) / (mask.sum(axis=1, keepdims=True) + 1e-10)
+    q = (q_avg @ f(wq).T).reshape(B, H, d)
+    k = x @ f(wk).T  # [B,S,d]
+    v = x @ f(wv).T
+    gate = x @ f(wg).T + f(bg)
+    scale = float(np.float32(1.0 / np.sqrt(float(d))))
+    logits = np.einsum("bhd,bsd->bhs", q, k) * scale
+    bias = (np.asarray(mask, dtype=np.float32) * np.float32(1e9) + np.float32(-1e9))
+    xl = (logits.astype(np.float32) + bias[:, None, :]).astype(np.float64)
+    xl = xl - xl.max(axis=-1, keepdims=True)
+    p = np.exp(xl)
+    p /= p.sum(axis=-1, keepdims=True)
+    wavg = np.einsum("bhs,bsd->bhd", p, v).reshape(B, 1, C)
+    gated = wavg / (1.0 + np.exp(-gate))
+    return gated @ f(wo).T + f(bo)
+
+
 # ---- independent numpy fp64 twin (used to pin the C code, and as R64 for golden fixtures) ---------
 def gating_attention_f64_numpy(x, wq, wk, wv, wg, bg, wo, bo, bias, nb, nheads, return_avg=False):
     """Textbook formulation in float64; the two bias additions are fp32 additions so that the -1e9

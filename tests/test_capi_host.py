@@ -39,7 +39,7 @@ def test_headers_and_binding_agree_on_symbol_list():
 
 def test_unimplemented_operators_resolve_and_report():
     L = capi.lib()
-    for name in ("kutacc_af2_transition", "kutacc_af2_global_attention", "kutacc_af2_transpose",
+    for name in ("kutacc_af2_transition", "kutacc_af2_transpose",
                  "kutacc_comm_init", "kutacc_af2_triangle_multiplication_last"):
         assert hasattr(L, name), name
     L.kutacc_af2_transition(None, None, None)
@@ -149,3 +149,28 @@ def test_launch_layer_rejects_bad_arguments_without_a_device():
     assert L.kutacc_hip_layernorm_rows(None, 1, None, None, None, 1, 1, 1, 1e-5, capi.K_BF16, None) == capi.EINVAL
     assert L.kutacc_hip_linear(None, 1, None, 1, None, None, 1, 1, 1, 0.0, capi.K_BF16, None) == capi.EINVAL
     assert L.kutacc_hip_pair_bias(None, None, None, None, None, None, 1, 1, 1, 1, 1e-5, capi.K_BF16, None) == capi.EINVAL
+
+
+# ---- kutacc_af2_global_attention: the five null-pointer cases of reference test/functest/cal/global_attention_test.cpp:18-190
+@pytest.mark.parametrize("null_index", range(5))
+def test_global_attention_null_pointers_are_rejected(null_index, capfd):
+    a, x, ap, xp, weights, inputs = _reference_style_arguments()
+    weights.nchannels = 64
+    args = [ctypes.byref(inputs), ap, ap, ctypes.byref(weights), ap]
+    args[null_index] = None
+    capi.lib().kutacc_af2_global_attention(*args)
+    assert capi.error_flag()
+    assert "nullptr error or invalid int value error" in capfd.readouterr().err
+
+
+def test_global_attention_needs_64_channels_and_checks_scalars_before_handles(capfd):
+    # handles are plain floats, as in the reference's tests: nothing may be read through them
+    a, x, ap, xp, weights, inputs = _reference_style_arguments()
+    capi.lib().kutacc_af2_global_attention(ctypes.byref(inputs), ap, ap, ctypes.byref(weights), ap)  # nchannels == 2
+    assert capi.error_flag()
+    capi.clear_error()
+    weights.nchannels = 64
+    inputs.batch = 0
+    capi.lib().kutacc_af2_global_attention(ctypes.byref(inputs), ap, ap, ctypes.byref(weights), ap)
+    assert capi.error_flag()
+    assert "input param <= 0 or overflow" in capfd.readouterr().err

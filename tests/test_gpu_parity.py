@@ -343,7 +343,7 @@ def test_linear_matches_oracle(torch_cuda):
     helpers.assert_within(helpers.to_numpy(res), ref2, 2.0 ** -7 * np.abs(ref2) + 1e-6, "linear beta=1")
 
 
-@pytest.mark.parametrize("config", [1, 3])
+@pytest.mark.parametrize("config", [1, 3, 2])
 def test_pair_bias_producer_matches_oracle(torch_cuda, config):
     """LN(z) -> [H, c_z] linear -> [H, S, S], one pass; against oracle LayerNorm + Linear + permute."""
     from oracle import oracle

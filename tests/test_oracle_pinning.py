@@ -329,3 +329,121 @@ def test_linear_matches_torch():
                                                     result_bits=oracle.to_bf16_bits(prev)))
     ref2 = ref - bias + prev
     assert np.all(np.abs(got2 - ref2) <= 2.0 ** -8 * np.abs(ref2) + 1e-6)
+
+
+# ---- global (extra-MSA column) attention: reference src/attention/global_attention.cpp:30-164 ---------------------
+def make_global_case(seed, B, S, H, d, mask_mode="random"):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    C = H * d
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
+    mask = np.ones((B, S), dtype=np.float32)
+    if mask_mode == "random":
+        mask = (rng.random((B, S)) > 0.3).astype(np.float32)
+        mask[:, 0] = 1
+    return dict(x=f(B, S, C), mask=mask, wq=f(C, C) / math.sqrt(C), wk=f(d, C) / math.sqrt(C), wv=f(d, C) / math.sqrt(C),
+                wg=f(C, C) / math.sqrt(C), bg=f(C), wo=f(C, C) / math.sqrt(C), bo=f(C), nheads=H)
+
+
+def run_global(c, fn=None, **kw):
+    fn = fn or oracle.global_attention_f32
+    return fn(c["x"], c["mask"], c["wq"], c["wk"], c["wv"], c["wg"], c["bg"], c["wo"], c["bo"], c["nheads"], **kw)
+
+
+@pytest.mark.parametrize("mask_mode", ["ones", "random"])
+def test_global_numpy_twin_matches_torch_sdpa(mask_mode):
+    """Library routine: torch scaled_dot_product_attention with one query per head and a shared key/value head."""
+    c = make_global_case(11, 3, 19, 4, 16, mask_mode)
+    t = lambda a: torch.from_numpy(np.asarray(a, dtype=np.float64))  # noqa: E731
+    x, mask = t(c["x"]), t(c["mask"])
+    B, S, C = x.shape
+    H, d = c["nheads"], C // c["nheads"]
+    q_avg = (mask[:, :, None] * x).sum(1) / (mask.sum(1, keepdim=True) + 1e-10)
+    q = torch.nn.functional.linear(q_avg, t(c["wq"])).reshape(B, H, 1, d)
+    k = torch.nn.functional.linear(x, t(c["wk"]))[:, None].expand(B, H, S, d)
+    v = torch.nn.functional.linear(x, t(c["wv"]))[:, None].expand(B, H, S, d)
+    bias = (1e9 * (mask - 1))[:, None, None, :]
+    wavg = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=bias, scale=1 / math.sqrt(d))
+    gate = torch.sigmoid(torch.nn.functional.linear(x, t(c["wg"]), t(c["bg"])))
+    out = torch.nn.functional.linear(gate * wavg.reshape(B, 1, C), t(c["wo"]), t(c["bo"]))
+    # the twin forms the mask bias and adds it in fp32, as the reference does: 1e-7-level differences to float64
+    np.testing.assert_allclose(run_global(c, oracle.global_attention_f64_numpy), out.numpy(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 2, 4), (3, 37, 8, 8), (1, 64, 4, 16)])
+def test_global_c_oracle_matches_numpy_twin(shape):
+    c = make_global_case(12, *shape)
+    c["mask"][-1] = 0  # one fully masked row
+    np.testing.assert_allclose(run_global(c), run_global(c, oracle.global_attention_f64_numpy), rtol=2e-5, atol=2e-6)
+
+
+def test_global_c_oracle_matches_python_bruteforce():
+    """Every index written out, on a case small enough for pure Python loops."""
+    c = make_global_case(13, 2, 4, 2, 3)
+    x, mask = c["x"].astype(float), c["mask"].astype(float)
+    B, S, C = x.shape
+    H, d = 2, 3
+    out = np.zeros((B, S, C))
+    for b in range(B):
+        msum = sum(mask[b, s] for s in range(S))
+        q_avg = [sum(mask[b, s] * x[b, s, ch] for s in range(S)) / (msum + 1e-10) for ch in range(C)]
+        q = [sum(q_avg[ch] * float(c["wq"][o, ch]) for ch in range(C)) for o in range(C)]
+        k = [[sum(x[b, s, ch] * float(c["wk"][e, ch]) for ch in range(C)) for e in range(d)] for s in range(S)]
+        v = [[sum(x[b, s, ch] * float(c["wv"][e, ch]) for ch in range(C)) for e in range(d)] for s in range(S)]
+        wavg = [0.0] * C
+        for h in range(H):
+            logit = [sum(q[h * d + e] * k[s][e] for e in range(d)) / math.sqrt(d) + 1e9 * (mask[b, s] - 1) for s in range(S)]
+            m = max(logit)
+            pe = [math.exp(v_ - m) for v_ in logit]
+            z = sum(pe)
+            for e in range(d):
+                wavg[h * d + e] = sum(pe[s] / z * v[s][e] for s in range(S))
+        for s in range(S):
+            gated = [wavg[o] / (1 + math.exp(-(sum(x[b, s, ch] * float(c["wg"][o, ch]) for ch in range(C)) + float(c["bg"][o]))))
+                     for o in range(C)]
+            for o in range(C):
+                out[b, s, o] = sum(gated[ch] * float(c["wo"][o, ch]) for ch in range(C)) + float(c["bo"][o])
+    np.testing.assert_allclose(run_global(c), out, rtol=2e-5, atol=2e-6)
+
+
+def test_global_closed_forms():
+    c = make_global_case(14, 2, 9, 4, 4, "ones")
+    C = 16
+    # zero query weight -> uniform attention -> the weighted average is the plain mean of v over the row
+    c0 = dict(c, wq=np.zeros_like(c["wq"]), wg=np.zeros_like(c["wg"]), bg=np.zeros(C, np.float32))
+    v = c["x"].astype(np.float64) @ c["wv"].astype(np.float64).T          # [B,S,d]
+    wavg = np.tile(v.mean(axis=1), (1, 4))                                # every head sees the same mean
+    expect = (0.5 * wavg) @ c["wo"].astype(np.float64).T + c["bo"]        # gate = sigmoid(0) = 0.5, same for every token
+    got = run_global(c0)
+    np.testing.assert_allclose(got, np.broadcast_to(expect[:, None, :], got.shape), rtol=2e-5, atol=2e-6)
+    # zero output weight -> the output bias
+    np.testing.assert_allclose(run_global(dict(c, wo=np.zeros_like(c["wo"]))), np.broadcast_to(c["bo"], got.shape),
+                               rtol=0, atol=1e-7)
+
+
+def test_global_masked_token_has_no_influence_on_the_others_and_q_avg_ignores_it():
+    c = make_global_case(15, 2, 11, 8, 8)
+    c["mask"][:, 3] = 0
+    base, qa = run_global(c, return_q_avg=True)
+    c2 = dict(c, x=c["x"].copy())
+    c2["x"][:, 3] = 7.0 * c2["x"][:, 3] + 1.0
+    moved, qa2 = run_global(c2, return_q_avg=True)
+    others = [s for s in range(11) if s != 3]
+    np.testing.assert_array_equal(qa, qa2)
+    np.testing.assert_array_equal(base[:, others], moved[:, others])
+    assert np.abs(base[:, 3] - moved[:, 3]).max() > 1e-3  # the token's own gate does change its own output
+
+
+def test_global_fully_masked_row_attends_uniformly():
+    c = make_global_case(16, 2, 13, 8, 8, "ones")
+    c["mask"][1] = 0
+    out, qa = run_global(c, return_q_avg=True)
+    assert np.all(qa[1] == 0)
+    uni = dict(c, mask=np.ones_like(c["mask"]), wq=np.zeros_like(c["wq"]))
+    np.testing.assert_allclose(out[1], run_global(uni)[1], rtol=2e-5, atol=2e-6)
+
+
+def test_global_token_permutation_permutes_output():
+    c = make_global_case(17, 2, 10, 4, 16)
+    perm = np.random.Generator(np.random.PCG64(5)).permutation(10)
+    c2 = dict(c, x=c["x"][:, perm].copy(), mask=c["mask"][:, perm].copy())
+    np.testing.assert_allclose(run_global(c2), run_global(c)[:, perm], rtol=2e-5, atol=2e-6)
