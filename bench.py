@@ -62,10 +62,11 @@ def cpu_baseline(w, budget_s=15.0):
 
 
 def producer_rates(config, reps=50):
-    """Achieved HBM rates of the two row kernels in front of the operator, at this configuration's pair
-    tensor z [S, S, 128]: LayerNorm over all rows, and the fused LN -> [H, c_z] projection -> [H, S, S] pair
-    bias (with and without writing the normalised z).  Algorithmic bytes: rows*c_z*2 read, plus what is
-    written (rows*c_z*2 for LN / z_norm, rows*H*2 for the pair bias)."""
+    """Achieved HBM rates of the HBM-bound kernels around the operator: the two row kernels in front of it, at this
+    configuration's pair tensor z [S, S, 128] (LayerNorm over all rows; the fused LN -> [H, c_z] projection ->
+    [H, S, S] pair bias, with and without writing the normalised z), and the global (extra-MSA column) attention.
+    Algorithmic bytes: rows*c_z*2 read plus what is written (rows*c_z*2 for LN / z_norm, rows*H*2 for the pair bias);
+    for the global attention its input read once and its output written once."""
     import numpy as np
     import torch
     from kutacc_amd import capi
@@ -104,7 +105,30 @@ def producer_rates(config, reps=50):
     t_pbz = timed(lambda: L.kutacc_hip_pair_bias(dz.data_ptr(), dg.data_ptr(), db.data_ptr(), dw.data_ptr(), nb.data_ptr(),
                                                  zn.data_ptr(), S, S, cz, H, 1e-5, capi.K_BF16, stream))
     zb = rows * cz * 2
+
+    # global (extra-MSA column) attention at an extra-MSA sized call: N_res batch rows of 1024 extra sequences, 64 channels
+    import math
+    gB, gS, gH, gd = (256 if config != 5 else 384), 1024, 8, 8
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rnd = lambda *sh: torch.randn(*sh, device="cuda", generator=g)  # noqa: E731
+    gx = rnd(gB, gS, 64).to(torch.bfloat16)
+    gmask = (torch.rand(gB, gS, 1, device="cuda", generator=g) > 0.25).to(torch.bfloat16)
+    gw = {n: (rnd(*sh) / math.sqrt(64)).to(torch.bfloat16)
+          for n, sh in (("wq", (64, 64)), ("wk", (gd, 64)), ("wv", (gd, 64)), ("wg", (64, 64)), ("wo", (64, 64)))}
+    gbg, gbo = torch.ones(64, device="cuda"), torch.zeros(64, device="cuda")
+    gout = torch.empty_like(gx)
+    gz = lambda *sh: torch.empty(sh, device="cuda", dtype=torch.bfloat16)  # noqa: E731
+    gop = capi.GlobalAttention(gx, gmask, gw["wq"], gw["wk"], gw["wv"], gw["wg"], gbg, gw["wo"], gbo, gH, gout,
+                               dict(q=gz(gB, 64), k=gz(gB * gS, gd), v=gz(gd, gB * gS), gate=gz(gB, gS, 64), avg=gz(gB, 64)))
+    capi.set_stream(stream)
+    capi.set_blocking(False)
+    t_ga = timed(gop.run)
+    capi.set_blocking(True)
+    capi.set_stream(None)
+    assert not capi.error_flag()
     return {
+        "global_attention": {"shape": f"B={gB} S={gS} C=64 H={gH}", "us": round(t_ga * 1e6, 2),
+                             "GB/s": round(2 * gB * gS * 64 * 2 / t_ga / 1e9, 1)},
         "shape": f"z [{S},{S},{cz}] bf16, H={H}",
         "layernorm_rows": {"us": round(t_ln * 1e6, 2), "GB/s": round(2 * zb / t_ln / 1e9, 1)},
         "pair_bias": {"us": round(t_pb * 1e6, 2), "GB/s": round((zb + rows * H * 2) / t_pb / 1e9, 1)},

@@ -6,10 +6,11 @@
 //   q_avg = sum_s mask[s] x[s,:] / (sum_s mask[s] + 1e-10);  q = q_avg.Wq^T  viewed [H, d]
 //   logit[h,s] = q[h].(Wk x[s]) / sqrt(d) + (mask[s]*1e9 - 1e9);  p = softmax_s
 //   wavg[h,:] = sum_s p[h,s] (Wv x[s]);  out[s,:] = (sigmoid(x[s].Wg^T + bg) * wavg).Wo^T + bo
-// One workgroup (four waves) owns a batch row and walks it three times in 32-token tiles, each tile
-// fetched with whole-cache-line loads through the wave's LDS staging panel: (A) masked mean, (B)
-// logits, online softmax and weighted average, (C) gate, gating and output projection.  Nothing but
-// q_avg and out is written to memory.  All contractions are v_mfma_f32_32x32x16_bf16:
+// One workgroup (four waves) owns a batch row and walks it in 32-token tiles in three phases: (A) masked
+// mean, (B) logits, online softmax and weighted average, (C) gate, gating and output projection.  Tiles
+// arrive with whole-cache-line loads through the wave's LDS staging panel, the next one in flight while
+// the current one is processed; up to seq_len 1024 a wave keeps the fragments of its tiles in registers
+// after phase A, so the row is read from memory once.  Nothing but q_avg and out is written to memory.  All contractions are v_mfma_f32_32x32x16_bf16:
 //   B: logits^T[s, h] = X[s, :] . QK^T with QK[h, :] = q[h].Wk / sqrt(d) folded per batch row (heads are the
 //      columns, 8 of 32 used for H = 8); V[s, e] = X . Wv^T; O^T[e, h] += V^T . P^T -- the accumulators
 //      of the first two products are directly the operands of the third, as in the gated attention
@@ -51,19 +52,14 @@ __device__ __forceinline__ int gate_channel(int rb, int v, int g)
     return 16 * (idx >> 3) + 8 * g + (idx & 7);
 }
 
-__device__ __forceinline__ void load_tile(const bf16_t *xb, int64_t ld, int t, int S, uint4 *panel, int lane, bf16x8 (&xf)[4])
-{
-    const int r = lane & 31, g = lane >> 5;
-    const PanelRegs pr = panel_load(xb, ld, t * 32, S - 1, 0, lane);
-    panel_store(panel, lane, pr);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
-    }
-}
-
+// CACHED: the row has at most 32 tiles (seq_len <= 1024), so each wave keeps the fragments of its (at most 8) tiles
+// in registers after phase A and the row is read from memory once; otherwise every phase streams the row again.
+template <bool CACHED>
 __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p)
 {
+    constexpr int MAXI = CACHED ? 8 : (1 << 24); // tiles per wave
+    constexpr int UNR = CACHED ? 8 : 1;          // the cached tile array needs compile-time indices
+    bf16x8 xs[CACHED ? 8 : 1][4];
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
@@ -124,9 +120,24 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
             }
         }
         float msum = 0.f;
-        for (int t = wave; t < NT; t += 4) {
+        // the loads of the next tile are in flight while this one is summed
+        PanelRegs nxt = panel_load(xb, p.x_ss, wave * 32, S - 1, 0, lane);
+#pragma unroll(UNR)
+        for (int i = 0; i < MAXI; ++i) {
+            const int t = wave + 4 * i;
+            if (t >= NT) {
+                break;
+            }
             bf16x8 xf[4];
-            load_tile(xb, p.x_ss, t, S, panel, lane, xf);
+            panel_store(panel, lane, nxt);
+            nxt = panel_load(xb, p.x_ss, (t + 4 < NT ? t + 4 : t) * 32, S - 1, 0, lane);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
+                if (CACHED) {
+                    xs[i][ks] = xf[ks];
+                }
+            }
             const float m = mask01[t * 32 + r];
             msum += g == 0 ? m : 0.f;
 #pragma unroll
@@ -210,9 +221,30 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
     {
         f32x16 o = zero16();
         float m_run = -1e30f, lsum = 0.f;
-        for (int t = wave; t < NT; t += 4) {
+        PanelRegs nxt;
+        if (!CACHED) {
+            nxt = panel_load(xb, p.x_ss, wave * 32, S - 1, 0, lane);
+        }
+#pragma unroll(UNR)
+        for (int i = 0; i < MAXI; ++i) {
+            const int t = wave + 4 * i;
+            if (t >= NT) {
+                break;
+            }
             bf16x8 xf[4];
-            load_tile(xb, p.x_ss, t, S, panel, lane, xf);
+            if (CACHED) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    xf[ks] = xs[i][ks];
+                }
+            } else {
+                panel_store(panel, lane, nxt);
+                nxt = panel_load(xb, p.x_ss, (t + 4 < NT ? t + 4 : t) * 32, S - 1, 0, lane);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
+                }
+            }
             f32x16 x1, vv = zero16();
             const f32x4 *mb4 = reinterpret_cast<const f32x4 *>(maskb + t * 32 + 4 * g);
 #pragma unroll
@@ -294,17 +326,39 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
 
     // ---- phase C: gate, gating, output projection ----
     {
-        float bgv[32], wv_[32], bov[32];
+        // per-channel constants of the gating, in the order the accumulators hold them
+        float bgv[32], wv_[32];
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
             const int ch = gate_channel(i >> 4, i & 15, g);
             bgv[i] = p.bg[ch];
             wv_[i] = wavg[ch];
-            bov[i] = p.bo[32 * (i >> 4) + 16 * g + (i & 15)];
         }
-        for (int t = wave; t < NT; t += 4) {
+        const float *bop = p.bo + 16 * g;
+        PanelRegs nxt;
+        if (!CACHED) {
+            nxt = panel_load(xb, p.x_ss, wave * 32, S - 1, 0, lane);
+        }
+#pragma unroll(UNR)
+        for (int i = 0; i < MAXI; ++i) {
+            const int t = wave + 4 * i;
+            if (t >= NT) {
+                break;
+            }
             bf16x8 xf[4];
-            load_tile(xb, p.x_ss, t, S, panel, lane, xf);
+            if (CACHED) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    xf[ks] = xs[i][ks];
+                }
+            } else {
+                panel_store(panel, lane, nxt);
+                nxt = panel_load(xb, p.x_ss, (t + 4 < NT ? t + 4 : t) * 32, S - 1, 0, lane);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
+                }
+            }
             bf16x8 gf[4];
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb) {
@@ -329,8 +383,12 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
                     oa = mfma(as_bf16x8(wo_frag[(ob * 4 + kk) * 64 + lane]), gf[kk], oa);
                 }
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    oa[v] += bov[ob * 16 + v];
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(bop + 32 * ob + 4 * a);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        oa[4 * a + c] += bv[c];
+                    }
                 }
                 if (s < S) {
                     bf16_t *dst = p.out + (int64_t)b * p.out_sb + (int64_t)s * p.out_ss + 32 * ob + 16 * g;
@@ -377,18 +435,24 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
     p.scale = (float)(1.0 / sqrt((double)a.head_size)); // reference :98
     const size_t lds_bytes = (size_t)(256 + 256 + 512 + 512 + 4 * 256) * 16 +
                              (size_t)(2 * p.NT * 32 + 4 * 68 + 3 * GC + 4 * 64 * MERGE_LD) * 4;
-    static size_t configured = 0;
-    if (lds_bytes > configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(global_attention_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    const bool cached = p.NT <= 32;
+    static size_t configured[2] = {0, 0};
+    if (lds_bytes > configured[cached]) {
+        const void *fn = cached ? reinterpret_cast<const void *>(global_attention_kernel<true>)
+                                : reinterpret_cast<const void *>(global_attention_kernel<false>);
+        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) {
             return (int)e;
         }
-        configured = lds_bytes;
+        configured[cached] = lds_bytes;
     }
     const double BS = (double)a.batch * (double)a.seq_len;
     kutacc_prof::KernelTimer t("global_attention_kernel", BS * (4.0 * GC * a.head_size + 4.0 * GC * GC + 4.0 * GC), stream);
-    global_attention_kernel<<<dim3((unsigned)a.batch), 256, lds_bytes, stream>>>(p);
+    if (cached) {
+        global_attention_kernel<true><<<dim3((unsigned)a.batch), 256, lds_bytes, stream>>>(p);
+    } else {
+        global_attention_kernel<false><<<dim3((unsigned)a.batch), 256, lds_bytes, stream>>>(p);
+    }
     return kutacc_hip_status(hipGetLastError());
 }
 
