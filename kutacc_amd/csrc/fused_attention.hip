@@ -6,24 +6,23 @@
 // (reference src/attention/gating_attention.cpp:47-66, 97-147) -- stays in LDS and registers:
 //
 //   persistent_head_kernel  seq_len <= 384 (C=128) / 256 (C=256).  One workgroup per CU keeps one head
-//       for its lifetime and walks batch rows.  Its waves are specialised: "projection" waves hold
-//       one weight matrix of the head in registers and produce K, V, Q, gate of the NEXT batch row
-//       into LDS (MFMA-bound) while the "attention" waves run the online softmax of the current one
-//       (VALU-bound); K/V are double-buffered, two workgroup barriers per batch row.
+//       for its lifetime (its four weight matrices staged once in LDS as MFMA fragments) and walks
+//       batch rows; wave j owns sequence block j: it projects the block's K, V, Q and gate, then
+//       attends its 32 queries against all keys of the row.
 //   fused_head_kernel       any seq_len <= 1024.  One workgroup per unit; projections first (weights
-//       staged through LDS in groups), then attention.
+//       staged through LDS in groups), then attention, up to four query blocks per wave.
 //
+// Both run the same attention blocks.  attend_block_l2 is the fast one (logits in log2 units, no running
+// maximum, pair bias from a fragment-major copy made by pair_bias_fragments_kernel, row sums on the
+// matrix core); attend_block and attend_block_direct are the general ones (running maximum with lazy
+// rescale, pair bias read in place) for calls whose pair bias cannot be copied.
 // A third kernel, output_projection_kernel, is the final GEMM with fp32 bias (reference :152-157).
 //
-// All contractions are v_mfma_f32_32x32x16_bf16 (fp32 accumulate).  Operand fragments use one
-// format throughout: a [32 rows x 16 k] slab, lane l holding row (l & 31), k-chunk (l >> 5)*8..+8,
-// i.e. 16 contiguous bytes of a row-major bf16 matrix.  Results come out as D[i][j] with
-// j = l & 31 and i = 8*(v/4) + 4*(l>>5) + (v&3) for accumulator register v.  Two consequences are
-// used everywhere below:
+// All contractions are v_mfma_f32_32x32x16_bf16 (fp32 accumulate); fragment and accumulator layouts
+// are described in mfma_tiles.h.  Two consequences of those layouts are used everywhere below:
 //   * a contraction index may be permuted freely as long as both operands agree, so an accumulator
-//     (rows i scattered as above) can be fed back as the k-dimension of the next MFMA without any
-//     cross-lane movement: Q^T and K^T share their head-dim order, and the probabilities share
-//     their key order with V;
+//     can be fed back as the k-dimension of the next MFMA without any cross-lane movement: Q^T and
+//     K^T share their head-dim order, and the probabilities share their key order with V;
 //   * the sequence position handled by "row r" of a 32-row block is pi(r) = 16*((r>>2)&1) +
 //     4*(r>>3) + (r&3), chosen so that the 16 logits a lane holds for its query are 16 CONSECUTIVE
 //     keys (pair-bias row loads become two 16-byte loads).
