@@ -457,11 +457,7 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
     auto exp4 = [&](f32x16 &x, int base) {
 #pragma unroll
         for (int v = base; v < base + 4; ++v) {
-#ifdef KUTACC_EXP_NOEXP
-            x[v] = SHIFT ? x[v] - shift : x[v] * 1.0001f;
-#else
             x[v] = __builtin_amdgcn_exp2f(SHIFT ? x[v] - shift : x[v]);
-#endif
         }
     };
     auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
@@ -472,17 +468,11 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
         bf16x8 p0, p1;
         xn = init(t_next);
         if (HAS_NB) {
-#ifndef KUTACC_EXP_NOSEL
             xn = mfma(sel0, as_bf16x8(w0), xn);
-#endif
             exp4(xc, 0);
             fence();
-#ifndef KUTACC_EXP_NOSEL
             xn = mfma(sel1, as_bf16x8(w1), xn);
-#endif
-#ifndef KUTACC_EXP_NOW
             w0 = nbf[t_w * 128], w1 = nbf[t_w * 128 + 64];
-#endif
             exp4(xc, 4);
             p0 = pack8(xc, 0);
             fence();
@@ -497,19 +487,13 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
         exp4(xc, 8);
         fence();
         xn = mfma(as_bf16x8(k1), q1, xn);
-#ifndef KUTACC_EXP_NOSUM
         lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sumsel, p0, lacc, 0, 0, 0);
-#endif
-#ifndef KUTACC_EXP_NOKV
         k0 = kp[(t_k * 2 + 0) * 64], k1 = kp[(t_k * 2 + 1) * 64];
-#endif
         exp4(xc, 12);
         p1 = pack8(xc, 8);
         fence();
         o = mfma(as_bf16x8(v1), p1, o);
-#ifndef KUTACC_EXP_NOSUM
         lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sumsel, p1, lacc, 0, 0, 0);
-#endif
     };
 
     for (int pair = 0; pair < npairs; ++pair) {
@@ -517,15 +501,11 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
         const int tn = pair + 1 < npairs ? 2 * pair + 2 : 2 * pair; // next pair's first tile, clamped
         // ---- odd tile's logits under the even tile's softmax ----
         half_step(xa, xb, t1, wb0, wb1, clampt(t1 + 2), tn);
-#ifndef KUTACC_EXP_NOKV
         v0 = vp[(t1 * 2 + 0) * 64], v1 = vp[(t1 * 2 + 1) * 64];
-#endif
         fence();
         // ---- next pair's even tile under the odd tile's softmax ----
         half_step(xb, xa, tn, wa0, wa1, clampt(tn + 2), tn + 1);
-#ifndef KUTACC_EXP_NOKV
         v0 = vp[(tn * 2 + 0) * 64], v1 = vp[(tn * 2 + 1) * 64];
-#endif
         fence();
     }
     o_out = o;
@@ -1000,17 +980,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                 }
             }
         }
-#ifdef KUTACC_OPT_TOUCH
-        // pull the next batch row's input block towards the L2 (one line per lane) while this row is
-        // projected; the value is only there to be waited for
-        uint32_t touch = 0;
-        if (n + 1 < nrows) {
-            const bf16_t *xn_ = p.x + (int64_t)(b + bstep) * S * p.x_ld;
-            int trow = j * 32 + (lane >> 1);
-            trow = trow < S ? trow : S - 1;
-            touch = *reinterpret_cast<const uint32_t *>(xn_ + (int64_t)trow * p.x_ld + (lane & 1) * 64);
-        }
-#endif
         if (n == 2) {
             TL(1);
         }
@@ -1064,9 +1033,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == 2) {
             TL(2);
         }
-#ifdef KUTACC_OPT_TOUCH
-        asm volatile("" ::"v"(touch));
-#endif
         __syncthreads(); // every wave is done with the previous row's attention: the K and V arrays are free
         lds_k[(j * 2 + 0) * 64 + lane] = kfrag0;
         lds_k[(j * 2 + 1) * 64 + lane] = kfrag1;
