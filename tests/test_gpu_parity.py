@@ -9,6 +9,7 @@ include masked rows where the configuration has them.
 Tolerances (stated by the task): fp32 storage within 1e-4 relative of the fp32 oracle; bf16 storage
 within 2e-2 absolute + 1e-2 relative of the fp32 oracle.
 """
+import ctypes
 import functools
 
 import numpy as np
@@ -225,6 +226,35 @@ def test_absent_pair_bias_equals_zero_pair_bias(torch_cuda, batch):
     else:
         a, b2 = helpers.to_numpy(ten["out"]), helpers.to_numpy(ten2["out"])
         helpers.assert_within(b2, a, 2.0 ** -7 * np.abs(a) + 3e-3, "zero pair bias vs none")
+
+
+@pytest.mark.parametrize("nb_pad", [16, 3], ids=["pair-bias rows 16B-aligned", "pair-bias rows unaligned"])
+@pytest.mark.parametrize("path", [capi.PATH_GENERIC, capi.PATH_FUSED])
+def test_strided_tensors_through_the_launch_layer(torch_cuda, path, nb_pad):
+    """Padded leading dimensions: input and out rows wider than C, a padded pair bias and mask bias.  Both kernel
+    families must read and write only what the strides describe."""
+    torch = torch_cuda
+    w = make_workload(3, batch=6, seq_len=96)
+    B, S, C, H = w.B, w.S, w.C, w.H
+    ten, scratch = helpers.to_device(w)
+    pad = 16
+    x_p = torch.full((B * S, C + pad), 7.0, dtype=torch.bfloat16, device="cuda")
+    x_p[:, :C] = ten["x"].reshape(B * S, C)
+    out_p = torch.full((B * S, C + pad), -3.0, dtype=torch.bfloat16, device="cuda")
+    nb_p = torch.full((H, S + 8, S + nb_pad), 5.0, dtype=torch.bfloat16, device="cuda")
+    nb_p[:, :S, :S] = ten["nb"]
+    bias_p = torch.full((B, S + pad), -1e9, dtype=torch.bfloat16, device="cuda")
+    bias_p[:, :S] = ten["bias"]
+    a = helpers.hip_args(w, ten, scratch, path)
+    a.input, a.input_ld = x_p.data_ptr(), C + pad
+    a.out, a.out_ld = out_p.data_ptr(), C + pad
+    a.nonbatched_bias, a.nb_stride_h, a.nb_stride_q = nb_p.data_ptr(), (S + 8) * (S + nb_pad), S + nb_pad
+    a.bias, a.bias_stride_b = bias_p.data_ptr(), S + pad
+    rc = capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None)
+    torch.cuda.synchronize()
+    assert rc == 0
+    helpers.check_close(helpers.to_numpy(out_p[:, :C]).reshape(B, S, C), helpers.oracle_out(w), w.dtype, "strided out")
+    assert bool((out_p[:, C:] == -3.0).all()), "columns beyond C of the padded out rows were written"
 
 
 # ---- boundary behaviour ------------------------------------------------------------------------------------
