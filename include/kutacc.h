@@ -129,6 +129,114 @@ kutacc_export void kutacc_af2_global_attention(kutacc_af2_attention_inputs_t *q_
                                                kutacc_tensor_h q_mask, kutacc_af2_attention_weights_t *weight_ptr,
                                                kutacc_tensor_h out);
 
+/* ---- transition and triangle multiplication: the pair/MSA-stack operators around the attention ---- */
+
+/* Weights of the transition (reference include/kutacc.h:194-202).  c_o = channels of the activation,
+ * c_i = channels of the hidden layer; linear1_w [c_i, c_o] and linear2_w [c_o, c_i] stored [out, in],
+ * linear1_b fp32 [c_i], linear2_b fp32 [c_o]. */
+typedef struct kutacc_af2_trans_weights {
+    int64_t c_o;
+    int64_t c_i;
+
+    kutacc_tensor_h linear1_w;
+    kutacc_tensor_h linear1_b;
+    kutacc_tensor_h linear2_w;
+    kutacc_tensor_h linear2_b;
+} kutacc_af2_trans_weights_t;
+
+/* Activations of the transition (reference include/kutacc.h:208-214): input_act dense [batch*n_res, c_o]
+ * (already layer-normalised), intermediate_act dense [batch*n_res, c_i] caller-owned scratch that receives
+ * relu(input_act . linear1_w^T + linear1_b). */
+typedef struct kutacc_af2_trans_act_inputs {
+    int64_t batch;
+    int64_t n_res;
+
+    kutacc_tensor_h input_act;
+    kutacc_tensor_h intermediate_act;
+} kutacc_af2_trans_act_inputs_t;
+
+/*
+ * out = relu(input_act . linear1_w^T + linear1_b) . linear2_w^T + linear2_b, out dense [batch*n_res, c_o]
+ * (reference include/kutacc.h:321-322, src/attention/transition.cpp:21-67).  Device pointers only.
+ */
+kutacc_export void kutacc_af2_transition(kutacc_af2_trans_act_inputs_t *trans_inputs_ptr,
+                                         kutacc_af2_trans_weights_t *trans_weights_ptr, kutacc_tensor_h out);
+
+/* Weights of one triangle projection, left or right (reference include/kutacc.h:154-162): proj_w and gate_w
+ * [c_i, c_o] stored [out, in] (c_o = channels of the pair activation, c_i = projected channels), proj_b and
+ * gate_b fp32 [c_i]. */
+typedef struct kutacc_af2_tm_proj_weights {
+    int64_t c_o;
+    int64_t c_i;
+
+    kutacc_tensor_h proj_w;
+    kutacc_tensor_h proj_b;
+    kutacc_tensor_h gate_w;
+    kutacc_tensor_h gate_b;
+} kutacc_af2_tm_proj_weights_t;
+
+/* Activations of the triangle multiplication (reference include/kutacc.h:168-175): input_act dense
+ * [n_res, n_res_gather, c_o] (layer-normalised pair activation), proj_act [c_i, n_res, n_res_gather] channel-first
+ * output of the projection step, proj_act_gate a scratch tensor of the same shape. */
+typedef struct kutacc_af2_tm_act_inputs {
+    int64_t n_res;
+    int64_t n_res_gather;
+
+    kutacc_tensor_h proj_act;
+    kutacc_tensor_h input_act;
+    kutacc_tensor_h proj_act_gate;
+} kutacc_af2_tm_act_inputs_t;
+
+/* Weights of the output step (reference include/kutacc.h:181-189): gating_w [c_o, c_o], output_proj_w [c_o, c_i],
+ * both stored [out, in]; gating_b, output_proj_b fp32 [c_o]. */
+typedef struct kutacc_af2_tm_linear_weights {
+    int64_t c_o;
+    int64_t c_i;
+
+    kutacc_tensor_h gating_w;
+    kutacc_tensor_h gating_b;
+    kutacc_tensor_h output_proj_w;
+    kutacc_tensor_h output_proj_b;
+} kutacc_af2_tm_linear_weights_t;
+
+/*
+ * proj_act[c, i, j] = (input_act[i, j, :] . proj_w[c, :] + proj_b[c]) * mask[i, j] * sigmoid(input_act[i, j, :] . gate_w[c, :] + gate_b[c])
+ * (reference include/kutacc.h:426-429, src/attention/triangle_multiplication.cpp:25-67, 152-178).
+ * mask bf16 [n_res, n_res_gather].  This backend forms both products in one kernel and leaves proj_act_gate
+ * untouched; `input_prepack` (a layout hint of the CPU GEMM) is ignored.  Device pointers only.
+ */
+kutacc_export void kutacc_af2_triangle_multiplication_calc_proj(kutacc_af2_tm_act_inputs_t *tm_acts_ptr,
+                                                                kutacc_tensor_h mask,
+                                                                kutacc_af2_tm_proj_weights_t *tm_weights_ptr,
+                                                                bool input_prepack);
+
+/*
+ * Per channel c of [c_i, n_res_gather, n_res_gather] tensors (reference include/kutacc.h:436-439,
+ * src/attention/triangle_multiplication.cpp:72-101, 180-195):
+ *   outgoing (is_incoming == false): center[c, i, j] = sum_k left[c, i, k] * right[c, j, k]
+ *   incoming (is_incoming == true) : center[c, i, j] = sum_k right[c, k, i] * left[c, k, j]
+ */
+kutacc_export void kutacc_af2_triangle_multiplication_equation(kutacc_tensor_h center_act,
+                                                               kutacc_tensor_h left_proj_act,
+                                                               kutacc_tensor_h right_proj_act, int64_t n_res_gather,
+                                                               bool is_incoming);
+
+/*
+ * gate = input_act . gating_w^T + gating_b and out = center_act . output_proj_w^T + output_proj_b, rows (i, j) of
+ * [n_res, n_res_gather, .] tensors; center_act is the channel-last, layer-normalised result of the equation
+ * (reference include/kutacc.h:446-448, src/attention/triangle_multiplication.cpp:106-127, 197-224).
+ */
+kutacc_export void kutacc_af2_triangle_multiplication_gate_and_out_linear(
+    kutacc_tensor_h gate, kutacc_tensor_h out, kutacc_af2_tm_act_inputs_t *tm_acts_ptr, kutacc_tensor_h center_act,
+    kutacc_af2_tm_linear_weights_t *tm_weights_ptr, bool input_prepack);
+
+/*
+ * out[i, j, :c_o] *= sigmoid(gate[i, j, :c_o]) (reference include/kutacc.h:455-456,
+ * src/attention/triangle_multiplication.cpp:129-150, 226-240).
+ */
+kutacc_export void kutacc_af2_triangle_multiplication_last(kutacc_tensor_h out, kutacc_tensor_h gate, int64_t n_res,
+                                                           int64_t n_res_gather, int64_t c_o);
+
 /*
  * LayerNorm of ONE row of `size` elements, bf16 in/out, fp32 gamma/beta
  * (reference include/kutacc.h:334, src/normalization/layernorm_kernel.h:21-53).

@@ -159,6 +159,46 @@ kutacc_export int kutacc_hip_pair_bias(const void *z, const float *gamma, const 
                                        void *nb, void *z_norm, int64_t rows_i, int64_t rows_j, int64_t c_z,
                                        int64_t nheads, float eps, int32_t dtype, void *stream);
 
+/*
+ * Strided bf16 matrix product with a fused epilogue: what kutacc::addmm (reference src/linear/mm.cpp:46-86) plus
+ * the BlasExtendParams epilogue flags (reference include/kutacc.h:474-482) hand to the GEMM backend, and the
+ * engine behind the transition and triangle-multiplication entry points below.
+ *   C(m, n) = epilogue( sum_k A(m, k) * B(n, k) ),  fp32 accumulation, result rounded to bf16
+ * A(m, k) sits at a + batch*a_stride_batch + m*a_stride_m + k*a_stride_k (one of the two strides must be 1 for
+ * the MFMA kernel; anything else runs on a scalar kernel), B(n, k) likewise, C(m, n) at
+ * c + batch*c_stride_batch + m*c_stride_m + n.  Epilogue: + bias (bias_axis 1: bias[n], the reference's
+ * row_bias; 2: bias[m], its col_bias; 0: none), then ReLU if `relu`.  Gated form (a_gate != NULL, used by the
+ * triangle projections, reference src/attention/triangle_multiplication.cpp:25-67): a second product
+ * G = A_gate * B^T (A_gate laid out like A, bias_gate like bias) and
+ *   C = bf16( bf16(A*B^T + bias) * mask[n] * sigmoid(bf16(G + bias_gate)) ),  mask bf16 at mask + batch*mask_stride_batch + n.
+ */
+typedef struct kutacc_hip_gemm_args {
+    int64_t m, n, k, batches;
+    int32_t dtype; /* KUTACC_DTYPE_BF16 */
+    int32_t path;  /* KUTACC_HIP_PATH_*: AUTO, GENERIC (scalar kernel), FUSED (MFMA kernel or EUNSUPPORTED) */
+    const void *a;
+    int64_t a_stride_m, a_stride_k, a_stride_batch;
+    const void *b;
+    int64_t b_stride_n, b_stride_k, b_stride_batch;
+    void *c;
+    int64_t c_stride_m, c_stride_batch;
+    const float *bias; /* fp32, NULL with bias_axis 0 */
+    int32_t bias_axis;
+    int32_t relu;
+    const void *a_gate; /* NULL = plain epilogue */
+    const float *bias_gate;
+    const void *mask;
+    int64_t mask_stride_batch;
+} kutacc_hip_gemm_args_t;
+
+kutacc_export int kutacc_hip_gemm(const kutacc_hip_gemm_args_t *args, void *stream);
+
+/* out[i, j, c] *= sigmoid(gate[i, j, c]) for c < size; element (i, j, c) of either tensor at i*stride0 + j*stride1 + c.
+ * The element-wise pass of kutacc::last (reference src/attention/triangle_multiplication.cpp:129-150). */
+kutacc_export int kutacc_hip_sigmoid_gate_rows(void *out, int64_t out_stride0, int64_t out_stride1, const void *gate,
+                                               int64_t gate_stride0, int64_t gate_stride1, int64_t n0, int64_t n1,
+                                               int64_t size, int32_t dtype, void *stream);
+
 /* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.

@@ -76,10 +76,50 @@ class HipGlobalAttentionArgs(ctypes.Structure):
     ]
 
 
+class HipGemmArgs(ctypes.Structure):
+    """kutacc_hip_gemm_args_t"""
+    _fields_ = [
+        ("m", _i64), ("n", _i64), ("k", _i64), ("batches", _i64), ("dtype", _i32), ("path", _i32),
+        ("a", _vp), ("a_stride_m", _i64), ("a_stride_k", _i64), ("a_stride_batch", _i64),
+        ("b", _vp), ("b_stride_n", _i64), ("b_stride_k", _i64), ("b_stride_batch", _i64),
+        ("c", _vp), ("c_stride_m", _i64), ("c_stride_batch", _i64),
+        ("bias", _vp), ("bias_axis", _i32), ("relu", _i32),
+        ("a_gate", _vp), ("bias_gate", _vp), ("mask", _vp), ("mask_stride_batch", _i64),
+    ]
+
+
+class TransWeights(ctypes.Structure):
+    """kutacc_af2_trans_weights_t"""
+    _fields_ = [("c_o", _i64), ("c_i", _i64), ("linear1_w", _vp), ("linear1_b", _vp), ("linear2_w", _vp), ("linear2_b", _vp)]
+
+
+class TransActInputs(ctypes.Structure):
+    """kutacc_af2_trans_act_inputs_t"""
+    _fields_ = [("batch", _i64), ("n_res", _i64), ("input_act", _vp), ("intermediate_act", _vp)]
+
+
+class TmProjWeights(ctypes.Structure):
+    """kutacc_af2_tm_proj_weights_t"""
+    _fields_ = [("c_o", _i64), ("c_i", _i64), ("proj_w", _vp), ("proj_b", _vp), ("gate_w", _vp), ("gate_b", _vp)]
+
+
+class TmActInputs(ctypes.Structure):
+    """kutacc_af2_tm_act_inputs_t"""
+    _fields_ = [("n_res", _i64), ("n_res_gather", _i64), ("proj_act", _vp), ("input_act", _vp), ("proj_act_gate", _vp)]
+
+
+class TmLinearWeights(ctypes.Structure):
+    """kutacc_af2_tm_linear_weights_t"""
+    _fields_ = [("c_o", _i64), ("c_i", _i64), ("gating_w", _vp), ("gating_b", _vp), ("output_proj_w", _vp),
+                ("output_proj_b", _vp)]
+
+
 # every symbol the two public headers declare; tests check that the library exports all of them
 DECLARED_SYMBOLS = [
     "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_global_attention", "kutacc_af2_layernorm",
-    "kutacc_af2_linear",
+    "kutacc_af2_linear", "kutacc_af2_transition", "kutacc_af2_triangle_multiplication_calc_proj",
+    "kutacc_af2_triangle_multiplication_equation", "kutacc_af2_triangle_multiplication_gate_and_out_linear",
+    "kutacc_af2_triangle_multiplication_last", "kutacc_hip_gemm", "kutacc_hip_sigmoid_gate_rows",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
@@ -129,6 +169,22 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_linear.restype = ctypes.c_int
     L.kutacc_hip_pair_bias.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _i32, _vp]
     L.kutacc_hip_pair_bias.restype = ctypes.c_int
+    L.kutacc_hip_gemm.argtypes = [ctypes.POINTER(HipGemmArgs), _vp]
+    L.kutacc_hip_gemm.restype = ctypes.c_int
+    L.kutacc_hip_sigmoid_gate_rows.argtypes = [_vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp]
+    L.kutacc_hip_sigmoid_gate_rows.restype = ctypes.c_int
+    L.kutacc_af2_transition.argtypes = [ctypes.POINTER(TransActInputs), ctypes.POINTER(TransWeights), _vp]
+    L.kutacc_af2_transition.restype = None
+    L.kutacc_af2_triangle_multiplication_calc_proj.argtypes = [ctypes.POINTER(TmActInputs), _vp,
+                                                               ctypes.POINTER(TmProjWeights), ctypes.c_bool]
+    L.kutacc_af2_triangle_multiplication_calc_proj.restype = None
+    L.kutacc_af2_triangle_multiplication_equation.argtypes = [_vp, _vp, _vp, _i64, ctypes.c_bool]
+    L.kutacc_af2_triangle_multiplication_equation.restype = None
+    L.kutacc_af2_triangle_multiplication_gate_and_out_linear.argtypes = [_vp, _vp, ctypes.POINTER(TmActInputs), _vp,
+                                                                         ctypes.POINTER(TmLinearWeights), ctypes.c_bool]
+    L.kutacc_af2_triangle_multiplication_gate_and_out_linear.restype = None
+    L.kutacc_af2_triangle_multiplication_last.argtypes = [_vp, _vp, _i64, _i64, _i64]
+    L.kutacc_af2_triangle_multiplication_last.restype = None
     L.kutacc_hip_set_stream.argtypes = [_vp]
     L.kutacc_hip_get_stream.restype = _vp
     L.kutacc_hip_set_blocking.argtypes = [ctypes.c_int]
@@ -281,3 +337,54 @@ class GlobalAttention:
 
     def run(self) -> None:
         kutacc_af2_global_attention(self.inputs, self.h["x"], self.h["mask"], self.weights, self.h["out"])
+
+
+# ---- transition and triangle multiplication (reference include/kutacc.h:321-322, 426-456) --------------------
+def _h(t):
+    return _vp(t.handle) if t is not None else None
+
+
+def _ref(s):
+    return ctypes.byref(s) if s is not None else None
+
+
+def kutacc_af2_transition(trans_inputs: TransActInputs, trans_weights: TransWeights, out) -> None:
+    lib().kutacc_af2_transition(_ref(trans_inputs), _ref(trans_weights), _h(out))
+
+
+def kutacc_af2_triangle_multiplication_calc_proj(tm_acts: TmActInputs, mask, tm_weights: TmProjWeights,
+                                                 input_prepack: bool = False) -> None:
+    lib().kutacc_af2_triangle_multiplication_calc_proj(_ref(tm_acts), _h(mask), _ref(tm_weights), input_prepack)
+
+
+def kutacc_af2_triangle_multiplication_equation(center_act, left_proj_act, right_proj_act, n_res_gather: int,
+                                                is_incoming: bool) -> None:
+    lib().kutacc_af2_triangle_multiplication_equation(_h(center_act), _h(left_proj_act), _h(right_proj_act), n_res_gather,
+                                                      is_incoming)
+
+
+def kutacc_af2_triangle_multiplication_gate_and_out_linear(gate, out, tm_acts: TmActInputs, center_act,
+                                                           tm_weights: TmLinearWeights, input_prepack: bool = False) -> None:
+    lib().kutacc_af2_triangle_multiplication_gate_and_out_linear(_h(gate), _h(out), _ref(tm_acts), _h(center_act),
+                                                                 _ref(tm_weights), input_prepack)
+
+
+def kutacc_af2_triangle_multiplication_last(out, gate, n_res: int, n_res_gather: int, c_o: int) -> None:
+    lib().kutacc_af2_triangle_multiplication_last(_h(out), _h(gate), n_res, n_res_gather, c_o)
+
+
+class Transition:
+    """Owner of the handles of one kutacc_af2_transition call.  x [batch, n_res, c_o]; w1 [c_i, c_o], w2 [c_o, c_i]
+    stored [out, in]; b1 fp32 [c_i], b2 fp32 [c_o]; mid [batch*n_res, c_i] scratch; out like x."""
+
+    def __init__(self, x, w1, b1, w2, b2, mid, out):
+        batch, n_res, c_o = x.shape
+        self.keep = (x, w1, b1, w2, b2, mid, out)
+        self.h = dict(x=tensor(x), w1=tensor(w1), b1=tensor(b1, K_FP32), w2=tensor(w2), b2=tensor(b2, K_FP32),
+                      mid=tensor(mid), out=tensor(out))
+        self.inputs = TransActInputs(batch, n_res, self.h["x"].handle, self.h["mid"].handle)
+        self.weights = TransWeights(c_o, w1.shape[0], self.h["w1"].handle, self.h["b1"].handle, self.h["w2"].handle,
+                                    self.h["b2"].handle)
+
+    def run(self) -> None:
+        kutacc_af2_transition(self.inputs, self.weights, self.h["out"])

@@ -15,6 +15,7 @@
 #include "check.h"
 #include "kutacc.h"
 #include "kutacc_hip.h"
+#include "api_internal.h"
 #include "launch_internal.h"
 #include "tensor_view.h"
 
@@ -263,6 +264,13 @@ int finish_device_call(int rc, hipStream_t s)
     return rc;
 }
 } // namespace
+
+namespace kutacc_api {
+hipStream_t default_stream() { return g_stream; }
+hipStream_t stream_or_default(void *s) { return pick_stream(s); }
+bool on_device(const void *p) { return space_of(p) == Space::Device; }
+int finish(int rc, hipStream_t s) { return finish_device_call(rc, s); }
+} // namespace kutacc_api
 
 void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inputs_t *q_based_ptr, kutacc_tensor_h bias,
                                  kutacc_tensor_h nonbatched_bias, kutacc_af2_attention_weights_t *weight_ptr,

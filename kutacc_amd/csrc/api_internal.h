@@ -1,0 +1,11 @@
+// Host-side state shared by the translation units that implement the handle-based entry points:
+// the library's default stream, the blocking switch and the host/device classification of a pointer.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace kutacc_api {
+hipStream_t default_stream();
+hipStream_t stream_or_default(void *stream); // an explicit stream argument, else the default stream
+bool on_device(const void *ptr);             // device or managed memory (plain and pinned host memory: false)
+int finish(int rc, hipStream_t stream);      // synchronise if the library is in blocking mode; passes rc through
+} // namespace kutacc_api

@@ -23,6 +23,11 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t 
 // global_attention.hip
 int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);
 
+// pair_stack.hip
+int pair_gemm(const kutacc_hip_gemm_args_t &args, hipStream_t stream);
+int sigmoid_gate_rows(void *out, int64_t out_s0, int64_t out_s1, const void *gate, int64_t gate_s0, int64_t gate_s1,
+                      int64_t n0, int64_t n1, int64_t size, hipStream_t stream);
+
 // row_kernels.hip
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                    int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream);

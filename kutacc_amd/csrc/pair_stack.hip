@@ -1,0 +1,484 @@
+// bf16 matrix products with fused epilogues for the operators next to the attention on the pair and
+// MSA stacks: transition (reference src/attention/transition.cpp:21-39) and the four steps of the
+// triangle multiplication (reference src/attention/triangle_multiplication.cpp:25-150).  All of them are
+// C = epilogue(A * B^T) on strided bf16 views with fp32 accumulation, which is what the reference hands
+// to its GEMM backend through addmm (src/linear/mm.cpp:46-86).
+//
+// One kernel covers them.  A workgroup of four waves owns a 128 x 128 tile of C and walks K in steps of
+// 64: each wave fetches a quarter of both operand tiles with whole-cache-line loads one step ahead,
+// parks it in registers while the current step is multiplied, and stores it into the other half of a
+// double-buffered LDS tile in MFMA fragment order (one barrier per step).  Operands may be stored
+// K-major (rows contiguous in k; 16-byte LDS writes) or M-major (the "incoming" triangle equation
+// contracts over the leading index of both operands; the transposition happens in the LDS write, two
+// bytes at a time).  The product is formed transposed (MFMA rows = columns of C) so that every lane
+// ends up with four consecutive columns of its own row of C; the tile is rounded to bf16 into LDS and
+// leaves as whole rows of 256 bytes.
+//
+// Epilogues: bias per column or per row of C, ReLU, and the gated form of the triangle projections,
+// where one launch multiplies the same B tile with 64 rows of the projection weights and the matching
+// 64 rows of the gate weights and writes bf16(bf16(proj) * mask * sigmoid(bf16(gate))) -- the rounding
+// points of the reference, which rounds both GEMM results to bf16 before its element-wise pass
+// (triangle_multiplication.cpp:37-66).
+//
+// Shapes the MFMA kernel does not take (k, n or a leading dimension not a multiple of 8, pointers not
+// 16-byte aligned) run on a scalar kernel with the same epilogues.
+#include <hip/hip_runtime.h>
+
+#include "launch_internal.h"
+#include "mfma_tiles.h"
+#include "profiler.h"
+
+namespace {
+using namespace kutacc_dev;
+
+struct GemmParams {
+    const bf16_t *a, *a_gate, *b;
+    bf16_t *c;
+    int64_t a_sm, a_sk, a_sb; // A(m, k) at a + m*a_sm + k*a_sk + batch*a_sb
+    int64_t b_sn, b_sk, b_sb; // B(n, k)
+    int64_t c_sm, c_sb;       // C(m, n) at c + m*c_sm + n + batch*c_sb
+    const float *bias, *bias_gate;
+    const bf16_t *mask; // gated epilogue: multiplier per column of C
+    int64_t mask_sb;
+    int M, N, K, batches;
+    int bias_axis; // 0 none, 1 per column n, 2 per row m
+    int relu;
+    int MT, NT; // tiles along m and n
+};
+
+constexpr int TILE = 128, KSTEP = 64;
+constexpr int OPERAND_SLOTS = 4 * 256;          // four 32-row panels of 256 16-byte slots
+constexpr int STAGE_SLOTS = 2 * OPERAND_SLOTS;  // A and B
+constexpr int CT_LD = 136;                      // bf16 elements per row of the C tile in LDS (272 bytes)
+constexpr size_t GEMM_LDS = 2 * STAGE_SLOTS * 16;
+
+// K-major operand: rows row0..row0+31 (clamped), 64 k from k0; chunks past K read as zero
+__device__ __forceinline__ PanelRegs load_kmajor(const bf16_t *base, int64_t ld, int row0, int last_row, int k0, int K, int lane)
+{
+    const int col = k0 + (lane & 7) * 8;
+    const bool ok = col < K;
+    const int colc = ok ? col : 0;
+    PanelRegs p;
+    uint4 *dst[4] = {&p.r0, &p.r1, &p.r2, &p.r3};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int row = row0 + 8 * i + (lane >> 3);
+        row = row < last_row ? row : last_row;
+        uint4 v = *reinterpret_cast<const uint4 *>(base + (int64_t)row * ld + colc);
+        if (!ok) {
+            v = make_uint4(0u, 0u, 0u, 0u);
+        }
+        *dst[i] = v;
+    }
+    return p;
+}
+
+// M-major operand (element (m, k) at base + k*ld + m): 64 rows m from m0, 32 k from k0.  Lane (kk, mc)
+// takes 8 consecutive m of row k0 + kk + 8i; a load instruction covers 8 k x 128 contiguous bytes.
+__device__ __forceinline__ PanelRegs load_mmajor(const bf16_t *base, int64_t ld, int m0, int rows, int k0, int K, int lane)
+{
+    int m = m0 + (lane & 7) * 8;
+    m = m + 8 <= rows ? m : rows - 8; // rows past the end are never stored; any valid address will do
+    PanelRegs p;
+    uint4 *dst[4] = {&p.r0, &p.r1, &p.r2, &p.r3};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int k = k0 + 8 * i + (lane >> 3);
+        const bool ok = k < K;
+        uint4 v = *reinterpret_cast<const uint4 *>(base + (int64_t)(ok ? k : 0) * ld + m);
+        if (!ok) {
+            v = make_uint4(0u, 0u, 0u, 0u);
+        }
+        *dst[i] = v;
+    }
+    return p;
+}
+
+// transposing store of what load_mmajor fetched: operand tile rows mrow0.., k columns kcol0..
+__device__ __forceinline__ void store_mmajor(uint4 *operand, int mrow0, int kcol0, int lane, const PanelRegs &p)
+{
+    uint16_t *o16 = reinterpret_cast<uint16_t *>(operand);
+    const uint4 regs[4] = {p.r0, p.r1, p.r2, p.r3};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int k = kcol0 + 8 * i + (lane >> 3);
+        const uint32_t w[4] = {regs[i].x, regs[i].y, regs[i].z, regs[i].w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int row = mrow0 + (lane & 7) * 8 + e;
+            const int slot = (row >> 5) * 256 + panel_slot(row & 31, k >> 3);
+            o16[slot * 8 + (k & 7)] = (uint16_t)(e & 1 ? w[e >> 1] >> 16 : w[e >> 1] & 0xffffu);
+        }
+    }
+}
+
+template <bool A_MMAJOR, bool B_MMAJOR, bool GATED>
+__global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
+{
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // Workgroup ids are dealt round robin over the 8 XCDs; give each XCD a contiguous run of tiles so
+    // that neighbours in the walk (which share an operand tile) share an L2.
+    int64_t bid = blockIdx.x;
+    {
+        const int64_t total = gridDim.x, per = total / 8;
+        if (bid < per * 8) {
+            bid = (bid % 8) * per + bid / 8;
+        }
+    }
+    const int64_t tiles = (int64_t)p.MT * p.NT;
+    const int batch = (int)(bid / tiles);
+    const int t = (int)(bid % tiles);
+    // the dimension with fewer tiles runs fastest: consecutive workgroups then share the tile of the larger operand
+    int mt, nt;
+    if (p.MT <= p.NT) {
+        mt = t % p.MT, nt = t / p.MT;
+    } else {
+        nt = t % p.NT, mt = t / p.NT;
+    }
+    constexpr int MROWS = GATED ? 64 : 128; // rows of C per tile
+    const int m0 = mt * MROWS, n0 = nt * TILE;
+
+    const bf16_t *a = p.a + (int64_t)batch * p.a_sb;
+    const bf16_t *a_gate = GATED ? p.a_gate + (int64_t)batch * p.a_sb : nullptr;
+    const bf16_t *b = p.b + (int64_t)batch * p.b_sb;
+
+    auto fetch_a = [&](int k0) -> PanelRegs {
+        if constexpr (A_MMAJOR) {
+            return load_mmajor(a, p.a_sk, m0 + 64 * (wave & 1), p.M, k0 + 32 * (wave >> 1), p.K, lane);
+        } else if constexpr (GATED) {
+            return load_kmajor(wave < 2 ? a : a_gate, p.a_sm, m0 + 32 * (wave & 1), p.M - 1, k0, p.K, lane);
+        } else {
+            return load_kmajor(a, p.a_sm, m0 + 32 * wave, p.M - 1, k0, p.K, lane);
+        }
+    };
+    auto fetch_b = [&](int k0) -> PanelRegs {
+        if constexpr (B_MMAJOR) {
+            return load_mmajor(b, p.b_sk, n0 + 64 * (wave & 1), p.N, k0 + 32 * (wave >> 1), p.K, lane);
+        } else {
+            return load_kmajor(b, p.b_sn, n0 + 32 * wave, p.N - 1, k0, p.K, lane);
+        }
+    };
+    auto park = [&](uint4 *stage, const PanelRegs &ra, const PanelRegs &rb) {
+        if constexpr (A_MMAJOR) {
+            store_mmajor(stage, 64 * (wave & 1), 32 * (wave >> 1), lane, ra);
+        } else {
+            panel_store(stage + wave * 256, lane, ra);
+        }
+        if constexpr (B_MMAJOR) {
+            store_mmajor(stage + OPERAND_SLOTS, 64 * (wave & 1), 32 * (wave >> 1), lane, rb);
+        } else {
+            panel_store(stage + OPERAND_SLOTS + wave * 256, lane, rb);
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            acc[i][j] = zero16();
+        }
+    }
+
+    const int KT = (p.K + KSTEP - 1) / KSTEP;
+    PanelRegs ra = fetch_a(0), rb = fetch_b(0);
+    for (int kt = 0; kt < KT; ++kt) {
+        uint4 *stage = lds + (kt & 1) * STAGE_SLOTS;
+        park(stage, ra, rb);
+        __syncthreads();
+        if (kt + 1 < KT) {
+            ra = fetch_a((kt + 1) * KSTEP);
+            rb = fetch_b((kt + 1) * KSTEP);
+        }
+        const uint4 *oa = stage + (2 * wm) * 256;
+        const uint4 *ob = stage + OPERAND_SLOTS + (2 * wn) * 256;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int slot = panel_slot(r, 2 * s + g);
+            const bf16x8 a0 = as_bf16x8(oa[slot]), a1 = as_bf16x8(oa[256 + slot]);
+            const bf16x8 b0 = as_bf16x8(ob[slot]), b1 = as_bf16x8(ob[256 + slot]);
+            acc[0][0] = mfma(b0, a0, acc[0][0]);
+            acc[0][1] = mfma(b1, a0, acc[0][1]);
+            acc[1][0] = mfma(b0, a1, acc[1][0]);
+            acc[1][1] = mfma(b1, a1, acc[1][1]);
+        }
+    }
+    __syncthreads(); // every wave is done with the operand tiles; the C tile takes their place
+
+    // accumulators (+ bias, ReLU) -> bf16 C tile in LDS: lane = row of C, four consecutive columns per group
+    bf16_t *ct = reinterpret_cast<bf16_t *>(lds);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int trow = 64 * wm + 32 * i + r; // row of the LDS tile
+        float row_bias = 0.f;
+        if (p.bias_axis == 2) {
+            const int gm = GATED ? m0 + 32 * i + r : m0 + trow;
+            const float *bsrc = (GATED && wm == 1) ? p.bias_gate : p.bias;
+            row_bias = gm < p.M ? bsrc[gm] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int tcol = 64 * wn + 32 * j + 8 * q + 4 * g;
+                f32x4 bv = {row_bias, row_bias, row_bias, row_bias};
+                if (p.bias_axis == 1 && n0 + tcol + 4 <= p.N) {
+                    bv = *reinterpret_cast<const f32x4 *>(p.bias + n0 + tcol);
+                }
+                bf16x4 ov;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float x = acc[i][j][4 * q + c] + bv[c];
+                    if (p.relu) {
+                        x = fmaxf(x, 0.f);
+                    }
+                    ov[c] = (bf16_t)x;
+                }
+                *reinterpret_cast<bf16x4 *>(ct + trow * CT_LD + tcol) = ov;
+            }
+        }
+    }
+    __syncthreads();
+
+    bf16_t *c = p.c + (int64_t)batch * p.c_sb;
+    if constexpr (GATED) {
+        const bf16_t *mask = p.mask + (int64_t)batch * p.mask_sb;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int piece = tid + 256 * i;
+            const int row = piece >> 4, chunk = piece & 15;
+            const int gm = m0 + row, gn = n0 + chunk * 8;
+            if (gm < p.M && gn < p.N) {
+                const bf16x8 pv = *reinterpret_cast<const bf16x8 *>(ct + row * CT_LD + chunk * 8);
+                const bf16x8 gv = *reinterpret_cast<const bf16x8 *>(ct + (64 + row) * CT_LD + chunk * 8);
+                const bf16x8 mv = *reinterpret_cast<const bf16x8 *>(mask + gn);
+                bf16x8 ov;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    ov[e] = (bf16_t)(to_f32(pv[e]) * to_f32(mv[e]) * sigmoid_fast(to_f32(gv[e])));
+                }
+                *reinterpret_cast<bf16x8 *>(c + (int64_t)gm * p.c_sm + gn) = ov;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int piece = tid + 256 * i;
+            const int row = piece >> 4, chunk = piece & 15;
+            const int gm = m0 + row, gn = n0 + chunk * 8;
+            if (gm < p.M && gn < p.N) {
+                *reinterpret_cast<uint4 *>(c + (int64_t)gm * p.c_sm + gn) =
+                    *reinterpret_cast<const uint4 *>(ct + row * CT_LD + chunk * 8);
+            }
+        }
+    }
+}
+
+// Any strides, any sizes: one thread per element of C, same epilogues and rounding points.
+__global__ __launch_bounds__(256) void pair_gemm_scalar_kernel(const GemmParams p)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t per = (int64_t)p.M * p.N;
+    if (idx >= per * p.batches) {
+        return;
+    }
+    const int batch = (int)(idx / per);
+    const int m = (int)((idx % per) / p.N), n = (int)(idx % p.N);
+    const bf16_t *a = p.a + (int64_t)batch * p.a_sb + (int64_t)m * p.a_sm;
+    const bf16_t *b = p.b + (int64_t)batch * p.b_sb + (int64_t)n * p.b_sn;
+    float s = 0.f, sg = 0.f;
+    for (int k = 0; k < p.K; ++k) {
+        const float bv = to_f32(b[(int64_t)k * p.b_sk]);
+        s = fmaf(to_f32(a[(int64_t)k * p.a_sk]), bv, s);
+        if (p.a_gate) {
+            sg = fmaf(to_f32(p.a_gate[(int64_t)batch * p.a_sb + (int64_t)m * p.a_sm + (int64_t)k * p.a_sk]), bv, sg);
+        }
+    }
+    const int bi = p.bias_axis == 1 ? n : m;
+    if (p.bias_axis != 0) {
+        s += p.bias[bi];
+    }
+    if (p.relu) {
+        s = fmaxf(s, 0.f);
+    }
+    float out = s;
+    if (p.a_gate) {
+        if (p.bias_axis != 0) {
+            sg += p.bias_gate[bi];
+        }
+        const float mv = to_f32(p.mask[(int64_t)batch * p.mask_sb + n]);
+        out = to_f32((bf16_t)s) * mv * sigmoid_fast(to_f32((bf16_t)sg));
+    }
+    p.c[(int64_t)batch * p.c_sb + (int64_t)m * p.c_sm + n] = (bf16_t)out;
+}
+
+// out[r][c] *= sigmoid(gate[r][c]) over rows r = (i, j) of two strided [n0, n1, size] tensors
+// (reference triangle_multiplication.cpp:129-150).
+template <bool VEC>
+__global__ __launch_bounds__(256) void sigmoid_gate_rows_kernel(bf16_t *__restrict__ out, int64_t out_s0, int64_t out_s1,
+                                                                const bf16_t *__restrict__ gate, int64_t gate_s0,
+                                                                int64_t gate_s1, int64_t n0, int64_t n1, int size)
+{
+    constexpr int W = VEC ? 8 : 1;
+    const int per_row = (size + W - 1) / W;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n0 * n1 * per_row) {
+        return;
+    }
+    const int64_t row = idx / per_row;
+    const int col = (int)(idx % per_row) * W;
+    const int64_t i = row / n1, j = row % n1;
+    bf16_t *o = out + i * out_s0 + j * out_s1 + col;
+    const bf16_t *gt = gate + i * gate_s0 + j * gate_s1 + col;
+    if constexpr (VEC) {
+        const bf16x8 ov = *reinterpret_cast<const bf16x8 *>(o), gv = *reinterpret_cast<const bf16x8 *>(gt);
+        bf16x8 res;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            res[e] = (bf16_t)(to_f32(ov[e]) * sigmoid_fast(to_f32(gv[e])));
+        }
+        *reinterpret_cast<bf16x8 *>(o) = res;
+    } else {
+        *o = (bf16_t)(to_f32(*o) * sigmoid_fast(to_f32(*gt)));
+    }
+}
+
+inline bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+// does this operand suit the 16-byte loads of the MFMA kernel?  rows = extent of the non-k index
+bool operand_ok(const void *ptr, int64_t s_row, int64_t s_k, int64_t s_batch, int64_t rows, int64_t K, bool &mmajor)
+{
+    if (!aligned16(ptr) || s_batch % 8 != 0) {
+        return false;
+    }
+    if (s_k == 1) {
+        mmajor = false;
+        return s_row % 8 == 0 && K % 8 == 0;
+    }
+    if (s_row == 1) {
+        mmajor = true;
+        return s_k % 8 == 0 && rows % 8 == 0 && rows >= 8;
+    }
+    return false;
+}
+
+template <bool AM, bool BM, bool G>
+hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
+{
+    static bool configured = false; // per instantiation: 64 KB of dynamic LDS needs the opt-in once
+    if (!configured) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_gemm_kernel<AM, BM, G>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_LDS);
+        if (e != hipSuccess) {
+            return e;
+        }
+        configured = true;
+    }
+    pair_gemm_kernel<AM, BM, G><<<dim3((unsigned)blocks), 256, GEMM_LDS, stream>>>(p);
+    return hipGetLastError();
+}
+} // namespace
+
+namespace kutacc_launch {
+
+int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
+{
+    if (g.m <= 0 || g.n <= 0 || g.k <= 0 || g.batches <= 0 || !g.a || !g.b || !g.c || g.dtype != KUTACC_DTYPE_BF16) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (g.m > INT32_MAX / 2 || g.n > INT32_MAX / 2 || g.k > INT32_MAX / 2 || g.batches > INT32_MAX ||
+        g.bias_axis < 0 || g.bias_axis > 2 || (g.bias_axis != 0 && !g.bias)) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const bool gated = g.a_gate != nullptr;
+    if (gated && (!g.mask || (g.bias_axis != 0 && !g.bias_gate))) {
+        return KUTACC_HIP_EINVAL;
+    }
+    GemmParams p;
+    p.a = (const bf16_t *)g.a, p.a_gate = (const bf16_t *)g.a_gate, p.b = (const bf16_t *)g.b, p.c = (bf16_t *)g.c;
+    p.a_sm = g.a_stride_m, p.a_sk = g.a_stride_k, p.a_sb = g.a_stride_batch;
+    p.b_sn = g.b_stride_n, p.b_sk = g.b_stride_k, p.b_sb = g.b_stride_batch;
+    p.c_sm = g.c_stride_m, p.c_sb = g.c_stride_batch;
+    p.bias = g.bias, p.bias_gate = g.bias_gate, p.mask = (const bf16_t *)g.mask, p.mask_sb = g.mask_stride_batch;
+    p.M = (int)g.m, p.N = (int)g.n, p.K = (int)g.k, p.batches = (int)g.batches;
+    p.bias_axis = g.bias_axis, p.relu = g.relu ? 1 : 0;
+
+    bool am = false, bm = false;
+    bool mfma_ok = operand_ok(g.a, g.a_stride_m, g.a_stride_k, g.a_stride_batch, g.m, g.k, am) &&
+                   operand_ok(g.b, g.b_stride_n, g.b_stride_k, g.b_stride_batch, g.n, g.k, bm) && aligned16(g.c) &&
+                   g.c_stride_m % 8 == 0 && g.c_stride_batch % 8 == 0 && g.n % 8 == 0 &&
+                   (g.bias_axis != 1 || aligned16(g.bias));
+    if (gated) {
+        mfma_ok = mfma_ok && !am && !bm && aligned16(g.a_gate) && aligned16(g.mask) && g.mask_stride_batch % 8 == 0;
+    }
+    if (g.path == KUTACC_HIP_PATH_GENERIC) {
+        mfma_ok = false;
+    } else if (g.path == KUTACC_HIP_PATH_FUSED && !mfma_ok) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    const double flops = 2.0 * (double)g.m * (double)g.n * (double)g.k * (double)g.batches * (gated ? 2.0 : 1.0);
+    if (!mfma_ok) {
+        const int64_t total = g.m * g.n * g.batches;
+        const int64_t blocks = (total + 255) / 256;
+        if (blocks > INT32_MAX) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        kutacc_prof::KernelTimer t("pair_gemm_scalar_kernel", flops, stream);
+        pair_gemm_scalar_kernel<<<dim3((unsigned)blocks), 256, 0, stream>>>(p);
+        return kutacc_hip_status(hipGetLastError());
+    }
+    p.MT = (int)((g.m + (gated ? 64 : 128) - 1) / (gated ? 64 : 128));
+    p.NT = (int)((g.n + 127) / 128);
+    const int64_t blocks = (int64_t)p.MT * p.NT * g.batches;
+    if (blocks > INT32_MAX) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    kutacc_prof::KernelTimer t(gated ? "pair_gemm_kernel<gated>" : (am || bm ? "pair_gemm_kernel<m-major>" : "pair_gemm_kernel"),
+                               flops, stream);
+    hipError_t e;
+    if (gated) {
+        e = launch_tiles<false, false, true>(p, blocks, stream);
+    } else if (am && bm) {
+        e = launch_tiles<true, true, false>(p, blocks, stream);
+    } else if (am) {
+        e = launch_tiles<true, false, false>(p, blocks, stream);
+    } else if (bm) {
+        e = launch_tiles<false, true, false>(p, blocks, stream);
+    } else {
+        e = launch_tiles<false, false, false>(p, blocks, stream);
+    }
+    return kutacc_hip_status(e);
+}
+
+int sigmoid_gate_rows(void *out, int64_t out_s0, int64_t out_s1, const void *gate, int64_t gate_s0, int64_t gate_s1,
+                      int64_t n0, int64_t n1, int64_t size, hipStream_t stream)
+{
+    if (!out || !gate || n0 <= 0 || n1 <= 0 || size <= 0 || size > INT32_MAX) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const bool vec = size % 8 == 0 && aligned16(out) && aligned16(gate) && out_s0 % 8 == 0 && out_s1 % 8 == 0 &&
+                     gate_s0 % 8 == 0 && gate_s1 % 8 == 0;
+    const int64_t per_row = vec ? size / 8 : size;
+    if (n0 > INT64_MAX / n1 || n0 * n1 > INT64_MAX / per_row) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int64_t blocks = (n0 * n1 * per_row + 255) / 256;
+    if (blocks > INT32_MAX) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    kutacc_prof::KernelTimer t("sigmoid_gate_rows_kernel", 0.0, stream);
+    if (vec) {
+        sigmoid_gate_rows_kernel<true><<<dim3((unsigned)blocks), 256, 0, stream>>>(
+            (bf16_t *)out, out_s0, out_s1, (const bf16_t *)gate, gate_s0, gate_s1, n0, n1, (int)size);
+    } else {
+        sigmoid_gate_rows_kernel<false><<<dim3((unsigned)blocks), 256, 0, stream>>>(
+            (bf16_t *)out, out_s0, out_s1, (const bf16_t *)gate, gate_s0, gate_s1, n0, n1, (int)size);
+    }
+    return kutacc_hip_status(hipGetLastError());
+}
+
+} // namespace kutacc_launch

@@ -1,7 +1,6 @@
-// Link-compatibility stubs.  The Kunpeng library exports more operators than the gated-attention
-// path this backend implements (reference include/kutacc.h:55-74, 266-280, 305-322, 367-388,
-// 426-456).  A program linked against that library must still resolve those names, so each is
-// exported here with C linkage; calling one reports "not implemented" through the usual
+// Link-compatibility stubs.  The Kunpeng library exports more operators than this backend implements
+// (reference include/kutacc.h:55-74, 266-280, 367-388).  A program linked against that library must
+// still resolve those names, so each is exported here with C linkage; calling one reports "not implemented" through the usual
 // KUTACC_CHECK channel (stderr line + sticky error flag) and touches none of its arguments.
 // With C linkage the parameter lists do not take part in symbol resolution, hence the opaque ones.
 #include "check.h"
@@ -19,11 +18,6 @@ KUTACC_UNSUPPORTED(kutacc_af2_transpose)
 KUTACC_UNSUPPORTED(kutacc_af2_all_gather)
 KUTACC_UNSUPPORTED(kutacc_af2_outer_product_mean_calc_left_and_right_mul)
 KUTACC_UNSUPPORTED(kutacc_af2_outer_product_mean_chunk)
-KUTACC_UNSUPPORTED(kutacc_af2_transition)
 KUTACC_UNSUPPORTED(kutacc_af2_invariant_point)
 KUTACC_UNSUPPORTED(kutacc_af2_rigid_rot_vec_mul)
 KUTACC_UNSUPPORTED(kutacc_af2_rigid_rot_matmul)
-KUTACC_UNSUPPORTED(kutacc_af2_triangle_multiplication_calc_proj)
-KUTACC_UNSUPPORTED(kutacc_af2_triangle_multiplication_equation)
-KUTACC_UNSUPPORTED(kutacc_af2_triangle_multiplication_gate_and_out_linear)
-KUTACC_UNSUPPORTED(kutacc_af2_triangle_multiplication_last)

@@ -14,8 +14,10 @@
  *                                 buffers, OpenMP.  This is the timed CPU baseline, and measures how
  *                                 far the reference itself sits from R32.
  *
- * plus the two row operators in front of the path (LayerNorm, Linear) and an R32 restatement of the
- * global (extra-MSA column) attention, reference src/attention/global_attention.cpp:30-164.
+ * plus the two row operators in front of the path (LayerNorm, Linear), an R32 restatement of the
+ * global (extra-MSA column) attention, reference src/attention/global_attention.cpp:30-164, and R32
+ * restatements of the transition (reference src/attention/transition.cpp:21-39) and of the steps of the
+ * triangle multiplication (reference src/attention/triangle_multiplication.cpp:25-150).
  *
  * Pinning status (the reference ships no numeric test for any of this):
  *   - R32 (both attentions), layernorm, linear: pinned by tests/test_oracle_pinning.py against library routines
@@ -574,6 +576,86 @@ void oracle_linear_f32(const float *act, int64_t ld_act, const float *w, int64_t
                 acc += (double)beta * result[r * n + o];
             }
             result[r * n + o] = (float)acc;
+        }
+    }
+}
+
+/* ---- transition and triangle multiplication (R32: fp32 operands, double accumulation, no rounding) ---- */
+
+/* mid = relu(x . w1^T + b1), out = mid . w2^T + b2 (reference src/attention/transition.cpp:31-38).
+ * x [rows, c_o], w1 [c_i, c_o], w2 [c_o, c_i] stored [out, in]; mid [rows, c_i] may be NULL. */
+void oracle_transition_f32(const float *x, const float *w1, const float *b1, const float *w2, const float *b2,
+                           int64_t rows, int64_t c_o, int64_t c_i, float *out, float *mid)
+{
+#pragma omp parallel
+    {
+        double *h = (double *)malloc((size_t)c_i * sizeof(double));
+#pragma omp for schedule(static)
+        for (int64_t r = 0; r < rows; ++r) {
+            for (int64_t j = 0; j < c_i; ++j) {
+                double acc = b1[j];
+                for (int64_t k = 0; k < c_o; ++k) {
+                    acc += (double)x[r * c_o + k] * (double)w1[j * c_o + k];
+                }
+                h[j] = acc > 0.0 ? acc : 0.0;
+                if (mid) {
+                    mid[r * c_i + j] = (float)h[j];
+                }
+            }
+            for (int64_t o = 0; o < c_o; ++o) {
+                double acc = b2[o];
+                for (int64_t j = 0; j < c_i; ++j) {
+                    acc += h[j] * (double)w2[o * c_i + j];
+                }
+                out[r * c_o + o] = (float)acc;
+            }
+        }
+        free(h);
+    }
+}
+
+/* proj[c, i, j] = (x[i, j, :] . pw[c, :] + pb[c]) * mask[i, j] * sigmoid(x[i, j, :] . gw[c, :] + gb[c])
+ * (reference src/attention/triangle_multiplication.cpp:37-66): x [n, c_o] with n = n_res*n_res_gather rows,
+ * pw, gw [c_i, c_o], mask [n], proj [c_i, n] channel-first. */
+void oracle_tm_calc_proj_f32(const float *x, const float *mask, const float *pw, const float *pb, const float *gw,
+                             const float *gb, int64_t n, int64_t c_o, int64_t c_i, float *proj)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < n; ++r) {
+        for (int64_t c = 0; c < c_i; ++c) {
+            double p = pb[c], g = gb[c];
+            for (int64_t k = 0; k < c_o; ++k) {
+                p += (double)x[r * c_o + k] * (double)pw[c * c_o + k];
+                g += (double)x[r * c_o + k] * (double)gw[c * c_o + k];
+            }
+            proj[c * n + r] = (float)(p * (double)mask[r] / (1.0 + exp(-g)));
+        }
+    }
+}
+
+/* Per channel c of dense [channels, n, n] tensors (reference src/attention/triangle_multiplication.cpp:72-101):
+ *   outgoing: center[c, i, j] = sum_k left[c, i, k] * right[c, j, k]
+ *   incoming: center[c, i, j] = sum_k right[c, k, i] * left[c, k, j] */
+void oracle_tm_equation_f32(const float *left, const float *right, int64_t channels, int64_t n, int incoming,
+                            float *center)
+{
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int64_t c = 0; c < channels; ++c) {
+        for (int64_t i = 0; i < n; ++i) {
+            const float *l = left + c * n * n, *r = right + c * n * n;
+            for (int64_t j = 0; j < n; ++j) {
+                double acc = 0.0;
+                if (!incoming) {
+                    for (int64_t k = 0; k < n; ++k) {
+                        acc += (double)l[i * n + k] * (double)r[j * n + k];
+                    }
+                } else {
+                    for (int64_t k = 0; k < n; ++k) {
+                        acc += (double)r[k * n + i] * (double)l[k * n + j];
+                    }
+                }
+                center[(c * n + i) * n + j] = (float)acc;
+            }
         }
     }
 }

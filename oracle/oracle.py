@@ -223,3 +223,53 @@ def gating_attention_f64_numpy(x, wq, wk, wv, wg, bg, wo, bo, bias, nb, nheads, 
     avg = avg.reshape(B, S, C)
     out = avg @ f(wo).T + f(bo)
     return (out, avg) if return_avg else out
+
+
+# ---- transition and triangle multiplication ---------------------------------------------------------
+def transition_f32(x, w1, b1, w2, b2, return_mid=False):
+    """x [rows, c_o]; w1 [c_i, c_o], w2 [c_o, c_i] stored [out, in]; b1 [c_i], b2 [c_o] -> out [rows, c_o]
+    (reference src/attention/transition.cpp:31-38)."""
+    x, w1, b1, w2, b2 = (_f32(a) for a in (x, w1, b1, w2, b2))
+    c_i, c_o = w1.shape
+    rows = x.size // c_o
+    out = np.empty((rows, c_o), dtype=np.float32)
+    mid = np.empty((rows, c_i), dtype=np.float32) if return_mid else None
+    lib().oracle_transition_f32(_ptr(x, _f32p), _ptr(w1, _f32p), _ptr(b1, _f32p), _ptr(w2, _f32p), _ptr(b2, _f32p),
+                                _i64(rows), _i64(c_o), _i64(c_i), _ptr(out, _f32p), _ptr(mid, _f32p))
+    return (out, mid) if return_mid else out
+
+
+def tm_calc_proj_f32(x, mask, pw, pb, gw, gb):
+    """x [n_res, n_gather, c_o]; mask [n_res, n_gather]; pw, gw [c_i, c_o]; pb, gb [c_i] -> proj [c_i, n_res, n_gather]
+    (reference src/attention/triangle_multiplication.cpp:37-66)."""
+    x, mask, pw, pb, gw, gb = (_f32(a) for a in (x, mask, pw, pb, gw, gb))
+    n_res, n_gather, c_o = x.shape
+    c_i = pw.shape[0]
+    proj = np.empty((c_i, n_res, n_gather), dtype=np.float32)
+    lib().oracle_tm_calc_proj_f32(_ptr(x, _f32p), _ptr(mask, _f32p), _ptr(pw, _f32p), _ptr(pb, _f32p), _ptr(gw, _f32p),
+                                  _ptr(gb, _f32p), _i64(n_res * n_gather), _i64(c_o), _i64(c_i), _ptr(proj, _f32p))
+    return proj
+
+
+def tm_equation_f32(left, right, incoming):
+    """left, right [c, n, n] -> center [c, n, n] (reference src/attention/triangle_multiplication.cpp:72-101)."""
+    left, right = _f32(left), _f32(right)
+    c, n, _ = left.shape
+    center = np.empty((c, n, n), dtype=np.float32)
+    lib().oracle_tm_equation_f32(_ptr(left, _f32p), _ptr(right, _f32p), _i64(c), _i64(n), ctypes.c_int(1 if incoming else 0),
+                                 _ptr(center, _f32p))
+    return center
+
+
+def tm_gate_and_out_f32(x, center, gating_w, gating_b, out_w, out_b):
+    """gate = x . gating_w^T + gating_b and out = center . out_w^T + out_b over rows (i, j): two plain linears
+    (reference src/attention/triangle_multiplication.cpp:115-126).  x [.., c_o], center [.., c_i]."""
+    gate = linear_f32(_f32(x).reshape(-1, np.shape(x)[-1]), gating_w, gating_b)
+    out = linear_f32(_f32(center).reshape(-1, np.shape(center)[-1]), out_w, out_b)
+    return gate, out
+
+
+def tm_last_f32(out, gate):
+    """out * sigmoid(gate) (reference src/attention/triangle_multiplication.cpp:139-146), evaluated in float64."""
+    o, g = np.asarray(out, dtype=np.float64), np.asarray(gate, dtype=np.float64)
+    return (o / (1.0 + np.exp(-g))).astype(np.float32)

@@ -39,10 +39,10 @@ def test_headers_and_binding_agree_on_symbol_list():
 
 def test_unimplemented_operators_resolve_and_report():
     L = capi.lib()
-    for name in ("kutacc_af2_transition", "kutacc_af2_transpose",
-                 "kutacc_comm_init", "kutacc_af2_triangle_multiplication_last"):
+    for name in ("kutacc_af2_invariant_point", "kutacc_af2_transpose", "kutacc_comm_init",
+                 "kutacc_af2_outer_product_mean_chunk"):
         assert hasattr(L, name), name
-    L.kutacc_af2_transition(None, None, None)
+    L.kutacc_af2_transpose(None, None)
     assert capi.error_flag()
 
 
@@ -174,3 +174,102 @@ def test_global_attention_needs_64_channels_and_checks_scalars_before_handles(ca
     capi.lib().kutacc_af2_global_attention(ctypes.byref(inputs), ap, ap, ctypes.byref(weights), ap)
     assert capi.error_flag()
     assert "input param <= 0 or overflow" in capfd.readouterr().err
+
+
+# ---- transition: reference test/functest/cal/transition_test.cpp:18-106 (each pointer null in turn) -------------
+def _pair_stack_arguments():
+    a = (ctypes.c_float * 1)(0.8)
+    x = (ctypes.c_float * 8)(1, 2, 3, 4, 7, 8, 9, 10)
+    ap, xp = ctypes.addressof(a), ctypes.addressof(x)
+    keep = (a, x)
+    return keep, ap, xp
+
+
+@pytest.mark.parametrize("null_index", range(3))
+def test_transition_null_pointers_are_rejected(null_index, capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    inputs = capi.TransActInputs(2, 2, xp, xp)
+    weights = capi.TransWeights(2, 2, xp, xp, xp, xp)
+    args = [ctypes.byref(inputs), ctypes.byref(weights), ap]
+    args[null_index] = None
+    capi.lib().kutacc_af2_transition(*args)
+    assert capi.error_flag()
+    assert "af2_transition: input args nullptr error" in capfd.readouterr().err
+
+
+def test_transition_checks_scalars_before_any_handle_is_read(capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    inputs = capi.TransActInputs(2, 0, xp, xp)  # handles are plain floats: nothing may be read through them
+    weights = capi.TransWeights(2, 2, xp, xp, xp, xp)
+    capi.lib().kutacc_af2_transition(ctypes.byref(inputs), ctypes.byref(weights), ap)
+    assert capi.error_flag()
+    assert "input param <= 0 or overflow" in capfd.readouterr().err
+
+
+# ---- triangle multiplication: reference test/functest/cal/triangle_multiplication_test.cpp:18-354 ---------------
+@pytest.mark.parametrize("null_index", range(3))
+def test_tm_calc_proj_null_pointers_are_rejected(null_index, capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    acts = capi.TmActInputs(2, 2, xp, xp, xp)
+    weights = capi.TmProjWeights(2, 2, xp, xp, xp, xp)
+    args = [ctypes.byref(acts), ap, ctypes.byref(weights)]
+    args[null_index] = None
+    capi.lib().kutacc_af2_triangle_multiplication_calc_proj(*args, True)
+    assert capi.error_flag()
+    assert "kutacc_af2_triangle_multiplication_calc_proj: input args nullptr error" in capfd.readouterr().err
+
+
+@pytest.mark.parametrize("null_index", range(3))
+def test_tm_equation_null_pointers_are_rejected(null_index, capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    args = [ap, ap, ap]
+    args[null_index] = None
+    capi.lib().kutacc_af2_triangle_multiplication_equation(*args, 5, True)
+    assert capi.error_flag()
+    assert "kutacc_af2_triangle_multiplication_equation: input args nullptr error" in capfd.readouterr().err
+
+
+def test_tm_equation_negative_extent_is_rejected_before_any_handle_is_read(capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    capi.lib().kutacc_af2_triangle_multiplication_equation(ap, ap, ap, -5, True)
+    assert capi.error_flag()
+    assert "less than or equal to zero" in capfd.readouterr().err
+
+
+@pytest.mark.parametrize("null_index", range(5))
+def test_tm_gate_and_out_linear_null_pointers_are_rejected(null_index, capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    acts = capi.TmActInputs(2, 2, xp, xp, xp)
+    weights = capi.TmLinearWeights(2, 2, xp, xp, xp, xp)
+    args = [ap, ap, ctypes.byref(acts), ap, ctypes.byref(weights)]
+    args[null_index] = None
+    capi.lib().kutacc_af2_triangle_multiplication_gate_and_out_linear(*args, True)
+    assert capi.error_flag()
+    assert "kutacc_af2_triangle_multiplication_gate_and_out_linear: input args nullptr error" in capfd.readouterr().err
+
+
+@pytest.mark.parametrize("null_index", range(2))
+def test_tm_last_null_pointers_are_rejected(null_index, capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    args = [ap, ap]
+    args[null_index] = None
+    capi.lib().kutacc_af2_triangle_multiplication_last(*args, 5, 5, 5)
+    assert capi.error_flag()
+    assert "kutacc_af2_triangle_multiplication_last: input args nullptr error" in capfd.readouterr().err
+
+
+@pytest.mark.parametrize("extents", [(-5, 5, 5), (5, -5, 5), (5, 5, -5)])
+def test_tm_last_negative_extents_are_rejected_before_any_handle_is_read(extents, capfd):
+    keep, ap, xp = _pair_stack_arguments()
+    capi.lib().kutacc_af2_triangle_multiplication_last(ap, ap, *extents)
+    assert capi.error_flag()
+    assert "less than or equal" in capfd.readouterr().err
+
+
+def test_gemm_launch_layer_rejects_bad_arguments_without_a_device():
+    L = capi.lib()
+    assert L.kutacc_hip_gemm(None, None) == capi.EINVAL
+    g = capi.HipGemmArgs()
+    g.m, g.n, g.k, g.batches, g.dtype = 4, 4, 4, 1, capi.K_BF16
+    assert L.kutacc_hip_gemm(ctypes.byref(g), None) == capi.EINVAL  # null operands
+    assert L.kutacc_hip_sigmoid_gate_rows(None, 1, 1, None, 1, 1, 1, 1, 1, capi.K_BF16, None) == capi.EINVAL

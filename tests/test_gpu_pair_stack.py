@@ -1,0 +1,288 @@
+"""Parity of the transition and triangle-multiplication operators (and of the strided bf16 GEMM under them)
+against the CPU oracle, through the C ABI, on a real MI355X.
+
+Inputs are bf16-representable fp32 draws, so the device and the oracle see the same numbers; the oracle
+works in fp32/fp64 without intermediate rounding.  Tolerances: a plain GEMM result is one bf16 rounding away
+from the exact value (relative 2^-9), checked at 6e-3 relative + 2e-3 absolute; results that pass through a
+second bf16-rounded intermediate (hidden layer of the transition, gated projections) are checked at the bar
+of the bf16 path, 2e-2 absolute + 1e-2 relative of the fp32 oracle.
+"""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+
+from kutacc_amd import capi
+from kutacc_amd.workloads import round_to_bf16
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    capi.set_stream(None)
+    capi.set_blocking(True)
+    return torch
+
+
+def draw(rng, *shape, scale=1.0):
+    return round_to_bf16((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+def dev(torch, a, dtype=None):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device="cuda", dtype=dtype or torch.bfloat16)
+
+
+GEMM_TOL = lambda ref: 2e-3 + 6e-3 * np.abs(ref)  # noqa: E731
+
+
+def run_gemm(torch, A, B, *, a_mmajor=False, b_mmajor=False, bias=None, bias_axis=0, relu=False, path=capi.PATH_AUTO,
+             c_pad=0):
+    """A [batches, M, K], B [batches, N, K] as fp32 numpy; operands are stored k-contiguous or transposed (m-major)."""
+    nb, M, K = A.shape
+    N = B.shape[1]
+    dA = dev(torch, A.transpose(0, 2, 1) if a_mmajor else A)
+    dB = dev(torch, B.transpose(0, 2, 1) if b_mmajor else B)
+    dC = torch.full((nb, M, N + c_pad), -7.0, dtype=torch.bfloat16, device="cuda")
+    g = capi.HipGemmArgs()
+    g.m, g.n, g.k, g.batches, g.dtype, g.path = M, N, K, nb, capi.K_BF16, path
+    g.a, g.a_stride_batch = dA.data_ptr(), M * K
+    g.a_stride_m, g.a_stride_k = (1, M) if a_mmajor else (K, 1)
+    g.b, g.b_stride_batch = dB.data_ptr(), N * K
+    g.b_stride_n, g.b_stride_k = (1, N) if b_mmajor else (K, 1)
+    g.c, g.c_stride_m, g.c_stride_batch = dC.data_ptr(), N + c_pad, M * (N + c_pad)
+    keep = None
+    if bias is not None:
+        keep = dev(torch, bias, torch.float32)
+        g.bias, g.bias_axis = keep.data_ptr(), bias_axis
+    g.relu = 1 if relu else 0
+    rc = capi.lib().kutacc_hip_gemm(ctypes.byref(g), None)
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    out = helpers.to_numpy(dC)
+    if c_pad:
+        assert np.all(out[:, :, N:] == -7.0), "columns beyond n were written"
+    return out[:, :, :N]
+
+
+def gemm_ref(A, B, bias=None, bias_axis=0, relu=False):
+    ref = np.einsum("bmk,bnk->bmn", A.astype(np.float64), B.astype(np.float64))
+    if bias_axis == 1:
+        ref = ref + bias[None, None, :]
+    elif bias_axis == 2:
+        ref = ref + bias[None, :, None]
+    return np.maximum(ref, 0) if relu else ref
+
+
+@pytest.mark.parametrize("path", [capi.PATH_FUSED, capi.PATH_GENERIC], ids=["mfma", "scalar"])
+@pytest.mark.parametrize("shape", [(1, 128, 128, 64), (1, 300, 136, 72), (3, 72, 264, 200), (2, 40, 8, 8)])
+def test_gemm_k_major_operands(torch_cuda, shape, path):
+    """Ragged tiles in m and n, a k tail that is not a multiple of the 64-wide step, batches."""
+    nb, M, N, K = shape
+    rng = np.random.Generator(np.random.PCG64(100 + M))
+    A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
+    got = run_gemm(torch_cuda, A, B, path=path, c_pad=8)
+    helpers.assert_within(got, gemm_ref(A, B), GEMM_TOL(gemm_ref(A, B)), f"gemm {shape}")
+
+
+@pytest.mark.parametrize("bias_axis,relu", [(1, False), (1, True), (2, False), (2, True)])
+@pytest.mark.parametrize("path", [capi.PATH_FUSED, capi.PATH_GENERIC], ids=["mfma", "scalar"])
+def test_gemm_bias_and_relu_epilogues(torch_cuda, path, bias_axis, relu):
+    nb, M, N, K = 2, 200, 168, 96
+    rng = np.random.Generator(np.random.PCG64(7))
+    A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
+    bias = rng.standard_normal(N if bias_axis == 1 else M).astype(np.float32)
+    got = run_gemm(torch_cuda, A, B, bias=bias, bias_axis=bias_axis, relu=relu, path=path)
+    ref = gemm_ref(A, B, bias, bias_axis, relu)
+    helpers.assert_within(got, ref, GEMM_TOL(ref), f"bias axis {bias_axis} relu {relu}")
+    if relu:
+        assert got.min() >= 0.0
+
+
+@pytest.mark.parametrize("a_mmajor,b_mmajor", [(True, True), (True, False), (False, True)])
+@pytest.mark.parametrize("shape", [(2, 128, 128, 64), (3, 200, 136, 100), (1, 64, 72, 45)])
+def test_gemm_m_major_operands(torch_cuda, shape, a_mmajor, b_mmajor):
+    """Operands stored transposed (contraction index slowest), as the incoming triangle equation has them."""
+    nb, M, N, K = shape
+    if not b_mmajor or not a_mmajor:
+        K = (K + 7) // 8 * 8  # a k-major operand next to it needs k in whole 16-byte chunks
+    rng = np.random.Generator(np.random.PCG64(200 + M + K))
+    A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
+    got = run_gemm(torch_cuda, A, B, a_mmajor=a_mmajor, b_mmajor=b_mmajor, path=capi.PATH_FUSED)
+    ref = gemm_ref(A, B)
+    helpers.assert_within(got, ref, GEMM_TOL(ref), f"m-major {a_mmajor}/{b_mmajor} {shape}")
+    same = run_gemm(torch_cuda, A, B, a_mmajor=a_mmajor, b_mmajor=b_mmajor, path=capi.PATH_GENERIC)
+    helpers.assert_within(got, same, 1e-3 + 8e-3 * np.abs(same), "mfma vs scalar kernel")
+
+
+def test_gemm_rejects_what_it_cannot_run(torch_cuda):
+    torch = torch_cuda
+    t = torch.zeros(64 * 64, dtype=torch.bfloat16, device="cuda")
+    g = capi.HipGemmArgs()
+    g.m, g.n, g.k, g.batches, g.dtype, g.path = 8, 8, 12, 1, capi.K_BF16, capi.PATH_FUSED  # k not a multiple of 8
+    g.a, g.a_stride_m, g.a_stride_k = t.data_ptr(), 12, 1
+    g.b, g.b_stride_n, g.b_stride_k = t.data_ptr(), 12, 1
+    g.c, g.c_stride_m = t.data_ptr(), 8
+    assert capi.lib().kutacc_hip_gemm(ctypes.byref(g), None) == capi.EUNSUPPORTED
+    g.path = capi.PATH_AUTO
+    assert capi.lib().kutacc_hip_gemm(ctypes.byref(g), None) == 0
+    g.dtype = capi.K_FP32
+    assert capi.lib().kutacc_hip_gemm(ctypes.byref(g), None) == capi.EINVAL
+    torch.cuda.synchronize()
+
+
+# ---- transition ------------------------------------------------------------------------------------------------
+def transition_case(seed, batch, n_res, c_o, c_i):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return dict(x=draw(rng, batch, n_res, c_o), w1=draw(rng, c_i, c_o, scale=1 / math.sqrt(c_o)),
+                b1=rng.standard_normal(c_i).astype(np.float32) * 0.5, w2=draw(rng, c_o, c_i, scale=1 / math.sqrt(c_i)),
+                b2=rng.standard_normal(c_o).astype(np.float32) * 0.5)
+
+
+def run_transition(torch, c):
+    batch, n_res, c_o = c["x"].shape
+    c_i = c["w1"].shape[0]
+    mid = torch.zeros((batch * n_res, c_i), dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros((batch, n_res, c_o), dtype=torch.bfloat16, device="cuda")
+    op = capi.Transition(dev(torch, c["x"]), dev(torch, c["w1"]), dev(torch, c["b1"], torch.float32), dev(torch, c["w2"]),
+                         dev(torch, c["b2"], torch.float32), mid, out)
+    op.run()
+    assert not capi.error_flag()
+    return out, mid
+
+
+@pytest.mark.parametrize("shape", [(2, 37, 128, 512), (3, 50, 256, 1024), (1, 9, 24, 40), (2, 5, 6, 10)])
+def test_transition_small(torch_cuda, shape):
+    """Pair (128 -> 512) and MSA (256 -> 1024) channel counts at ragged row counts, and channel counts that run on
+    the scalar kernel."""
+    from oracle import oracle
+    c = transition_case(300 + shape[2], *shape)
+    out, mid = run_transition(torch_cuda, c)
+    ref, ref_mid = oracle.transition_f32(c["x"].reshape(-1, shape[2]), c["w1"], c["b1"], c["w2"], c["b2"], return_mid=True)
+    helpers.assert_within(helpers.to_numpy(mid), ref_mid, GEMM_TOL(ref_mid), "hidden layer")
+    helpers.check_close(helpers.to_numpy(out).reshape(ref.shape), ref, "bf16", f"transition {shape}")
+
+
+def test_transition_full_pair_size(torch_cuda):
+    """The pair transition of a 384-residue model at its real shape (147456 rows); the oracle checks a sample of
+    rows (rows are independent), and a second call on a row permutation must give the permuted result bit for bit."""
+    from oracle import oracle
+    torch = torch_cuda
+    c = transition_case(310, 384, 384, 128, 512)
+    out, _ = run_transition(torch, c)
+    rows = np.random.Generator(np.random.PCG64(1)).choice(384 * 384, size=1024, replace=False)
+    ref = oracle.transition_f32(c["x"].reshape(-1, 128)[rows], c["w1"], c["b1"], c["w2"], c["b2"])
+    helpers.check_close(helpers.to_numpy(out).reshape(-1, 128)[rows], ref, "bf16", "transition 384x384")
+    c2 = dict(c, x=np.ascontiguousarray(c["x"][::-1]))
+    out2, _ = run_transition(torch, c2)
+    assert helpers.same_bits(out2, torch.flip(out, dims=[0]))
+
+
+# ---- triangle multiplication -----------------------------------------------------------------------------------
+def tm_case(seed, n, c_o, c_i):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    w = lambda o, i: draw(rng, o, i, scale=1 / math.sqrt(i))  # noqa: E731
+    b = lambda k: (rng.standard_normal(k) * 0.5).astype(np.float32)  # noqa: E731
+    return dict(x=draw(rng, n, n, c_o), mask=(rng.random((n, n)) > 0.15).astype(np.float32),
+                lpw=w(c_i, c_o), lpb=b(c_i), lgw=w(c_i, c_o), lgb=b(c_i),
+                rpw=w(c_i, c_o), rpb=b(c_i), rgw=w(c_i, c_o), rgb=b(c_i),
+                gating_w=w(c_o, c_o), gating_b=b(c_o), out_w=w(c_o, c_i), out_b=b(c_o))
+
+
+def calc_proj(torch, c, side, n, c_o, c_i, dx, dmask):
+    proj = torch.zeros((c_i, n, n), dtype=torch.bfloat16, device="cuda")
+    gate = torch.zeros_like(proj)
+    keep = [dev(torch, c[side + "pw"]), dev(torch, c[side + "pb"], torch.float32), dev(torch, c[side + "gw"]),
+            dev(torch, c[side + "gb"], torch.float32)]
+    h = [capi.tensor(t) if t.dtype == torch.bfloat16 else capi.tensor(t, capi.K_FP32) for t in keep]
+    hp, hx, hg, hm = capi.tensor(proj), capi.tensor(dx), capi.tensor(gate), capi.tensor(dmask)
+    acts = capi.TmActInputs(n, n, hp.handle, hx.handle, hg.handle)
+    weights = capi.TmProjWeights(c_o, c_i, h[0].handle, h[1].handle, h[2].handle, h[3].handle)
+    capi.kutacc_af2_triangle_multiplication_calc_proj(acts, hm, weights, False)
+    assert not capi.error_flag()
+    return proj
+
+
+def equation(torch, left, right, n, incoming):
+    center = torch.zeros_like(left)
+    hc, hl, hr = capi.tensor(center), capi.tensor(left), capi.tensor(right)
+    capi.kutacc_af2_triangle_multiplication_equation(hc, hl, hr, n, incoming)
+    assert not capi.error_flag()
+    return center
+
+
+@pytest.mark.parametrize("n,c_o,c_i", [(40, 128, 128), (24, 64, 32), (7, 6, 5)])
+@pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
+def test_triangle_multiplication_steps(torch_cuda, n, c_o, c_i, incoming):
+    """Each of the four entry points against its oracle function, on the oracle's (unrounded) inputs to that step
+    rounded to bf16, so that an error in one step is not hidden by the tolerance of the next."""
+    from oracle import oracle
+    torch = torch_cuda
+    c = tm_case(400 + n, n, c_o, c_i)
+    dx, dmask = dev(torch, c["x"]), dev(torch, c["mask"])
+    # 1. projections
+    left = calc_proj(torch, c, "l", n, c_o, c_i, dx, dmask)
+    right = calc_proj(torch, c, "r", n, c_o, c_i, dx, dmask)
+    ref_l = oracle.tm_calc_proj_f32(c["x"], c["mask"], c["lpw"], c["lpb"], c["lgw"], c["lgb"])
+    ref_r = oracle.tm_calc_proj_f32(c["x"], c["mask"], c["rpw"], c["rpb"], c["rgw"], c["rgb"])
+    helpers.check_close(helpers.to_numpy(left), ref_l, "bf16", "left projection")
+    helpers.check_close(helpers.to_numpy(right), ref_r, "bf16", "right projection")
+    assert bool((left[:, dmask == 0] == 0).all()), "masked positions must be exactly zero"
+    # 2. equation, on bf16-rounded oracle projections
+    in_l, in_r = round_to_bf16(ref_l), round_to_bf16(ref_r)
+    center = equation(torch, dev(torch, in_l), dev(torch, in_r), n, incoming)
+    ref_c = oracle.tm_equation_f32(in_l, in_r, incoming)
+    helpers.assert_within(helpers.to_numpy(center), ref_c, GEMM_TOL(ref_c), "equation")
+    # 3. gate and output projection on a channel-last, normalised centre (the caller's layer norm is not part of the step)
+    ctr = round_to_bf16(np.ascontiguousarray(ref_c.transpose(1, 2, 0)) / math.sqrt(n))
+    d_ctr = dev(torch, ctr)
+    gate = torch.zeros((n, n, c_o), dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros_like(gate)
+    keep = [dev(torch, c["gating_w"]), dev(torch, c["gating_b"], torch.float32), dev(torch, c["out_w"]),
+            dev(torch, c["out_b"], torch.float32)]
+    h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]
+    hx, hg, ho, hc = capi.tensor(dx), capi.tensor(gate), capi.tensor(out), capi.tensor(d_ctr)
+    acts = capi.TmActInputs(n, n, None, hx.handle, None)
+    weights = capi.TmLinearWeights(c_o, c_i, h[0].handle, h[1].handle, h[2].handle, h[3].handle)
+    capi.kutacc_af2_triangle_multiplication_gate_and_out_linear(hg, ho, acts, hc, weights, False)
+    assert not capi.error_flag()
+    ref_gate, ref_out = oracle.tm_gate_and_out_f32(c["x"], ctr, c["gating_w"], c["gating_b"], c["out_w"], c["out_b"])
+    helpers.assert_within(helpers.to_numpy(gate).reshape(ref_gate.shape), ref_gate, GEMM_TOL(ref_gate), "gate")
+    helpers.assert_within(helpers.to_numpy(out).reshape(ref_out.shape), ref_out, GEMM_TOL(ref_out), "output projection")
+    # 4. last: out *= sigmoid(gate), on the device's own gate and out
+    want = oracle.tm_last_f32(helpers.to_numpy(out), helpers.to_numpy(gate))
+    capi.kutacc_af2_triangle_multiplication_last(ho, hg, n, n, c_o)
+    assert not capi.error_flag()
+    helpers.assert_within(helpers.to_numpy(out), want, 1e-3 + 6e-3 * np.abs(want), "gated output")
+
+
+def test_triangle_multiplication_full_size_properties(torch_cuda):
+    """384 residues, 128 channels at the real shape.  The oracle checks a sample of channels of the equation and a
+    sample of positions of the projection; size-independent properties cover the rest: the incoming equation equals
+    the outgoing one on transposed operands, and a masked position is exactly zero."""
+    from oracle import oracle
+    torch = torch_cuda
+    n, c_o, c_i = 384, 128, 128
+    c = tm_case(500, n, c_o, c_i)
+    dx, dmask = dev(torch, c["x"]), dev(torch, c["mask"])
+    left = calc_proj(torch, c, "l", n, c_o, c_i, dx, dmask)
+    right = calc_proj(torch, c, "r", n, c_o, c_i, dx, dmask)
+    rows = np.random.Generator(np.random.PCG64(2)).choice(n, size=6, replace=False)
+    ref_rows = oracle.tm_calc_proj_f32(c["x"][rows], c["mask"][rows], c["lpw"], c["lpb"], c["lgw"], c["lgb"])
+    helpers.check_close(helpers.to_numpy(left[:, torch.from_numpy(rows).cuda()]), ref_rows, "bf16", "left projection rows")
+    assert bool((right[:, dmask == 0] == 0).all())
+    out_c = equation(torch, left, right, n, False)
+    in_c = equation(torch, left, right, n, True)
+    chans = [0, 77, 127]
+    l_np, r_np = helpers.to_numpy(left[chans]), helpers.to_numpy(right[chans])
+    for incoming, got in ((False, out_c), (True, in_c)):
+        ref = oracle.tm_equation_f32(l_np, r_np, incoming)
+        helpers.assert_within(helpers.to_numpy(got[chans]), ref, 2e-2 + 6e-3 * np.abs(ref), f"equation incoming={incoming}")
+    lt, rt = left.transpose(1, 2).contiguous(), right.transpose(1, 2).contiguous()
+    swapped = equation(torch, rt, lt, n, False)  # outgoing(right^T, left^T) == incoming(left, right)
+    assert helpers.same_bits(swapped, in_c)

@@ -447,3 +447,115 @@ def test_global_token_permutation_permutes_output():
     perm = np.random.Generator(np.random.PCG64(5)).permutation(10)
     c2 = dict(c, x=c["x"][:, perm].copy(), mask=c["mask"][:, perm].copy())
     np.testing.assert_allclose(run_global(c2), run_global(c)[:, perm], rtol=2e-5, atol=2e-6)
+
+
+# ---- transition and triangle multiplication: reference src/attention/transition.cpp:21-39,
+# ---- src/attention/triangle_multiplication.cpp:25-150 -------------------------------------------------------------
+def make_pair_case(seed, n_res, n_gather, c_o, c_i):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
+    return dict(x=f(n_res, n_gather, c_o), mask=(rng.random((n_res, n_gather)) > 0.2).astype(np.float32),
+                pw=f(c_i, c_o) / math.sqrt(c_o), pb=f(c_i), gw=f(c_i, c_o) / math.sqrt(c_o), gb=f(c_i),
+                w1=f(c_i, c_o) / math.sqrt(c_o), b1=f(c_i), w2=f(c_o, c_i) / math.sqrt(c_i), b2=f(c_o),
+                left=f(c_i, n_gather, n_gather), right=f(c_i, n_gather, n_gather))
+
+
+def test_transition_matches_torch_and_bruteforce():
+    c = make_pair_case(50, 3, 5, 8, 12)
+    out, mid = oracle.transition_f32(c["x"].reshape(-1, 8), c["w1"], c["b1"], c["w2"], c["b2"], return_mid=True)
+    t = lambda a: torch.from_numpy(a).double()  # noqa: E731
+    h = torch.relu(torch.nn.functional.linear(t(c["x"]).reshape(-1, 8), t(c["w1"]), t(c["b1"])))
+    ref = torch.nn.functional.linear(h, t(c["w2"]), t(c["b2"]))
+    np.testing.assert_allclose(mid, h.numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(out, ref.numpy(), rtol=1e-6, atol=1e-6)
+    # pure-Python loops, index by index, on the first two rows
+    x = c["x"].reshape(-1, 8).astype(float)
+    for r in range(2):
+        hid = [max(0.0, sum(x[r][k] * float(c["w1"][j][k]) for k in range(8)) + float(c["b1"][j])) for j in range(12)]
+        for o in range(8):
+            want = sum(hid[j] * float(c["w2"][o][j]) for j in range(12)) + float(c["b2"][o])
+            assert abs(out[r][o] - want) < 1e-5
+
+
+def test_transition_closed_forms():
+    c = make_pair_case(51, 2, 4, 8, 12)
+    x = c["x"].reshape(-1, 8)
+    # zero first weight: the hidden layer is relu(b1) for every row
+    out = oracle.transition_f32(x, np.zeros_like(c["w1"]), c["b1"], c["w2"], c["b2"])
+    want = np.maximum(c["b1"].astype(np.float64), 0) @ c["w2"].astype(np.float64).T + c["b2"]
+    np.testing.assert_allclose(out, np.broadcast_to(want, out.shape), rtol=1e-6, atol=1e-6)
+    # a very negative first bias switches every hidden unit off: out == b2
+    out = oracle.transition_f32(x, c["w1"], np.full(12, -1e4, np.float32), c["w2"], c["b2"])
+    np.testing.assert_allclose(out, np.broadcast_to(c["b2"], out.shape), rtol=0, atol=0)
+    # a very positive first bias makes the ReLU the identity: the layer pair collapses to one affine map
+    big = np.full(12, 1e3, np.float32)
+    out = oracle.transition_f32(x, c["w1"], big, c["w2"], c["b2"])
+    w = c["w2"].astype(np.float64) @ c["w1"].astype(np.float64)
+    want = x.astype(np.float64) @ w.T + c["w2"].astype(np.float64) @ big + c["b2"]
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-3)
+
+
+def test_tm_calc_proj_matches_torch_and_closed_forms():
+    c = make_pair_case(52, 4, 6, 8, 5)
+    got = oracle.tm_calc_proj_f32(c["x"], c["mask"], c["pw"], c["pb"], c["gw"], c["gb"])
+    t = lambda a: torch.from_numpy(a).double()  # noqa: E731
+    p = torch.nn.functional.linear(t(c["x"]), t(c["pw"]), t(c["pb"]))       # [i, j, c]
+    g = torch.sigmoid(torch.nn.functional.linear(t(c["x"]), t(c["gw"]), t(c["gb"])))
+    ref = (p * t(c["mask"])[..., None] * g).permute(2, 0, 1)               # channel-first, as the reference stores it
+    np.testing.assert_allclose(got, ref.numpy(), rtol=1e-6, atol=1e-6)
+    assert got.shape == (5, 4, 6)
+    # masked positions are exactly zero, in every channel
+    assert np.all(got[:, c["mask"] == 0] == 0)
+    # gate weights zero and gate bias 0 -> sigmoid(0) = 1/2; gate bias +40 -> gate 1
+    half = oracle.tm_calc_proj_f32(c["x"], c["mask"], c["pw"], c["pb"], np.zeros_like(c["gw"]), np.zeros_like(c["gb"]))
+    one = oracle.tm_calc_proj_f32(c["x"], c["mask"], c["pw"], c["pb"], np.zeros_like(c["gw"]), np.full(5, 40, np.float32))
+    np.testing.assert_allclose(2 * half, one, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(one, (p * t(c["mask"])[..., None]).permute(2, 0, 1).numpy(), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("incoming", [False, True])
+def test_tm_equation_matches_einsum_and_bruteforce(incoming):
+    c = make_pair_case(53, 7, 7, 4, 3)
+    got = oracle.tm_equation_f32(c["left"], c["right"], incoming)
+    le, ri = torch.from_numpy(c["left"]).double(), torch.from_numpy(c["right"]).double()
+    # AlphaFold's equations with channel-first operands: outgoing 'ikc,jkc->ijc', incoming 'kjc,kic->ijc'
+    ref = torch.einsum("ckj,cki->cij", le, ri) if incoming else torch.einsum("cik,cjk->cij", le, ri)
+    np.testing.assert_allclose(got, ref.numpy(), rtol=1e-6, atol=1e-6)
+    ch, i, j = 2, 3, 5
+    if incoming:
+        want = sum(float(c["right"][ch, k, i]) * float(c["left"][ch, k, j]) for k in range(7))
+    else:
+        want = sum(float(c["left"][ch, i, k]) * float(c["right"][ch, j, k]) for k in range(7))
+    assert abs(got[ch, i, j] - want) < 1e-5
+
+
+def test_tm_equation_identities():
+    c = make_pair_case(54, 6, 6, 4, 2)
+    eye = np.broadcast_to(np.eye(6, dtype=np.float32), (2, 6, 6)).copy()
+    # outgoing with right = I returns left; incoming with right = I returns left as well (sum_k I[k,i] left[k,j])
+    np.testing.assert_array_equal(oracle.tm_equation_f32(c["left"], eye, False), c["left"])
+    np.testing.assert_array_equal(oracle.tm_equation_f32(c["left"], eye, True), c["left"])
+    # outgoing with left = I returns right transposed; the two equations are not symmetric in their operands
+    np.testing.assert_array_equal(oracle.tm_equation_f32(eye, c["right"], False), c["right"].transpose(0, 2, 1))
+    np.testing.assert_array_equal(oracle.tm_equation_f32(eye, c["right"], True), c["right"].transpose(0, 2, 1))
+    # incoming(left, right) == outgoing(right^T, left^T)
+    a = oracle.tm_equation_f32(c["left"], c["right"], True)
+    b = oracle.tm_equation_f32(np.ascontiguousarray(c["right"].transpose(0, 2, 1)),
+                               np.ascontiguousarray(c["left"].transpose(0, 2, 1)), False)
+    np.testing.assert_allclose(a, b, rtol=1e-6, atol=1e-6)
+
+
+def test_tm_output_step_matches_torch():
+    c = make_pair_case(55, 3, 4, 8, 5)
+    rng = np.random.Generator(np.random.PCG64(56))
+    center = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    gating_w, gating_b = rng.standard_normal((8, 8)).astype(np.float32), rng.standard_normal(8).astype(np.float32)
+    out_w, out_b = rng.standard_normal((8, 5)).astype(np.float32), rng.standard_normal(8).astype(np.float32)
+    gate, out = oracle.tm_gate_and_out_f32(c["x"], center, gating_w, gating_b, out_w, out_b)
+    t = lambda a: torch.from_numpy(a).double()  # noqa: E731
+    g_ref = torch.nn.functional.linear(t(c["x"]).reshape(-1, 8), t(gating_w), t(gating_b))
+    o_ref = torch.nn.functional.linear(t(center).reshape(-1, 5), t(out_w), t(out_b))
+    np.testing.assert_allclose(gate, g_ref.numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(out, o_ref.numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oracle.tm_last_f32(out, gate), (o_ref * torch.sigmoid(g_ref)).numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_array_equal(oracle.tm_last_f32(out, np.full_like(gate, 100.0)), out)
