@@ -137,6 +137,87 @@ def producer_rates(config, reps=50):
     }
 
 
+def pair_stack_rates(config, reps=20):
+    """Times of the transition and of the four steps of the triangle multiplication (outgoing and incoming equation)
+    at this configuration's pair tensor: n = S residues, 128 pair channels, 128 projected channels, hidden layer 512.
+    Called through the handle-based entry points, asynchronously on torch's stream, hipEvent-bracketed.  Per step:
+    microseconds, algorithmic TFLOP/s (2 flops per multiply-add of the products) and algorithmic GB/s (every operand
+    and result of the step once, intermediates the reference also materialises included)."""
+    import torch
+    from kutacc_amd import capi
+    from kutacc_amd.workloads import CONFIGS
+
+    n = CONFIGS[config]["S"]
+    c_o, c_i, hid = 128, 128, 512
+    rows = n * n
+    g = torch.Generator(device="cuda").manual_seed(11)
+    bf = lambda *sh, scale=1.0: (torch.randn(*sh, device="cuda", generator=g) * scale).to(torch.bfloat16)  # noqa: E731
+    f32 = lambda k: torch.randn(k, device="cuda", generator=g) * 0.5  # noqa: E731
+    x = bf(n, n, c_o)
+    mask = (torch.rand(n, n, device="cuda", generator=g) > 0.1).to(torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+    capi.set_stream(stream)
+    capi.set_blocking(False)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        assert not capi.error_flag()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    res = {"shape": f"pair activation [{n},{n},{c_o}] bf16, c_i={c_i}, transition hidden {hid}"}
+
+    def report(name, t, flops, nbytes):
+        res[name] = {"us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1), "GB/s": round(nbytes / t / 1e9, 1)}
+
+    # transition
+    mid = torch.empty(rows, hid, device="cuda", dtype=torch.bfloat16)
+    out = torch.empty(n, n, c_o, device="cuda", dtype=torch.bfloat16)
+    tr = capi.Transition(x, bf(hid, c_o, scale=c_o ** -0.5), f32(hid), bf(c_o, hid, scale=hid ** -0.5), f32(c_o), mid, out)
+    report("transition", timed(tr.run), 4.0 * rows * c_o * hid, 2.0 * rows * (2 * c_o + 2 * hid))
+    del mid
+    # triangle multiplication
+    keep = [bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i), bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i)]
+    h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]
+    left = torch.empty(c_i, n, n, device="cuda", dtype=torch.bfloat16)
+    right = torch.empty_like(left)
+    gate_scratch = torch.empty_like(left)
+    hx, hm, hl, hr, hgs = capi.tensor(x), capi.tensor(mask), capi.tensor(left), capi.tensor(right), capi.tensor(gate_scratch)
+    pw = capi.TmProjWeights(c_o, c_i, h[0].handle, h[1].handle, h[2].handle, h[3].handle)
+    acts_l = capi.TmActInputs(n, n, hl.handle, hx.handle, hgs.handle)
+    acts_r = capi.TmActInputs(n, n, hr.handle, hx.handle, hgs.handle)
+    capi.kutacc_af2_triangle_multiplication_calc_proj(acts_r, hm, pw, False)
+    t = timed(lambda: capi.kutacc_af2_triangle_multiplication_calc_proj(acts_l, hm, pw, False))
+    report("tm_calc_proj (one side)", t, 4.0 * rows * c_o * c_i, 2.0 * rows * (c_o + c_i + 1))
+    center = torch.empty_like(left)
+    hc = capi.tensor(center)
+    for name, incoming in (("tm_equation outgoing", False), ("tm_equation incoming", True)):
+        t = timed(lambda: capi.kutacc_af2_triangle_multiplication_equation(hc, hl, hr, n, incoming))
+        report(name, t, 2.0 * c_i * n * n * n, 2.0 * 3 * c_i * rows)
+    del gate_scratch
+    ctr = bf(n, n, c_i)
+    gate = torch.empty(n, n, c_o, device="cuda", dtype=torch.bfloat16)
+    keep2 = [bf(c_o, c_o, scale=c_o ** -0.5), f32(c_o), bf(c_o, c_i, scale=c_i ** -0.5), f32(c_o)]
+    h2 = [capi.tensor(keep2[0]), capi.tensor(keep2[1], capi.K_FP32), capi.tensor(keep2[2]), capi.tensor(keep2[3], capi.K_FP32)]
+    lw = capi.TmLinearWeights(c_o, c_i, h2[0].handle, h2[1].handle, h2[2].handle, h2[3].handle)
+    hg, ho, hctr = capi.tensor(gate), capi.tensor(out), capi.tensor(ctr)
+    acts = capi.TmActInputs(n, n, None, hx.handle, None)
+    t = timed(lambda: capi.kutacc_af2_triangle_multiplication_gate_and_out_linear(hg, ho, acts, hctr, lw, False))
+    report("tm_gate_and_out_linear", t, 2.0 * rows * c_o * (c_o + c_i), 2.0 * rows * (3 * c_o + c_i))
+    t = timed(lambda: capi.kutacc_af2_triangle_multiplication_last(ho, hg, n, n, c_o))
+    report("tm_last", t, 0.0, 2.0 * rows * 3 * c_o)
+    capi.set_blocking(True)
+    capi.set_stream(None)
+    res["peaks"] = {"bf16_mfma_TFLOP/s": MFMA_BF16_PEAK_TFLOPS, "hbm_GB/s": HBM_PEAK_GBS}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -147,6 +228,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy: a kernel of known traffic to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run against")
+    ap.add_argument("--pair-stack", action="store_true",
+                    help="also time the transition and the triangle-multiplication steps at this configuration's pair "
+                         "tensor and report them in a \"pair_stack\" object")
     ap.add_argument("--producers", action="store_true",
                     help="also time the LayerNorm and pair-bias producer kernels at this configuration's pair tensor "
                          "and report their HBM rates in a \"producers\" object")
@@ -230,6 +314,8 @@ def main():
     }
     if a.producers:
         rec["producers"] = producer_rates(a.config)
+    if a.pair_stack:
+        rec["pair_stack"] = pair_stack_rates(a.config)
     print(json.dumps(rec))
 
 

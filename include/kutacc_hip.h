@@ -193,6 +193,18 @@ typedef struct kutacc_hip_gemm_args {
 
 kutacc_export int kutacc_hip_gemm(const kutacc_hip_gemm_args_t *args, void *stream);
 
+/*
+ * Transition: out = relu(x . w1^T + b1) . w2^T + b2 over `rows` dense rows (x, out [rows, c_o]; w1 [c_i, c_o] and
+ * w2 [c_o, c_i] stored [out, in]; b1 fp32 [c_i], b2 fp32 [c_o]).  Replaces kutacc::transition_kernel (reference
+ * src/attention/transition.cpp:21-39).  path AUTO: one kernel that keeps the hidden layer on chip when c_o is 128
+ * or 256 and c_i a multiple of 64 (`intermediate` is then not touched and may be NULL), else two kutacc_hip_gemm
+ * launches through `intermediate` ([rows, c_i], required); GENERIC: always the two launches; FUSED: the one kernel
+ * or KUTACC_HIP_EUNSUPPORTED.
+ */
+kutacc_export int kutacc_hip_transition(const void *x, const void *w1, const float *b1, const void *w2, const float *b2,
+                                        void *intermediate, void *out, int64_t rows, int64_t c_o, int64_t c_i,
+                                        int32_t dtype, int32_t path, void *stream);
+
 /* out[i, j, c] *= sigmoid(gate[i, j, c]) for c < size; element (i, j, c) of either tensor at i*stride0 + j*stride1 + c.
  * The element-wise pass of kutacc::last (reference src/attention/triangle_multiplication.cpp:129-150). */
 kutacc_export int kutacc_hip_sigmoid_gate_rows(void *out, int64_t out_stride0, int64_t out_stride1, const void *gate,

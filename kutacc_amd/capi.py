@@ -119,7 +119,7 @@ DECLARED_SYMBOLS = [
     "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_global_attention", "kutacc_af2_layernorm",
     "kutacc_af2_linear", "kutacc_af2_transition", "kutacc_af2_triangle_multiplication_calc_proj",
     "kutacc_af2_triangle_multiplication_equation", "kutacc_af2_triangle_multiplication_gate_and_out_linear",
-    "kutacc_af2_triangle_multiplication_last", "kutacc_hip_gemm", "kutacc_hip_sigmoid_gate_rows",
+    "kutacc_af2_triangle_multiplication_last", "kutacc_hip_gemm", "kutacc_hip_sigmoid_gate_rows", "kutacc_hip_transition",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
@@ -173,6 +173,8 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_gemm.restype = ctypes.c_int
     L.kutacc_hip_sigmoid_gate_rows.argtypes = [_vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp]
     L.kutacc_hip_sigmoid_gate_rows.restype = ctypes.c_int
+    L.kutacc_hip_transition.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]
+    L.kutacc_hip_transition.restype = ctypes.c_int
     L.kutacc_af2_transition.argtypes = [ctypes.POINTER(TransActInputs), ctypes.POINTER(TransWeights), _vp]
     L.kutacc_af2_transition.restype = None
     L.kutacc_af2_triangle_multiplication_calc_proj.argtypes = [ctypes.POINTER(TmActInputs), _vp,

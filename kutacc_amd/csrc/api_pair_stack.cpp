@@ -92,6 +92,42 @@ int kutacc_hip_sigmoid_gate_rows(void *out, int64_t out_stride0, int64_t out_str
                                             kutacc_api::stream_or_default(stream));
 }
 
+int kutacc_hip_transition(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *intermediate,
+                          void *out, int64_t rows, int64_t c_o, int64_t c_i, int32_t dtype, int32_t path, void *stream)
+{
+    if (!x || !w1 || !b1 || !w2 || !b2 || !out || rows <= 0 || c_o <= 0 || c_i <= 0 || dtype != KUTACC_DTYPE_BF16) {
+        return KUTACC_HIP_EINVAL;
+    }
+    hipStream_t s = kutacc_api::stream_or_default(stream);
+    const bool fused_ok = kutacc_launch::transition_fused_supports(rows, c_o, c_i, x, w1, b1, w2, b2, out);
+    if (path == KUTACC_HIP_PATH_FUSED && !fused_ok) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    if (path != KUTACC_HIP_PATH_GENERIC && fused_ok) {
+        return kutacc_launch::transition_fused(x, w1, b1, w2, b2, out, rows, c_o, c_i, s);
+    }
+    if (!intermediate) {
+        return KUTACC_HIP_EINVAL;
+    }
+    kutacc_hip_gemm_args_t g = blank_gemm();
+    g.m = rows, g.n = c_i, g.k = c_o;
+    g.a = x, g.a_stride_m = c_o, g.a_stride_k = 1;
+    g.b = w1, g.b_stride_n = c_o, g.b_stride_k = 1;
+    g.c = intermediate, g.c_stride_m = c_i;
+    g.bias = b1, g.bias_axis = 1, g.relu = 1;
+    int rc = kutacc_launch::pair_gemm(g, s);
+    if (rc != 0) {
+        return rc;
+    }
+    g = blank_gemm();
+    g.m = rows, g.n = c_o, g.k = c_i;
+    g.a = intermediate, g.a_stride_m = c_i, g.a_stride_k = 1;
+    g.b = w2, g.b_stride_n = c_i, g.b_stride_k = 1;
+    g.c = out, g.c_stride_m = c_o;
+    g.bias = b2, g.bias_axis = 1;
+    return kutacc_launch::pair_gemm(g, s);
+}
+
 void kutacc_af2_transition(kutacc_af2_trans_act_inputs_t *trans_inputs_ptr, kutacc_af2_trans_weights_t *trans_weights_ptr,
                            kutacc_tensor_h out)
 {
@@ -121,24 +157,9 @@ void kutacc_af2_transition(kutacc_af2_trans_act_inputs_t *trans_inputs_ptr, kuta
         return;
     }
     hipStream_t s = kutacc_api::default_stream();
-    const int64_t rows = batch * n_res;
     // the reference's views: every tensor dense with its channel count as the row stride (transition.cpp:31-38)
-    kutacc_hip_gemm_args_t g = blank_gemm();
-    g.m = rows, g.n = c_i, g.k = c_o;
-    g.a = x.data, g.a_stride_m = c_o, g.a_stride_k = 1;
-    g.b = w1.data, g.b_stride_n = c_o, g.b_stride_k = 1;
-    g.c = mid.data, g.c_stride_m = c_i;
-    g.bias = (const float *)b1.data, g.bias_axis = 1, g.relu = 1;
-    int rc = kutacc_launch::pair_gemm(g, s);
-    if (rc == 0) {
-        g = blank_gemm();
-        g.m = rows, g.n = c_o, g.k = c_i;
-        g.a = mid.data, g.a_stride_m = c_i, g.a_stride_k = 1;
-        g.b = w2.data, g.b_stride_n = c_i, g.b_stride_k = 1;
-        g.c = o.data, g.c_stride_m = c_o;
-        g.bias = (const float *)b2.data, g.bias_axis = 1;
-        rc = kutacc_launch::pair_gemm(g, s);
-    }
+    const int rc = kutacc_hip_transition(x.data, w1.data, (const float *)b1.data, w2.data, (const float *)b2.data, mid.data,
+                                         o.data, batch * n_res, c_o, c_i, KUTACC_DTYPE_BF16, KUTACC_HIP_PATH_AUTO, s);
     report("kutacc_af2_transition", kutacc_api::finish(rc, s));
 }
 

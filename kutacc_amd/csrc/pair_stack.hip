@@ -278,6 +278,177 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
     }
 }
 
+// Transition with the hidden layer kept on chip: out = relu(x . W1^T + b1) . W2^T + b2 for row tiles of x
+// (reference src/attention/transition.cpp:31-38 runs two GEMMs through a [rows, c_i] intermediate; with
+// c_i = 4 c_o that intermediate is four fifths of the HBM traffic).  A wave owns RB blocks of 32 rows, whose
+// input fragments stay in registers; the workgroup streams the two weight matrices through LDS in slices
+// of 64 hidden units, double buffered, one barrier per slice.  Both products are formed transposed
+// (MFMA rows = hidden units, then output channels; columns = rows of x): the accumulators of the first,
+// after bias, ReLU and rounding to bf16 (the reference's rounding point: its intermediate is a bf16
+// tensor), are the B operand of the second without leaving the registers.  For that the lane that feeds
+// MFMA row i with a row of W1 takes hidden unit sigma(i) (bits 2 and 3 of i swapped), which makes the
+// eight values a lane holds per k-step consecutive hidden units.
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+__device__ __forceinline__ int sigma_row(int r) { return (r & 0x13) | ((r & 4) << 1) | ((r & 8) >> 1); }
+
+template <int CO, int RB>
+__global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *__restrict__ x,
+                                                                 const bf16_t *__restrict__ w1,
+                                                                 const float *__restrict__ b1,
+                                                                 const bf16_t *__restrict__ w2,
+                                                                 const float *__restrict__ b2, bf16_t *__restrict__ out,
+                                                                 int64_t rows, int c_i)
+{
+    constexpr int KS = CO / 16; // k-steps of the first product
+    constexpr int CP = CO / 64; // 64-column panels across a row of x or W1
+    constexpr int CB = CO / 32; // 32-channel blocks of the output
+    constexpr int W1_PANELS = 2 * CP, STAGE_PANELS = W1_PANELS + CB, PPW = STAGE_PANELS / 4;
+    extern __shared__ uint4 lds[]; // [2 stages][STAGE_PANELS][256 slots], one private panel per wave, b1 as fp32
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, g = lane >> 5, sr = sigma_row(r);
+    uint4 *xpanel = lds + 2 * STAGE_PANELS * 256 + wave * 256;
+    float *b1s = reinterpret_cast<float *>(lds + 2 * STAGE_PANELS * 256 + 4 * 256);
+    for (int i = tid; i < c_i; i += 256) {
+        b1s[i] = b1[i]; // visible after the first barrier of the slice loop
+    }
+
+    int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (32 * RB);
+    const bool active = row0 < rows;
+    if (!active) {
+        row0 = rows - 1; // keeps every address valid; nothing is stored
+    }
+    const int last_local = (int)((rows - row0 < 32 * RB ? rows - row0 : 32 * RB) - 1);
+    const bf16_t *xb = x + row0 * CO;
+
+    auto fetch = [&](int jc, PanelRegs *wr) {
+        const int h0 = jc * 64;
+#pragma unroll
+        for (int i = 0; i < PPW; ++i) {
+            const int pnl = wave * PPW + i;
+            if (pnl < W1_PANELS) {
+                wr[i] = panel_load(w1 + (int64_t)(h0 + 32 * (pnl / CP)) * CO, CO, 0, 31, (pnl % CP) * 64, lane);
+            } else {
+                wr[i] = panel_load(w2 + (int64_t)((pnl - W1_PANELS) * 32) * c_i, c_i, 0, 31, h0, lane);
+            }
+        }
+    };
+    PanelRegs wr[PPW];
+    fetch(0, wr);
+
+    bf16x8 xf[RB][KS];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+        for (int cp = 0; cp < CP; ++cp) {
+            const PanelRegs t = panel_load(xb, CO, rb * 32, last_local, cp * 64, lane);
+            panel_store(xpanel, lane, t);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                xf[rb][cp * 4 + k] = as_bf16x8(xpanel[panel_slot(r, 2 * k + g)]);
+            }
+        }
+    }
+
+    f32x16 oacc[RB][CB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            oacc[rb][cb] = zero16();
+        }
+    }
+
+    const int NJ = c_i / 64;
+    for (int jc = 0; jc < NJ; ++jc) {
+        uint4 *stage = lds + (jc & 1) * STAGE_PANELS * 256;
+#pragma unroll
+        for (int i = 0; i < PPW; ++i) {
+            panel_store(stage + (wave * PPW + i) * 256, lane, wr[i]);
+        }
+        __syncthreads();
+        if (jc + 1 < NJ) {
+            fetch(jc + 1, wr);
+        }
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+            f32x16 hacc[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                hacc[rb] = zero16();
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8 a = as_bf16x8(stage[(hb * CP + ks / 4) * 256 + panel_slot(sr, 2 * (ks % 4) + g)]);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    hacc[rb] = mfma(a, xf[rb][ks], hacc[rb]);
+                }
+            }
+            // + b1, ReLU, round to bf16 pairwise (the pair form maps onto one conversion instruction)
+            const float *bp = b1s + jc * 64 + 32 * hb + 8 * g;
+            bf16x8 hf[RB][2];
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                const f32x4 ba = *reinterpret_cast<const f32x4 *>(bp + 16 * s2);
+                const f32x4 bb = *reinterpret_cast<const f32x4 *>(bp + 16 * s2 + 4);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    bf16x2 w[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float b0 = q < 2 ? ba[2 * q] : bb[2 * q - 4], b1v = q < 2 ? ba[2 * q + 1] : bb[2 * q - 3];
+                        const f32x2 pr = {fmaxf(hacc[rb][8 * s2 + 2 * q] + b0, 0.f), fmaxf(hacc[rb][8 * s2 + 2 * q + 1] + b1v, 0.f)};
+                        w[q] = __builtin_convertvector(pr, bf16x2);
+                    }
+                    const bf16x8 all = {w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
+                    hf[rb][s2] = all;
+                }
+            }
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                    const bf16x8 a2 = as_bf16x8(stage[(W1_PANELS + cb) * 256 + panel_slot(r, 2 * (2 * hb + s2) + g)]);
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        oacc[rb][cb] = mfma(a2, hf[rb][s2], oacc[rb][cb]);
+                    }
+                }
+            }
+        }
+    }
+
+    // accumulators (+ b2) -> bf16 through the private panel, 64 channels at a time, out as whole 128-byte runs
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+        for (int half = 0; half < CB / 2; ++half) {
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(b2 + (2 * half + n) * 32 + 8 * a + 4 * g);
+                    bf16x4 ov;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        ov[c] = (bf16_t)(oacc[rb][2 * half + n][4 * a + c] + bv[c]);
+                    }
+                    *(reinterpret_cast<bf16x4 *>(xpanel + panel_slot(r, n * 4 + a)) + g) = ov;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int prow = 8 * i + (lane >> 3);
+                const uint4 v = xpanel[panel_slot(prow, lane & 7)];
+                if (active && rb * 32 + prow <= last_local) {
+                    *reinterpret_cast<uint4 *>(out + (row0 + rb * 32 + prow) * CO + half * 64 + (lane & 7) * 8) = v;
+                }
+            }
+        }
+    }
+}
+
 // Any strides, any sizes: one thread per element of C, same epilogues and rounding points.
 __global__ __launch_bounds__(256) void pair_gemm_scalar_kernel(const GemmParams p)
 {
@@ -381,9 +552,52 @@ hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
     pair_gemm_kernel<AM, BM, G><<<dim3((unsigned)blocks), 256, GEMM_LDS, stream>>>(p);
     return hipGetLastError();
 }
+constexpr int MAX_HIDDEN = 2048; // hidden units whose bias fits next to the weight stages in LDS
+
+template <int CO, int RB>
+hipError_t launch_transition(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
+                             int64_t rows, int c_i, hipStream_t stream)
+{
+    constexpr int STAGE_PANELS = 2 * (CO / 64) + CO / 32;
+    const size_t lds_bytes = (size_t)(2 * STAGE_PANELS + 4) * 4096 + (size_t)c_i * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 (2 * STAGE_PANELS + 4) * 4096 + MAX_HIDDEN * (int)sizeof(float));
+        if (e != hipSuccess) {
+            return e;
+        }
+        configured = true;
+    }
+    const int64_t blocks = (rows + 128 * RB - 1) / (128 * RB);
+    transition_fused_kernel<CO, RB><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(
+        (const bf16_t *)x, (const bf16_t *)w1, b1, (const bf16_t *)w2, b2, (bf16_t *)out, rows, c_i);
+    return hipGetLastError();
+}
 } // namespace
 
 namespace kutacc_launch {
+
+bool transition_fused_supports(int64_t rows, int64_t c_o, int64_t c_i, const void *x, const void *w1, const float *b1,
+                               const void *w2, const float *b2, const void *out)
+{
+    return (c_o == 128 || c_o == 256) && c_i >= 64 && c_i % 64 == 0 && c_i <= MAX_HIDDEN && rows > 0 &&
+           rows <= ((int64_t)1 << 31) * 64 && aligned16(x) && aligned16(w1) && aligned16(b1) && aligned16(w2) &&
+           aligned16(b2) && aligned16(out);
+}
+
+int transition_fused(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
+                     int64_t rows, int64_t c_o, int64_t c_i, hipStream_t stream)
+{
+    if (!transition_fused_supports(rows, c_o, c_i, x, w1, b1, w2, b2, out)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    kutacc_prof::KernelTimer t("transition_fused_kernel", 4.0 * (double)rows * (double)c_o * (double)c_i, stream);
+    const hipError_t e = c_o == 128 ? launch_transition<128, 2>(x, w1, b1, w2, b2, out, rows, (int)c_i, stream)
+                                    : launch_transition<256, 1>(x, w1, b1, w2, b2, out, rows, (int)c_i, stream);
+    return kutacc_hip_status(e);
+}
 
 int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
 {

@@ -144,28 +144,56 @@ def transition_case(seed, batch, n_res, c_o, c_i):
                 b2=rng.standard_normal(c_o).astype(np.float32) * 0.5)
 
 
-def run_transition(torch, c):
+def run_transition(torch, c, path=None):
+    """path None: the handle-based entry point; else kutacc_hip_transition with that path."""
     batch, n_res, c_o = c["x"].shape
     c_i = c["w1"].shape[0]
-    mid = torch.zeros((batch * n_res, c_i), dtype=torch.bfloat16, device="cuda")
+    mid = torch.full((batch * n_res, c_i), -5.0, dtype=torch.bfloat16, device="cuda")
     out = torch.zeros((batch, n_res, c_o), dtype=torch.bfloat16, device="cuda")
-    op = capi.Transition(dev(torch, c["x"]), dev(torch, c["w1"]), dev(torch, c["b1"], torch.float32), dev(torch, c["w2"]),
-                         dev(torch, c["b2"], torch.float32), mid, out)
-    op.run()
-    assert not capi.error_flag()
+    t = [dev(torch, c["x"]), dev(torch, c["w1"]), dev(torch, c["b1"], torch.float32), dev(torch, c["w2"]),
+         dev(torch, c["b2"], torch.float32)]
+    if path is None:
+        op = capi.Transition(*t, mid, out)
+        op.run()
+        assert not capi.error_flag()
+    else:
+        rc = capi.lib().kutacc_hip_transition(*[a.data_ptr() for a in t], mid.data_ptr(), out.data_ptr(), batch * n_res,
+                                              c_o, c_i, capi.K_BF16, path, None)
+        torch.cuda.synchronize()
+        assert rc == 0, rc
     return out, mid
 
 
-@pytest.mark.parametrize("shape", [(2, 37, 128, 512), (3, 50, 256, 1024), (1, 9, 24, 40), (2, 5, 6, 10)])
-def test_transition_small(torch_cuda, shape):
-    """Pair (128 -> 512) and MSA (256 -> 1024) channel counts at ragged row counts, and channel counts that run on
-    the scalar kernel."""
+@pytest.mark.parametrize("shape", [(2, 37, 128, 512), (3, 50, 256, 1024), (1, 300, 128, 64), (1, 9, 24, 40), (2, 5, 6, 10)])
+@pytest.mark.parametrize("path", [None, capi.PATH_GENERIC], ids=["entry point", "two launches"])
+def test_transition_small(torch_cuda, shape, path):
+    """Pair (128 -> 512) and MSA (256 -> 1024) channel counts at ragged row counts (the one-kernel form through the
+    entry point, the two-GEMM form when forced), and channel counts that only the GEMM kernels take."""
     from oracle import oracle
     c = transition_case(300 + shape[2], *shape)
-    out, mid = run_transition(torch_cuda, c)
+    out, mid = run_transition(torch_cuda, c, path)
     ref, ref_mid = oracle.transition_f32(c["x"].reshape(-1, shape[2]), c["w1"], c["b1"], c["w2"], c["b2"], return_mid=True)
-    helpers.assert_within(helpers.to_numpy(mid), ref_mid, GEMM_TOL(ref_mid), "hidden layer")
+    one_kernel = path is None and shape[2] in (128, 256)
+    if one_kernel:
+        assert bool((mid == -5.0).all()), "the one-kernel form must leave the intermediate tensor alone"
+    else:
+        helpers.assert_within(helpers.to_numpy(mid), ref_mid, GEMM_TOL(ref_mid), "hidden layer")
     helpers.check_close(helpers.to_numpy(out).reshape(ref.shape), ref, "bf16", f"transition {shape}")
+
+
+def test_transition_forced_paths(torch_cuda):
+    c = transition_case(305, 1, 70, 128, 256)
+    a, _ = run_transition(torch_cuda, c, capi.PATH_FUSED)
+    b, _ = run_transition(torch_cuda, c, capi.PATH_GENERIC)
+    # same rounding points (bf16 hidden layer, fp32 accumulation): the two forms differ by summation order only
+    helpers.assert_within(helpers.to_numpy(a), helpers.to_numpy(b), 1e-2 + 1e-2 * np.abs(helpers.to_numpy(b)), "fused vs two launches")
+    t = torch_cuda.zeros(64, dtype=torch_cuda.bfloat16, device="cuda")
+    f = torch_cuda.zeros(64, dtype=torch_cuda.float32, device="cuda")
+    L = capi.lib()
+    assert L.kutacc_hip_transition(t.data_ptr(), t.data_ptr(), f.data_ptr(), t.data_ptr(), f.data_ptr(), None, t.data_ptr(),
+                                   2, 8, 8, capi.K_BF16, capi.PATH_FUSED, None) == capi.EUNSUPPORTED
+    assert L.kutacc_hip_transition(t.data_ptr(), t.data_ptr(), f.data_ptr(), t.data_ptr(), f.data_ptr(), None, t.data_ptr(),
+                                   2, 8, 8, capi.K_BF16, capi.PATH_AUTO, None) == capi.EINVAL  # needs the intermediate
 
 
 def test_transition_full_pair_size(torch_cuda):
