@@ -8,9 +8,9 @@
 // 64: each wave fetches a quarter of both operand tiles with whole-cache-line loads one step ahead,
 // parks it in registers while the current step is multiplied, and stores it into the other half of a
 // double-buffered LDS tile in MFMA fragment order (one barrier per step).  Operands may be stored
-// K-major (rows contiguous in k; 16-byte LDS writes) or M-major (the "incoming" triangle equation
-// contracts over the leading index of both operands; the transposition happens in the LDS write, two
-// bytes at a time).  The product is formed transposed (MFMA rows = columns of C) so that every lane
+// K-major (rows contiguous in k) or M-major (the "incoming" triangle equation contracts over the leading
+// index of both operands; those tiles are transposed in registers, eight lanes at a time, on their way
+// into LDS).  The product is formed transposed (MFMA rows = columns of C) so that every lane
 // ends up with four consecutive columns of its own row of C; the tile is rounded to bf16 into LDS and
 // leaves as whole rows of 256 bytes.
 //
@@ -94,21 +94,44 @@ __device__ __forceinline__ PanelRegs load_mmajor(const bf16_t *base, int64_t ld,
     return p;
 }
 
-// transposing store of what load_mmajor fetched: operand tile rows mrow0.., k columns kcol0..
+// Transposing store of what load_mmajor fetched: operand tile rows mrow0.., k columns kcol0...
+// Register i of lane (kk, mc) holds 8 consecutive m (8mc..8mc+7) of row k = 8i + kk; the fragment layout wants
+// 8 consecutive k of one m in a lane.  That is an 8 x 8 transposition of 16-bit elements over the eight lanes
+// that share mc (lane bits 3, 4, 5), done in three exchange steps in registers: halves of a dword against
+// lane bit 3 (row rotation by 8 + byte permute), dword pairs against lane bit 4 (v_permlane16_swap) and
+// against lane bit 5 (v_permlane32_swap).  Afterwards lane (kk, mc) holds k = 8i..8i+7 of m = 8mc + kk, one
+// 16-byte slot.
+__device__ __forceinline__ uint4 transpose8x8_lanes(uint4 v, uint32_t sel)
+{
+    uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t partner = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d[j], 0x128, 0xf, 0xf, false); // lane ^ 8
+        d[j] = __builtin_amdgcn_perm(partner, d[j], sel);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j += 2) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(d[j], d[j + 1], false, false);
+        d[j] = sw[0], d[j + 1] = sw[1];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(d[j], d[j + 2], false, false);
+        d[j] = sw[0], d[j + 2] = sw[1];
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
 __device__ __forceinline__ void store_mmajor(uint4 *operand, int mrow0, int kcol0, int lane, const PanelRegs &p)
 {
-    uint16_t *o16 = reinterpret_cast<uint16_t *>(operand);
+    // even lanes of bit 3 keep their low halves and take the partner's low halves on top; odd ones the high halves
+    const uint32_t sel = (lane & 8) ? 0x03020706u : 0x05040100u;
+    const int row = mrow0 + (lane & 7) * 8 + (lane >> 3);
+    uint4 *dst = operand + (row >> 5) * 256;
     const uint4 regs[4] = {p.r0, p.r1, p.r2, p.r3};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int k = kcol0 + 8 * i + (lane >> 3);
-        const uint32_t w[4] = {regs[i].x, regs[i].y, regs[i].z, regs[i].w};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int row = mrow0 + (lane & 7) * 8 + e;
-            const int slot = (row >> 5) * 256 + panel_slot(row & 31, k >> 3);
-            o16[slot * 8 + (k & 7)] = (uint16_t)(e & 1 ? w[e >> 1] >> 16 : w[e >> 1] & 0xffffu);
-        }
+        dst[panel_slot(row & 31, (kcol0 >> 3) + i)] = transpose8x8_lanes(regs[i], sel);
     }
 }
 
