@@ -1416,8 +1416,10 @@ int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t strea
     }
 }
 
+// out[M, N] = a[M, K] . w[N, K]^T + bias with K = C and N a multiple of 128 (one grid row per 128-feature slab)
 template <int C>
-int launch_output_projection(const kutacc_hip_attention_args_t &a, hipStream_t stream)
+int launch_output_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld,
+                             int64_t M, int64_t N, hipStream_t stream)
 {
     auto kern = output_projection_kernel<C>;
     const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16 + 4 * 4096;
@@ -1425,16 +1427,14 @@ int launch_output_projection(const kutacc_hip_attention_args_t &a, hipStream_t s
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
         return rc;
     }
-    const int64_t M = a.batch * a.seq_len;
     const int64_t tiles = (M + 31) / 32;
     // two resident workgroups per CU, each wave with an equal share of the rows
     int64_t gx = (tiles + 3) / 4;
     const int64_t cap = (int64_t)num_cus() * 2;
     gx = gx > cap ? cap : gx;
     const int64_t rpw = ((M + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
-    kern<<<dim3((unsigned)gx, (unsigned)(C / 128)), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a.avg, a.avg_stride_s, (const bf16_t *)a.output_w, a.output_b, (bf16_t *)a.out, a.out_ld, M,
-        (int)rpw);
+    kern<<<dim3((unsigned)gx, (unsigned)(N / 128)), 256, lds_bytes, stream>>>(
+        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)rpw);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -1535,7 +1535,30 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
         }
     }
     kutacc_prof::KernelTimer t("output_projection_kernel", 2.0 * BS * C * C, stream);
-    return (C == 128) ? launch_output_projection<128>(a, stream) : launch_output_projection<256>(a, stream);
+    const int64_t M = a.batch * a.seq_len;
+    return (C == 128) ? launch_output_projection<128>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out, a.out_ld, M, C, stream)
+                      : launch_output_projection<256>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out, a.out_ld, M, C, stream);
+}
+
+// The attention's output-projection kernel on its own: out[m, n] = sum_k a[m, k] * w[n, k] + bias[n] for rows of
+// 128 or 256 input features (w dense [n, k]) and n a multiple of 128.  HBM-bound; every row is read and written
+// once per 128-feature slab of the output.
+bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
+                             int64_t m, int64_t n, int64_t k)
+{
+    return (k == 128 || k == 256) && n > 0 && n % 128 == 0 && n / 128 <= 65535 && m > 0 && m <= INT32_MAX - 64 && bias &&
+           a_ld % 8 == 0 && out_ld % 8 == 0 && aligned(a, 16) && aligned(w, 16) && aligned(bias, 16) && aligned(out, 16);
+}
+
+int row_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld, int64_t m,
+                   int64_t n, int64_t k, hipStream_t stream)
+{
+    if (!row_projection_supports(a, a_ld, w, bias, out, out_ld, m, n, k)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    kutacc_prof::KernelTimer t("output_projection_kernel", 2.0 * (double)m * (double)n * (double)k, stream);
+    return k == 128 ? launch_output_projection<128>(a, a_ld, w, bias, out, out_ld, m, n, stream)
+                    : launch_output_projection<256>(a, a_ld, w, bias, out, out_ld, m, n, stream);
 }
 
 } // namespace kutacc_launch

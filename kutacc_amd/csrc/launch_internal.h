@@ -20,6 +20,11 @@ int gemm_nt(int32_t dtype, const void *a, int64_t lda, const void *w, int64_t ld
 bool fused_attention_supports(const kutacc_hip_attention_args_t &args);
 int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream);
 
+bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
+                             int64_t m, int64_t n, int64_t k);
+int row_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld, int64_t m,
+                   int64_t n, int64_t k, hipStream_t stream);
+
 // global_attention.hip
 int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);
 

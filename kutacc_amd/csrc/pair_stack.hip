@@ -657,6 +657,12 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
     } else if (g.path == KUTACC_HIP_PATH_FUSED && !mfma_ok) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
+    // rows of 128 or 256 features against a dense weight matrix: the attention's output-projection kernel keeps
+    // the weight slab in LDS and streams the rows, which suits these HBM-bound shapes better than square tiles
+    if (mfma_ok && !gated && !am && !bm && g.batches == 1 && g.bias_axis == 1 && !g.relu && g.b_stride_n == g.k &&
+        kutacc_launch::row_projection_supports(g.a, g.a_stride_m, g.b, g.bias, g.c, g.c_stride_m, g.m, g.n, g.k)) {
+        return kutacc_launch::row_projection(g.a, g.a_stride_m, g.b, g.bias, g.c, g.c_stride_m, g.m, g.n, g.k, stream);
+    }
     const double flops = 2.0 * (double)g.m * (double)g.n * (double)g.k * (double)g.batches * (gated ? 2.0 : 1.0);
     if (!mfma_ok) {
         const int64_t total = g.m * g.n * g.batches;
