@@ -212,6 +212,19 @@ def pair_stack_rates(config, reps=20):
     report("tm_gate_and_out_linear", t, 2.0 * rows * c_o * (c_o + c_i), 2.0 * rows * (3 * c_o + c_i))
     t = timed(lambda: capi.kutacc_af2_triangle_multiplication_last(ho, hg, n, n, c_o))
     report("tm_last", t, 0.0, 2.0 * rows * 3 * c_o)
+    # whole triangle-attention block (LayerNorm + pair bias, mask bias, attention, residual), both orientations
+    heads = c_o // 32
+    wts = [bf(c_o, c_o, scale=c_o ** -0.5) for _ in range(5)]
+    blk_args = (x.clone(), mask, torch.ones(c_o, device="cuda"), torch.zeros(c_o, device="cuda"),
+                bf(heads, c_o, scale=c_o ** -0.5), wts[0], wts[1], wts[2], wts[3], torch.ones(c_o, device="cuda"), wts[4],
+                torch.zeros(c_o, device="cuda"), heads)
+    attn_flops = 10.0 * rows * c_o * c_o + 4.0 * rows * n * c_o + 2.0 * rows * c_o * heads
+    for name, ending in (("triangle_attention_block starting node", False), ("triangle_attention_block ending node", True)):
+        blk = capi.TriangleAttentionBlock(*blk_args, ending)
+
+        def run_blk():
+            assert blk.run(stream) == 0
+        report(name, timed(run_blk), attn_flops, 2.0 * rows * (2 * c_o + 1))
     capi.set_blocking(True)
     capi.set_stream(None)
     res["peaks"] = {"bf16_mfma_TFLOP/s": MFMA_BF16_PEAK_TFLOPS, "hbm_GB/s": HBM_PEAK_GBS}

@@ -211,6 +211,60 @@ kutacc_export int kutacc_hip_sigmoid_gate_rows(void *out, int64_t out_stride0, i
                                                int64_t gate_stride0, int64_t gate_stride1, int64_t n0, int64_t n1,
                                                int64_t size, int32_t dtype, void *stream);
 
+/* ---- between the operators: what a caller of the reference does in its framework, here on the device ---- */
+
+/* kutacc_hip_pair_bias reading the pair tensor transposed: output row (i, j) (of nb[h, i, j] and of z_norm[i, j, :])
+ * is computed from z[j, i, :], z dense [rows_j, rows_i, c_z].  This is the "ending node" orientation of triangle
+ * attention without a separate pass that swaps the axes of z. */
+kutacc_export int kutacc_hip_pair_bias_transposed(const void *z, const float *gamma, const float *beta, const void *w,
+                                                  void *nb, void *z_norm, int64_t rows_i, int64_t rows_j, int64_t c_z,
+                                                  int64_t nheads, float eps, int32_t dtype, void *stream);
+
+/* bias[i, j] = 1e9 * (mask[i, j] - 1), formed as one fp32 multiply-add (the convention of reference
+ * src/attention/global_attention.cpp:120-121) and rounded to `dtype`; dense [n0, n1].  transposed != 0 reads
+ * mask[j, i] from a dense [n1, n0] mask.  The result is the `bias` argument of kutacc_af2_gating_attention. */
+kutacc_export int kutacc_hip_mask_bias(const void *mask, void *bias, int64_t n0, int64_t n1, int32_t transposed,
+                                       int32_t dtype, void *stream);
+
+/* out[j, i, :] = in[i, j, :] for dense in [n0, n1, inner], out [n1, n0, inner]; in != out. */
+kutacc_export int kutacc_hip_swap_leading_axes(const void *in, void *out, int64_t n0, int64_t n1, int64_t inner,
+                                               int32_t dtype, void *stream);
+
+/* acc[i, j, :] += delta[i, j, :], or delta[j, i, :] (delta dense [n1, n0, inner]) when swapped != 0; fp32 sum. */
+kutacc_export int kutacc_hip_residual_add(void *acc, const void *delta, int64_t n0, int64_t n1, int64_t inner,
+                                          int32_t swapped, int32_t dtype, void *stream);
+
+/*
+ * One triangle-attention block of the pair stack, in place:
+ *   pair_act += gating_attention(input = LN(pair_act), nonbatched_bias = LN(pair_act) . bias_w^T, bias = 1e9*(pair_mask-1))
+ * around the starting node (ending_node == 0: row i attends over j) or the ending node (ending_node != 0: the same
+ * on the transposed pair tensor, result transposed back).  Four device passes on `stream`: LayerNorm + pair-bias
+ * projection (one read of pair_act), mask bias, the attention operator, residual update.  bf16, head_size 32,
+ * c_z = nheads * 32 in {128, 256}, n_res <= 1024 (the shapes of the MFMA attention kernels; otherwise
+ * KUTACC_HIP_EUNSUPPORTED).  `workspace`: device memory, 256-byte aligned, at least
+ * kutacc_hip_triangle_attention_workspace(n_res, nheads) bytes; contents unspecified afterwards.
+ */
+typedef struct kutacc_hip_triangle_attention_args {
+    int64_t n_res;
+    int64_t nheads;
+    int32_t dtype;       /* KUTACC_DTYPE_BF16 */
+    int32_t ending_node; /* 0 starting node, 1 ending node */
+    void *pair_act;        /* [n_res, n_res, c_z], updated in place */
+    const void *pair_mask; /* [n_res, n_res], 1 = valid, 0 = padding */
+    const float *ln_gamma; /* fp32 [c_z] */
+    const float *ln_beta;  /* fp32 [c_z] */
+    float ln_eps;
+    int32_t reserved;
+    const void *bias_w;    /* [nheads, c_z] pair-bias projection, stored [out, in] */
+    const void *query_w, *key_w, *value_w, *gating_w, *output_w; /* [c_z, c_z] stored [out, in] */
+    const float *gating_b, *output_b;                             /* fp32 [c_z] */
+    void *workspace;
+    int64_t workspace_bytes;
+} kutacc_hip_triangle_attention_args_t;
+
+kutacc_export int64_t kutacc_hip_triangle_attention_workspace(int64_t n_res, int64_t nheads);
+kutacc_export int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *args, void *stream);
+
 /* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.

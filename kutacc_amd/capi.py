@@ -114,12 +114,25 @@ class TmLinearWeights(ctypes.Structure):
                 ("output_proj_b", _vp)]
 
 
+class HipTriangleAttentionArgs(ctypes.Structure):
+    """kutacc_hip_triangle_attention_args_t"""
+    _fields_ = [
+        ("n_res", _i64), ("nheads", _i64), ("dtype", _i32), ("ending_node", _i32),
+        ("pair_act", _vp), ("pair_mask", _vp), ("ln_gamma", _vp), ("ln_beta", _vp), ("ln_eps", ctypes.c_float),
+        ("reserved", _i32), ("bias_w", _vp),
+        ("query_w", _vp), ("key_w", _vp), ("value_w", _vp), ("gating_w", _vp), ("output_w", _vp),
+        ("gating_b", _vp), ("output_b", _vp), ("workspace", _vp), ("workspace_bytes", _i64),
+    ]
+
+
 # every symbol the two public headers declare; tests check that the library exports all of them
 DECLARED_SYMBOLS = [
     "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_global_attention", "kutacc_af2_layernorm",
     "kutacc_af2_linear", "kutacc_af2_transition", "kutacc_af2_triangle_multiplication_calc_proj",
     "kutacc_af2_triangle_multiplication_equation", "kutacc_af2_triangle_multiplication_gate_and_out_linear",
     "kutacc_af2_triangle_multiplication_last", "kutacc_hip_gemm", "kutacc_hip_sigmoid_gate_rows", "kutacc_hip_transition",
+    "kutacc_hip_pair_bias_transposed", "kutacc_hip_mask_bias", "kutacc_hip_swap_leading_axes", "kutacc_hip_residual_add",
+    "kutacc_hip_triangle_attention_workspace", "kutacc_hip_triangle_attention",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
@@ -187,6 +200,18 @@ def lib() -> ctypes.CDLL:
     L.kutacc_af2_triangle_multiplication_gate_and_out_linear.restype = None
     L.kutacc_af2_triangle_multiplication_last.argtypes = [_vp, _vp, _i64, _i64, _i64]
     L.kutacc_af2_triangle_multiplication_last.restype = None
+    L.kutacc_hip_pair_bias_transposed.argtypes = L.kutacc_hip_pair_bias.argtypes
+    L.kutacc_hip_pair_bias_transposed.restype = ctypes.c_int
+    L.kutacc_hip_mask_bias.argtypes = [_vp, _vp, _i64, _i64, _i32, _i32, _vp]
+    L.kutacc_hip_mask_bias.restype = ctypes.c_int
+    L.kutacc_hip_swap_leading_axes.argtypes = [_vp, _vp, _i64, _i64, _i64, _i32, _vp]
+    L.kutacc_hip_swap_leading_axes.restype = ctypes.c_int
+    L.kutacc_hip_residual_add.argtypes = [_vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]
+    L.kutacc_hip_residual_add.restype = ctypes.c_int
+    L.kutacc_hip_triangle_attention_workspace.argtypes = [_i64, _i64]
+    L.kutacc_hip_triangle_attention_workspace.restype = _i64
+    L.kutacc_hip_triangle_attention.argtypes = [ctypes.POINTER(HipTriangleAttentionArgs), _vp]
+    L.kutacc_hip_triangle_attention.restype = ctypes.c_int
     L.kutacc_hip_set_stream.argtypes = [_vp]
     L.kutacc_hip_get_stream.restype = _vp
     L.kutacc_hip_set_blocking.argtypes = [ctypes.c_int]
@@ -390,3 +415,30 @@ class Transition:
 
     def run(self) -> None:
         kutacc_af2_transition(self.inputs, self.weights, self.h["out"])
+
+
+class TriangleAttentionBlock:
+    """One triangle-attention block on device tensors, in place on `pair_act` [n, n, c_z]:
+    pair_act += gating_attention(LN(pair_act), pair bias from LN(pair_act) . bias_w^T, mask bias from pair_mask),
+    around the starting or the ending node.  Owns the workspace; `run()` is one kutacc_hip_triangle_attention call."""
+
+    def __init__(self, pair_act, pair_mask, ln_gamma, ln_beta, bias_w, wq, wk, wv, wg, bg, wo, bo, nheads, ending_node,
+                 eps=1e-5):
+        import torch
+        n = pair_act.shape[0]
+        nbytes = lib().kutacc_hip_triangle_attention_workspace(n, nheads)
+        assert nbytes > 0
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=pair_act.device)
+        self.keep = (pair_act, pair_mask, ln_gamma, ln_beta, bias_w, wq, wk, wv, wg, bg, wo, bo)
+        a = HipTriangleAttentionArgs()
+        a.n_res, a.nheads, a.dtype, a.ending_node = n, nheads, K_BF16, 1 if ending_node else 0
+        a.pair_act, a.pair_mask = pair_act.data_ptr(), pair_mask.data_ptr()
+        a.ln_gamma, a.ln_beta, a.ln_eps = ln_gamma.data_ptr(), ln_beta.data_ptr(), eps
+        a.bias_w = bias_w.data_ptr()
+        a.query_w, a.key_w, a.value_w, a.gating_w, a.output_w = (t.data_ptr() for t in (wq, wk, wv, wg, wo))
+        a.gating_b, a.output_b = bg.data_ptr(), bo.data_ptr()
+        a.workspace, a.workspace_bytes = self.workspace.data_ptr(), nbytes
+        self.args = a
+
+    def run(self, stream_ptr=None) -> int:
+        return lib().kutacc_hip_triangle_attention(ctypes.byref(self.args), stream_ptr)

@@ -243,7 +243,7 @@ int kutacc_hip_pair_bias(const void *z, const float *gamma, const float *beta, c
                          int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype,
                          void *stream)
 {
-    return kutacc_launch::pair_bias(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, dtype,
+    return kutacc_launch::pair_bias(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, dtype, 0,
                                     pick_stream(stream));
 }
 

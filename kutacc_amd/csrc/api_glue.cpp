@@ -1,0 +1,125 @@
+// extern "C" layer of the glue between operators (mask bias, axis swap, residual update, the pair-bias
+// producer reading a transposed pair tensor) and of the triangle-attention block built from them:
+//   pair_act += attention(LayerNorm(pair_act))        along rows (starting node) or columns (ending node)
+// with the pair bias projected from the same normalised tensor.  The reference leaves these steps to its
+// caller (a PyTorch extension that is not part of the repository); the operator calls in between are
+// kutacc_af2_layernorm / kutacc_af2_linear (reference src/normalization/layernorm.cpp:17-20,
+// src/linear/linear.cpp:45-50) and kutacc_af2_gating_attention (reference src/attention/gating_attention.cpp:160-200).
+// Everything here runs on the device, on one stream, without host round trips.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "api_internal.h"
+#include "kutacc_hip.h"
+#include "launch_internal.h"
+
+namespace {
+constexpr int64_t HEAD = 32;
+
+inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+struct Workspace {
+    int64_t z_norm, nb, bias, q, avg, total; // byte offsets; z_norm doubles as the attention output
+};
+
+Workspace layout(int64_t n, int64_t heads)
+{
+    const int64_t c = heads * HEAD, act = align256(n * n * c * 2);
+    Workspace w;
+    w.z_norm = 0;
+    w.nb = w.z_norm + act;
+    w.bias = w.nb + align256(heads * n * n * 2);
+    w.q = w.bias + align256(n * n * 2);
+    w.avg = w.q + act;
+    w.total = w.avg + act;
+    return w;
+}
+} // namespace
+
+extern "C" {
+
+int kutacc_hip_pair_bias_transposed(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
+                                    int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype,
+                                    void *stream)
+{
+    return kutacc_launch::pair_bias(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, dtype, 1,
+                                    kutacc_api::stream_or_default(stream));
+}
+
+int kutacc_hip_mask_bias(const void *mask, void *bias, int64_t n0, int64_t n1, int32_t transposed, int32_t dtype, void *stream)
+{
+    return kutacc_launch::mask_bias(mask, bias, n0, n1, transposed != 0, dtype, kutacc_api::stream_or_default(stream));
+}
+
+int kutacc_hip_swap_leading_axes(const void *in, void *out, int64_t n0, int64_t n1, int64_t inner, int32_t dtype, void *stream)
+{
+    return kutacc_launch::swap_leading_axes(in, out, n0, n1, inner, dtype, kutacc_api::stream_or_default(stream));
+}
+
+int kutacc_hip_residual_add(void *acc, const void *delta, int64_t n0, int64_t n1, int64_t inner, int32_t swapped, int32_t dtype,
+                            void *stream)
+{
+    return kutacc_launch::residual_add(acc, delta, n0, n1, inner, swapped != 0, dtype, kutacc_api::stream_or_default(stream));
+}
+
+int64_t kutacc_hip_triangle_attention_workspace(int64_t n_res, int64_t nheads)
+{
+    if (n_res <= 0 || nheads <= 0 || n_res > 65536 || nheads > 64) {
+        return -1;
+    }
+    return layout(n_res, nheads).total;
+}
+
+int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a, void *stream)
+{
+    if (!a || !a->pair_act || !a->pair_mask || !a->ln_gamma || !a->ln_beta || !a->bias_w || !a->query_w || !a->key_w ||
+        !a->value_w || !a->gating_w || !a->output_w || !a->gating_b || !a->output_b || !a->workspace) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (a->dtype != KUTACC_DTYPE_BF16 || a->n_res <= 0 || a->n_res > 65536 || a->nheads <= 0 || a->nheads > 64) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int64_t n = a->n_res, heads = a->nheads, c = heads * HEAD;
+    const Workspace w = layout(n, heads);
+    if (a->workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
+        return KUTACC_HIP_EINVAL;
+    }
+    char *ws = static_cast<char *>(a->workspace);
+    hipStream_t s = kutacc_api::stream_or_default(stream);
+    const int ending = a->ending_node != 0;
+
+    kutacc_hip_attention_args_t g;
+    std::memset(&g, 0, sizeof(g));
+    g.batch = n, g.seq_len = n, g.nheads = heads, g.head_size = HEAD;
+    g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_FUSED;
+    g.input = ws + w.z_norm, g.input_ld = c;
+    g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
+    g.gating_b = a->gating_b, g.output_b = a->output_b;
+    g.bias = ws + w.bias, g.bias_stride_b = n;
+    g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n * n, g.nb_stride_q = n;
+    g.q = ws + w.q, g.q_stride_b = n * c, g.q_stride_s = c, g.q_stride_h = HEAD;
+    g.avg = ws + w.avg, g.avg_stride_b = n * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
+    g.out = ws + w.z_norm, g.out_ld = c; // the normalised input is dead once the head kernel has run
+    if (!kutacc_launch::fused_attention_supports(g)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    // 1. LayerNorm + pair-bias projection in one pass over the pair tensor; the ending node reads it transposed
+    int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, ws + w.z_norm, n, n, c, heads,
+                                      a->ln_eps, KUTACC_DTYPE_BF16, ending, s);
+    if (rc != 0) {
+        return rc;
+    }
+    // 2. mask -> additive bias of the keys of every row
+    if ((rc = kutacc_launch::mask_bias(a->pair_mask, ws + w.bias, n, n, ending, KUTACC_DTYPE_BF16, s)) != 0) {
+        return rc;
+    }
+    // 3. the operator
+    if ((rc = kutacc_launch::gating_attention_fused(g, s)) != 0) {
+        return rc;
+    }
+    // 4. residual update; the ending node's result goes back transposed
+    return kutacc_launch::residual_add(a->pair_act, ws + w.z_norm, n, n, c, ending, KUTACC_DTYPE_BF16, s);
+}
+
+} // extern "C"

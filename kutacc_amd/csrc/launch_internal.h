@@ -37,11 +37,17 @@ int transition_fused(const void *x, const void *w1, const float *b1, const void 
 int sigmoid_gate_rows(void *out, int64_t out_s0, int64_t out_s1, const void *gate, int64_t gate_s0, int64_t gate_s1,
                       int64_t n0, int64_t n1, int64_t size, hipStream_t stream);
 
+// glue_kernels.hip
+int mask_bias(const void *mask, void *bias, int64_t n0, int64_t n1, int transposed, int32_t dtype, hipStream_t stream);
+int swap_leading_axes(const void *in, void *out, int64_t n0, int64_t n1, int64_t inner, int32_t dtype, hipStream_t stream);
+int residual_add(void *acc, const void *delta, int64_t n0, int64_t n1, int64_t inner, int swapped, int32_t dtype,
+                 hipStream_t stream);
+
 // row_kernels.hip
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                    int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream);
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
-              int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype,
+              int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
               hipStream_t stream);
 
 } // namespace kutacc_launch

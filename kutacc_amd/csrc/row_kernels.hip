@@ -66,7 +66,8 @@ __global__ __launch_bounds__(64 * ROW_WAVES) void pair_bias_kernel(const T *__re
                                                                   const float *__restrict__ beta,
                                                                   const T *__restrict__ w, T *__restrict__ nb,
                                                                   T *__restrict__ z_norm, int64_t rows_i,
-                                                                  int64_t rows_j, int64_t c_z, int64_t nheads, float eps)
+                                                                  int64_t rows_j, int64_t c_z, int64_t nheads, float eps,
+                                                                  int transposed)
 {
     const int lane = threadIdx.x % 64;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + threadIdx.x / 64;
@@ -74,7 +75,8 @@ __global__ __launch_bounds__(64 * ROW_WAVES) void pair_bias_kernel(const T *__re
     if (r >= rows) {
         return;
     }
-    const T *row = z + r * c_z;
+    // transposed: output row (i, j) is computed from row (j, i) of z, stored [rows_j, rows_i, c_z]
+    const T *row = z + (transposed ? (r % rows_j) * rows_i + r / rows_j : r) * c_z;
     float rstd, shift;
     row_stats(row, c_z, lane, eps, rstd, shift);
     for (int64_t h0 = 0; h0 < nheads; h0 += 8) {
@@ -224,7 +226,8 @@ template <int H>
 __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__restrict__ z, const float *__restrict__ gamma,
                                                              const float *__restrict__ beta, const bf16_t *__restrict__ w,
                                                              bf16_t *__restrict__ nb, bf16_t *__restrict__ z_norm,
-                                                             int64_t rows, float eps)
+                                                             int64_t rows, float eps, int64_t rows_i, int64_t rows_j,
+                                                             int transposed)
 {
     constexpr int LPR = 16, CZ = 128;
     const int lane = threadIdx.x & 63;
@@ -234,11 +237,21 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
         return;
     }
     Pack16 in[16];
+    {
+        // transposed: output row (i, j) is computed from row (j, i) of z, stored [rows_j, rows_i, c_z]; the walk
+        // over 16 consecutive output rows then steps through z with stride rows_i rows
+        int64_t r = r0 + grp * 16;
+        int64_t i = transposed ? r / rows_j : 0, j = transposed ? r % rows_j : 0;
 #pragma unroll
-    for (int s = 0; s < 16; ++s) {
-        int64_t r = r0 + grp * 16 + s;
-        r = r < rows ? r : rows - 1;
-        in[s].u = *reinterpret_cast<const uint4 *>(z + r * CZ + sub * 8);
+        for (int s = 0; s < 16; ++s) {
+            int64_t src = transposed ? j * rows_i + i : r;
+            src = r < rows ? src : 0;
+            in[s].u = *reinterpret_cast<const uint4 *>(z + src * CZ + sub * 8);
+            ++r;
+            if (++j == rows_j) {
+                j = 0, ++i;
+            }
+        }
     }
     float gm[8], bt[8];
 #pragma unroll
@@ -328,7 +341,8 @@ int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const floa
 
 template <typename T>
 int launch_pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
-                     int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, hipStream_t stream)
+                     int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int transposed,
+                     hipStream_t stream)
 {
     const int64_t rows = rows_i * rows_j;
     if (sizeof(T) == 2 && c_z == 128 && (nheads == 4 || nheads == 8) &&
@@ -339,10 +353,12 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
         }
         if (nheads == 4) {
             pair_bias_bf16_kernel<4><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
-                                                                        (bf16_t *)nb, (bf16_t *)z_norm, rows, eps);
+                                                                        (bf16_t *)nb, (bf16_t *)z_norm, rows, eps, rows_i, rows_j,
+                                                                        transposed);
         } else {
             pair_bias_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
-                                                                        (bf16_t *)nb, (bf16_t *)z_norm, rows, eps);
+                                                                        (bf16_t *)nb, (bf16_t *)z_norm, rows, eps, rows_i, rows_j,
+                                                                        transposed);
         }
         return kutacc_hip_status(hipGetLastError());
     }
@@ -351,7 +367,7 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
         return KUTACC_HIP_EUNSUPPORTED;
     }
     pair_bias_kernel<T><<<(unsigned)blocks, 64 * ROW_WAVES, 0, stream>>>(
-        (const T *)z, gamma, beta, (const T *)w, (T *)nb, (T *)z_norm, rows_i, rows_j, c_z, nheads, eps);
+        (const T *)z, gamma, beta, (const T *)w, (T *)nb, (T *)z_norm, rows_i, rows_j, c_z, nheads, eps, transposed);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -375,17 +391,17 @@ int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float 
 }
 
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
-              int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype,
+              int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
               hipStream_t stream)
 {
     if (!z || !gamma || !beta || !w || !nb || rows_i <= 0 || rows_j <= 0 || c_z <= 0 || nheads <= 0) {
         return KUTACC_HIP_EINVAL;
     }
     if (dtype == KUTACC_DTYPE_BF16) {
-        return launch_pair_bias<bf16_t>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, stream);
+        return launch_pair_bias<bf16_t>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream);
     }
     if (dtype == KUTACC_DTYPE_FP32) {
-        return launch_pair_bias<float>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, stream);
+        return launch_pair_bias<float>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream);
     }
     return KUTACC_HIP_EINVAL;
 }

@@ -273,3 +273,17 @@ def test_gemm_launch_layer_rejects_bad_arguments_without_a_device():
     g.m, g.n, g.k, g.batches, g.dtype = 4, 4, 4, 1, capi.K_BF16
     assert L.kutacc_hip_gemm(ctypes.byref(g), None) == capi.EINVAL  # null operands
     assert L.kutacc_hip_sigmoid_gate_rows(None, 1, 1, None, 1, 1, 1, 1, 1, capi.K_BF16, None) == capi.EINVAL
+
+
+def test_glue_launch_layer_rejects_bad_arguments_without_a_device():
+    L = capi.lib()
+    assert L.kutacc_hip_mask_bias(None, None, 4, 4, 0, capi.K_BF16, None) == capi.EINVAL
+    assert L.kutacc_hip_swap_leading_axes(None, None, 4, 4, 8, capi.K_BF16, None) == capi.EINVAL
+    assert L.kutacc_hip_residual_add(None, None, 4, 4, 8, 0, capi.K_BF16, None) == capi.EINVAL
+    assert L.kutacc_hip_pair_bias_transposed(None, None, None, None, None, None, 1, 1, 1, 1, 1e-5, capi.K_BF16, None) == capi.EINVAL
+    assert L.kutacc_hip_triangle_attention(None, None) == capi.EINVAL
+    # activation, pair bias, mask bias and two scratch activations, each rounded up to 256 bytes
+    n, h = 384, 4
+    act = n * n * h * 32 * 2
+    assert L.kutacc_hip_triangle_attention_workspace(n, h) == 3 * act + h * n * n * 2 + n * n * 2
+    assert L.kutacc_hip_triangle_attention_workspace(-1, h) == -1

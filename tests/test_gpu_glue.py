@@ -1,0 +1,184 @@
+"""The steps between the operators (mask bias, axis swap, residual update, transposed pair-bias producer) and the
+triangle-attention block assembled from them, on a real MI355X through the C ABI.
+
+The copies and the residual update are checked bit for bit against torch's own indexing and bf16 addition; the
+block is checked against the CPU oracle's LayerNorm, Linear and gated attention composed in numpy (fp32, no
+intermediate rounding) at the tolerance of the bf16 path, and, at a full-size pair tensor, through the identity
+ending_node(z, mask) == starting_node(z^T, mask^T)^T, which must hold bit for bit.
+"""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+
+from kutacc_amd import capi
+from kutacc_amd.workloads import round_to_bf16
+
+import helpers
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    capi.set_stream(None)
+    capi.set_blocking(True)
+    return torch
+
+
+def code(torch, t):
+    return capi.K_BF16 if t.dtype == torch.bfloat16 else capi.K_FP32
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("transposed", [0, 1])
+def test_mask_bias(torch_cuda, dtype, transposed):
+    torch = torch_cuda
+    dt = getattr(torch, dtype)
+    n0, n1 = 37, 52
+    g = torch.Generator(device="cuda").manual_seed(3)
+    mask_ij = (torch.rand(n0, n1, device="cuda", generator=g) > 0.3).to(dt)
+    stored = mask_ij.t().contiguous() if transposed else mask_ij
+    bias = torch.full((n0, n1), 7.0, dtype=dt, device="cuda")
+    rc = capi.lib().kutacc_hip_mask_bias(stored.data_ptr(), bias.data_ptr(), n0, n1, transposed, code(torch, bias), None)
+    torch.cuda.synchronize()
+    assert rc == 0
+    want = (mask_ij.float() * 1e9 - 1e9).to(dt)
+    assert helpers.same_bits(bias, want)
+    assert float(bias.max()) == 0.0 and float(bias.min()) < -9e8
+
+
+@pytest.mark.parametrize("shape,dtype", [((40, 24, 128), "bfloat16"), ((9, 31, 5), "bfloat16"), ((17, 6, 12), "float32"),
+                                         ((384, 384, 128), "bfloat16")])
+def test_swap_leading_axes_and_residual_add(torch_cuda, shape, dtype):
+    torch = torch_cuda
+    dt = getattr(torch, dtype)
+    n0, n1, c = shape
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(n0, n1, c, device="cuda", generator=g).to(dt)
+    out = torch.zeros(n1, n0, c, dtype=dt, device="cuda")
+    L = capi.lib()
+    assert L.kutacc_hip_swap_leading_axes(x.data_ptr(), out.data_ptr(), n0, n1, c, code(torch, x), None) == 0
+    torch.cuda.synchronize()
+    assert helpers.same_bits(out, x.transpose(0, 1).contiguous())
+    # acc[i, j] += delta[i, j] and acc[i, j] += delta[j, i]
+    acc = torch.randn(n0, n1, c, device="cuda", generator=g).to(dt)
+    want_plain = (acc.float() + x.float()).to(dt)
+    want_swapped = (acc.float() + out.transpose(0, 1).float()).to(dt)
+    a1, a2 = acc.clone(), acc.clone()
+    assert L.kutacc_hip_residual_add(a1.data_ptr(), x.data_ptr(), n0, n1, c, 0, code(torch, x), None) == 0
+    assert L.kutacc_hip_residual_add(a2.data_ptr(), out.data_ptr(), n0, n1, c, 1, code(torch, x), None) == 0
+    torch.cuda.synchronize()
+    assert helpers.same_bits(a1, want_plain)
+    assert helpers.same_bits(a2, want_swapped)
+    assert L.kutacc_hip_swap_leading_axes(x.data_ptr(), x.data_ptr(), n0, n1, c, code(torch, x), None) == capi.EINVAL
+
+
+@pytest.mark.parametrize("n_i,n_j,c_z,heads,dtype", [(48, 48, 128, 4, "bfloat16"), (40, 56, 128, 8, "bfloat16"),
+                                                      (9, 14, 64, 3, "bfloat16"), (7, 5, 32, 2, "float32")])
+def test_pair_bias_transposed_equals_pair_bias_of_the_swapped_tensor(torch_cuda, n_i, n_j, c_z, heads, dtype):
+    torch = torch_cuda
+    dt = getattr(torch, dtype)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    z_t = torch.randn(n_j, n_i, c_z, device="cuda", generator=g).to(dt)  # stored transposed: [j, i, c]
+    z = z_t.transpose(0, 1).contiguous()
+    w = (torch.randn(heads, c_z, device="cuda", generator=g) / math.sqrt(c_z)).to(dt)
+    gamma = torch.rand(c_z, device="cuda", generator=g) + 0.5
+    beta = torch.randn(c_z, device="cuda", generator=g) * 0.1
+    L = capi.lib()
+    res = []
+    for fn, src in ((L.kutacc_hip_pair_bias, z), (L.kutacc_hip_pair_bias_transposed, z_t)):
+        nb = torch.zeros(heads, n_i, n_j, dtype=dt, device="cuda")
+        zn = torch.zeros(n_i, n_j, c_z, dtype=dt, device="cuda")
+        assert fn(src.data_ptr(), gamma.data_ptr(), beta.data_ptr(), w.data_ptr(), nb.data_ptr(), zn.data_ptr(), n_i, n_j, c_z,
+                  heads, 1e-5, code(torch, z), None) == 0
+        torch.cuda.synchronize()
+        res.append((nb, zn))
+    assert helpers.same_bits(res[0][0], res[1][0]) and helpers.same_bits(res[0][1], res[1][1])
+
+
+# ---- the block ---------------------------------------------------------------------------------------------------
+def block_case(seed, n, heads):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    c = heads * 32
+    w = lambda o, i: round_to_bf16((rng.standard_normal((o, i)) / math.sqrt(i)).astype(np.float32))  # noqa: E731
+    mask = (rng.random((n, n)) > 0.1).astype(np.float32)
+    mask[:, -3:] = 0.0  # padded residues: masked as keys for the starting node, whole rows for the ending node
+    return dict(z=round_to_bf16(rng.standard_normal((n, n, c)).astype(np.float32)), mask=mask,
+                gamma=(rng.random(c) + 0.5).astype(np.float32), beta=(rng.standard_normal(c) * 0.1).astype(np.float32),
+                bias_w=w(heads, c), wq=w(c, c), wk=w(c, c), wv=w(c, c), wg=w(c, c), wo=w(c, c),
+                bg=np.ones(c, np.float32), bo=(rng.standard_normal(c) * 0.1).astype(np.float32), heads=heads)
+
+
+def block_oracle(c, ending):
+    """AlphaFold's TriangleAttention in numpy on the oracle's operators: orientation swap, LayerNorm, pair bias from
+    the normalised tensor, mask bias, gated attention, swap back, residual."""
+    from oracle import oracle
+    z, mask = c["z"], c["mask"]
+    if ending:
+        z, mask = z.transpose(1, 0, 2), mask.T
+    n, _, ch = z.shape
+    zn = oracle.layernorm_rows_f32(np.ascontiguousarray(z).reshape(-1, ch), c["gamma"], c["beta"], 1e-5).reshape(n, n, ch)
+    nb = oracle.linear_f32(zn.reshape(-1, ch), c["bias_w"]).reshape(n, n, c["heads"]).transpose(2, 0, 1)
+    bias = (mask * np.float32(1e9) - np.float32(1e9)).astype(np.float32)
+    out = oracle.gating_attention_f32(zn, c["wq"], c["wk"], c["wv"], c["wg"], c["bg"], c["wo"], c["bo"], bias,
+                                      np.ascontiguousarray(nb), c["heads"])
+    if ending:
+        out = out.transpose(1, 0, 2)
+    return c["z"] + out
+
+
+def run_block(torch, c, ending, z=None, mask=None):
+    dev = lambda a, dt=torch.bfloat16: torch.from_numpy(np.ascontiguousarray(a)).to(device="cuda", dtype=dt)  # noqa: E731
+    pair = dev(c["z"]) if z is None else z.clone()
+    dmask = dev(c["mask"]) if mask is None else mask
+    f32 = torch.float32
+    blk = capi.TriangleAttentionBlock(pair, dmask, dev(c["gamma"], f32), dev(c["beta"], f32), dev(c["bias_w"]), dev(c["wq"]),
+                                      dev(c["wk"]), dev(c["wv"]), dev(c["wg"]), dev(c["bg"], f32), dev(c["wo"]),
+                                      dev(c["bo"], f32), c["heads"], ending)
+    rc = blk.run()
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    return pair
+
+
+@pytest.mark.parametrize("ending", [False, True], ids=["starting node", "ending node"])
+@pytest.mark.parametrize("n,heads", [(48, 4), (70, 4), (40, 8)])
+def test_triangle_attention_block_against_the_oracle(torch_cuda, n, heads, ending):
+    c = block_case(600 + n, n, heads)
+    got = run_block(torch_cuda, c, ending)
+    helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block n={n} ending={ending}")
+
+
+def test_triangle_attention_block_full_size_orientation_identity(torch_cuda):
+    """384 residues: the ending-node block equals the starting-node block on the transposed pair tensor and mask,
+    transposed back -- the two orientations differ only in which element is read or written where."""
+    torch = torch_cuda
+    c = block_case(700, 384, 4)
+    z = torch.from_numpy(c["z"]).to(device="cuda", dtype=torch.bfloat16)
+    mask = torch.from_numpy(c["mask"]).to(device="cuda", dtype=torch.bfloat16)
+    end = run_block(torch, c, True, z, mask)
+    start_t = run_block(torch, c, False, z.transpose(0, 1).contiguous(), mask.t().contiguous())
+    assert helpers.same_bits(end, start_t.transpose(0, 1).contiguous())
+    assert not helpers.same_bits(end, z)
+
+
+def test_triangle_attention_block_rejects_bad_arguments(torch_cuda):
+    torch = torch_cuda
+    L = capi.lib()
+    assert L.kutacc_hip_triangle_attention(None, None) == capi.EINVAL
+    assert L.kutacc_hip_triangle_attention_workspace(0, 4) == -1
+    c = block_case(1, 40, 4)
+    dev = lambda a, dt=torch.bfloat16: torch.from_numpy(np.ascontiguousarray(a)).to(device="cuda", dtype=dt)  # noqa: E731
+    blk = capi.TriangleAttentionBlock(dev(c["z"]), dev(c["mask"]), dev(c["gamma"], torch.float32), dev(c["beta"], torch.float32),
+                                      dev(c["bias_w"]), dev(c["wq"]), dev(c["wk"]), dev(c["wv"]), dev(c["wg"]),
+                                      dev(c["bg"], torch.float32), dev(c["wo"]), dev(c["bo"], torch.float32), 4, False)
+    blk.args.workspace_bytes -= 1
+    assert blk.run() == capi.EINVAL
+    blk.args.workspace_bytes += 1
+    blk.args.nheads = 3  # 96 channels: no MFMA attention kernel
+    assert blk.run() in (capi.EUNSUPPORTED, capi.EINVAL)
+    torch.cuda.synchronize()
