@@ -142,7 +142,7 @@ def pair_stack_rates(config, reps=20):
     at this configuration's pair tensor: n = S residues, 128 pair channels, 128 projected channels, hidden layer 512.
     Called through the handle-based entry points, asynchronously on torch's stream, hipEvent-bracketed.  Per step:
     microseconds, algorithmic TFLOP/s (2 flops per multiply-add of the products) and algorithmic GB/s (every operand
-    and result of the step once, intermediates the reference also materialises included)."""
+    and result of the step once)."""
     import torch
     from kutacc_amd import capi
     from kutacc_amd.workloads import CONFIGS
@@ -180,7 +180,7 @@ def pair_stack_rates(config, reps=20):
     mid = torch.empty(rows, hid, device="cuda", dtype=torch.bfloat16)
     out = torch.empty(n, n, c_o, device="cuda", dtype=torch.bfloat16)
     tr = capi.Transition(x, bf(hid, c_o, scale=c_o ** -0.5), f32(hid), bf(c_o, hid, scale=hid ** -0.5), f32(c_o), mid, out)
-    report("transition", timed(tr.run), 4.0 * rows * c_o * hid, 2.0 * rows * (2 * c_o + 2 * hid))
+    report("transition", timed(tr.run), 4.0 * rows * c_o * hid, 2.0 * rows * 2 * c_o)  # input and output; the hidden layer stays on chip
     del mid
     # triangle multiplication
     keep = [bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i), bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i)]
