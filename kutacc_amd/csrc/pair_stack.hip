@@ -472,6 +472,145 @@ __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *
     }
 }
 
+// Gated projection of the triangle multiplication for 128 pair channels and 128 projected channels
+// (reference src/attention/triangle_multiplication.cpp:37-66):
+//   out[c][p] = bf16( bf16(x[p] . wp[c] + bp[c]) * mask[p] * sigmoid(x[p] . wg[c] + bg[c]) )
+// over positions p of the pair tensor, written channel-first (the gate is not rounded to bf16 on its way into the
+// sigmoid as it is in the reference, which stores it; the result is the closer one to exact arithmetic).  HBM-bound (256 bytes in, 256 bytes out per
+// position), so the layout follows the row-projection kernel of the attention: both weight matrices stay in
+// LDS in fragment order for the life of the workgroup (64 KB), every wave streams ranges of 64 positions whose
+// rows it fetches as whole cache lines one step ahead, and the products are formed with positions as MFMA rows
+// and channels as columns: a lane then owns one channel and four consecutive positions per accumulator group,
+// which is the order of the channel-first output -- an 8-byte panel write, then 128-byte runs per channel.
+__global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ wp,
+                                                                  const float *__restrict__ bp, const bf16_t *__restrict__ wg,
+                                                                  const float *__restrict__ bg, const bf16_t *__restrict__ mask,
+                                                                  bf16_t *__restrict__ out, int64_t out_ld, int64_t n_pos,
+                                                                  int pos_per_wave)
+{
+    constexpr int C = 128, CK = C / 16;
+    extern __shared__ uint4 lds[]; // [2 matrices][4 channel blocks][CK][64 lanes], then one panel per wave
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    uint4 *panel = lds + 2 * 4 * CK * 64 + wave * 256;
+    const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * pos_per_wave;
+    const int64_t stop = start + pos_per_wave < n_pos ? start + pos_per_wave : n_pos;
+    const int last = (int)(stop - start) - 1; // last valid position of the range, relative to start
+    const bf16_t *xb = x + start * C;
+    PanelRegs t[4]; // two 32-row blocks x two 64-column halves of the current step
+    if (start < stop) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            t[q] = panel_load(xb, C, (q >> 1) * 32, last, (q & 1) * 64, lane);
+        }
+    }
+    {
+        constexpr int PER = 2 * 4 * CK * 64 / 256;
+        uint4 wreg[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = tid + i * 256;
+            const int mat = idx / (4 * CK * 64), nb_ = (idx / (CK * 64)) % 4, ks = (idx >> 6) % CK, ln = idx & 63;
+            const bf16_t *w = mat ? wg : wp;
+            wreg[i] = *reinterpret_cast<const uint4 *>(w + (int64_t)(nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            lds[tid + i * 256] = wreg[i];
+        }
+    }
+    __syncthreads();
+    for (int64_t base = start; base < stop; base += 64) {
+        const int rel = (int)(base - start);
+        bf16x8 af[2][CK];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            panel_store(panel, lane, t[q]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                af[q >> 1][(q & 1) * 4 + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+            }
+        }
+        {
+            const int nrel = base + 64 < stop ? rel + 64 : rel; // clamped: one harmless re-read at the end
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                t[q] = panel_load(xb, C, nrel + (q >> 1) * 32, last, (q & 1) * 64, lane);
+            }
+        }
+#pragma unroll 1
+        for (int n = 0; n < 4; ++n) { // 32 channels at a time
+            // projection first, rounded to bf16 and parked as packed pairs, then the gate: half the accumulators live
+            const float pbias = bp[n * 32 + r], gneg = -LOG2E * bg[n * 32 + r];
+            bf16x8 pp[2][2];
+            {
+                f32x16 pa[2];
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    pa[rb] = zero16();
+                }
+#pragma unroll
+                for (int ks = 0; ks < CK; ++ks) {
+                    const bf16x8 wpf = as_bf16x8(lds[(n * CK + ks) * 64 + lane]);
+#pragma unroll
+                    for (int rb = 0; rb < 2; ++rb) {
+                        pa[rb] = mfma(af[rb][ks], wpf, pa[rb]);
+                    }
+                }
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        pa[rb][v] += pbias;
+                    }
+                    pp[rb][0] = pack8(pa[rb], 0), pp[rb][1] = pack8(pa[rb], 8);
+                }
+            }
+            f32x16 ga[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                ga[rb] = zero16();
+            }
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                const bf16x8 wgf = as_bf16x8(lds[((4 + n) * CK + ks) * 64 + lane]);
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    ga[rb] = mfma(af[rb][ks], wgf, ga[rb]);
+                }
+            }
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    // mask of the lane's four consecutive positions (re-read per channel block: it stays in the L1)
+                    int64_t p0 = base + rb * 32 + 8 * a + 4 * g;
+                    p0 = p0 + 4 <= n_pos ? p0 : n_pos - 4; // positions past the end are never stored
+                    const bf16x4 mk = *reinterpret_cast<const bf16x4 *>(mask + p0);
+                    bf16x4 ov;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float pv = to_f32(pp[rb][a >> 1][4 * (a & 1) + c]) * to_f32(mk[c]);
+                        // sigmoid(gate + bias) = 1 / (1 + 2^-(gate*log2e + bias*log2e)); the gate stays in fp32
+                        const float e = __builtin_amdgcn_exp2f(fmaf(ga[rb][4 * a + c], -LOG2E, gneg));
+                        ov[c] = (bf16_t)(pv * __builtin_amdgcn_rcpf(1.0f + e));
+                    }
+                    *(reinterpret_cast<bf16x4 *>(panel + panel_slot(r, rb * 4 + a)) + g) = ov;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ch = 8 * i + (lane >> 3);
+                const uint4 v = panel[panel_slot(ch, lane & 7)];
+                const int64_t p0 = base + (lane & 7) * 8;
+                if (p0 < stop) {
+                    *reinterpret_cast<uint4 *>(out + (int64_t)(n * 32 + ch) * out_ld + p0) = v;
+                }
+            }
+        }
+    }
+}
+
 // Any strides, any sizes: one thread per element of C, same epilogues and rounding points.
 __global__ __launch_bounds__(256) void pair_gemm_scalar_kernel(const GemmParams p)
 {
@@ -575,6 +714,50 @@ hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
     pair_gemm_kernel<AM, BM, G><<<dim3((unsigned)blocks), 256, GEMM_LDS, stream>>>(p);
     return hipGetLastError();
 }
+constexpr int64_t GATED_STREAMING_MIN_POSITIONS = 512 * 512;
+
+// the dedicated kernel of the gated projection: 128 -> 128 channels, dense operands, positions in whole 16-byte runs
+bool gated_projection_fits(const kutacc_hip_gemm_args_t &g)
+{
+    return g.a_gate && g.mask && g.bias_axis == 2 && g.bias && g.bias_gate && g.batches == 1 && g.m == 128 && g.k == 128 &&
+           g.a_stride_k == 1 && g.a_stride_m == 128 && g.b_stride_k == 1 && g.b_stride_n == 128 && g.n % 8 == 0 && g.n >= 8 &&
+           g.c_stride_m % 8 == 0 && aligned16(g.a) && aligned16(g.a_gate) && aligned16(g.b) && aligned16(g.c) &&
+           (reinterpret_cast<uintptr_t>(g.mask) & 7u) == 0 && !g.relu;
+}
+
+hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = (size_t)2 * 4 * 8 * 64 * 16 + 4 * 4096;
+    static bool configured = false;
+    static int cus = 0;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gated_projection_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        int dev = 0;
+        if (e == hipSuccess) {
+            e = hipGetDevice(&dev);
+        }
+        if (e == hipSuccess) {
+            e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        }
+        if (e != hipSuccess) {
+            return e;
+        }
+        configured = true;
+    }
+    // two resident workgroups per CU, every wave an equal range of positions (a multiple of 8; the last step of a
+    // range may be partial)
+    const int64_t tiles = (g.n + 63) / 64;
+    int64_t gx = (tiles + 3) / 4;
+    const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * 2;
+    gx = gx > cap ? cap : gx;
+    const int64_t ppw = ((g.n + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
+    gated_projection_kernel<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>(
+        (const bf16_t *)g.b, (const bf16_t *)g.a, g.bias, (const bf16_t *)g.a_gate, g.bias_gate, (const bf16_t *)g.mask,
+        (bf16_t *)g.c, g.c_stride_m, g.n, (int)ppw);
+    return hipGetLastError();
+}
+
 constexpr int MAX_HIDDEN = 2048; // hidden units whose bias fits next to the weight stages in LDS
 
 template <int CO, int RB>
@@ -656,6 +839,14 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
         mfma_ok = false;
     } else if (g.path == KUTACC_HIP_PATH_FUSED && !mfma_ok) {
         return KUTACC_HIP_EUNSUPPORTED;
+    }
+    // The streaming kernel pays a 64 KB weight load per workgroup and works in steps of 64 positions per wave: it
+    // wins once every wave has several steps (measured: 182 us against 225 us at 1024 x 1024 positions, but 44 us
+    // against 32 us at 384 x 384), so small pair tensors stay on the tiled kernel.
+    if (g.path != KUTACC_HIP_PATH_GENERIC && gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 &&
+        g.n >= GATED_STREAMING_MIN_POSITIONS) {
+        kutacc_prof::KernelTimer t("gated_projection_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);
+        return kutacc_hip_status(launch_gated_projection(g, stream));
     }
     // rows of 128 or 256 features against a dense weight matrix: the attention's output-projection kernel keeps
     // the weight slab in LDS and streams the rows, which suits these HBM-bound shapes better than square tiles
