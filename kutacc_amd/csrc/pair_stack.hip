@@ -382,64 +382,135 @@ __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *
         }
     }
 
-    const int NJ = c_i / 64;
-    for (int jc = 0; jc < NJ; ++jc) {
-        uint4 *stage = lds + (jc & 1) * STAGE_PANELS * 256;
+    // Blocks of 32 hidden units, t = 0 .. c_i/32 - 1; block t lives in slice t/2.  The loop is software-pipelined by
+    // hand: while the matrix core runs the first product of block t+1, the vector ALU turns the finished accumulators
+    // of block t into the bf16 operand of its second product (bias, ReLU, rounding), whose MFMAs follow.  Fences keep
+    // the compiler from pulling the two instruction streams apart again.
+    auto first_product = [&](const uint4 *stage, int hb, f32x16 (&hn)[RB]) {
 #pragma unroll
-        for (int i = 0; i < PPW; ++i) {
-            panel_store(stage + (wave * PPW + i) * 256, lane, wr[i]);
-        }
-        __syncthreads();
-        if (jc + 1 < NJ) {
-            fetch(jc + 1, wr);
+        for (int rb = 0; rb < RB; ++rb) {
+            hn[rb] = zero16();
         }
 #pragma unroll
-        for (int hb = 0; hb < 2; ++hb) {
-            f32x16 hacc[RB];
+        for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 a = as_bf16x8(stage[(hb * CP + ks / 4) * 256 + panel_slot(sr, 2 * (ks % 4) + g)]);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
-                hacc[rb] = zero16();
+                hn[rb] = mfma(a, xf[rb][ks], hn[rb]);
+            }
+        }
+    };
+    // element pair q of k-step s2 of block t: + b1, ReLU, round to bf16 (the pair form maps onto one conversion)
+    auto convert_pair = [&](const f32x16 (&hc)[RB], const float *bp, int s2, int q, bf16x2 (&w)[RB][2][4]) {
+        const f32x2 bias = *reinterpret_cast<const f32x2 *>(bp + 16 * s2 + 2 * q);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const f32x2 pr = {fmaxf(hc[rb][8 * s2 + 2 * q] + bias[0], 0.f), fmaxf(hc[rb][8 * s2 + 2 * q + 1] + bias[1], 0.f)};
+            w[rb][s2][q] = __builtin_convertvector(pr, bf16x2);
+        }
+    };
+    // first product of the next block (if any) interleaved with the conversion of the current one
+    auto overlap = [&](const uint4 *stage_next, int hb_next, bool have_next, f32x16 (&hn)[RB], const f32x16 (&hc)[RB], int t,
+                       bf16x8 (&hf)[RB][2]) {
+        const float *bp = b1s + t * 32 + 8 * g;
+        bf16x2 w[RB][2][4];
+        if (have_next) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                hn[rb] = zero16();
+            }
+            constexpr int PER = KS / 8; // k-steps per converted pair
+            // all weight fragments of the block are requested up front: with one wave per SIMD nothing else hides an
+            // LDS round trip, and the fences below would otherwise pin each read right in front of its MFMA
+            bf16x8 af[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                af[ks] = as_bf16x8(stage_next[(hb_next * CP + ks / 4) * 256 + panel_slot(sr, 2 * (ks % 4) + g)]);
             }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8 a = as_bf16x8(stage[(hb * CP + ks / 4) * 256 + panel_slot(sr, 2 * (ks % 4) + g)]);
+                const bf16x8 a = af[ks];
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
-                    hacc[rb] = mfma(a, xf[rb][ks], hacc[rb]);
+                    hn[rb] = mfma(a, xf[rb][ks], hn[rb]);
                 }
+                if (ks % PER == 0) {
+                    convert_pair(hc, bp, (ks / PER) >> 2, (ks / PER) & 3, w);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            // + b1, ReLU, round to bf16 pairwise (the pair form maps onto one conversion instruction)
-            const float *bp = b1s + jc * 64 + 32 * hb + 8 * g;
-            bf16x8 hf[RB][2];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                convert_pair(hc, bp, i >> 2, i & 3, w);
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-                const f32x4 ba = *reinterpret_cast<const f32x4 *>(bp + 16 * s2);
-                const f32x4 bb = *reinterpret_cast<const f32x4 *>(bp + 16 * s2 + 4);
+                const bf16x8 all = {w[rb][s2][0][0], w[rb][s2][0][1], w[rb][s2][1][0], w[rb][s2][1][1],
+                                    w[rb][s2][2][0], w[rb][s2][2][1], w[rb][s2][3][0], w[rb][s2][3][1]};
+                hf[rb][s2] = all;
+            }
+        }
+    };
+    auto second_fragments = [&](const uint4 *stage, int hb, bf16x8 (&a2)[CB][2]) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                a2[cb][s2] = as_bf16x8(stage[(W1_PANELS + cb) * 256 + panel_slot(r, 2 * (2 * hb + s2) + g)]);
+            }
+        }
+    };
+    auto second_product = [&](const bf16x8 (&a2)[CB][2], const bf16x8 (&hf)[RB][2]) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
-                    bf16x2 w[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float b0 = q < 2 ? ba[2 * q] : bb[2 * q - 4], b1v = q < 2 ? ba[2 * q + 1] : bb[2 * q - 3];
-                        const f32x2 pr = {fmaxf(hacc[rb][8 * s2 + 2 * q] + b0, 0.f), fmaxf(hacc[rb][8 * s2 + 2 * q + 1] + b1v, 0.f)};
-                        w[q] = __builtin_convertvector(pr, bf16x2);
-                    }
-                    const bf16x8 all = {w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
-                    hf[rb][s2] = all;
-                }
-            }
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
-                    const bf16x8 a2 = as_bf16x8(stage[(W1_PANELS + cb) * 256 + panel_slot(r, 2 * (2 * hb + s2) + g)]);
-#pragma unroll
-                    for (int rb = 0; rb < RB; ++rb) {
-                        oacc[rb][cb] = mfma(a2, hf[rb][s2], oacc[rb][cb]);
-                    }
+                    oacc[rb][cb] = mfma(a2[cb][s2], hf[rb][s2], oacc[rb][cb]);
                 }
             }
         }
+    };
+
+    const int NJ = c_i / 64;
+#pragma unroll
+    for (int i = 0; i < PPW; ++i) {
+        panel_store(lds + (wave * PPW + i) * 256, lane, wr[i]);
+    }
+    __syncthreads();
+    if (NJ > 1) {
+        fetch(1, wr);
+    }
+    f32x16 ha[RB], hb_[RB];
+    first_product(lds, 0, ha);
+    for (int jc = 0; jc < NJ; ++jc) {
+        const uint4 *stage = lds + (jc & 1) * STAGE_PANELS * 256;
+        uint4 *other = lds + ((jc + 1) & 1) * STAGE_PANELS * 256;
+        const bool more = jc + 1 < NJ;
+        // every wave is done with the other stage (its last readers were the second products of the previous slice)
+        __syncthreads();
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < PPW; ++i) {
+                panel_store(other + (wave * PPW + i) * 256, lane, wr[i]);
+            }
+            if (jc + 2 < NJ) {
+                fetch(jc + 2, wr);
+            }
+        }
+        bf16x8 hf[RB][2], a2[CB][2];
+        second_fragments(stage, 0, a2); // on their way while the first product of the next block runs
+        overlap(stage, 1, true, hb_, ha, 2 * jc, hf);
+        second_product(a2, hf);
+        __syncthreads(); // the other stage is complete and visible before the first product of its block 0 reads it
+        second_fragments(stage, 1, a2);
+        overlap(other, 0, more, ha, hb_, 2 * jc + 1, hf);
+        second_product(a2, hf);
     }
 
     // accumulators (+ b2) -> bf16 through the private panel, 64 channels at a time, out as whole 128-byte runs
