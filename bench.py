@@ -225,6 +225,22 @@ def pair_stack_rates(config, reps=20):
         def run_blk():
             assert blk.run(stream) == 0
         report(name, timed(run_blk), attn_flops, 2.0 * rows * (2 * c_o + 1))
+    # whole triangle-multiplication block (two LayerNorms, projections, equation, output step, residual)
+    tw = {"ln_in_gamma": torch.ones(c_o, device="cuda"), "ln_in_beta": torch.zeros(c_o, device="cuda"),
+          "ln_center_gamma": torch.ones(c_i, device="cuda"), "ln_center_beta": torch.zeros(c_i, device="cuda"),
+          "output_w": bf(c_o, c_i, scale=c_i ** -0.5), "output_b": f32(c_o), "gating_w": bf(c_o, c_o, scale=c_o ** -0.5),
+          "gating_b": f32(c_o)}
+    for side in ("left", "right"):
+        tw[side + "_proj_w"], tw[side + "_proj_b"] = bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i)
+        tw[side + "_gate_w"], tw[side + "_gate_b"] = bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i)
+    tm_flops = 2.0 * rows * c_o * (4 * c_i) + 2.0 * c_i * n * n * n + 2.0 * rows * c_o * (c_o + c_i)
+    zt = x.clone()
+    for name, incoming in (("triangle_multiplication_block outgoing", False), ("triangle_multiplication_block incoming", True)):
+        tmb = capi.TriangleMultiplicationBlock(zt, mask, tw, incoming)
+
+        def run_tmb():
+            assert tmb.run(stream) == 0
+        report(name, timed(run_tmb), tm_flops, 2.0 * rows * (2 * c_o + 1))
     capi.set_blocking(True)
     capi.set_stream(None)
     res["peaks"] = {"bf16_mfma_TFLOP/s": MFMA_BF16_PEAK_TFLOPS, "hbm_GB/s": HBM_PEAK_GBS}

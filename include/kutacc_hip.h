@@ -265,6 +265,57 @@ typedef struct kutacc_hip_triangle_attention_args {
 kutacc_export int64_t kutacc_hip_triangle_attention_workspace(int64_t n_res, int64_t nheads);
 kutacc_export int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *args, void *stream);
 
+/* LayerNorm over the channel axis of a channel-first tensor, written channel-last: out[p, c] = LN_c(x[c, p]) * gamma[c]
+ * + beta[c], x element (c, p) at c*ld_x + p, out row stride ld_out.  The step between the triangle equation, which
+ * leaves [c_i, n, n], and the output projection, which reads [n, n, c_i]; arithmetic as kutacc_af2_layernorm
+ * (reference src/normalization/layernorm_kernel.h:21-53). */
+kutacc_export int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, const float *beta,
+                                                     void *out, int64_t ld_out, int64_t channels, int64_t positions,
+                                                     float eps, int32_t dtype, void *stream);
+
+/*
+ * One triangle-multiplication block of the pair stack, in place (outgoing or incoming edges):
+ *   act    = LN_in(pair_act)
+ *   left   = mask * (act . left_proj_w^T + left_proj_b) * sigmoid(act . left_gate_w^T + left_gate_b)       (right alike)
+ *   center = sum_k left[i, k] * right[j, k]   (outgoing)      or      sum_k right[k, i] * left[k, j]   (incoming)
+ *   pair_act += (LN_center(center) . output_w^T + output_b) * sigmoid(act . gating_w^T + gating_b)
+ * i.e. the four kutacc_af2_triangle_multiplication_* steps (reference src/attention/triangle_multiplication.cpp:25-150)
+ * with the two LayerNorms, the layout change and the residual a caller of the reference adds around them; nine
+ * launches on `stream`.  bf16; weights stored [out, in]: *_proj_w, *_gate_w [c_i, c_z], output_w [c_z, c_i], gating_w
+ * [c_z, c_z]; all biases and LayerNorm parameters fp32.  `workspace`: device memory, 256-byte aligned, at least
+ * kutacc_hip_triangle_multiplication_workspace(n_res, c_z, c_i) bytes.
+ */
+typedef struct kutacc_hip_triangle_multiplication_args {
+    int64_t n_res;
+    int64_t c_z; /* channels of the pair activation */
+    int64_t c_i; /* projected channels */
+    int32_t dtype;    /* KUTACC_DTYPE_BF16 */
+    int32_t incoming; /* 0 outgoing edges, 1 incoming edges */
+    void *pair_act;        /* [n_res, n_res, c_z], updated in place */
+    const void *pair_mask; /* [n_res, n_res] */
+    const float *ln_in_gamma, *ln_in_beta; /* [c_z] */
+    float ln_eps;
+    int32_t reserved;
+    const void *left_proj_w;
+    const float *left_proj_b;
+    const void *left_gate_w;
+    const float *left_gate_b;
+    const void *right_proj_w;
+    const float *right_proj_b;
+    const void *right_gate_w;
+    const float *right_gate_b;
+    const float *ln_center_gamma, *ln_center_beta; /* [c_i] */
+    const void *output_w;
+    const float *output_b;
+    const void *gating_w;
+    const float *gating_b;
+    void *workspace;
+    int64_t workspace_bytes;
+} kutacc_hip_triangle_multiplication_args_t;
+
+kutacc_export int64_t kutacc_hip_triangle_multiplication_workspace(int64_t n_res, int64_t c_z, int64_t c_i);
+kutacc_export int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_args_t *args, void *stream);
+
 /* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.

@@ -125,6 +125,20 @@ class HipTriangleAttentionArgs(ctypes.Structure):
     ]
 
 
+class HipTriangleMultiplicationArgs(ctypes.Structure):
+    """kutacc_hip_triangle_multiplication_args_t"""
+    _fields_ = [
+        ("n_res", _i64), ("c_z", _i64), ("c_i", _i64), ("dtype", _i32), ("incoming", _i32),
+        ("pair_act", _vp), ("pair_mask", _vp), ("ln_in_gamma", _vp), ("ln_in_beta", _vp), ("ln_eps", ctypes.c_float),
+        ("reserved", _i32),
+        ("left_proj_w", _vp), ("left_proj_b", _vp), ("left_gate_w", _vp), ("left_gate_b", _vp),
+        ("right_proj_w", _vp), ("right_proj_b", _vp), ("right_gate_w", _vp), ("right_gate_b", _vp),
+        ("ln_center_gamma", _vp), ("ln_center_beta", _vp),
+        ("output_w", _vp), ("output_b", _vp), ("gating_w", _vp), ("gating_b", _vp),
+        ("workspace", _vp), ("workspace_bytes", _i64),
+    ]
+
+
 # every symbol the two public headers declare; tests check that the library exports all of them
 DECLARED_SYMBOLS = [
     "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_global_attention", "kutacc_af2_layernorm",
@@ -132,7 +146,8 @@ DECLARED_SYMBOLS = [
     "kutacc_af2_triangle_multiplication_equation", "kutacc_af2_triangle_multiplication_gate_and_out_linear",
     "kutacc_af2_triangle_multiplication_last", "kutacc_hip_gemm", "kutacc_hip_sigmoid_gate_rows", "kutacc_hip_transition",
     "kutacc_hip_pair_bias_transposed", "kutacc_hip_mask_bias", "kutacc_hip_swap_leading_axes", "kutacc_hip_residual_add",
-    "kutacc_hip_triangle_attention_workspace", "kutacc_hip_triangle_attention",
+    "kutacc_hip_triangle_attention_workspace", "kutacc_hip_triangle_attention", "kutacc_hip_layernorm_channel_first",
+    "kutacc_hip_triangle_multiplication_workspace", "kutacc_hip_triangle_multiplication",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
@@ -212,6 +227,12 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_triangle_attention_workspace.restype = _i64
     L.kutacc_hip_triangle_attention.argtypes = [ctypes.POINTER(HipTriangleAttentionArgs), _vp]
     L.kutacc_hip_triangle_attention.restype = ctypes.c_int
+    L.kutacc_hip_layernorm_channel_first.argtypes = [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_float, _i32, _vp]
+    L.kutacc_hip_layernorm_channel_first.restype = ctypes.c_int
+    L.kutacc_hip_triangle_multiplication_workspace.argtypes = [_i64, _i64, _i64]
+    L.kutacc_hip_triangle_multiplication_workspace.restype = _i64
+    L.kutacc_hip_triangle_multiplication.argtypes = [ctypes.POINTER(HipTriangleMultiplicationArgs), _vp]
+    L.kutacc_hip_triangle_multiplication.restype = ctypes.c_int
     L.kutacc_hip_set_stream.argtypes = [_vp]
     L.kutacc_hip_get_stream.restype = _vp
     L.kutacc_hip_set_blocking.argtypes = [ctypes.c_int]
@@ -442,3 +463,31 @@ class TriangleAttentionBlock:
 
     def run(self, stream_ptr=None) -> int:
         return lib().kutacc_hip_triangle_attention(ctypes.byref(self.args), stream_ptr)
+
+
+class TriangleMultiplicationBlock:
+    """One triangle-multiplication block on device tensors, in place on `pair_act` [n, n, c_z].  `w` is a dict of
+    device tensors: ln_in_gamma/beta [c_z], left/right_proj_w and left/right_gate_w [c_i, c_z] with their fp32 biases
+    left/right_proj_b, left/right_gate_b [c_i], ln_center_gamma/beta [c_i], output_w [c_z, c_i], output_b [c_z],
+    gating_w [c_z, c_z], gating_b [c_z].  Owns the workspace; `run()` is one kutacc_hip_triangle_multiplication call."""
+
+    def __init__(self, pair_act, pair_mask, w, incoming, eps=1e-5):
+        import torch
+        n, _, c_z = pair_act.shape
+        c_i = w["left_proj_w"].shape[0]
+        nbytes = lib().kutacc_hip_triangle_multiplication_workspace(n, c_z, c_i)
+        assert nbytes > 0
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=pair_act.device)
+        self.keep = (pair_act, pair_mask, w)
+        a = HipTriangleMultiplicationArgs()
+        a.n_res, a.c_z, a.c_i, a.dtype, a.incoming = n, c_z, c_i, K_BF16, 1 if incoming else 0
+        a.pair_act, a.pair_mask, a.ln_eps = pair_act.data_ptr(), pair_mask.data_ptr(), eps
+        for name in ("ln_in_gamma", "ln_in_beta", "left_proj_w", "left_proj_b", "left_gate_w", "left_gate_b", "right_proj_w",
+                     "right_proj_b", "right_gate_w", "right_gate_b", "ln_center_gamma", "ln_center_beta", "output_w",
+                     "output_b", "gating_w", "gating_b"):
+            setattr(a, name, w[name].data_ptr())
+        a.workspace, a.workspace_bytes = self.workspace.data_ptr(), nbytes
+        self.args = a
+
+    def run(self, stream_ptr=None) -> int:
+        return lib().kutacc_hip_triangle_multiplication(ctypes.byref(self.args), stream_ptr)

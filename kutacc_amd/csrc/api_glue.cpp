@@ -5,6 +5,8 @@
 // caller (a PyTorch extension that is not part of the repository); the operator calls in between are
 // kutacc_af2_layernorm / kutacc_af2_linear (reference src/normalization/layernorm.cpp:17-20,
 // src/linear/linear.cpp:45-50) and kutacc_af2_gating_attention (reference src/attention/gating_attention.cpp:160-200).
+// The triangle-multiplication block is assembled the same way from the steps of reference
+// src/attention/triangle_multiplication.cpp:25-150, with the two LayerNorms and the residual a caller adds around them.
 // Everything here runs on the device, on one stream, without host round trips.
 #include <hip/hip_runtime.h>
 
@@ -120,6 +122,100 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     }
     // 4. residual update; the ending node's result goes back transposed
     return kutacc_launch::residual_add(a->pair_act, ws + w.z_norm, n, n, c, ending, KUTACC_DTYPE_BF16, s);
+}
+
+int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out,
+                                       int64_t ld_out, int64_t channels, int64_t positions, float eps, int32_t dtype,
+                                       void *stream)
+{
+    return kutacc_launch::layernorm_channel_first(x, ld_x, gamma, beta, out, ld_out, channels, positions, eps, dtype,
+                                                  kutacc_api::stream_or_default(stream));
+}
+
+int64_t kutacc_hip_triangle_multiplication_workspace(int64_t n_res, int64_t c_z, int64_t c_i)
+{
+    if (n_res <= 0 || c_z <= 0 || c_i <= 0 || n_res > 65536 || c_z > 4096 || c_i > 4096) {
+        return -1;
+    }
+    return 4 * align256(n_res * n_res * (c_z > c_i ? c_z : c_i) * 2);
+}
+
+int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_args_t *a, void *stream)
+{
+    if (!a || !a->pair_act || !a->pair_mask || !a->ln_in_gamma || !a->ln_in_beta || !a->left_proj_w || !a->left_proj_b ||
+        !a->left_gate_w || !a->left_gate_b || !a->right_proj_w || !a->right_proj_b || !a->right_gate_w || !a->right_gate_b ||
+        !a->ln_center_gamma || !a->ln_center_beta || !a->output_w || !a->output_b || !a->gating_w || !a->gating_b ||
+        !a->workspace) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int64_t need = kutacc_hip_triangle_multiplication_workspace(a->n_res, a->c_z, a->c_i);
+    if (a->dtype != KUTACC_DTYPE_BF16 || need < 0 || a->workspace_bytes < need ||
+        (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int64_t n = a->n_res, cz = a->c_z, ci = a->c_i, rows = n * n, buf = need / 4;
+    char *ws = static_cast<char *>(a->workspace);
+    void *act = ws, *left = ws + buf, *right = ws + 2 * buf, *center_cf = ws + 3 * buf;
+    void *center = left, *gate = right, *out = center_cf; // each is free again by the time its second tenant arrives
+    hipStream_t s = kutacc_api::stream_or_default(stream);
+
+    // 1. layer_norm_input
+    int rc = kutacc_launch::layernorm_rows(a->pair_act, cz, a->ln_in_gamma, a->ln_in_beta, act, cz, rows, cz, a->ln_eps,
+                                           KUTACC_DTYPE_BF16, s);
+    // 2. gated projections, channel-first
+    for (int side = 0; side < 2 && rc == 0; ++side) {
+        kutacc_hip_gemm_args_t g;
+        std::memset(&g, 0, sizeof(g));
+        g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO, g.batches = 1;
+        g.m = ci, g.n = rows, g.k = cz;
+        g.a = side ? a->right_proj_w : a->left_proj_w, g.a_gate = side ? a->right_gate_w : a->left_gate_w;
+        g.a_stride_m = cz, g.a_stride_k = 1;
+        g.b = act, g.b_stride_n = cz, g.b_stride_k = 1;
+        g.c = side ? right : left, g.c_stride_m = rows;
+        g.bias = side ? a->right_proj_b : a->left_proj_b, g.bias_gate = side ? a->right_gate_b : a->left_gate_b;
+        g.bias_axis = 2, g.mask = a->pair_mask;
+        rc = kutacc_launch::pair_gemm(g, s);
+    }
+    // 3. the equation, one n x n product per channel
+    if (rc == 0) {
+        kutacc_hip_gemm_args_t g;
+        std::memset(&g, 0, sizeof(g));
+        g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO;
+        g.m = g.n = g.k = n, g.batches = ci;
+        if (!a->incoming) {
+            g.a = left, g.a_stride_m = n, g.a_stride_k = 1, g.b = right, g.b_stride_n = n, g.b_stride_k = 1;
+        } else {
+            g.a = right, g.a_stride_m = 1, g.a_stride_k = n, g.b = left, g.b_stride_n = 1, g.b_stride_k = n;
+        }
+        g.a_stride_batch = g.b_stride_batch = g.c_stride_batch = rows;
+        g.c = center_cf, g.c_stride_m = n;
+        rc = kutacc_launch::pair_gemm(g, s);
+    }
+    // 4. center_layer_norm, channel-first in, channel-last out
+    if (rc == 0) {
+        rc = kutacc_launch::layernorm_channel_first(center_cf, rows, a->ln_center_gamma, a->ln_center_beta, center, ci, ci, rows,
+                                                    a->ln_eps, KUTACC_DTYPE_BF16, s);
+    }
+    // 5. gate from the normalised input, output projection from the normalised centre
+    for (int which = 0; which < 2 && rc == 0; ++which) {
+        kutacc_hip_gemm_args_t g;
+        std::memset(&g, 0, sizeof(g));
+        g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO, g.batches = 1;
+        g.m = rows, g.n = cz, g.k = which ? ci : cz;
+        g.a = which ? center : act, g.a_stride_m = g.k, g.a_stride_k = 1;
+        g.b = which ? a->output_w : a->gating_w, g.b_stride_n = g.k, g.b_stride_k = 1;
+        g.c = which ? out : gate, g.c_stride_m = cz;
+        g.bias = which ? a->output_b : a->gating_b, g.bias_axis = 1;
+        rc = kutacc_launch::pair_gemm(g, s);
+    }
+    // 6. out *= sigmoid(gate), 7. residual
+    if (rc == 0) {
+        rc = kutacc_launch::sigmoid_gate_rows(out, n * cz, cz, gate, n * cz, cz, n, n, cz, s);
+    }
+    if (rc == 0) {
+        rc = kutacc_launch::residual_add(a->pair_act, out, n, n, cz, 0, KUTACC_DTYPE_BF16, s);
+    }
+    return rc;
 }
 
 } // extern "C"

@@ -43,6 +43,9 @@ int swap_leading_axes(const void *in, void *out, int64_t n0, int64_t n1, int64_t
 int residual_add(void *acc, const void *delta, int64_t n0, int64_t n1, int64_t inner, int swapped, int32_t dtype,
                  hipStream_t stream);
 
+int layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
+                            int64_t channels, int64_t positions, float eps, int32_t dtype, hipStream_t stream);
+
 // row_kernels.hip
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                    int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream);

@@ -119,6 +119,39 @@ __device__ __forceinline__ void panel_store(uint4 *panel, int lane, const PanelR
     panel[panel_slot(row + 24, chunk)] = p.r3;
 }
 
+// 8 x 8 transposition of 16-bit elements over the eight lanes that differ in lane bits 3, 4, 5 (same lane & 7).
+// Before: lane with index kk = lane >> 3 holds elements (kk, 0..7) as four dwords; after: elements (0..7, kk).
+// Three exchange steps in registers: halves of a dword against lane bit 3 (row rotation by 8 + byte permute;
+// `sel` must be transpose8x8_selector(lane)), dword pairs against lane bit 4 (v_permlane16_swap) and against lane
+// bit 5 (v_permlane32_swap).  Used where memory is contiguous along the index an MFMA fragment (or a row kernel)
+// wants spread over lanes.
+__device__ __forceinline__ uint32_t transpose8x8_selector(int lane)
+{
+    // even lanes of bit 3 keep their low halves and take the partner's low halves on top; odd ones the high halves
+    return (lane & 8) ? 0x03020706u : 0x05040100u;
+}
+
+__device__ __forceinline__ uint4 transpose8x8_lanes(uint4 v, uint32_t sel)
+{
+    uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t partner = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d[j], 0x128, 0xf, 0xf, false); // lane ^ 8
+        d[j] = __builtin_amdgcn_perm(partner, d[j], sel);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j += 2) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(d[j], d[j + 1], false, false);
+        d[j] = sw[0], d[j + 1] = sw[1];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(d[j], d[j + 2], false, false);
+        d[j] = sw[0], d[j + 2] = sw[1];
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
 __device__ __forceinline__ float sigmoid_fast(float x)
 {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));

@@ -95,37 +95,11 @@ __device__ __forceinline__ PanelRegs load_mmajor(const bf16_t *base, int64_t ld,
 }
 
 // Transposing store of what load_mmajor fetched: operand tile rows mrow0.., k columns kcol0...
-// Register i of lane (kk, mc) holds 8 consecutive m (8mc..8mc+7) of row k = 8i + kk; the fragment layout wants
-// 8 consecutive k of one m in a lane.  That is an 8 x 8 transposition of 16-bit elements over the eight lanes
-// that share mc (lane bits 3, 4, 5), done in three exchange steps in registers: halves of a dword against
-// lane bit 3 (row rotation by 8 + byte permute), dword pairs against lane bit 4 (v_permlane16_swap) and
-// against lane bit 5 (v_permlane32_swap).  Afterwards lane (kk, mc) holds k = 8i..8i+7 of m = 8mc + kk, one
-// 16-byte slot.
-__device__ __forceinline__ uint4 transpose8x8_lanes(uint4 v, uint32_t sel)
-{
-    uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t partner = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)d[j], 0x128, 0xf, 0xf, false); // lane ^ 8
-        d[j] = __builtin_amdgcn_perm(partner, d[j], sel);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; j += 2) {
-        const auto sw = __builtin_amdgcn_permlane16_swap(d[j], d[j + 1], false, false);
-        d[j] = sw[0], d[j + 1] = sw[1];
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const auto sw = __builtin_amdgcn_permlane32_swap(d[j], d[j + 2], false, false);
-        d[j] = sw[0], d[j + 2] = sw[1];
-    }
-    return make_uint4(d[0], d[1], d[2], d[3]);
-}
-
+// Register i of lane (kk, mc) holds 8 consecutive m (8mc..8mc+7) of row k = 8i + kk; after transpose8x8_lanes the
+// lane holds k = 8i..8i+7 of m = 8mc + kk, one 16-byte fragment slot.
 __device__ __forceinline__ void store_mmajor(uint4 *operand, int mrow0, int kcol0, int lane, const PanelRegs &p)
 {
-    // even lanes of bit 3 keep their low halves and take the partner's low halves on top; odd ones the high halves
-    const uint32_t sel = (lane & 8) ? 0x03020706u : 0x05040100u;
+    const uint32_t sel = transpose8x8_selector(lane);
     const int row = mrow0 + (lane & 7) * 8 + (lane >> 3);
     uint4 *dst = operand + (row >> 5) * 256;
     const uint4 regs[4] = {p.r0, p.r1, p.r2, p.r3};

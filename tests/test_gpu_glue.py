@@ -182,3 +182,109 @@ def test_triangle_attention_block_rejects_bad_arguments(torch_cuda):
     blk.args.nheads = 3  # 96 channels: no MFMA attention kernel
     assert blk.run() in (capi.EUNSUPPORTED, capi.EINVAL)
     torch.cuda.synchronize()
+
+
+# ---- channel-first LayerNorm and the triangle-multiplication block ------------------------------------------------
+@pytest.mark.parametrize("channels,positions,dtype", [(128, 4096, "bfloat16"), (128, 1000, "bfloat16"), (128, 40, "bfloat16"),
+                                                      (96, 77, "bfloat16"), (20, 33, "float32")])
+def test_layernorm_channel_first(torch_cuda, channels, positions, dtype):
+    """Against the oracle's row LayerNorm on the transposed tensor: fast path (128 channels, ragged position counts) and
+    the generic kernel."""
+    from oracle import oracle
+    torch = torch_cuda
+    dt = getattr(torch, dtype)
+    rng = np.random.Generator(np.random.PCG64(31 + positions))
+    x = (rng.standard_normal((channels, positions)) * 2 + rng.standard_normal((1, positions))).astype(np.float32)
+    if dtype == "bfloat16":
+        x = round_to_bf16(x)
+    gamma = (rng.random(channels) + 0.5).astype(np.float32)
+    beta = (rng.standard_normal(channels) * 0.2).astype(np.float32)
+    dx = torch.from_numpy(x).to(device="cuda", dtype=dt)
+    out = torch.full((positions, channels + 8), 9.0, dtype=dt, device="cuda")
+    g, b = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    rc = capi.lib().kutacc_hip_layernorm_channel_first(dx.data_ptr(), positions, g.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                       channels + 8, channels, positions, 1e-5, code(torch, dx), None)
+    torch.cuda.synchronize()
+    assert rc == 0
+    ref = oracle.layernorm_rows_f32(np.ascontiguousarray(x.T), gamma, beta, 1e-5)
+    helpers.check_close(helpers.to_numpy(out[:, :channels]), ref, "bf16" if dtype == "bfloat16" else "fp32", "channel-first LN")
+    assert bool((out[:, channels:] == 9.0).all())
+
+
+def tm_block_case(seed, n, c_z, c_i):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    w = lambda o, i: round_to_bf16((rng.standard_normal((o, i)) / math.sqrt(i)).astype(np.float32))  # noqa: E731
+    b = lambda k: (rng.standard_normal(k) * 0.3).astype(np.float32)  # noqa: E731
+    g = lambda k: (rng.random(k) + 0.5).astype(np.float32)  # noqa: E731
+    return dict(z=round_to_bf16(rng.standard_normal((n, n, c_z)).astype(np.float32)),
+                mask=(rng.random((n, n)) > 0.15).astype(np.float32),
+                ln_in_gamma=g(c_z), ln_in_beta=b(c_z), left_proj_w=w(c_i, c_z), left_proj_b=b(c_i), left_gate_w=w(c_i, c_z),
+                left_gate_b=b(c_i), right_proj_w=w(c_i, c_z), right_proj_b=b(c_i), right_gate_w=w(c_i, c_z), right_gate_b=b(c_i),
+                ln_center_gamma=g(c_i), ln_center_beta=b(c_i), output_w=w(c_z, c_i), output_b=b(c_z), gating_w=w(c_z, c_z),
+                gating_b=b(c_z))
+
+
+def tm_block_oracle(c, incoming):
+    """AlphaFold's TriangleMultiplication in numpy on the oracle's operators (fp32, no intermediate rounding)."""
+    from oracle import oracle
+    n, _, c_z = c["z"].shape
+    c_i = c["left_proj_w"].shape[0]
+    act = oracle.layernorm_rows_f32(c["z"].reshape(-1, c_z), c["ln_in_gamma"], c["ln_in_beta"], 1e-5).reshape(n, n, c_z)
+    left = oracle.tm_calc_proj_f32(act, c["mask"], c["left_proj_w"], c["left_proj_b"], c["left_gate_w"], c["left_gate_b"])
+    right = oracle.tm_calc_proj_f32(act, c["mask"], c["right_proj_w"], c["right_proj_b"], c["right_gate_w"], c["right_gate_b"])
+    center = oracle.tm_equation_f32(left, right, incoming)
+    center = oracle.layernorm_rows_f32(np.ascontiguousarray(center.transpose(1, 2, 0)).reshape(-1, c_i), c["ln_center_gamma"],
+                                       c["ln_center_beta"], 1e-5)
+    gate, out = oracle.tm_gate_and_out_f32(act, center, c["gating_w"], c["gating_b"], c["output_w"], c["output_b"])
+    return c["z"] + oracle.tm_last_f32(out, gate).reshape(n, n, c_z)
+
+
+@pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
+@pytest.mark.parametrize("n,c_z,c_i", [(48, 128, 128), (40, 64, 32), (9, 12, 6)])
+def test_triangle_multiplication_block_against_the_oracle(torch_cuda, n, c_z, c_i, incoming):
+    torch = torch_cuda
+    c = tm_block_case(800 + n, n, c_z, c_i)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    pair = dev(c["z"])
+    w = {k: dev(v) for k, v in c.items() if k not in ("z", "mask")}
+    blk = capi.TriangleMultiplicationBlock(pair, dev(c["mask"]), w, incoming)
+    rc = blk.run()
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    helpers.check_close(helpers.to_numpy(pair), tm_block_oracle(c, incoming), "bf16", f"TM block n={n} incoming={incoming}")
+
+
+@pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
+def test_triangle_multiplication_block_full_size(torch_cuda, incoming):
+    """384 residues, 128 channels, the real shape.  The oracle follows a sample of output positions (i, j) through the
+    whole block: their centre needs the left projections of row i and the right projections of row j (columns for the
+    incoming form), which the oracle computes for just those rows."""
+    from oracle import oracle
+    torch = torch_cuda
+    n, c = 384, 128
+    case = tm_block_case(900, n, c, c)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    w = {k: dev(v) for k, v in case.items() if k not in ("z", "mask")}
+    pair = dev(case["z"])
+    assert capi.TriangleMultiplicationBlock(pair, dev(case["mask"]), w, incoming).run() == 0
+    torch.cuda.synchronize()
+    got = helpers.to_numpy(pair)
+    I, J = [0, 77, 200, 383], [5, 100, 383]
+    act = oracle.layernorm_rows_f32(case["z"].reshape(-1, c), case["ln_in_gamma"], case["ln_in_beta"], 1e-5).reshape(n, n, c)
+    proj = lambda side, x, m: oracle.tm_calc_proj_f32(x, m, case[side + "_proj_w"], case[side + "_proj_b"],  # noqa: E731
+                                                       case[side + "_gate_w"], case[side + "_gate_b"])
+    if not incoming:  # center[c, i, j] = sum_k left[c, i, k] right[c, j, k]
+        left, right = proj("left", act[I], case["mask"][I]), proj("right", act[J], case["mask"][J])
+        center = np.einsum("cik,cjk->ijc", left.astype(np.float64), right.astype(np.float64))
+    else:             # center[c, i, j] = sum_k right[c, k, i] left[c, k, j]
+        right = proj("right", np.ascontiguousarray(act[:, I]), np.ascontiguousarray(case["mask"][:, I]))
+        left = proj("left", np.ascontiguousarray(act[:, J]), np.ascontiguousarray(case["mask"][:, J]))
+        center = np.einsum("cki,ckj->ijc", right.astype(np.float64), left.astype(np.float64))
+    center = oracle.layernorm_rows_f32(center.reshape(-1, c).astype(np.float32), case["ln_center_gamma"], case["ln_center_beta"], 1e-5)
+    act_ij = act[np.ix_(I, J)].reshape(-1, c)
+    gate, out = oracle.tm_gate_and_out_f32(act_ij, center, case["gating_w"], case["gating_b"], case["output_w"], case["output_b"])
+    want = case["z"][np.ix_(I, J)].reshape(-1, c) + oracle.tm_last_f32(out, gate)
+    helpers.check_close(got[np.ix_(I, J)].reshape(-1, c), want, "bf16", f"TM block 384 incoming={incoming}")
+    assert not np.array_equal(got, case["z"])
