@@ -273,6 +273,15 @@ kutacc_export int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x
                                                      void *out, int64_t ld_out, int64_t channels, int64_t positions,
                                                      float eps, int32_t dtype, void *stream);
 
+/* acc[m, n] += bf16(sum_k a[m, k] * w[n, k] + bias[n]) * sigmoid(gate[m, n]) in one pass: the output projection of the
+ * triangle multiplication with its gating (kutacc::last, reference src/attention/triangle_multiplication.cpp:129-150)
+ * and the residual update folded into the epilogue.  bf16; k in {128, 256}, n a multiple of 128, w dense [n, k], row
+ * strides multiples of 8 elements, 16-byte aligned pointers; otherwise KUTACC_HIP_EUNSUPPORTED (run
+ * kutacc_hip_gemm, kutacc_hip_sigmoid_gate_rows and kutacc_hip_residual_add instead). */
+kutacc_export int kutacc_hip_gated_residual_projection(const void *a, int64_t a_ld, const void *w, const float *bias,
+                                                       const void *gate, int64_t gate_ld, void *acc, int64_t acc_ld,
+                                                       int64_t m, int64_t n, int64_t k, int32_t dtype, void *stream);
+
 /*
  * One triangle-multiplication block of the pair stack, in place (outgoing or incoming edges):
  *   act    = LN_in(pair_act)
@@ -280,8 +289,9 @@ kutacc_export int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x
  *   center = sum_k left[i, k] * right[j, k]   (outgoing)      or      sum_k right[k, i] * left[k, j]   (incoming)
  *   pair_act += (LN_center(center) . output_w^T + output_b) * sigmoid(act . gating_w^T + gating_b)
  * i.e. the four kutacc_af2_triangle_multiplication_* steps (reference src/attention/triangle_multiplication.cpp:25-150)
- * with the two LayerNorms, the layout change and the residual a caller of the reference adds around them; nine
- * launches on `stream`.  bf16; weights stored [out, in]: *_proj_w, *_gate_w [c_i, c_z], output_w [c_z, c_i], gating_w
+ * with the two LayerNorms, the layout change and the residual a caller of the reference adds around them; seven
+ * launches on `stream` (the output projection, its gating and the residual are one kernel when c_i is 128 or 256
+ * and c_z a multiple of 128).  bf16; weights stored [out, in]: *_proj_w, *_gate_w [c_i, c_z], output_w [c_z, c_i], gating_w
  * [c_z, c_z]; all biases and LayerNorm parameters fp32.  `workspace`: device memory, 256-byte aligned, at least
  * kutacc_hip_triangle_multiplication_workspace(n_res, c_z, c_i) bytes.
  */

@@ -132,6 +132,17 @@ int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x, const float 
                                                   kutacc_api::stream_or_default(stream));
 }
 
+int kutacc_hip_gated_residual_projection(const void *a, int64_t a_ld, const void *w, const float *bias, const void *gate,
+                                         int64_t gate_ld, void *acc, int64_t acc_ld, int64_t m, int64_t n, int64_t k,
+                                         int32_t dtype, void *stream)
+{
+    if (!a || !w || !bias || !gate || !acc || m <= 0 || n <= 0 || k <= 0 || dtype != KUTACC_DTYPE_BF16) {
+        return KUTACC_HIP_EINVAL;
+    }
+    return kutacc_launch::row_projection_gated_residual(a, a_ld, w, bias, gate, gate_ld, acc, acc_ld, m, n, k,
+                                                        kutacc_api::stream_or_default(stream));
+}
+
 int64_t kutacc_hip_triangle_multiplication_workspace(int64_t n_res, int64_t c_z, int64_t c_i)
 {
     if (n_res <= 0 || c_z <= 0 || c_i <= 0 || n_res > 65536 || c_z > 4096 || c_i > 4096) {
@@ -196,24 +207,40 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
         rc = kutacc_launch::layernorm_channel_first(center_cf, rows, a->ln_center_gamma, a->ln_center_beta, center, ci, ci, rows,
                                                     a->ln_eps, KUTACC_DTYPE_BF16, s);
     }
-    // 5. gate from the normalised input, output projection from the normalised centre
-    for (int which = 0; which < 2 && rc == 0; ++which) {
+    // 5. gate from the normalised input
+    if (rc == 0) {
         kutacc_hip_gemm_args_t g;
         std::memset(&g, 0, sizeof(g));
         g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO, g.batches = 1;
-        g.m = rows, g.n = cz, g.k = which ? ci : cz;
-        g.a = which ? center : act, g.a_stride_m = g.k, g.a_stride_k = 1;
-        g.b = which ? a->output_w : a->gating_w, g.b_stride_n = g.k, g.b_stride_k = 1;
-        g.c = which ? out : gate, g.c_stride_m = cz;
-        g.bias = which ? a->output_b : a->gating_b, g.bias_axis = 1;
+        g.m = rows, g.n = cz, g.k = cz;
+        g.a = act, g.a_stride_m = cz, g.a_stride_k = 1;
+        g.b = a->gating_w, g.b_stride_n = cz, g.b_stride_k = 1;
+        g.c = gate, g.c_stride_m = cz;
+        g.bias = a->gating_b, g.bias_axis = 1;
         rc = kutacc_launch::pair_gemm(g, s);
     }
-    // 6. out *= sigmoid(gate), 7. residual
+    // 6. output projection of the normalised centre, times sigmoid(gate), added to the pair activation: one kernel
+    //    when the shape allows, else projection, gating and residual as three passes
     if (rc == 0) {
-        rc = kutacc_launch::sigmoid_gate_rows(out, n * cz, cz, gate, n * cz, cz, n, n, cz, s);
-    }
-    if (rc == 0) {
-        rc = kutacc_launch::residual_add(a->pair_act, out, n, n, cz, 0, KUTACC_DTYPE_BF16, s);
+        rc = kutacc_launch::row_projection_gated_residual(center, ci, a->output_w, a->output_b, gate, cz, a->pair_act, cz, rows,
+                                                          cz, ci, s);
+        if (rc == KUTACC_HIP_EUNSUPPORTED) {
+            kutacc_hip_gemm_args_t g;
+            std::memset(&g, 0, sizeof(g));
+            g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO, g.batches = 1;
+            g.m = rows, g.n = cz, g.k = ci;
+            g.a = center, g.a_stride_m = ci, g.a_stride_k = 1;
+            g.b = a->output_w, g.b_stride_n = ci, g.b_stride_k = 1;
+            g.c = out, g.c_stride_m = cz;
+            g.bias = a->output_b, g.bias_axis = 1;
+            rc = kutacc_launch::pair_gemm(g, s);
+            if (rc == 0) {
+                rc = kutacc_launch::sigmoid_gate_rows(out, n * cz, cz, gate, n * cz, cz, n, n, cz, s);
+            }
+            if (rc == 0) {
+                rc = kutacc_launch::residual_add(a->pair_act, out, n, n, cz, 0, KUTACC_DTYPE_BF16, s);
+            }
+        }
     }
     return rc;
 }

@@ -1100,10 +1100,14 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 // slab of Wo once and its four waves walk 32-row tiles.  The product is formed transposed
 // (rows = output features, columns = tokens), which leaves every lane with 4 consecutive features
 // of its own token per accumulator group -- an 8-byte panel write.
-template <int C>
+// GATED_RESIDUAL: the rounded result is not stored but folded into `out`, out += result * sigmoid(gate), with gate
+// and out read in the order they are written, 16 bytes per lane -- the last two steps of the triangle multiplication
+// (reference src/attention/triangle_multiplication.cpp:129-150) and the residual update fused into its output
+// projection.
+template <int C, bool GATED_RESIDUAL>
 __global__ __launch_bounds__(256, 2) void output_projection_kernel(
     const bf16_t *__restrict__ avg, int64_t avg_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
-    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave)
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave, const bf16_t *__restrict__ gate, int64_t gate_ld)
 {
     constexpr int CK = C / 16;
     constexpr int NP = CK / 4;
@@ -1173,6 +1177,17 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
         }
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
+            uint4 gq[4], zq[4];
+            if constexpr (GATED_RESIDUAL) { // requested before the MFMAs, used after them
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    int64_t row = (int64_t)row0 + 8 * i + (lane >> 3);
+                    row = row < stop ? row : stop - 1;
+                    const int64_t col = n0 + half * 64 + (lane & 7) * 8;
+                    gq[i] = *reinterpret_cast<const uint4 *>(gate + row * gate_ld + col);
+                    zq[i] = *reinterpret_cast<const uint4 *>(out + row * out_ld + col);
+                }
+            }
             f32x16 acc[2];
             acc[0] = zero16(), acc[1] = zero16();
 #pragma unroll
@@ -1200,8 +1215,19 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int prow_ = 8 * i + (lane >> 3);
-                const uint4 v = panel[panel_slot(prow_, lane & 7)];
+                uint4 v = panel[panel_slot(prow_, lane & 7)];
                 const int64_t row = (int64_t)row0 + prow_;
+                if constexpr (GATED_RESIDUAL) {
+                    const bf16x8 o = as_bf16x8(v), gt = as_bf16x8(gq[i]), z = as_bf16x8(zq[i]);
+                    bf16x8 res;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        // bf16(out * sigmoid(gate)) as the reference stores it, then the residual sum in fp32
+                        const float upd = to_f32((bf16_t)(to_f32(o[e]) * sigmoid_fast(to_f32(gt[e]))));
+                        res[e] = (bf16_t)(to_f32(z[e]) + upd);
+                    }
+                    v = as_uint4(res);
+                }
                 if (row < stop) {
                     *reinterpret_cast<uint4 *>(out + row * out_ld + n0 + half * 64 + (lane & 7) * 8) = v;
                 }
@@ -1417,11 +1443,11 @@ int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t strea
 }
 
 // out[M, N] = a[M, K] . w[N, K]^T + bias with K = C and N a multiple of 128 (one grid row per 128-feature slab)
-template <int C>
+template <int C, bool GATED_RESIDUAL = false>
 int launch_output_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld,
-                             int64_t M, int64_t N, hipStream_t stream)
+                             int64_t M, int64_t N, hipStream_t stream, const void *gate = nullptr, int64_t gate_ld = 0)
 {
-    auto kern = output_projection_kernel<C>;
+    auto kern = output_projection_kernel<C, GATED_RESIDUAL>;
     const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16 + 4 * 4096;
     static size_t configured = 0;
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
@@ -1434,7 +1460,7 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
     gx = gx > cap ? cap : gx;
     const int64_t rpw = ((M + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
     kern<<<dim3((unsigned)gx, (unsigned)(N / 128)), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)rpw);
+        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)rpw, (const bf16_t *)gate, gate_ld);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -1559,6 +1585,19 @@ int row_projection(const void *a, int64_t a_ld, const void *w, const float *bias
     kutacc_prof::KernelTimer t("output_projection_kernel", 2.0 * (double)m * (double)n * (double)k, stream);
     return k == 128 ? launch_output_projection<128>(a, a_ld, w, bias, out, out_ld, m, n, stream)
                     : launch_output_projection<256>(a, a_ld, w, bias, out, out_ld, m, n, stream);
+}
+
+// acc[m, n] += bf16(sum_k a[m, k] * w[n, k] + bias[n]) * sigmoid(gate[m, n]): same shapes as row_projection
+int row_projection_gated_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *gate,
+                                  int64_t gate_ld, void *acc, int64_t acc_ld, int64_t m, int64_t n, int64_t k,
+                                  hipStream_t stream)
+{
+    if (!row_projection_supports(a, a_ld, w, bias, acc, acc_ld, m, n, k) || !gate || gate_ld % 8 != 0 || !aligned(gate, 16)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    kutacc_prof::KernelTimer t("output_projection_kernel<gated residual>", 2.0 * (double)m * (double)n * (double)k, stream);
+    return k == 128 ? launch_output_projection<128, true>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld)
+                    : launch_output_projection<256, true>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld);
 }
 
 } // namespace kutacc_launch

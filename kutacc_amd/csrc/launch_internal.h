@@ -25,6 +25,10 @@ bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const f
 int row_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld, int64_t m,
                    int64_t n, int64_t k, hipStream_t stream);
 
+int row_projection_gated_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *gate,
+                                  int64_t gate_ld, void *acc, int64_t acc_ld, int64_t m, int64_t n, int64_t k,
+                                  hipStream_t stream);
+
 // global_attention.hip
 int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);
 

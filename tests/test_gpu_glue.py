@@ -288,3 +288,28 @@ def test_triangle_multiplication_block_full_size(torch_cuda, incoming):
     want = case["z"][np.ix_(I, J)].reshape(-1, c) + oracle.tm_last_f32(out, gate)
     helpers.check_close(got[np.ix_(I, J)].reshape(-1, c), want, "bf16", f"TM block 384 incoming={incoming}")
     assert not np.array_equal(got, case["z"])
+
+
+@pytest.mark.parametrize("m,n,k", [(1000, 128, 128), (333, 256, 128), (520, 128, 256)])
+def test_gated_residual_projection(torch_cuda, m, n, k):
+    """acc += bf16(a . w^T + bias) * sigmoid(gate) in one kernel, against the same three steps in float64."""
+    torch = torch_cuda
+    rng = np.random.Generator(np.random.PCG64(40 + m))
+    a = round_to_bf16(rng.standard_normal((m, k)).astype(np.float32))
+    w = round_to_bf16((rng.standard_normal((n, k)) / math.sqrt(k)).astype(np.float32))
+    bias = (rng.standard_normal(n) * 0.3).astype(np.float32)
+    gate = round_to_bf16(rng.standard_normal((m, n)).astype(np.float32) * 2)
+    acc = round_to_bf16(rng.standard_normal((m, n)).astype(np.float32))
+    dev = lambda x, dt=torch.bfloat16: torch.from_numpy(x).to(device="cuda", dtype=dt)  # noqa: E731
+    d_acc = dev(acc)
+    t = [dev(a), dev(w), dev(bias, torch.float32), dev(gate)]
+    rc = capi.lib().kutacc_hip_gated_residual_projection(t[0].data_ptr(), k, t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr(), n,
+                                                         d_acc.data_ptr(), n, m, n, k, capi.K_BF16, None)
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    o = a.astype(np.float64) @ w.astype(np.float64).T + bias
+    want = acc + o / (1.0 + np.exp(-gate.astype(np.float64)))
+    helpers.check_close(helpers.to_numpy(d_acc), want, "bf16", "gated residual projection")
+    rc = capi.lib().kutacc_hip_gated_residual_projection(t[0].data_ptr(), k, t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr(), n,
+                                                         d_acc.data_ptr(), n, m, 96, k, capi.K_BF16, None)
+    assert rc == capi.EUNSUPPORTED
