@@ -22,7 +22,7 @@ constexpr int64_t HEAD = 32;
 inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 struct Workspace {
-    int64_t z_norm, nb, bias, q, avg, total; // byte offsets; z_norm doubles as the attention output
+    int64_t z_norm, nb, bias, q, avg, total; // byte offsets
 };
 
 Workspace layout(int64_t n, int64_t heads)
@@ -102,7 +102,7 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n * n, g.nb_stride_q = n;
     g.q = ws + w.q, g.q_stride_b = n * c, g.q_stride_s = c, g.q_stride_h = HEAD;
     g.avg = ws + w.avg, g.avg_stride_b = n * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
-    g.out = ws + w.z_norm, g.out_ld = c; // the normalised input is dead once the head kernel has run
+    g.out = a->pair_act, g.out_ld = c;
     if (!kutacc_launch::fused_attention_supports(g)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
@@ -116,12 +116,9 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     if ((rc = kutacc_launch::mask_bias(a->pair_mask, ws + w.bias, n, n, ending, KUTACC_DTYPE_BF16, s)) != 0) {
         return rc;
     }
-    // 3. the operator
-    if ((rc = kutacc_launch::gating_attention_fused(g, s)) != 0) {
-        return rc;
-    }
-    // 4. residual update; the ending node's result goes back transposed
-    return kutacc_launch::residual_add(a->pair_act, ws + w.z_norm, n, n, c, ending, KUTACC_DTYPE_BF16, s);
+    // 3. the operator, its output projection adding straight into the pair activation (transposed back for the ending
+    //    node): the residual update costs no pass of its own
+    return kutacc_launch::gating_attention_fused(g, s, ending ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD);
 }
 
 int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out,

@@ -1100,15 +1100,27 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 // slab of Wo once and its four waves walk 32-row tiles.  The product is formed transposed
 // (rows = output features, columns = tokens), which leaves every lane with 4 consecutive features
 // of its own token per accumulator group -- an 8-byte panel write.
-// GATED_RESIDUAL: the rounded result is not stored but folded into `out`, out += result * sigmoid(gate), with gate
-// and out read in the order they are written, 16 bytes per lane -- the last two steps of the triangle multiplication
-// (reference src/attention/triangle_multiplication.cpp:129-150) and the residual update fused into its output
-// projection.
-template <int C, bool GATED_RESIDUAL>
+// EPILOGUE 1 (gated residual): the rounded result is not stored but folded into `out`, out += result * sigmoid(gate),
+// with gate and out read in the order they are written, 16 bytes per lane -- the last two steps of the triangle
+// multiplication (reference src/attention/triangle_multiplication.cpp:129-150) and the residual update fused into
+// its output projection.  EPILOGUE 2 (residual): out += result, where row (i, j) of the result goes to row (j, i)
+// of `out` when swap_n != 0 (rows are pairs of an n x n grid): the residual update of a triangle-attention block,
+// transposed back for the ending node.
+constexpr int EPILOGUE_STORE = 0, EPILOGUE_GATED_RESIDUAL = 1, EPILOGUE_RESIDUAL = 2;
+
+template <int C, int EPILOGUE>
 __global__ __launch_bounds__(256, 2) void output_projection_kernel(
     const bf16_t *__restrict__ avg, int64_t avg_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
-    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave, const bf16_t *__restrict__ gate, int64_t gate_ld)
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave, const bf16_t *__restrict__ gate, int64_t gate_ld,
+    int64_t swap_n)
 {
+    // row of `out` that receives row `row` of the result
+    auto target_row = [&](int64_t row) -> int64_t {
+        if constexpr (EPILOGUE == EPILOGUE_RESIDUAL) {
+            return swap_n ? (row % swap_n) * swap_n + row / swap_n : row;
+        }
+        return row;
+    };
     constexpr int CK = C / 16;
     constexpr int NP = CK / 4;
     extern __shared__ uint4 lds[]; // W slab [4 feature blocks][CK][64 lanes], then 4 panels of 256
@@ -1178,14 +1190,16 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
             uint4 gq[4], zq[4];
-            if constexpr (GATED_RESIDUAL) { // requested before the MFMAs, used after them
+            if constexpr (EPILOGUE != EPILOGUE_STORE) { // requested before the MFMAs, used after them
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     int64_t row = (int64_t)row0 + 8 * i + (lane >> 3);
                     row = row < stop ? row : stop - 1;
                     const int64_t col = n0 + half * 64 + (lane & 7) * 8;
-                    gq[i] = *reinterpret_cast<const uint4 *>(gate + row * gate_ld + col);
-                    zq[i] = *reinterpret_cast<const uint4 *>(out + row * out_ld + col);
+                    if constexpr (EPILOGUE == EPILOGUE_GATED_RESIDUAL) {
+                        gq[i] = *reinterpret_cast<const uint4 *>(gate + row * gate_ld + col);
+                    }
+                    zq[i] = *reinterpret_cast<const uint4 *>(out + target_row(row) * out_ld + col);
                 }
             }
             f32x16 acc[2];
@@ -1217,7 +1231,7 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
                 const int prow_ = 8 * i + (lane >> 3);
                 uint4 v = panel[panel_slot(prow_, lane & 7)];
                 const int64_t row = (int64_t)row0 + prow_;
-                if constexpr (GATED_RESIDUAL) {
+                if constexpr (EPILOGUE == EPILOGUE_GATED_RESIDUAL) {
                     const bf16x8 o = as_bf16x8(v), gt = as_bf16x8(gq[i]), z = as_bf16x8(zq[i]);
                     bf16x8 res;
 #pragma unroll
@@ -1227,9 +1241,17 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
                         res[e] = (bf16_t)(to_f32(z[e]) + upd);
                     }
                     v = as_uint4(res);
+                } else if constexpr (EPILOGUE == EPILOGUE_RESIDUAL) {
+                    const bf16x8 o = as_bf16x8(v), z = as_bf16x8(zq[i]);
+                    bf16x8 res;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        res[e] = (bf16_t)(to_f32(z[e]) + to_f32(o[e]));
+                    }
+                    v = as_uint4(res);
                 }
                 if (row < stop) {
-                    *reinterpret_cast<uint4 *>(out + row * out_ld + n0 + half * 64 + (lane & 7) * 8) = v;
+                    *reinterpret_cast<uint4 *>(out + target_row(row) * out_ld + n0 + half * 64 + (lane & 7) * 8) = v;
                 }
             }
         }
@@ -1443,11 +1465,12 @@ int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t strea
 }
 
 // out[M, N] = a[M, K] . w[N, K]^T + bias with K = C and N a multiple of 128 (one grid row per 128-feature slab)
-template <int C, bool GATED_RESIDUAL = false>
+template <int C, int EPILOGUE = EPILOGUE_STORE>
 int launch_output_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld,
-                             int64_t M, int64_t N, hipStream_t stream, const void *gate = nullptr, int64_t gate_ld = 0)
+                             int64_t M, int64_t N, hipStream_t stream, const void *gate = nullptr, int64_t gate_ld = 0,
+                             int64_t swap_n = 0)
 {
-    auto kern = output_projection_kernel<C, GATED_RESIDUAL>;
+    auto kern = output_projection_kernel<C, EPILOGUE>;
     const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16 + 4 * 4096;
     static size_t configured = 0;
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
@@ -1460,7 +1483,8 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
     gx = gx > cap ? cap : gx;
     const int64_t rpw = ((M + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
     kern<<<dim3((unsigned)gx, (unsigned)(N / 128)), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)rpw, (const bf16_t *)gate, gate_ld);
+        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)rpw, (const bf16_t *)gate, gate_ld,
+        swap_n);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -1494,7 +1518,7 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
     return make_plan(a.seq_len, (int)C, pl);
 }
 
-int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t stream)
+int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t stream, int residual)
 {
     const int C = (int)(a.nheads * a.head_size);
     Plan pl;
@@ -1560,8 +1584,20 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
             return rc;
         }
     }
-    kutacc_prof::KernelTimer t("output_projection_kernel", 2.0 * BS * C * C, stream);
     const int64_t M = a.batch * a.seq_len;
+    if (residual != FUSED_OUT_STORE) {
+        // out += result, row (b, s) of the result going to row (s, b) of out in the transposed form
+        if (residual == FUSED_OUT_ADD_TRANSPOSED && a.batch != a.seq_len) {
+            return KUTACC_HIP_EINVAL;
+        }
+        const int64_t swap_n = residual == FUSED_OUT_ADD_TRANSPOSED ? a.seq_len : 0;
+        kutacc_prof::KernelTimer t("output_projection_kernel<residual>", 2.0 * BS * C * C, stream);
+        return (C == 128) ? launch_output_projection<128, EPILOGUE_RESIDUAL>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out,
+                                                                             a.out_ld, M, C, stream, nullptr, 0, swap_n)
+                          : launch_output_projection<256, EPILOGUE_RESIDUAL>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out,
+                                                                             a.out_ld, M, C, stream, nullptr, 0, swap_n);
+    }
+    kutacc_prof::KernelTimer t("output_projection_kernel", 2.0 * BS * C * C, stream);
     return (C == 128) ? launch_output_projection<128>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out, a.out_ld, M, C, stream)
                       : launch_output_projection<256>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out, a.out_ld, M, C, stream);
 }
@@ -1596,8 +1632,8 @@ int row_projection_gated_residual(const void *a, int64_t a_ld, const void *w, co
         return KUTACC_HIP_EUNSUPPORTED;
     }
     kutacc_prof::KernelTimer t("output_projection_kernel<gated residual>", 2.0 * (double)m * (double)n * (double)k, stream);
-    return k == 128 ? launch_output_projection<128, true>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld)
-                    : launch_output_projection<256, true>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld);
+    return k == 128 ? launch_output_projection<128, EPILOGUE_GATED_RESIDUAL>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld)
+                    : launch_output_projection<256, EPILOGUE_GATED_RESIDUAL>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld);
 }
 
 } // namespace kutacc_launch

@@ -18,7 +18,10 @@ int gemm_nt(int32_t dtype, const void *a, int64_t lda, const void *w, int64_t ld
 
 // fused_attention.hip
 bool fused_attention_supports(const kutacc_hip_attention_args_t &args);
-int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream);
+// `residual`: what the output projection does with its result -- store it in args.out (the operator as the reference
+// defines it), add it to args.out, or add row (b, s) of it to row (s, b) of args.out (batch == seq_len)
+constexpr int FUSED_OUT_STORE = 0, FUSED_OUT_ADD = 1, FUSED_OUT_ADD_TRANSPOSED = 2;
+int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream, int residual = FUSED_OUT_STORE);
 
 bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
                              int64_t m, int64_t n, int64_t k);
