@@ -182,6 +182,16 @@ def pair_stack_rates(config, reps=20):
     tr = capi.Transition(x, bf(hid, c_o, scale=c_o ** -0.5), f32(hid), bf(c_o, hid, scale=hid ** -0.5), f32(c_o), mid, out)
     report("transition", timed(tr.run), 4.0 * rows * c_o * hid, 2.0 * rows * 2 * c_o)  # input and output; the hidden layer stays on chip
     del mid
+    # the whole block in place: act += transition(LN(act)), one kernel
+    zb = x.clone().reshape(rows, c_o)
+    gam, bet = torch.ones(c_o, device="cuda"), torch.zeros(c_o, device="cuda")
+    tw1, tb1, tw2, tb2 = bf(hid, c_o, scale=c_o ** -0.5), f32(hid), bf(c_o, hid, scale=hid ** -0.5) * 0.1, f32(c_o) * 0.1
+
+    def run_tb():
+        assert capi.lib().kutacc_hip_transition_block(zb.data_ptr(), gam.data_ptr(), bet.data_ptr(), 1e-5, tw1.data_ptr(),
+                                                      tb1.data_ptr(), tw2.data_ptr(), tb2.data_ptr(), None, 0, rows, c_o, hid,
+                                                      capi.K_BF16, stream) == 0
+    report("transition_block (LN + transition + residual)", timed(run_tb), 4.0 * rows * c_o * hid, 2.0 * rows * 2 * c_o)
     # triangle multiplication
     keep = [bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i), bf(c_i, c_o, scale=c_o ** -0.5), f32(c_i)]
     h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]

@@ -326,6 +326,20 @@ typedef struct kutacc_hip_triangle_multiplication_args {
 kutacc_export int64_t kutacc_hip_triangle_multiplication_workspace(int64_t n_res, int64_t c_z, int64_t c_i);
 kutacc_export int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_args_t *args, void *stream);
 
+/*
+ * One transition block in place: act += relu(LN(act) . w1^T + b1) . w2^T + b2 over `rows` dense rows of c_o channels
+ * (kutacc_af2_transition, reference src/attention/transition.cpp:21-39, with the LayerNorm in front of it and the
+ * residual behind it that a caller of the reference runs itself).  bf16.  With c_o in {128, 256} and c_i a multiple of
+ * 64 (<= 2048) this is one kernel and one read and one write of the activation; `workspace` may then be NULL.
+ * Other shapes run LayerNorm, the two GEMMs and the residual as separate passes through `workspace` (256-byte
+ * aligned, kutacc_hip_transition_block_workspace(rows, c_o, c_i) bytes).
+ */
+kutacc_export int64_t kutacc_hip_transition_block_workspace(int64_t rows, int64_t c_o, int64_t c_i);
+kutacc_export int kutacc_hip_transition_block(void *act, const float *ln_gamma, const float *ln_beta, float ln_eps,
+                                              const void *w1, const float *b1, const void *w2, const float *b2,
+                                              void *workspace, int64_t workspace_bytes, int64_t rows, int64_t c_o,
+                                              int64_t c_i, int32_t dtype, void *stream);
+
 /* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.

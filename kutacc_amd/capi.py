@@ -148,7 +148,7 @@ DECLARED_SYMBOLS = [
     "kutacc_hip_pair_bias_transposed", "kutacc_hip_mask_bias", "kutacc_hip_swap_leading_axes", "kutacc_hip_residual_add",
     "kutacc_hip_triangle_attention_workspace", "kutacc_hip_triangle_attention", "kutacc_hip_layernorm_channel_first",
     "kutacc_hip_triangle_multiplication_workspace", "kutacc_hip_triangle_multiplication",
-    "kutacc_hip_gated_residual_projection",
+    "kutacc_hip_gated_residual_projection", "kutacc_hip_transition_block_workspace", "kutacc_hip_transition_block",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
@@ -236,6 +236,11 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_triangle_multiplication.restype = ctypes.c_int
     L.kutacc_hip_gated_residual_projection.argtypes = [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _i32, _vp]
     L.kutacc_hip_gated_residual_projection.restype = ctypes.c_int
+    L.kutacc_hip_transition_block_workspace.argtypes = [_i64, _i64, _i64]
+    L.kutacc_hip_transition_block_workspace.restype = _i64
+    L.kutacc_hip_transition_block.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                                              _i32, _vp]
+    L.kutacc_hip_transition_block.restype = ctypes.c_int
     L.kutacc_hip_set_stream.argtypes = [_vp]
     L.kutacc_hip_get_stream.restype = _vp
     L.kutacc_hip_set_blocking.argtypes = [ctypes.c_int]

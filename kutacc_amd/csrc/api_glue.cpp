@@ -10,6 +10,7 @@
 // Everything here runs on the device, on one stream, without host round trips.
 #include <hip/hip_runtime.h>
 
+#include <climits>
 #include <cstring>
 
 #include "api_internal.h"
@@ -238,6 +239,47 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
                 rc = kutacc_launch::residual_add(a->pair_act, out, n, n, cz, 0, KUTACC_DTYPE_BF16, s);
             }
         }
+    }
+    return rc;
+}
+
+int64_t kutacc_hip_transition_block_workspace(int64_t rows, int64_t c_o, int64_t c_i)
+{
+    if (rows <= 0 || c_o <= 0 || c_i <= 0 || rows > INT64_MAX / 4 / (c_o + c_i)) {
+        return -1;
+    }
+    if ((c_o == 128 || c_o == 256) && c_i % 64 == 0 && c_i <= 2048) {
+        return 0; // the one-kernel form needs none
+    }
+    return align256(rows * c_o * 2) + align256(rows * c_i * 2);
+}
+
+int kutacc_hip_transition_block(void *act, const float *ln_gamma, const float *ln_beta, float ln_eps, const void *w1,
+                                const float *b1, const void *w2, const float *b2, void *workspace, int64_t workspace_bytes,
+                                int64_t rows, int64_t c_o, int64_t c_i, int32_t dtype, void *stream)
+{
+    if (!act || !ln_gamma || !ln_beta || !w1 || !b1 || !w2 || !b2 || rows <= 0 || c_o <= 0 || c_i <= 0 ||
+        dtype != KUTACC_DTYPE_BF16) {
+        return KUTACC_HIP_EINVAL;
+    }
+    hipStream_t s = kutacc_api::stream_or_default(stream);
+    int rc = kutacc_launch::transition_block_fused(act, ln_gamma, ln_beta, ln_eps, w1, b1, w2, b2, rows, c_o, c_i, s);
+    if (rc != KUTACC_HIP_EUNSUPPORTED) {
+        return rc;
+    }
+    // three passes through the workspace: LayerNorm, the transition (its result takes the place of its input), residual
+    const int64_t norm_bytes = align256(rows * c_o * 2), need = norm_bytes + align256(rows * c_i * 2);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) {
+        return KUTACC_HIP_EINVAL;
+    }
+    char *ws = static_cast<char *>(workspace);
+    rc = kutacc_launch::layernorm_rows(act, c_o, ln_gamma, ln_beta, ws, c_o, rows, c_o, ln_eps, KUTACC_DTYPE_BF16, s);
+    if (rc == 0) {
+        rc = kutacc_hip_transition(ws, w1, b1, w2, b2, ws + norm_bytes, ws, rows, c_o, c_i, KUTACC_DTYPE_BF16, KUTACC_HIP_PATH_GENERIC,
+                                   s);
+    }
+    if (rc == 0) {
+        rc = kutacc_launch::residual_add(act, ws, rows, 1, c_o, 0, KUTACC_DTYPE_BF16, s);
     }
     return rc;
 }

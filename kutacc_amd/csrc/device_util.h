@@ -45,6 +45,33 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
+// lane-group sums without LDS: a row spread over LPR consecutive lanes (LPR = 8, 16, 32 or 64)
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(moved);
+}
+
+// sum over the LPR lanes that hold one row; every lane of the group gets the total
+template <int LPR>
+__device__ __forceinline__ float group_sum(float v)
+{
+    v = dpp_add<0xB1>(v);  // quad_perm [1,0,3,2]: lane ^ 1
+    v = dpp_add<0x4E>(v);  // quad_perm [2,3,0,1]: lane ^ 2
+    v = dpp_add<0x141>(v); // row_half_mirror: pairs the two quads of 8 lanes
+    if (LPR >= 16) {
+        v = dpp_add<0x140>(v); // row_mirror: pairs the two halves of 16 lanes
+    }
+    if (LPR >= 32) {
+        v += __shfl_xor(v, 16, 64);
+    }
+    if (LPR >= 64) {
+        v += __shfl_xor(v, 32, 64);
+    }
+    return v;
+}
+
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 } // namespace kutacc_dev

@@ -41,6 +41,8 @@ bool transition_fused_supports(int64_t rows, int64_t c_o, int64_t c_i, const voi
                                const void *w2, const float *b2, const void *out);
 int transition_fused(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
                      int64_t rows, int64_t c_o, int64_t c_i, hipStream_t stream);
+int transition_block_fused(void *act, const float *ln_gamma, const float *ln_beta, float ln_eps, const void *w1, const float *b1,
+                           const void *w2, const float *b2, int64_t rows, int64_t c_o, int64_t c_i, hipStream_t stream);
 int sigmoid_gate_rows(void *out, int64_t out_s0, int64_t out_s1, const void *gate, int64_t gate_s0, int64_t gate_s1,
                       int64_t n0, int64_t n1, int64_t size, hipStream_t stream);
 

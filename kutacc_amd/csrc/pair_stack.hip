@@ -289,13 +289,20 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 
 __device__ __forceinline__ int sigma_row(int r) { return (r & 0x13) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
-template <int CO, int RB>
+//
+// BLOCK: the whole transition block of an Evoformer layer in place, out += transition(LayerNorm(out)) with x == out.
+// The rows are normalised between their coalesced load and the fragment staging (a row's 16-byte chunks sit in the 8
+// lanes that loaded them: sums by DPP adds, arithmetic of reference src/normalization/layernorm_kernel.h:21-53), and
+// the epilogue re-reads the rows in the order it writes them and adds.  One read and one write of the activation
+// for LayerNorm, both linears and the residual.
+template <int CO, int RB, bool BLOCK>
 __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *__restrict__ x,
                                                                  const bf16_t *__restrict__ w1,
                                                                  const float *__restrict__ b1,
                                                                  const bf16_t *__restrict__ w2,
                                                                  const float *__restrict__ b2, bf16_t *__restrict__ out,
-                                                                 int64_t rows, int c_i)
+                                                                 int64_t rows, int c_i, const float *__restrict__ ln_gamma,
+                                                                 const float *__restrict__ ln_beta, float ln_eps)
 {
     constexpr int KS = CO / 16; // k-steps of the first product
     constexpr int CP = CO / 64; // 64-column panels across a row of x or W1
@@ -336,10 +343,63 @@ __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *
     bf16x8 xf[RB][KS];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
+        PanelRegs t[CP];
 #pragma unroll
         for (int cp = 0; cp < CP; ++cp) {
-            const PanelRegs t = panel_load(xb, CO, rb * 32, last_local, cp * 64, lane);
-            panel_store(xpanel, lane, t);
+            t[cp] = panel_load(xb, CO, rb * 32, last_local, cp * 64, lane);
+        }
+        if constexpr (BLOCK) {
+            // lane (lane >> 3, lane & 7) holds chunk lane & 7 of every 64-channel panel of rows 8i + (lane >> 3)
+            float gm[CP][8], bt[CP][8];
+#pragma unroll
+            for (int cp = 0; cp < CP; ++cp) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    gm[cp][e] = ln_gamma[cp * 64 + (lane & 7) * 8 + e];
+                    bt[cp][e] = ln_beta[cp * 64 + (lane & 7) * 8 + e];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint4 *regs[CP];
+#pragma unroll
+                for (int cp = 0; cp < CP; ++cp) {
+                    regs[cp] = i == 0 ? &t[cp].r0 : i == 1 ? &t[cp].r1 : i == 2 ? &t[cp].r2 : &t[cp].r3;
+                }
+                const float x0 = __shfl(to_f32(as_bf16x8(*regs[0])[0]), lane & ~7, 64); // first element of the row
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int cp = 0; cp < CP; ++cp) {
+                    const bf16x8 b = as_bf16x8(*regs[cp]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float d = to_f32(b[e]) - x0;
+                        s1 += d;
+                        s2 = fmaf(d, d, s2);
+                    }
+                }
+                s1 = group_sum<8>(s1);
+                s2 = group_sum<8>(s2);
+                const float n = (float)CO;
+                const float mean = s1 / n + x0;
+                const float var = fmaxf((s2 - s1 * s1 / n) / n, 0.f);
+                const float rstd = 1.0f / sqrtf(var + ln_eps);
+                const float shift = -rstd * mean;
+#pragma unroll
+                for (int cp = 0; cp < CP; ++cp) {
+                    const bf16x8 b = as_bf16x8(*regs[cp]);
+                    bf16x8 o;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        o[e] = (bf16_t)fmaf(fmaf(to_f32(b[e]), rstd, shift), gm[cp][e], bt[cp][e]);
+                    }
+                    *regs[cp] = as_uint4(o);
+                }
+            }
+        }
+#pragma unroll
+        for (int cp = 0; cp < CP; ++cp) {
+            panel_store(xpanel, lane, t[cp]);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 xf[rb][cp * 4 + k] = as_bf16x8(xpanel[panel_slot(r, 2 * k + g)]);
@@ -508,9 +568,19 @@ __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int prow = 8 * i + (lane >> 3);
-                const uint4 v = xpanel[panel_slot(prow, lane & 7)];
+                uint4 v = xpanel[panel_slot(prow, lane & 7)];
                 if (active && rb * 32 + prow <= last_local) {
-                    *reinterpret_cast<uint4 *>(out + (row0 + rb * 32 + prow) * CO + half * 64 + (lane & 7) * 8) = v;
+                    bf16_t *dst = out + (row0 + rb * 32 + prow) * CO + half * 64 + (lane & 7) * 8;
+                    if constexpr (BLOCK) { // residual: the row as it was before the LayerNorm
+                        const bf16x8 o = as_bf16x8(v), z = as_bf16x8(*reinterpret_cast<const uint4 *>(dst));
+                        bf16x8 res;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            res[e] = (bf16_t)(to_f32(z[e]) + to_f32(o[e]));
+                        }
+                        v = as_uint4(res);
+                    }
+                    *reinterpret_cast<uint4 *>(dst) = v;
                 }
             }
         }
@@ -805,15 +875,16 @@ hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, hipStream_t 
 
 constexpr int MAX_HIDDEN = 2048; // hidden units whose bias fits next to the weight stages in LDS
 
-template <int CO, int RB>
+template <int CO, int RB, bool BLOCK>
 hipError_t launch_transition(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
-                             int64_t rows, int c_i, hipStream_t stream)
+                             int64_t rows, int c_i, const float *ln_gamma, const float *ln_beta, float ln_eps,
+                             hipStream_t stream)
 {
     constexpr int STAGE_PANELS = 2 * (CO / 64) + CO / 32;
     const size_t lds_bytes = (size_t)(2 * STAGE_PANELS + 4) * 4096 + (size_t)c_i * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB, BLOCK>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize,
                                                  (2 * STAGE_PANELS + 4) * 4096 + MAX_HIDDEN * (int)sizeof(float));
         if (e != hipSuccess) {
@@ -822,8 +893,8 @@ hipError_t launch_transition(const void *x, const void *w1, const float *b1, con
         configured = true;
     }
     const int64_t blocks = (rows + 128 * RB - 1) / (128 * RB);
-    transition_fused_kernel<CO, RB><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(
-        (const bf16_t *)x, (const bf16_t *)w1, b1, (const bf16_t *)w2, b2, (bf16_t *)out, rows, c_i);
+    transition_fused_kernel<CO, RB, BLOCK><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(
+        (const bf16_t *)x, (const bf16_t *)w1, b1, (const bf16_t *)w2, b2, (bf16_t *)out, rows, c_i, ln_gamma, ln_beta, ln_eps);
     return hipGetLastError();
 }
 } // namespace
@@ -845,8 +916,22 @@ int transition_fused(const void *x, const void *w1, const float *b1, const void 
         return KUTACC_HIP_EUNSUPPORTED;
     }
     kutacc_prof::KernelTimer t("transition_fused_kernel", 4.0 * (double)rows * (double)c_o * (double)c_i, stream);
-    const hipError_t e = c_o == 128 ? launch_transition<128, 2>(x, w1, b1, w2, b2, out, rows, (int)c_i, stream)
-                                    : launch_transition<256, 1>(x, w1, b1, w2, b2, out, rows, (int)c_i, stream);
+    const hipError_t e = c_o == 128 ? launch_transition<128, 2, false>(x, w1, b1, w2, b2, out, rows, (int)c_i, nullptr, nullptr, 0.f, stream)
+                                    : launch_transition<256, 1, false>(x, w1, b1, w2, b2, out, rows, (int)c_i, nullptr, nullptr, 0.f, stream);
+    return kutacc_hip_status(e);
+}
+
+// act += transition(LayerNorm(act)) in place, one kernel
+int transition_block_fused(void *act, const float *ln_gamma, const float *ln_beta, float ln_eps, const void *w1, const float *b1,
+                           const void *w2, const float *b2, int64_t rows, int64_t c_o, int64_t c_i, hipStream_t stream)
+{
+    if (!ln_gamma || !ln_beta || !transition_fused_supports(rows, c_o, c_i, act, w1, b1, w2, b2, act)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    kutacc_prof::KernelTimer t("transition_fused_kernel<block>", 4.0 * (double)rows * (double)c_o * (double)c_i, stream);
+    const hipError_t e =
+        c_o == 128 ? launch_transition<128, 2, true>(act, w1, b1, w2, b2, act, rows, (int)c_i, ln_gamma, ln_beta, ln_eps, stream)
+                   : launch_transition<256, 1, true>(act, w1, b1, w2, b2, act, rows, (int)c_i, ln_gamma, ln_beta, ln_eps, stream);
     return kutacc_hip_status(e);
 }
 

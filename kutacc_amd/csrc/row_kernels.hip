@@ -118,32 +118,6 @@ __global__ __launch_bounds__(64 * ROW_WAVES) void pair_bias_kernel(const T *__re
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v)
-{
-    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
-    return v + __int_as_float(moved);
-}
-
-// sum over the LPR lanes that hold one row; every lane of the group gets the total
-template <int LPR>
-__device__ __forceinline__ float group_sum(float v)
-{
-    v = dpp_add<0xB1>(v);  // quad_perm [1,0,3,2]: lane ^ 1
-    v = dpp_add<0x4E>(v);  // quad_perm [2,3,0,1]: lane ^ 2
-    v = dpp_add<0x141>(v); // row_half_mirror: pairs the two quads of 8 lanes
-    if (LPR >= 16) {
-        v = dpp_add<0x140>(v); // row_mirror: pairs the two halves of 16 lanes
-    }
-    if (LPR >= 32) {
-        v += __shfl_xor(v, 16, 64);
-    }
-    if (LPR >= 64) {
-        v += __shfl_xor(v, 32, 64);
-    }
-    return v;
-}
-
 union Pack16 {
     uint4 u;
     bf16x8 b;

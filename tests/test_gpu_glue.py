@@ -313,3 +313,36 @@ def test_gated_residual_projection(torch_cuda, m, n, k):
     rc = capi.lib().kutacc_hip_gated_residual_projection(t[0].data_ptr(), k, t[1].data_ptr(), t[2].data_ptr(), t[3].data_ptr(), n,
                                                          d_acc.data_ptr(), n, m, 96, k, capi.K_BF16, None)
     assert rc == capi.EUNSUPPORTED
+
+
+@pytest.mark.parametrize("rows,c_o,c_i", [(300, 128, 512), (200, 256, 1024), (64 * 64, 128, 512), (50, 24, 40)])
+def test_transition_block(torch_cuda, rows, c_o, c_i):
+    """act += transition(LN(act)) in place: the one-kernel form (pair and MSA channel counts, ragged row counts) and the
+    separate-pass form through a workspace, against the oracle's LayerNorm and transition composed in numpy."""
+    from oracle import oracle
+    torch = torch_cuda
+    rng = np.random.Generator(np.random.PCG64(70 + rows))
+    x = round_to_bf16((rng.standard_normal((rows, c_o)) * 1.5 + 0.3).astype(np.float32))
+    gamma, beta = (rng.random(c_o) + 0.5).astype(np.float32), (rng.standard_normal(c_o) * 0.2).astype(np.float32)
+    w1 = round_to_bf16((rng.standard_normal((c_i, c_o)) / math.sqrt(c_o)).astype(np.float32))
+    w2 = round_to_bf16((rng.standard_normal((c_o, c_i)) / math.sqrt(c_i)).astype(np.float32))
+    b1, b2 = (rng.standard_normal(c_i) * 0.3).astype(np.float32), (rng.standard_normal(c_o) * 0.3).astype(np.float32)
+    dev = lambda a, dt=torch.bfloat16: torch.from_numpy(a).to(device="cuda", dtype=dt)  # noqa: E731
+    f32 = torch.float32
+    act = dev(x)
+    t = [dev(gamma, f32), dev(beta, f32), dev(w1), dev(b1, f32), dev(w2), dev(b2, f32)]
+    L = capi.lib()
+    nbytes = L.kutacc_hip_transition_block_workspace(rows, c_o, c_i)
+    assert (nbytes == 0) == (c_o in (128, 256))
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device="cuda")
+    rc = L.kutacc_hip_transition_block(act.data_ptr(), t[0].data_ptr(), t[1].data_ptr(), 1e-5, t[2].data_ptr(), t[3].data_ptr(),
+                                       t[4].data_ptr(), t[5].data_ptr(), ws.data_ptr() if nbytes else None, nbytes, rows, c_o, c_i,
+                                       capi.K_BF16, None)
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    want = x + oracle.transition_f32(oracle.layernorm_rows_f32(x, gamma, beta, 1e-5), w1, b1, w2, b2)
+    helpers.check_close(helpers.to_numpy(act), want, "bf16", f"transition block {rows}x{c_o}->{c_i}")
+    if nbytes:  # without its workspace the separate-pass form must refuse
+        assert L.kutacc_hip_transition_block(act.data_ptr(), t[0].data_ptr(), t[1].data_ptr(), 1e-5, t[2].data_ptr(),
+                                             t[3].data_ptr(), t[4].data_ptr(), t[5].data_ptr(), None, 0, rows, c_o, c_i,
+                                             capi.K_BF16, None) == capi.EINVAL
