@@ -257,6 +257,44 @@ def pair_stack_rates(config, reps=20):
     return res
 
 
+def msa_block_rates(reps=20):
+    """Times of the two MSA attention blocks at the shapes of configurations 2 and 4: row-wise with pair bias
+    (512 sequences x 256 residues, 256 channels, pair bias from a [256, 256, 128] pair tensor) and column-wise
+    (1024 sequences x 384 residues).  One kutacc_hip_msa_attention call each, in place, hipEvent-bracketed."""
+    import torch
+    from kutacc_amd import capi
+
+    g = torch.Generator(device="cuda").manual_seed(13)
+    bf = lambda *sh, scale=1.0: (torch.randn(*sh, device="cuda", generator=g) * scale).to(torch.bfloat16)  # noqa: E731
+    stream = torch.cuda.current_stream().cuda_stream
+    heads, c, cz = 8, 256, 128
+    w = {"ln_gamma": torch.ones(c, device="cuda"), "ln_beta": torch.zeros(c, device="cuda"), "bg": torch.ones(c, device="cuda"),
+         "bo": torch.zeros(c, device="cuda")}
+    for k in ("wq", "wk", "wv", "wg", "wo"):
+        w[k] = bf(c, c, scale=c ** -0.5) * (0.1 if k == "wo" else 1.0)
+    res = {}
+    for name, n_seq, n_res, column in (("msa_row_attention_with_pair_bias 512x256", 512, 256, False),
+                                       ("msa_column_attention 1024x384", 1024, 384, True)):
+        msa = bf(n_seq, n_res, c)
+        mask = (torch.rand(n_seq, n_res, device="cuda", generator=g) > 0.05).to(torch.bfloat16)
+        pair = None if column else {"pair_act": bf(n_res, n_res, cz), "pair_ln_gamma": torch.ones(cz, device="cuda"),
+                                    "pair_ln_beta": torch.zeros(cz, device="cuda"), "bias_w": bf(heads, cz, scale=cz ** -0.5)}
+        blk = capi.MsaAttentionBlock(msa, mask, w, heads, pair)
+        for _ in range(3):
+            assert blk.run(stream) == 0
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            assert blk.run(stream) == 0
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) / reps * 1e-3
+        B, S = (n_res, n_seq) if column else (n_seq, n_res)
+        flops = 10.0 * B * S * c * c + 4.0 * B * S * S * c
+        res[name] = {"us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -267,6 +305,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy: a kernel of known traffic to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run against")
+    ap.add_argument("--msa-blocks", action="store_true",
+                    help="also time the row-wise (with pair bias) and column-wise MSA attention blocks at the shapes of "
+                         "configurations 2 and 4 and report them in an \"msa_blocks\" object")
     ap.add_argument("--pair-stack", action="store_true",
                     help="also time the transition and the triangle-multiplication steps at this configuration's pair "
                          "tensor and report them in a \"pair_stack\" object")
@@ -355,6 +396,8 @@ def main():
         rec["producers"] = producer_rates(a.config)
     if a.pair_stack:
         rec["pair_stack"] = pair_stack_rates(a.config)
+    if a.msa_blocks:
+        rec["msa_blocks"] = msa_block_rates()
     print(json.dumps(rec))
 
 

@@ -340,6 +340,47 @@ kutacc_export int kutacc_hip_transition_block(void *act, const float *ln_gamma, 
                                               void *workspace, int64_t workspace_bytes, int64_t rows, int64_t c_o,
                                               int64_t c_i, int32_t dtype, void *stream);
 
+/* kutacc_hip_layernorm_rows on a grid of rows read transposed: out row (i, j) of a dense [rows_i, rows_j, size] tensor is
+ * the LayerNorm of row (j, i) of the dense [rows_j, rows_i, size] input.  The column-wise MSA attention's input without
+ * a separate pass that swaps the axes of the msa. */
+kutacc_export int kutacc_hip_layernorm_rows_transposed(const void *x, const float *gamma, const float *beta, void *out,
+                                                       int64_t rows_i, int64_t rows_j, int64_t size, float eps,
+                                                       int32_t dtype, void *stream);
+
+/*
+ * One MSA attention block, in place on msa_act [n_seq, n_res, c_m] (c_m = nheads * 32):
+ *   column == 0, row-wise with pair bias: msa_act += gating_attention(LN(msa_act), bias from msa_mask,
+ *                nonbatched_bias = LN_pair(pair_act) . bias_w^T), every sequence attending over the residues;
+ *   column != 0, column-wise: the same operator without pair bias on the msa with its leading axes exchanged, every
+ *                residue attending over the sequences; no transposed copy of the msa is made (the LayerNorm reads it
+ *                transposed, the output projection adds its result back transposed).
+ * bf16; shapes of the MFMA attention kernels (c_m in {128, 256}, attended axis <= 1024), else KUTACC_HIP_EUNSUPPORTED.
+ * pair_act [n_res, n_res, c_z], its LayerNorm parameters and bias_w [nheads, c_z] are read by the row-wise form only.
+ */
+typedef struct kutacc_hip_msa_attention_args {
+    int64_t n_seq;
+    int64_t n_res;
+    int64_t nheads;
+    int64_t c_z;     /* channels of pair_act (row-wise form) */
+    int32_t dtype;   /* KUTACC_DTYPE_BF16 */
+    int32_t column;  /* 0 row-wise with pair bias, 1 column-wise */
+    void *msa_act;          /* [n_seq, n_res, c_m], updated in place */
+    const void *msa_mask;   /* [n_seq, n_res], 1 = valid */
+    const float *ln_gamma, *ln_beta; /* [c_m] */
+    float ln_eps;
+    int32_t reserved;
+    const void *pair_act;
+    const float *pair_ln_gamma, *pair_ln_beta; /* [c_z] */
+    const void *bias_w;
+    const void *query_w, *key_w, *value_w, *gating_w, *output_w; /* [c_m, c_m] stored [out, in] */
+    const float *gating_b, *output_b;
+    void *workspace;
+    int64_t workspace_bytes; /* >= kutacc_hip_msa_attention_workspace(n_seq, n_res, nheads, column), 256-byte aligned */
+} kutacc_hip_msa_attention_args_t;
+
+kutacc_export int64_t kutacc_hip_msa_attention_workspace(int64_t n_seq, int64_t n_res, int64_t nheads, int32_t column);
+kutacc_export int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *args, void *stream);
+
 /* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.

@@ -139,6 +139,17 @@ class HipTriangleMultiplicationArgs(ctypes.Structure):
     ]
 
 
+class HipMsaAttentionArgs(ctypes.Structure):
+    """kutacc_hip_msa_attention_args_t"""
+    _fields_ = [
+        ("n_seq", _i64), ("n_res", _i64), ("nheads", _i64), ("c_z", _i64), ("dtype", _i32), ("column", _i32),
+        ("msa_act", _vp), ("msa_mask", _vp), ("ln_gamma", _vp), ("ln_beta", _vp), ("ln_eps", ctypes.c_float), ("reserved", _i32),
+        ("pair_act", _vp), ("pair_ln_gamma", _vp), ("pair_ln_beta", _vp), ("bias_w", _vp),
+        ("query_w", _vp), ("key_w", _vp), ("value_w", _vp), ("gating_w", _vp), ("output_w", _vp),
+        ("gating_b", _vp), ("output_b", _vp), ("workspace", _vp), ("workspace_bytes", _i64),
+    ]
+
+
 # every symbol the two public headers declare; tests check that the library exports all of them
 DECLARED_SYMBOLS = [
     "kutacc_get_version", "kutacc_af2_gating_attention", "kutacc_af2_global_attention", "kutacc_af2_layernorm",
@@ -149,6 +160,7 @@ DECLARED_SYMBOLS = [
     "kutacc_hip_triangle_attention_workspace", "kutacc_hip_triangle_attention", "kutacc_hip_layernorm_channel_first",
     "kutacc_hip_triangle_multiplication_workspace", "kutacc_hip_triangle_multiplication",
     "kutacc_hip_gated_residual_projection", "kutacc_hip_transition_block_workspace", "kutacc_hip_transition_block",
+    "kutacc_hip_layernorm_rows_transposed", "kutacc_hip_msa_attention_workspace", "kutacc_hip_msa_attention",
     "kutacc_af2_linear_weight_prepack", "kutacc_af2_gemm_pack_get_size", "world_size", "rank",
     "_ZN6kutacc13TensorWrapperC1EPvOSt6vectorIlSaIlEES5_lNS_14TensorDataTypeE",
     "_ZN6kutacc13TensorWrapperC1Ev", "_ZN6kutacc13TensorWrapperD1Ev",
@@ -241,6 +253,12 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_transition_block.argtypes = [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                               _i32, _vp]
     L.kutacc_hip_transition_block.restype = ctypes.c_int
+    L.kutacc_hip_layernorm_rows_transposed.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_float, _i32, _vp]
+    L.kutacc_hip_layernorm_rows_transposed.restype = ctypes.c_int
+    L.kutacc_hip_msa_attention_workspace.argtypes = [_i64, _i64, _i64, _i32]
+    L.kutacc_hip_msa_attention_workspace.restype = _i64
+    L.kutacc_hip_msa_attention.argtypes = [ctypes.POINTER(HipMsaAttentionArgs), _vp]
+    L.kutacc_hip_msa_attention.restype = ctypes.c_int
     L.kutacc_hip_set_stream.argtypes = [_vp]
     L.kutacc_hip_get_stream.restype = _vp
     L.kutacc_hip_set_blocking.argtypes = [ctypes.c_int]
@@ -499,3 +517,33 @@ class TriangleMultiplicationBlock:
 
     def run(self, stream_ptr=None) -> int:
         return lib().kutacc_hip_triangle_multiplication(ctypes.byref(self.args), stream_ptr)
+
+
+class MsaAttentionBlock:
+    """One MSA attention block on device tensors, in place on `msa_act` [n_seq, n_res, c_m]: row-wise with pair bias
+    (`pair` = dict with pair_act [n_res, n_res, c_z], pair_ln_gamma, pair_ln_beta [c_z], bias_w [nheads, c_z]) or
+    column-wise (`pair` None).  `w`: ln_gamma, ln_beta, wq, wk, wv, wg, bg, wo, bo.  Owns the workspace."""
+
+    def __init__(self, msa_act, msa_mask, w, nheads, pair=None, eps=1e-5):
+        import torch
+        n_seq, n_res, _ = msa_act.shape
+        column = pair is None
+        nbytes = lib().kutacc_hip_msa_attention_workspace(n_seq, n_res, nheads, 1 if column else 0)
+        assert nbytes > 0
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=msa_act.device)
+        self.keep = (msa_act, msa_mask, w, pair)
+        a = HipMsaAttentionArgs()
+        a.n_seq, a.n_res, a.nheads, a.dtype, a.column = n_seq, n_res, nheads, K_BF16, 1 if column else 0
+        a.msa_act, a.msa_mask, a.ln_eps = msa_act.data_ptr(), msa_mask.data_ptr(), eps
+        a.ln_gamma, a.ln_beta = w["ln_gamma"].data_ptr(), w["ln_beta"].data_ptr()
+        if pair is not None:
+            a.c_z = pair["pair_act"].shape[-1]
+            a.pair_act, a.bias_w = pair["pair_act"].data_ptr(), pair["bias_w"].data_ptr()
+            a.pair_ln_gamma, a.pair_ln_beta = pair["pair_ln_gamma"].data_ptr(), pair["pair_ln_beta"].data_ptr()
+        a.query_w, a.key_w, a.value_w, a.gating_w, a.output_w = (w[k].data_ptr() for k in ("wq", "wk", "wv", "wg", "wo"))
+        a.gating_b, a.output_b = w["bg"].data_ptr(), w["bo"].data_ptr()
+        a.workspace, a.workspace_bytes = self.workspace.data_ptr(), nbytes
+        self.args = a
+
+    def run(self, stream_ptr=None) -> int:
+        return lib().kutacc_hip_msa_attention(ctypes.byref(self.args), stream_ptr)

@@ -284,4 +284,101 @@ int kutacc_hip_transition_block(void *act, const float *ln_gamma, const float *l
     return rc;
 }
 
+int kutacc_hip_layernorm_rows_transposed(const void *x, const float *gamma, const float *beta, void *out, int64_t rows_i,
+                                         int64_t rows_j, int64_t size, float eps, int32_t dtype, void *stream)
+{
+    if (rows_i <= 0 || rows_j <= 0 || rows_i > INT64_MAX / rows_j) {
+        return KUTACC_HIP_EINVAL;
+    }
+    return kutacc_launch::layernorm_rows(x, size, gamma, beta, out, size, rows_i * rows_j, size, eps, dtype,
+                                         kutacc_api::stream_or_default(stream), rows_j);
+}
+
+namespace {
+struct MsaWorkspace {
+    int64_t m_norm, nb, bias, q, avg, total;
+};
+
+MsaWorkspace msa_layout(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
+{
+    const int64_t act = align256(n_seq * n_res * heads * HEAD * 2);
+    MsaWorkspace w;
+    w.m_norm = 0;
+    w.nb = w.m_norm + act;
+    w.bias = w.nb + (column ? 0 : align256(heads * n_res * n_res * 2));
+    w.q = w.bias + align256(n_seq * n_res * 2);
+    w.avg = w.q + act;
+    w.total = w.avg + act;
+    return w;
+}
+} // namespace
+
+int64_t kutacc_hip_msa_attention_workspace(int64_t n_seq, int64_t n_res, int64_t nheads, int32_t column)
+{
+    if (n_seq <= 0 || n_res <= 0 || nheads <= 0 || n_seq > 1 << 20 || n_res > 65536 || nheads > 64) {
+        return -1;
+    }
+    return msa_layout(n_seq, n_res, nheads, column != 0).total;
+}
+
+int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *stream)
+{
+    if (!a || !a->msa_act || !a->msa_mask || !a->ln_gamma || !a->ln_beta || !a->query_w || !a->key_w || !a->value_w ||
+        !a->gating_w || !a->output_w || !a->gating_b || !a->output_b || !a->workspace) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const bool column = a->column != 0;
+    if (!column && (!a->pair_act || !a->pair_ln_gamma || !a->pair_ln_beta || !a->bias_w || a->c_z <= 0)) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (a->dtype != KUTACC_DTYPE_BF16 || kutacc_hip_msa_attention_workspace(a->n_seq, a->n_res, a->nheads, a->column) < 0) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int64_t n_seq = a->n_seq, n_res = a->n_res, heads = a->nheads, c = heads * HEAD;
+    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column);
+    if (a->workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
+        return KUTACC_HIP_EINVAL;
+    }
+    char *ws = static_cast<char *>(a->workspace);
+    hipStream_t s = kutacc_api::stream_or_default(stream);
+    // row-wise: every sequence attends over the residues; column-wise: every residue attends over the sequences,
+    // i.e. the same operator on the msa with its two leading axes exchanged
+    const int64_t batch = column ? n_res : n_seq, seq = column ? n_seq : n_res;
+
+    kutacc_hip_attention_args_t g;
+    std::memset(&g, 0, sizeof(g));
+    g.batch = batch, g.seq_len = seq, g.nheads = heads, g.head_size = HEAD;
+    g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_FUSED;
+    g.input = ws + w.m_norm, g.input_ld = c;
+    g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
+    g.gating_b = a->gating_b, g.output_b = a->output_b;
+    g.bias = ws + w.bias, g.bias_stride_b = seq;
+    if (!column) {
+        g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n_res * n_res, g.nb_stride_q = n_res;
+    }
+    g.q = ws + w.q, g.q_stride_b = seq * c, g.q_stride_s = c, g.q_stride_h = HEAD;
+    g.avg = ws + w.avg, g.avg_stride_b = seq * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
+    g.out = a->msa_act, g.out_ld = c;
+    if (!kutacc_launch::fused_attention_supports(g)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    // 1. LayerNorm of the msa rows, read transposed for the column-wise form
+    int rc = kutacc_launch::layernorm_rows(a->msa_act, c, a->ln_gamma, a->ln_beta, ws + w.m_norm, c, n_seq * n_res, c, a->ln_eps,
+                                           KUTACC_DTYPE_BF16, s, column ? n_seq : 0);
+    // 2. pair bias from the pair activation (row-wise form only)
+    if (rc == 0 && !column) {
+        rc = kutacc_launch::pair_bias(a->pair_act, a->pair_ln_gamma, a->pair_ln_beta, a->bias_w, ws + w.nb, nullptr, n_res, n_res,
+                                      a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s);
+    }
+    // 3. mask bias [batch, seq]
+    if (rc == 0) {
+        rc = kutacc_launch::mask_bias(a->msa_mask, ws + w.bias, batch, seq, column, KUTACC_DTYPE_BF16, s);
+    }
+    // 4. the operator; its output projection adds into the msa (transposed back for the column-wise form)
+    if (rc == 0) {
+        rc = kutacc_launch::gating_attention_fused(g, s, column ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD);
+    }
+    return rc;
+}
+
 } // extern "C"

@@ -1104,7 +1104,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 // with gate and out read in the order they are written, 16 bytes per lane -- the last two steps of the triangle
 // multiplication (reference src/attention/triangle_multiplication.cpp:129-150) and the residual update fused into
 // its output projection.  EPILOGUE 2 (residual): out += result, where row (i, j) of the result goes to row (j, i)
-// of `out` when swap_n != 0 (rows are pairs of an n x n grid): the residual update of a triangle-attention block,
+// of `out` when swap_n != 0 (rows are pairs (i, j) of an [M / swap_n, swap_n] grid): the residual update of a triangle-attention block,
 // transposed back for the ending node.
 constexpr int EPILOGUE_STORE = 0, EPILOGUE_GATED_RESIDUAL = 1, EPILOGUE_RESIDUAL = 2;
 
@@ -1117,7 +1117,7 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
     // row of `out` that receives row `row` of the result
     auto target_row = [&](int64_t row) -> int64_t {
         if constexpr (EPILOGUE == EPILOGUE_RESIDUAL) {
-            return swap_n ? (row % swap_n) * swap_n + row / swap_n : row;
+            return swap_n ? (row % swap_n) * (M / swap_n) + row / swap_n : row; // row (b, s) of [M / n, n] -> (s, b)
         }
         return row;
     };
@@ -1586,10 +1586,7 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     }
     const int64_t M = a.batch * a.seq_len;
     if (residual != FUSED_OUT_STORE) {
-        // out += result, row (b, s) of the result going to row (s, b) of out in the transposed form
-        if (residual == FUSED_OUT_ADD_TRANSPOSED && a.batch != a.seq_len) {
-            return KUTACC_HIP_EINVAL;
-        }
+        // out += result, row (b, s) of the result going to row (s, b) of out ([seq_len, batch, C]) in the transposed form
         const int64_t swap_n = residual == FUSED_OUT_ADD_TRANSPOSED ? a.seq_len : 0;
         kutacc_prof::KernelTimer t("output_projection_kernel<residual>", 2.0 * BS * C * C, stream);
         return (C == 128) ? launch_output_projection<128, EPILOGUE_RESIDUAL>(a.avg, a.avg_stride_s, a.output_w, a.output_b, a.out,

@@ -19,7 +19,7 @@ int gemm_nt(int32_t dtype, const void *a, int64_t lda, const void *w, int64_t ld
 // fused_attention.hip
 bool fused_attention_supports(const kutacc_hip_attention_args_t &args);
 // `residual`: what the output projection does with its result -- store it in args.out (the operator as the reference
-// defines it), add it to args.out, or add row (b, s) of it to row (s, b) of args.out (batch == seq_len)
+// defines it), add it to args.out, or add row (b, s) of it to row (s, b) of args.out, then [seq_len, batch, C]
 constexpr int FUSED_OUT_STORE = 0, FUSED_OUT_ADD = 1, FUSED_OUT_ADD_TRANSPOSED = 2;
 int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream, int residual = FUSED_OUT_STORE);
 
@@ -56,8 +56,10 @@ int layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, con
                             int64_t channels, int64_t positions, float eps, int32_t dtype, hipStream_t stream);
 
 // row_kernels.hip
+// swap_j != 0: rows are pairs (i, j) of an [rows / swap_j, swap_j] grid and output row (i, j) is computed from input
+// row (j, i) of the transposed grid
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
-                   int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream);
+                   int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream, int64_t swap_j = 0);
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
               int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
               hipStream_t stream);

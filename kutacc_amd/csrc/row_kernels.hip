@@ -40,14 +40,16 @@ __global__ __launch_bounds__(64 * ROW_WAVES) void layernorm_rows_kernel(const T 
                                                                        const float *__restrict__ gamma,
                                                                        const float *__restrict__ beta,
                                                                        T *__restrict__ out, int64_t ld_out,
-                                                                       int64_t rows, int64_t size, float eps)
+                                                                       int64_t rows, int64_t size, float eps, int64_t swap_j)
 {
     const int lane = threadIdx.x % 64;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + threadIdx.x / 64;
     if (r >= rows) {
         return;
     }
-    const T *row = x + r * ld_x;
+    // swap_j != 0: rows are pairs (i, j) of an [rows / swap_j, swap_j] grid and output row (i, j) is computed from
+    // input row (j, i) of the transposed grid
+    const T *row = x + (swap_j ? (r % swap_j) * (rows / swap_j) + r / swap_j : r) * ld_x;
     float rstd, shift;
     row_stats(row, size, lane, eps, rstd, shift);
     T *orow = out + r * ld_out;
@@ -147,7 +149,7 @@ template <int LPR>
 __global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *__restrict__ x, int64_t ld_x,
                                                                   const float *__restrict__ gamma,
                                                                   const float *__restrict__ beta, bf16_t *__restrict__ out,
-                                                                  int64_t ld_out, int64_t rows, float eps)
+                                                                  int64_t ld_out, int64_t rows, float eps, int64_t swap_j)
 {
     constexpr int RPS = 64 / LPR; // rows per step of a wave
     constexpr int U = 4;          // steps in flight
@@ -166,6 +168,7 @@ __global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *
     for (int u = 0; u < U; ++u) {
         int64_t r = r0 + u * RPS + grp;
         r = r < rows ? r : rows - 1;
+        r = swap_j ? (r % swap_j) * (rows / swap_j) + r / swap_j : r; // input row (j, i) for output row (i, j)
         in[u].u = *reinterpret_cast<const uint4 *>(x + r * ld_x + sub * 8);
     }
 #pragma unroll
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
 
 template <typename T>
 int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
-                     int64_t rows, int64_t size, float eps, hipStream_t stream)
+                     int64_t rows, int64_t size, float eps, int64_t swap_j, hipStream_t stream)
 {
     if (sizeof(T) == 2 && (size == 64 || size == 128 || size == 256 || size == 512) && ld_x % 8 == 0 && ld_out % 8 == 0 &&
         (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % 16 == 0) {
@@ -297,10 +300,10 @@ int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const floa
         const bf16_t *xi = (const bf16_t *)x;
         bf16_t *oi = (bf16_t *)out;
         switch (lpr) {
-            case 8: layernorm_rows_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
-            case 16: layernorm_rows_bf16_kernel<16><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
-            case 32: layernorm_rows_bf16_kernel<32><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
-            default: layernorm_rows_bf16_kernel<64><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps); break;
+            case 8: layernorm_rows_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
+            case 16: layernorm_rows_bf16_kernel<16><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
+            case 32: layernorm_rows_bf16_kernel<32><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
+            default: layernorm_rows_bf16_kernel<64><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
         }
         return kutacc_hip_status(hipGetLastError());
     }
@@ -309,7 +312,7 @@ int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const floa
         return KUTACC_HIP_EUNSUPPORTED;
     }
     layernorm_rows_kernel<T><<<(unsigned)blocks, 64 * ROW_WAVES, 0, stream>>>((const T *)x, ld_x, gamma, beta, (T *)out,
-                                                                               ld_out, rows, size, eps);
+                                                                               ld_out, rows, size, eps, swap_j);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -350,16 +353,17 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
 namespace kutacc_launch {
 
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
-                   int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream)
+                   int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream, int64_t swap_j)
 {
-    if (!x || !gamma || !beta || !out || rows <= 0 || size <= 0 || ld_x < size || ld_out < size) {
+    if (!x || !gamma || !beta || !out || rows <= 0 || size <= 0 || ld_x < size || ld_out < size || swap_j < 0 ||
+        (swap_j > 0 && rows % swap_j != 0)) {
         return KUTACC_HIP_EINVAL;
     }
     if (dtype == KUTACC_DTYPE_BF16) {
-        return launch_layernorm<bf16_t>(x, ld_x, gamma, beta, out, ld_out, rows, size, eps, stream);
+        return launch_layernorm<bf16_t>(x, ld_x, gamma, beta, out, ld_out, rows, size, eps, swap_j, stream);
     }
     if (dtype == KUTACC_DTYPE_FP32) {
-        return launch_layernorm<float>(x, ld_x, gamma, beta, out, ld_out, rows, size, eps, stream);
+        return launch_layernorm<float>(x, ld_x, gamma, beta, out, ld_out, rows, size, eps, swap_j, stream);
     }
     return KUTACC_HIP_EINVAL;
 }

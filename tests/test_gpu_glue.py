@@ -346,3 +346,76 @@ def test_transition_block(torch_cuda, rows, c_o, c_i):
         assert L.kutacc_hip_transition_block(act.data_ptr(), t[0].data_ptr(), t[1].data_ptr(), 1e-5, t[2].data_ptr(),
                                              t[3].data_ptr(), t[4].data_ptr(), t[5].data_ptr(), None, 0, rows, c_o, c_i,
                                              capi.K_BF16, None) == capi.EINVAL
+
+
+# ---- MSA attention blocks ------------------------------------------------------------------------------------------
+def msa_case(seed, n_seq, n_res, heads, c_z):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    c = heads * 32
+    w = lambda o, i: round_to_bf16((rng.standard_normal((o, i)) / math.sqrt(i)).astype(np.float32))  # noqa: E731
+    mask = (rng.random((n_seq, n_res)) > 0.1).astype(np.float32)
+    mask[:, -2:] = 0.0  # padded residues
+    mask[-1, :] = 0.0   # a padded sequence: a fully masked row for the row-wise form
+    return dict(m=round_to_bf16(rng.standard_normal((n_seq, n_res, c)).astype(np.float32)), mask=mask,
+                z=round_to_bf16(rng.standard_normal((n_res, n_res, c_z)).astype(np.float32)),
+                ln_gamma=(rng.random(c) + 0.5).astype(np.float32), ln_beta=(rng.standard_normal(c) * 0.1).astype(np.float32),
+                pair_ln_gamma=(rng.random(c_z) + 0.5).astype(np.float32),
+                pair_ln_beta=(rng.standard_normal(c_z) * 0.1).astype(np.float32), bias_w=w(heads, c_z),
+                wq=w(c, c), wk=w(c, c), wv=w(c, c), wg=w(c, c), wo=w(c, c), bg=np.ones(c, np.float32),
+                bo=(rng.standard_normal(c) * 0.1).astype(np.float32), heads=heads)
+
+
+def msa_oracle(c, column):
+    """AlphaFold's MSARowAttentionWithPairBias / MSAColumnAttention in numpy on the oracle's operators."""
+    from oracle import oracle
+    m, mask = c["m"], c["mask"]
+    if column:
+        m, mask = m.transpose(1, 0, 2), mask.T
+    B, S, ch = m.shape
+    mn = oracle.layernorm_rows_f32(np.ascontiguousarray(m).reshape(-1, ch), c["ln_gamma"], c["ln_beta"], 1e-5).reshape(B, S, ch)
+    nb = None
+    if not column:
+        n_res, _, cz = c["z"].shape
+        zn = oracle.layernorm_rows_f32(c["z"].reshape(-1, cz), c["pair_ln_gamma"], c["pair_ln_beta"], 1e-5)
+        nb = np.ascontiguousarray(oracle.linear_f32(zn, c["bias_w"]).reshape(n_res, n_res, c["heads"]).transpose(2, 0, 1))
+    bias = (np.ascontiguousarray(mask) * np.float32(1e9) - np.float32(1e9)).astype(np.float32)
+    out = oracle.gating_attention_f32(mn, c["wq"], c["wk"], c["wv"], c["wg"], c["bg"], c["wo"], c["bo"], bias, nb, c["heads"])
+    if column:
+        out = out.transpose(1, 0, 2)
+    return c["m"] + out
+
+
+@pytest.mark.parametrize("column", [False, True], ids=["row-wise with pair bias", "column-wise"])
+@pytest.mark.parametrize("n_seq,n_res,heads,c_z", [(24, 40, 8, 128), (50, 20, 8, 128), (33, 33, 4, 64)])
+def test_msa_attention_block_against_the_oracle(torch_cuda, n_seq, n_res, heads, c_z, column):
+    torch = torch_cuda
+    c = msa_case(1000 + n_seq, n_seq, n_res, heads, c_z)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    msa = dev(c["m"])
+    w = {k: dev(c[k]) for k in ("ln_gamma", "ln_beta", "wq", "wk", "wv", "wg", "bg", "wo", "bo")}
+    pair = None if column else {"pair_act": dev(c["z"]), "pair_ln_gamma": dev(c["pair_ln_gamma"]),
+                                "pair_ln_beta": dev(c["pair_ln_beta"]), "bias_w": dev(c["bias_w"])}
+    blk = capi.MsaAttentionBlock(msa, dev(c["mask"]), w, heads, pair)
+    rc = blk.run()
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    helpers.check_close(helpers.to_numpy(msa), msa_oracle(c, column), "bf16", f"msa block {n_seq}x{n_res} column={column}")
+
+
+def test_layernorm_rows_transposed(torch_cuda):
+    torch = torch_cuda
+    g = torch.Generator(device="cuda").manual_seed(4)
+    for rows_i, rows_j, size, dt in ((20, 36, 256, torch.bfloat16), (7, 9, 24, torch.float32)):
+        x_t = torch.randn(rows_j, rows_i, size, device="cuda", generator=g).to(dt)
+        gamma = torch.rand(size, device="cuda", generator=g) + 0.5
+        beta = torch.randn(size, device="cuda", generator=g) * 0.1
+        a, b = torch.zeros(rows_i, rows_j, size, dtype=dt, device="cuda"), torch.zeros(rows_i, rows_j, size, dtype=dt, device="cuda")
+        L = capi.lib()
+        x = x_t.transpose(0, 1).contiguous()
+        assert L.kutacc_hip_layernorm_rows(x.data_ptr(), size, gamma.data_ptr(), beta.data_ptr(), a.data_ptr(), size,
+                                           rows_i * rows_j, size, 1e-5, code(torch, x), None) == 0
+        assert L.kutacc_hip_layernorm_rows_transposed(x_t.data_ptr(), gamma.data_ptr(), beta.data_ptr(), b.data_ptr(), rows_i,
+                                                      rows_j, size, 1e-5, code(torch, x), None) == 0
+        torch.cuda.synchronize()
+        assert helpers.same_bits(a, b)
