@@ -400,8 +400,6 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
     }
 }
 
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
 } // namespace
 
 namespace kutacc_launch {
@@ -418,8 +416,8 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
     }
     // 16-byte row loads of x and the weights, 16-byte stores of out rows
     if (a.q_data_stride_s % 8 != 0 || a.q_data_stride_b % 8 != 0 || a.out_stride_s % 8 != 0 || a.out_stride_b % 8 != 0 ||
-        !aligned16(a.q_data) || !aligned16(a.out) || !aligned16(a.query_w) || !aligned16(a.key_w) ||
-        !aligned16(a.value_w) || !aligned16(a.gating_w) || !aligned16(a.output_w)) {
+        !kutacc_hip_aligned16(a.q_data) || !kutacc_hip_aligned16(a.out) || !kutacc_hip_aligned16(a.query_w) || !kutacc_hip_aligned16(a.key_w) ||
+        !kutacc_hip_aligned16(a.value_w) || !kutacc_hip_aligned16(a.gating_w) || !kutacc_hip_aligned16(a.output_w)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
     GlobalParams p;

@@ -171,8 +171,6 @@ __global__ __launch_bounds__(256) void layernorm_channel_first_kernel(const T *_
     }
 }
 
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
 inline bool grid_for(int64_t work, unsigned &blocks)
 {
     const int64_t b = (work + 255) / 256;
@@ -219,7 +217,7 @@ int swap_leading_axes(const void *in, void *out, int64_t n0, int64_t n1, int64_t
     }
     unsigned blocks;
     kutacc_prof::KernelTimer t("swap_axes_kernel", 0.0, stream);
-    if (row_bytes % 16 == 0 && aligned16(in) && aligned16(out)) {
+    if (row_bytes % 16 == 0 && kutacc_hip_aligned16(in) && kutacc_hip_aligned16(out)) {
         if (!grid_for(n0 * n1 * (row_bytes / 16), blocks)) {
             return KUTACC_HIP_EUNSUPPORTED;
         }
@@ -246,7 +244,7 @@ int residual_add(void *acc, const void *delta, int64_t n0, int64_t n1, int64_t i
         return KUTACC_HIP_EINVAL;
     }
     const int vw = dtype == KUTACC_DTYPE_BF16 ? 8 : 4; // elements per 16 bytes
-    const bool vec = inner % vw == 0 && aligned16(acc) && aligned16(delta);
+    const bool vec = inner % vw == 0 && kutacc_hip_aligned16(acc) && kutacc_hip_aligned16(delta);
     unsigned blocks;
     if (!grid_for(n0 * n1 * (vec ? inner / vw : inner), blocks)) {
         return KUTACC_HIP_EUNSUPPORTED;
@@ -278,7 +276,7 @@ int layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, con
     kutacc_prof::KernelTimer t("layernorm_channel_first_kernel", 0.0, stream);
     unsigned blocks;
     if (dtype == KUTACC_DTYPE_BF16 && channels == 128 && positions % 8 == 0 && ld_x % 8 == 0 && ld_out % 8 == 0 &&
-        aligned16(x) && aligned16(out)) {
+        kutacc_hip_aligned16(x) && kutacc_hip_aligned16(out)) {
         if (!grid_for(positions, blocks)) { // 256 positions per workgroup
             return KUTACC_HIP_EUNSUPPORTED;
         }

@@ -9,6 +9,9 @@
 // Turn a HIP status into the int the C ABI returns (0 = success, else the hipError_t value).
 static inline int kutacc_hip_status(hipError_t e) { return e == hipSuccess ? 0 : (int)e; }
 
+// 16-byte alignment of a pointer: what the vector loads and stores of the fast kernels need
+static inline bool kutacc_hip_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 namespace kutacc_launch {
 
 // generic_kernels.hip

@@ -795,12 +795,10 @@ __global__ __launch_bounds__(256) void sigmoid_gate_rows_kernel(bf16_t *__restri
     }
 }
 
-inline bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
-
 // does this operand suit the 16-byte loads of the MFMA kernel?  rows = extent of the non-k index
 bool operand_ok(const void *ptr, int64_t s_row, int64_t s_k, int64_t s_batch, int64_t rows, int64_t K, bool &mmajor)
 {
-    if (!aligned16(ptr) || s_batch % 8 != 0) {
+    if (!kutacc_hip_aligned16(ptr) || s_batch % 8 != 0) {
         return false;
     }
     if (s_k == 1) {
@@ -836,7 +834,7 @@ bool gated_projection_fits(const kutacc_hip_gemm_args_t &g)
 {
     return g.a_gate && g.mask && g.bias_axis == 2 && g.bias && g.bias_gate && g.batches == 1 && g.m == 128 && g.k == 128 &&
            g.a_stride_k == 1 && g.a_stride_m == 128 && g.b_stride_k == 1 && g.b_stride_n == 128 && g.n % 8 == 0 && g.n >= 8 &&
-           g.c_stride_m % 8 == 0 && aligned16(g.a) && aligned16(g.a_gate) && aligned16(g.b) && aligned16(g.c) &&
+           g.c_stride_m % 8 == 0 && kutacc_hip_aligned16(g.a) && kutacc_hip_aligned16(g.a_gate) && kutacc_hip_aligned16(g.b) && kutacc_hip_aligned16(g.c) &&
            (reinterpret_cast<uintptr_t>(g.mask) & 7u) == 0 && !g.relu;
 }
 
@@ -905,8 +903,8 @@ bool transition_fused_supports(int64_t rows, int64_t c_o, int64_t c_i, const voi
                                const void *w2, const float *b2, const void *out)
 {
     return (c_o == 128 || c_o == 256) && c_i >= 64 && c_i % 64 == 0 && c_i <= MAX_HIDDEN && rows > 0 &&
-           rows <= ((int64_t)1 << 31) * 64 && aligned16(x) && aligned16(w1) && aligned16(b1) && aligned16(w2) &&
-           aligned16(b2) && aligned16(out);
+           rows <= ((int64_t)1 << 31) * 64 && kutacc_hip_aligned16(x) && kutacc_hip_aligned16(w1) && kutacc_hip_aligned16(b1) && kutacc_hip_aligned16(w2) &&
+           kutacc_hip_aligned16(b2) && kutacc_hip_aligned16(out);
 }
 
 int transition_fused(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
@@ -959,11 +957,11 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
 
     bool am = false, bm = false;
     bool mfma_ok = operand_ok(g.a, g.a_stride_m, g.a_stride_k, g.a_stride_batch, g.m, g.k, am) &&
-                   operand_ok(g.b, g.b_stride_n, g.b_stride_k, g.b_stride_batch, g.n, g.k, bm) && aligned16(g.c) &&
+                   operand_ok(g.b, g.b_stride_n, g.b_stride_k, g.b_stride_batch, g.n, g.k, bm) && kutacc_hip_aligned16(g.c) &&
                    g.c_stride_m % 8 == 0 && g.c_stride_batch % 8 == 0 && g.n % 8 == 0 &&
-                   (g.bias_axis != 1 || aligned16(g.bias));
+                   (g.bias_axis != 1 || kutacc_hip_aligned16(g.bias));
     if (gated) {
-        mfma_ok = mfma_ok && !am && !bm && aligned16(g.a_gate) && aligned16(g.mask) && g.mask_stride_batch % 8 == 0;
+        mfma_ok = mfma_ok && !am && !bm && kutacc_hip_aligned16(g.a_gate) && kutacc_hip_aligned16(g.mask) && g.mask_stride_batch % 8 == 0;
     }
     if (g.path == KUTACC_HIP_PATH_GENERIC) {
         mfma_ok = false;
@@ -1024,7 +1022,7 @@ int sigmoid_gate_rows(void *out, int64_t out_s0, int64_t out_s1, const void *gat
     if (!out || !gate || n0 <= 0 || n1 <= 0 || size <= 0 || size > INT32_MAX) {
         return KUTACC_HIP_EINVAL;
     }
-    const bool vec = size % 8 == 0 && aligned16(out) && aligned16(gate) && out_s0 % 8 == 0 && out_s1 % 8 == 0 &&
+    const bool vec = size % 8 == 0 && kutacc_hip_aligned16(out) && kutacc_hip_aligned16(gate) && out_s0 % 8 == 0 && out_s1 % 8 == 0 &&
                      gate_s0 % 8 == 0 && gate_s1 % 8 == 0;
     const int64_t per_row = vec ? size / 8 : size;
     if (n0 > INT64_MAX / n1 || n0 * n1 > INT64_MAX / per_row) {
