@@ -7,6 +7,7 @@
 
 #include "device_util.h"
 #include "launch_internal.h"
+#include "mfma_tiles.h"
 
 using namespace kutacc_dev;
 
@@ -193,12 +194,15 @@ __global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *
     }
 }
 
-// Pair-bias producer, bf16, c_z = 128 (16 lanes per row), H <= 8.  A wave owns 64 consecutive rows of
-// z; its four 16-lane groups walk 16 rows each (all 16 loads of a lane are issued up front: 16 KB in
-// flight per wave).  The normalised row is rounded to bf16, as a caller of the reference would hand it
-// to kutacc_af2_linear, and dotted with the H weight rows by packed bf16 dot products with fp32
-// accumulation.  Lane 16q+s keeps the results of the row that group q handled in step s, so that at the end
-// lane L holds the H results of row r0+L and every head's 64 values leave as one 128-byte store.
+// Pair-bias producer, bf16, c_z = 128 (16 lanes per row), H <= 8.  A wave owns 32 consecutive rows of
+// z; its four 16-lane groups walk 8 rows each (all loads of a lane are issued up front: 8 KB in
+// flight per wave, and the small LDS tile leaves room for five workgroups per CU).  The normalised row is rounded to bf16, as a caller of the reference would hand it
+// to kutacc_af2_linear, written out (if wanted) and parked in a wave-private LDS tile; when the rows
+// are done, the [H, c_z] projection of all of them is 8 MFMAs (heads as MFMA rows, z rows as columns,
+// fp32 accumulation), whose result has one z row per lane: every head's 32 values leave as one 64-byte store.
+// The vector ALU, which bounds this kernel, is left with the LayerNorm alone.
+constexpr int PAIR_BIAS_ROWS_PER_WAVE = 32; // a multiple of 32; LDS per workgroup = 1 KB per row
+
 template <int H>
 __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__restrict__ z, const float *__restrict__ gamma,
                                                              const float *__restrict__ beta, const bf16_t *__restrict__ w,
@@ -206,21 +210,23 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
                                                              int64_t rows, float eps, int64_t rows_i, int64_t rows_j,
                                                              int transposed)
 {
-    constexpr int LPR = 16, CZ = 128;
+    constexpr int LPR = 16, CZ = 128, STEPS = PAIR_BIAS_ROWS_PER_WAVE / 4, RB = PAIR_BIAS_ROWS_PER_WAVE / 32;
+    __shared__ uint4 tiles[4][RB * 2 * 256]; // per wave: its rows x 128 channels as 32 x 64 panels
     const int lane = threadIdx.x & 63;
     const int sub = lane & 15, grp = lane >> 4;
-    const int64_t r0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;
+    const int64_t r0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * PAIR_BIAS_ROWS_PER_WAVE;
     if (r0 >= rows) {
         return;
     }
-    Pack16 in[16];
+    uint4 *tile = tiles[threadIdx.x >> 6];
+    Pack16 in[STEPS];
     {
         // transposed: output row (i, j) is computed from row (j, i) of z, stored [rows_j, rows_i, c_z]; the walk
-        // over 16 consecutive output rows then steps through z with stride rows_i rows
-        int64_t r = r0 + grp * 16;
+        // over consecutive output rows then steps through z with stride rows_i rows
+        int64_t r = r0 + grp * STEPS;
         int64_t i = transposed ? r / rows_j : 0, j = transposed ? r % rows_j : 0;
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
+        for (int s = 0; s < STEPS; ++s) {
             int64_t src = transposed ? j * rows_i + i : r;
             src = r < rows ? src : 0;
             in[s].u = *reinterpret_cast<const uint4 *>(z + src * CZ + sub * 8);
@@ -236,19 +242,23 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
         gm[e] = gamma[sub * 8 + e];
         bt[e] = beta[sub * 8 + e];
     }
-    Pack16 wv[H];
+    // weight fragments, heads as MFMA rows (rows >= H are zero): lane (head, g) holds w[head][16 ks + 8 g .. + 8]
+    kutacc_dev::bf16x8 wf[8];
+    {
+        const int head = lane & 31, g = lane >> 5;
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
-        wv[h].u = *reinterpret_cast<const uint4 *>(w + h * CZ + sub * 8);
+        for (int ks = 0; ks < 8; ++ks) {
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (head < H) {
+                v = *reinterpret_cast<const uint4 *>(w + head * CZ + ks * 16 + g * 8);
+            }
+            wf[ks] = kutacc_dev::as_bf16x8(v);
+        }
     }
-    float keep[H];
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
-        keep[h] = 0.f;
-    }
-#pragma unroll
-    for (int s = 0; s < 16; ++s) {
-        const int64_t r = r0 + grp * 16 + s;
+    for (int s = 0; s < STEPS; ++s) {
+        const int row_local = grp * STEPS + s;
+        const int64_t r = r0 + row_local;
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -265,22 +275,27 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
         if (z_norm != nullptr && r < rows) {
             *reinterpret_cast<uint4 *>(z_norm + r * CZ + sub * 8) = o.u;
         }
-#pragma unroll
-        for (int h = 0; h < H; ++h) {
-            float acc = 0.f;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                acc = __builtin_amdgcn_fdot2_f32_bf16(o.p[k], wv[h].p[k], acc, false);
-            }
-            acc = group_sum<LPR>(acc);
-            keep[h] = sub == s ? acc : keep[h];
-        }
+        tile[((row_local >> 5) * 2 + (sub >> 3)) * 256 + kutacc_dev::panel_slot(row_local & 31, sub & 7)] = o.u;
     }
-    const int64_t r = r0 + lane;
-    if (r < rows) {
+    // the tile is private to the wave and LDS operations of a wave complete in order: no barrier
+    const int col = lane & 31, g = lane >> 5;
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
-            nb[(int64_t)h * rows + r] = (bf16_t)keep[h];
+    for (int rb = 0; rb < RB; ++rb) {
+        kutacc_dev::f32x16 acc = kutacc_dev::zero16();
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const uint4 zf = tile[(rb * 2 + (ks >> 2)) * 256 + kutacc_dev::panel_slot(col, 2 * (ks & 3) + g)];
+            acc = kutacc_dev::mfma(wf[ks], kutacc_dev::as_bf16x8(zf), acc);
+        }
+        // accumulator v < 4 of lane (col, g) is head 4 g + v of z row r0 + 32 rb + col
+        const int64_t r = r0 + rb * 32 + col;
+        if (r < rows) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if (4 * g + v < H) {
+                    nb[(int64_t)(4 * g + v) * rows + r] = (bf16_t)acc[v];
+                }
+            }
         }
     }
 }
@@ -324,7 +339,7 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
     const int64_t rows = rows_i * rows_j;
     if (sizeof(T) == 2 && c_z == 128 && (nheads == 4 || nheads == 8) &&
         (reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(z_norm)) % 16 == 0) {
-        const int64_t nblk = (rows + 255) / 256;
+        const int64_t nblk = (rows + 4 * PAIR_BIAS_ROWS_PER_WAVE - 1) / (4 * PAIR_BIAS_ROWS_PER_WAVE);
         if (nblk > INT32_MAX) {
             return KUTACC_HIP_EUNSUPPORTED;
         }
