@@ -99,7 +99,7 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     g.input = ws + w.z_norm, g.input_ld = c;
     g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
     g.gating_b = a->gating_b, g.output_b = a->output_b;
-    g.bias = ws + w.bias, g.bias_stride_b = n;
+    g.bias = a->pair_mask, g.bias_stride_b = ending ? 1 : n;
     g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n * n, g.nb_stride_q = n;
     g.q = ws + w.q, g.q_stride_b = n * c, g.q_stride_s = c, g.q_stride_h = HEAD;
     g.avg = ws + w.avg, g.avg_stride_b = n * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
@@ -113,13 +113,13 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     if (rc != 0) {
         return rc;
     }
-    // 2. mask -> additive bias of the keys of every row
-    if ((rc = kutacc_launch::mask_bias(a->pair_mask, ws + w.bias, n, n, ending, KUTACC_DTYPE_BF16, s)) != 0) {
-        return rc;
-    }
-    // 3. the operator, its output projection adding straight into the pair activation (transposed back for the ending
-    //    node): the residual update costs no pass of its own
-    return kutacc_launch::gating_attention_fused(g, s, ending ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD);
+    // 2. the operator: it forms the mask bias from the pair mask itself, and its output projection adds straight into
+    //    the pair activation (transposed back for the ending node), so neither costs a pass of its own
+    kutacc_launch::FusedAttentionOptions opt;
+    opt.out_mode = ending ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
+    opt.bias_is_mask = true; // element (b, k) of the mask bias comes from mask[b, k], or mask[k, b] for the ending node
+    opt.bias_stride_k = ending ? n : 1;
+    return kutacc_launch::gating_attention_fused(g, s, opt);
 }
 
 int kutacc_hip_layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out,
@@ -352,7 +352,7 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
     g.input = ws + w.m_norm, g.input_ld = c;
     g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
     g.gating_b = a->gating_b, g.output_b = a->output_b;
-    g.bias = ws + w.bias, g.bias_stride_b = seq;
+    g.bias = a->msa_mask, g.bias_stride_b = column ? 1 : n_res;
     if (!column) {
         g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n_res * n_res, g.nb_stride_q = n_res;
     }
@@ -370,13 +370,14 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
         rc = kutacc_launch::pair_bias(a->pair_act, a->pair_ln_gamma, a->pair_ln_beta, a->bias_w, ws + w.nb, nullptr, n_res, n_res,
                                       a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s);
     }
-    // 3. mask bias [batch, seq]
+    // 3. the operator: mask bias formed from the msa mask on the fly, output projection adding into the msa (transposed
+    //    back for the column-wise form)
     if (rc == 0) {
-        rc = kutacc_launch::mask_bias(a->msa_mask, ws + w.bias, batch, seq, column, KUTACC_DTYPE_BF16, s);
-    }
-    // 4. the operator; its output projection adds into the msa (transposed back for the column-wise form)
-    if (rc == 0) {
-        rc = kutacc_launch::gating_attention_fused(g, s, column ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD);
+        kutacc_launch::FusedAttentionOptions opt;
+        opt.out_mode = column ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
+        opt.bias_is_mask = true; // msa_mask[s, r] is element (b = s, k = r) row-wise and (b = r, k = s) column-wise
+        opt.bias_stride_k = column ? n_res : 1;
+        rc = kutacc_launch::gating_attention_fused(g, s, opt);
     }
     return rc;
 }

@@ -85,7 +85,8 @@ struct FusedParams {
     const bf16_t *bias;
     const bf16_t *nb;
     bf16_t *avg;
-    int64_t x_ld, bias_sb, nb_sh, nb_sq, avg_sb, avg_ss, avg_sh;
+    int64_t x_ld, bias_sb, bias_sk, nb_sh, nb_sq, avg_sb, avg_ss, avg_sh;
+    int bias_is_mask; // bias holds the 0/1 mask; the kernels form 1e9*(mask-1) themselves
     int B, S, H, NB, NW, GW;
     int nb_vec;   // pair-bias rows may be read with 16-byte loads
     float qscale; // 1 / sqrt(head_size)
@@ -114,14 +115,21 @@ __device__ __forceinline__ void make_selectors(int lane, bf16x8 &sel0, bf16x8 &s
 // Mask bias of one batch row -> LDS as fp32 (keys past S get -inf), plus one flag bit per 32-key tile
 // saying "this tile needs the mask added" (non-zero bias or ragged tail).  Wave w covers keys
 // [64w, 64w+64); *flag_word must have been zeroed before, with a barrier in between.
+// bias_row[k * stride_k] is the mask bias itself, or (from_mask) the 0/1 mask, turned into 1e9*(mask-1) here with the
+// same multiply-add and bf16 rounding as the stand-alone mask-bias pass.
 __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *mask, uint32_t *flag_word, int S, int NB,
-                                                int wave, int lane, float scale = 1.0f)
+                                                int wave, int lane, float scale = 1.0f, int64_t stride_k = 1,
+                                                bool from_mask = false)
 {
     const int k = wave * 64 + lane;
     if (wave * 64 < NB * 32) {
         float mv = -INFINITY;
         if (k < S) {
-            mv = to_f32(bias_row[k]) * scale;
+            mv = to_f32(bias_row[k * stride_k]);
+            if (from_mask) {
+                mv = to_f32((bf16_t)fmaf(mv, 1e9f, -1e9f));
+            }
+            mv *= scale;
         }
         if (k < NB * 32) {
             mask[k] = mv;
@@ -726,7 +734,8 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     }
     __syncthreads();
     for (int part = wave; part * 64 < NT * 32; part += NW) {
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, part, lane, p.l2mode ? LOG2E : 1.0f);
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, part, lane, p.l2mode ? LOG2E : 1.0f, p.bias_sk,
+                        p.bias_is_mask != 0);
     }
 
     const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
@@ -950,7 +959,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == nrows - 1) {
             TL(10);
         }
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane, p.l2mode ? LOG2E : 1.0f);
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane, p.l2mode ? LOG2E : 1.0f, p.bias_sk,
+                        p.bias_is_mask != 0);
 
         // ---- input rows of the block -> fragments, 64 channels per staging panel ----
         const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
@@ -1518,8 +1528,9 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
     return make_plan(a.seq_len, (int)C, pl);
 }
 
-int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t stream, int residual)
+int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t stream, const FusedAttentionOptions &opt)
 {
+    const int residual = opt.out_mode;
     const int C = (int)(a.nheads * a.head_size);
     Plan pl;
     if (!make_plan(a.seq_len, C, pl)) {
@@ -1534,6 +1545,7 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     p.nb = (const bf16_t *)a.nonbatched_bias;
     p.avg = (bf16_t *)a.avg;
     p.x_ld = a.input_ld, p.bias_sb = a.bias_stride_b, p.nb_sh = a.nb_stride_h, p.nb_sq = a.nb_stride_q;
+    p.bias_sk = opt.bias_stride_k, p.bias_is_mask = opt.bias_is_mask ? 1 : 0;
     p.avg_sb = a.avg_stride_b, p.avg_ss = a.avg_stride_s, p.avg_sh = a.avg_stride_h;
     p.B = (int)a.batch, p.S = (int)a.seq_len, p.H = (int)a.nheads, p.NB = pl.NB, p.NW = pl.NW, p.GW = pl.GW;
     p.NT = (pl.NB + 1) & ~1;

@@ -24,7 +24,15 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &args);
 // `residual`: what the output projection does with its result -- store it in args.out (the operator as the reference
 // defines it), add it to args.out, or add row (b, s) of it to row (s, b) of args.out, then [seq_len, batch, C]
 constexpr int FUSED_OUT_STORE = 0, FUSED_OUT_ADD = 1, FUSED_OUT_ADD_TRANSPOSED = 2;
-int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream, int residual = FUSED_OUT_STORE);
+// bias_is_mask: args.bias holds the 0/1 mask instead of the mask bias, element (b, k) at b*bias_stride_b + k*bias_stride_k,
+// and the kernels form 1e9*(mask-1) themselves (no separate mask-bias pass; a transposed mask is a stride choice)
+struct FusedAttentionOptions {
+    int out_mode = FUSED_OUT_STORE;
+    bool bias_is_mask = false;
+    int64_t bias_stride_k = 1;
+};
+int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream,
+                           const FusedAttentionOptions &opt = FusedAttentionOptions());
 
 bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
                              int64_t m, int64_t n, int64_t k);
