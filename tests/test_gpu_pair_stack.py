@@ -359,3 +359,50 @@ def test_gated_projection_streaming_kernel(torch_cuda):
     a, b = helpers.to_numpy(outs[0][1]), helpers.to_numpy(outs[1][1])
     helpers.assert_within(a, b, 4e-3 + 1.2e-2 * np.abs(b), "streaming vs tiled kernel")
     assert bool((outs[0][1][:, t["mask"] == 0] == 0).all())
+
+
+def test_pair_stack_against_the_golden_fixture(torch_cuda):
+    """The committed float64 fixture (tests/golden/pair_stack_tiny.npz) through the handle-based entry points.  Its
+    inputs are rounded to bf16 on the way to the device, so the comparison runs at the bf16 bar."""
+    import os
+    torch = torch_cuda
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "pair_stack_tiny.npz"))
+    n, c_o, c_i, hid = 6, 8, 4, 12
+    d = lambda k, dt=torch.bfloat16: torch.from_numpy(g["in." + k]).to(device="cuda", dtype=dt)  # noqa: E731
+    f32 = torch.float32
+    # transition
+    x = d("x")
+    mid = torch.zeros(n * n, hid, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(n, n, c_o, dtype=torch.bfloat16, device="cuda")
+    capi.Transition(x, d("w1"), d("b1", f32), d("w2"), d("b2", f32), mid, out).run()
+    assert not capi.error_flag()
+    helpers.check_close(helpers.to_numpy(out), g["transition.out"], "bf16", "fixture transition")
+    # projections and equation
+    proj = {}
+    for side in ("left", "right"):
+        p = torch.zeros(c_i, n, n, dtype=torch.bfloat16, device="cuda")
+        keep = [d(side + "_w"), d(side + "_b", f32), d(side + "_gw"), d(side + "_gb", f32), d("mask"), torch.zeros_like(p)]
+        h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]
+        hp, hx, hm, hg = capi.tensor(p), capi.tensor(x), capi.tensor(keep[4]), capi.tensor(keep[5])
+        capi.kutacc_af2_triangle_multiplication_calc_proj(capi.TmActInputs(n, n, hp.handle, hx.handle, hg.handle), hm,
+                                                          capi.TmProjWeights(c_o, c_i, h[0].handle, h[1].handle, h[2].handle,
+                                                                             h[3].handle), False)
+        assert not capi.error_flag()
+        helpers.check_close(helpers.to_numpy(p), g["tm." + side], "bf16", f"fixture {side} projection")
+        proj[side] = p
+    for name, incoming in (("tm.outgoing", False), ("tm.incoming", True)):
+        center = equation(torch, proj["left"], proj["right"], n, incoming)
+        helpers.check_close(helpers.to_numpy(center), g[name], "bf16", "fixture " + name)
+    # output step
+    gate = torch.zeros(n, n, c_o, dtype=torch.bfloat16, device="cuda")
+    res = torch.zeros_like(gate)
+    keep = [d("gating_w"), d("gating_b", f32), d("out_w"), d("out_b", f32), d("center")]
+    h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]
+    hx, hgt, hres, hc = capi.tensor(x), capi.tensor(gate), capi.tensor(res), capi.tensor(keep[4])
+    capi.kutacc_af2_triangle_multiplication_gate_and_out_linear(hgt, hres, capi.TmActInputs(n, n, None, hx.handle, None), hc,
+                                                                capi.TmLinearWeights(c_o, c_i, h[0].handle, h[1].handle,
+                                                                                     h[2].handle, h[3].handle), False)
+    capi.kutacc_af2_triangle_multiplication_last(hres, hgt, n, n, c_o)
+    assert not capi.error_flag()
+    helpers.check_close(helpers.to_numpy(gate), g["tm.gate"], "bf16", "fixture gate")
+    helpers.check_close(helpers.to_numpy(res), g["tm.last"], "bf16", "fixture gated output")

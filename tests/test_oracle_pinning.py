@@ -559,3 +559,22 @@ def test_tm_output_step_matches_torch():
     np.testing.assert_allclose(out, o_ref.numpy(), rtol=1e-6, atol=1e-6)
     np.testing.assert_allclose(oracle.tm_last_f32(out, gate), (o_ref * torch.sigmoid(g_ref)).numpy(), rtol=1e-6, atol=1e-6)
     np.testing.assert_array_equal(oracle.tm_last_f32(out, np.full_like(gate, 100.0)), out)
+
+
+def test_pair_stack_oracle_matches_golden_fixture():
+    """tests/golden/pair_stack_tiny.npz (float64 einsum expressions, made by tests/golden/make_golden_pair_stack.py)."""
+    g = np.load(os.path.join(HERE, "golden", "pair_stack_tiny.npz"))
+    i = lambda k: g["in." + k]  # noqa: E731
+    out, mid = oracle.transition_f32(i("x").reshape(-1, 8), i("w1"), i("b1"), i("w2"), i("b2"), return_mid=True)
+    np.testing.assert_allclose(mid.reshape(6, 6, 12), g["transition.mid"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(out.reshape(6, 6, 8), g["transition.out"], rtol=1e-5, atol=1e-5)
+    left = oracle.tm_calc_proj_f32(i("x"), i("mask"), i("left_w"), i("left_b"), i("left_gw"), i("left_gb"))
+    right = oracle.tm_calc_proj_f32(i("x"), i("mask"), i("right_w"), i("right_b"), i("right_gw"), i("right_gb"))
+    np.testing.assert_allclose(left, g["tm.left"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(right, g["tm.right"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(oracle.tm_equation_f32(left, right, False), g["tm.outgoing"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(oracle.tm_equation_f32(left, right, True), g["tm.incoming"], rtol=1e-5, atol=1e-5)
+    gate, proj = oracle.tm_gate_and_out_f32(i("x"), i("center"), i("gating_w"), i("gating_b"), i("out_w"), i("out_b"))
+    np.testing.assert_allclose(gate.reshape(6, 6, 8), g["tm.gate"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(proj.reshape(6, 6, 8), g["tm.out"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(oracle.tm_last_f32(proj, gate).reshape(6, 6, 8), g["tm.last"], rtol=1e-5, atol=1e-5)
