@@ -419,3 +419,51 @@ def test_layernorm_rows_transposed(torch_cuda):
                                                       rows_j, size, 1e-5, code(torch, x), None) == 0
         torch.cuda.synchronize()
         assert helpers.same_bits(a, b)
+
+
+def test_pair_stack_blocks_replay_from_a_hip_graph(torch_cuda):
+    """The three pair-stack blocks (triangle multiplication, triangle attention, transition) captured into one HIP graph
+    on a side stream and replayed three times, with eager work (restoring the pair tensor) between the replays; every
+    replay must reproduce the eager result bit for bit.  Nothing in the launch path allocates, frees, memsets or
+    synchronises, which is what makes the blocks capturable."""
+    torch = torch_cuda
+    n, heads = 64, 4
+    c = heads * 32
+    ca, ct = block_case(1200, n, heads), tm_block_case(1201, n, c, c)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    z0 = dev(ca["z"])
+    z = z0.clone()
+    mask = dev(ca["mask"])
+    tm = capi.TriangleMultiplicationBlock(z, mask, {k: dev(v) for k, v in ct.items() if k not in ("z", "mask")}, False)
+    ta = capi.TriangleAttentionBlock(z, mask, dev(ca["gamma"]), dev(ca["beta"]), dev(ca["bias_w"]), dev(ca["wq"]), dev(ca["wk"]),
+                                     dev(ca["wv"]), dev(ca["wg"]), dev(ca["bg"]), dev(ca["wo"]), dev(ca["bo"]), heads, True)
+    rng = np.random.Generator(np.random.PCG64(5))
+    w1 = dev(round_to_bf16((rng.standard_normal((4 * c, c)) / math.sqrt(c)).astype(np.float32)))
+    w2 = dev(round_to_bf16((rng.standard_normal((c, 4 * c)) / math.sqrt(4 * c)).astype(np.float32)))
+    b1, b2 = dev((rng.standard_normal(4 * c) * 0.1).astype(np.float32)), dev((rng.standard_normal(c) * 0.1).astype(np.float32))
+    gam, bet = dev(ca["gamma"]), dev(ca["beta"])
+    L = capi.lib()
+
+    def blocks(stream_ptr):
+        assert tm.run(stream_ptr) == 0
+        assert ta.run(stream_ptr) == 0
+        assert L.kutacc_hip_transition_block(z.data_ptr(), gam.data_ptr(), bet.data_ptr(), 1e-5, w1.data_ptr(), b1.data_ptr(),
+                                             w2.data_ptr(), b2.data_ptr(), None, 0, n * n, c, 4 * c, capi.K_BF16, stream_ptr) == 0
+
+    blocks(None)  # eager, also takes every first-call set-up (kernel attributes) out of the capture
+    torch.cuda.synchronize()
+    want = z.clone()
+    assert not helpers.same_bits(want, z0)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    z.copy_(z0)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        blocks(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        z.copy_(z0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert helpers.same_bits(z, want)
