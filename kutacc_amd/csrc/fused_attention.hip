@@ -417,7 +417,8 @@ __device__ __forceinline__ float rowsum_fetch(const f32x4 &lacc, int lane)
 template <bool HAS_NB, bool WITH_MASK, bool SHIFT>
 __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4,
                                                 const uint4 *nbf, bf16x8 q0, bf16x8 q1, bf16x8 sel0, bf16x8 sel1,
-                                                bf16x8 sumsel, int NB, int lane, float shift, f32x16 &o_out, float &l_out)
+                                                bf16x8 sumsel, int NB, int lane, float shift, f32x16 &o_out, float &l_out,
+                                                int prio_phase = -1)
 {
     const int npairs = NB >> 1;
     const uint4 *kp = lds_k + lane;
@@ -505,6 +506,15 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
     };
 
     for (int pair = 0; pair < npairs; ++pair) {
+        if (prio_phase >= 0) {
+            // two waves of one workgroup share a SIMD in lock step; the arbiter prefers the older one, which then runs
+            // ahead and leaves the other to finish alone.  Alternating the issue priority per tile pair keeps them level.
+            if ((pair + prio_phase) & 1) {
+                __builtin_amdgcn_s_setprio(1);
+            } else {
+                __builtin_amdgcn_s_setprio(0);
+            }
+        }
         const int t1 = 2 * pair + 1;
         const int tn = pair + 1 < npairs ? 2 * pair + 2 : 2 * pair; // next pair's first tile, clamped
         // ---- odd tile's logits under the even tile's softmax ----
@@ -743,9 +753,18 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     bf16x8 qf[BPW][2];   // Q^T fragments (B operand of the logits MFMA), scaled by 1/sqrt(d)
     bf16x8 gate[BPW][2]; // sigmoid(gate) in accumulator order, packed
     const int npass = 4 / GW;
-    for (int pass = 0; pass < npass; ++pass) {
+    // With at least two matrices per group K and V (matrices 0 and 1) share a group; the groups are then walked from the
+    // last to the first, so that K and V come last and the K/V fragment slots of a block stay free until that block's
+    // own results land in them.  That lets the input rows take the coalesced route: a 4 KB staging panel aliased onto
+    // the block's K slot (rows 0-15) and V slot (rows 16-31), private to the wave that owns the block.  With one matrix
+    // per group there is no such free space (LDS is full at that sequence length) and the fragments are loaded from
+    // global memory directly.
+    const bool staged_input = GW >= 2;
+    const int prow = pi_row(r);
+    for (int pi = 0; pi < npass; ++pi) {
+        const int pass = staged_input ? npass - 1 - pi : pi;
         __syncthreads(); // previous group's fragments are no longer being read
-        if (pass == 0) {
+        if (pi == 0) {
             TL(1);
         }
         for (int idx = tid; idx < GW * CK * 64; idx += nthreads) {
@@ -756,7 +775,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             lds_w[idx] = *reinterpret_cast<const uint4 *>(src);
         }
         __syncthreads();
-        if (pass == 0) {
+        if (pi == 0) {
             TL(2);
         }
 #pragma unroll
@@ -765,13 +784,35 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             if (j >= NB) {
                 continue;
             }
-            int srow = j * 32 + pi_row(r);
-            srow = srow < S ? srow : S - 1; // rows past the end repeat the last row; they are never stored
-            const bf16_t *xrow = p.x + ((int64_t)b * S + srow) * p.x_ld + g * 8;
             bf16x8 xf[CK];
+            if (staged_input) {
+                const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
+                uint4 *kslot = lds_k + j * 128, *vslot = lds_v + j * 128 - 128; // panel slots 0-127 and 128-255
+                const uint4 *fsrc = prow < 16 ? kslot : vslot;
+                const int srow8 = lane >> 3, chunk = lane & 7;
+                PanelRegs t = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane);
 #pragma unroll
-            for (int ks = 0; ks < CK; ++ks) {
-                xf[ks] = as_bf16x8(*reinterpret_cast<const uint4 *>(xrow + ks * 16));
+                for (int c = 0; c < CK / 4; ++c) {
+                    kslot[panel_slot(srow8, chunk)] = t.r0;
+                    kslot[panel_slot(srow8 + 8, chunk)] = t.r1;
+                    vslot[panel_slot(srow8 + 16, chunk)] = t.r2;
+                    vslot[panel_slot(srow8 + 24, chunk)] = t.r3;
+                    if (c + 1 < CK / 4) {
+                        t = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 1) * 64, lane);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        xf[4 * c + k] = as_bf16x8(fsrc[panel_slot(prow, 2 * k + g)]);
+                    }
+                }
+            } else {
+                int srow = j * 32 + prow;
+                srow = srow < S ? srow : S - 1; // rows past the end repeat the last row; they are never stored
+                const bf16_t *xrow = p.x + ((int64_t)b * S + srow) * p.x_ld + g * 8;
+#pragma unroll
+                for (int ks = 0; ks < CK; ++ks) {
+                    xf[ks] = as_bf16x8(*reinterpret_cast<const uint4 *>(xrow + ks * 16));
+                }
             }
             for (int mm = 0; mm < GW; ++mm) {
                 const int m = pass * GW + mm;
@@ -843,11 +884,12 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NT * 2) * 64 + lane : nullptr;
             if (flags == 0u) {
                 attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
-                                                      lane, 0.f, o, l);
+                                                      lane, 0.f, o, l, (wave >> 2) & 1);
             } else {
                 attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
-                                                     lane, 0.f, o, l);
+                                                     lane, 0.f, o, l, (wave >> 2) & 1);
             }
+            __builtin_amdgcn_s_setprio(0);
             if (__any(!(l > 1e-30f && l < 1e30f))) {
                 // some probability overflowed or a whole row underflowed: shift by the true row maxima
                 const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, NT, lane);
