@@ -142,6 +142,21 @@ __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *m
     }
 }
 
+// The value stage_mask_part would store for key k, for kernels that fetch the mask early and store it later.
+__device__ __forceinline__ float mask_bias_value(const bf16_t *bias_row, int S, int k, float scale, int64_t stride_k,
+                                                 bool from_mask)
+{
+    float mv = -INFINITY;
+    if (k < S) {
+        mv = to_f32(bias_row[k * stride_k]);
+        if (from_mask) {
+            mv = to_f32((bf16_t)fmaf(mv, 1e9f, -1e9f));
+        }
+        mv *= scale;
+    }
+    return mv;
+}
+
 // Flash-style attention of one 32-query block against all keys of the unit.
 //   lds_k / lds_v : K and V fragments of the unit, [tile][kstep][lane] in 16-byte units
 //   mask4         : fp32 mask bias in LDS, already offset by 16*g floats; flags: one bit per tile
@@ -699,9 +714,12 @@ __device__ __forceinline__ void store_gated(bf16_t *dst, const f32x16 &o, float 
 // fused_head_kernel: one workgroup per (b, h) unit
 // LDS carve-up, in 16-byte units unless noted:
 //   [0, GW*CK*64)               staged weight fragments  [slot][kstep][lane]
-//   [.., +NB*2*64)              K fragments              [tile][kstep][lane]
-//   [.., +NB*2*64)              V fragments              [tile][kstep][lane]
-//   then floats: mask[NB*32] (-inf past S), then one uint32 of tile flags
+//   [.., +NT*2*64)              K fragments              [tile][kstep][lane]
+//   [.., +NT*2*64)              V fragments              [tile][kstep][lane]
+// The mask of the batch row (floats, -inf past S) and the tile flags are needed only by the attention phase and take
+// the place of the weight fragments once the projections are done; every thread fetches its mask values at the start
+// and keeps them in registers until then.  At 1024 keys that leaves room for all four weight matrices of a
+// 128-channel head (two of a 256-channel one) beside K and V, so the input rows are read once (twice).
 // ------------------------------------------------------------------------------------------------
 template <int C, int BPW, bool HAS_NB>
 __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(FusedParams p)
@@ -729,12 +747,9 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     uint4 *lds_w = lds;
     uint4 *lds_k = lds_w + GW * CK * 64;
     uint4 *lds_v = lds_k + NT * 2 * 64;
-    float *mask = reinterpret_cast<float *>(lds_v + NT * 2 * 64);
-    uint32_t *flag_word = reinterpret_cast<uint32_t *>(mask + NT * 32);
+    float *mask = reinterpret_cast<float *>(lds_w);
+    uint32_t *part_flags = reinterpret_cast<uint32_t *>(mask + NT * 32); // two flag bits per 64 keys, one word each
 
-    if (tid == 0) {
-        *flag_word = 0;
-    }
     if (NT > NB) { // phantom key tile: zero K and V fragments
         const uint4 z4 = {0u, 0u, 0u, 0u};
         for (int idx = tid; idx < 128; idx += nthreads) {
@@ -742,10 +757,13 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             lds_v[NB * 2 * 64 + idx] = z4;
         }
     }
-    __syncthreads();
-    for (int part = wave; part * 64 < NT * 32; part += NW) {
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, part, lane, p.l2mode ? LOG2E : 1.0f, p.bias_sk,
-                        p.bias_is_mask != 0);
+    // wave w holds the mask of keys [64(w + q NW), +64): NT <= 4 NW + 1 tiles are at most 2 NW such parts
+    constexpr int MASK_PARTS = (BPW + 1) / 2;
+    float mask_value[MASK_PARTS];
+#pragma unroll
+    for (int q = 0; q < MASK_PARTS; ++q) {
+        mask_value[q] = mask_bias_value(p.bias + (int64_t)b * p.bias_sb, S, (wave + q * NW) * 64 + lane,
+                                        p.l2mode ? LOG2E : 1.0f, p.bias_sk, p.bias_is_mask != 0);
     }
 
     const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
@@ -860,11 +878,27 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         }
     }
     TL(3);
-    __syncthreads(); // K and V of the whole sequence are in LDS
+    __syncthreads(); // K and V of the whole sequence are in LDS; the weight fragments are no longer read
+#pragma unroll
+    for (int q = 0; q < MASK_PARTS; ++q) {
+        const int part = wave + q * NW;
+        if (part * 64 < NT * 32) {
+            const float mv = mask_value[q];
+            mask[part * 64 + lane] = mv;
+            const unsigned long long nz = __ballot(mv != 0.f);
+            if (lane == 0) {
+                part_flags[part] = ((uint32_t)nz != 0u ? 1u : 0u) | ((uint32_t)(nz >> 32) != 0u ? 2u : 0u);
+            }
+        }
+    }
+    __syncthreads();
     TL(4);
 
     // ---- attention: each wave walks the key tiles for its own query blocks ----
-    const uint32_t flags = *flag_word;
+    uint32_t flags = 0; // bit t: key tile t needs the mask added (non-zero bias or ragged tail)
+    for (int part = 0; part * 64 < NT * 32; ++part) {
+        flags |= part_flags[part] << (2 * part);
+    }
     const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
     bf16x8 sel0, sel1;
     make_selectors(lane, sel0, sel1);
@@ -1387,7 +1421,8 @@ int num_cus()
 size_t head_kernel_lds(int C, int NB, int GW)
 {
     const int NT = (NB + 1) & ~1; // key tiles, padded to a pair
-    return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NT * 2 * 64 * 16 * 2 + (size_t)NT * 32 * 4 + 16;
+    // weight fragments (the mask, 4 bytes per key, and 16 flag words take their place later), K and V
+    return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NT * 2 * 64 * 16 * 2;
 }
 
 size_t persistent_kernel_lds(int C, int NB)
