@@ -798,10 +798,14 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         }
 #pragma unroll
         for (int i = 0; i < BPW; ++i) {
-            const int j = wave + i * NW;
+            int j = wave + i * NW;
             if (j >= NB) {
                 continue;
             }
+            // Opaque to the optimiser: otherwise the row addresses of every block of the wave are computed once, ahead
+            // of the loop over the groups, and with three or four blocks of 256-channel rows they no longer fit the
+            // registers -- each spilled address then costs a scratch round trip in front of the load it feeds.
+            asm volatile("" : "+v"(j));
             bf16x8 xf[CK];
             if (staged_input) {
                 const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
