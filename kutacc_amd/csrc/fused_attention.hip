@@ -973,7 +973,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     extern __shared__ uint4 lds[];
     TL(7);
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: values derived from it stay in scalar registers
     const int r = lane & 31, g = lane >> 5;
     const int S = p.S, NB = p.NB, NT = p.NT;
     const int nthreads = NB * 64;
@@ -994,7 +994,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     uint4 *lds_k = lds_w + 4 * CK * 64;
     uint4 *lds_v = lds_k + NT * 2 * 64;
     uint4 *panel = lds_v + NT * 2 * 64 + wave * 256;
-    uint4 *gate_park = lds_v + NT * 2 * 64 + NB * 256 + wave * 128 + lane; // sigmoid(gate) waits here during attention
+    uint4 *gate_park_base = lds_v + NT * 2 * 64 + NB * 256 + wave * 128; // sigmoid(gate) waits here during attention
     float *mask_base = reinterpret_cast<float *>(lds_v + NT * 2 * 64 + NB * 256 + NB * 128); // two buffers of NT*32
     uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 2 * NT * 32);            // two, alternating by batch row
 
@@ -1024,8 +1024,9 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     TL(8);
     const int j = wave; // this wave's sequence block
     const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
+    // uniform, and kept in a scalar register
+    const float mask_scale = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(p.l2mode ? LOG2E : 1.0f)));
     const bf16x8 sumsel = rowsum_selector(lane);
-    const int qpos = j * 32 + prow;
     for (int n = 0; n < nrows; ++n) {
         const int b = b0 + n * bstep;
         uint32_t *flag_word = flag_words + (n & 1);
@@ -1039,33 +1040,39 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         if (n == nrows - 1) {
             TL(10);
         }
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane, p.l2mode ? LOG2E : 1.0f, p.bias_sk,
+        // The lane index is opaque to the optimiser here: the row addresses and panel offsets derived from it are then
+        // formed anew for every batch row (a few dozen vector instructions) instead of being kept across the attention
+        // loop, where there is no register for them -- spilled, each costs a scratch round trip per batch row.
+        int lane_x = lane;
+        asm volatile("" : "+v"(lane_x));
+        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane_x, mask_scale, p.bias_sk,
                         p.bias_is_mask != 0);
 
         // ---- input rows of the block -> fragments, 64 channels per staging panel ----
+        const int prow_x = pi_row(lane_x & 31), g_x = lane_x >> 5;
         const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
         bf16x8 xf[CK];
         {
             PanelRegs ta, tb;
-            ta = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane);
+            ta = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane_x);
 #pragma unroll
             for (int c = 0; c < NP; c += 2) {
                 if (c + 1 < NP) {
-                    tb = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 1) * 64, lane);
+                    tb = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 1) * 64, lane_x);
                 }
-                panel_store(panel, lane, ta);
+                panel_store(panel, lane_x, ta);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    xf[4 * c + k] = as_bf16x8(panel[panel_slot(prow, 2 * k + g)]);
+                    xf[4 * c + k] = as_bf16x8(panel[panel_slot(prow_x, 2 * k + g_x)]);
                 }
                 if (c + 1 < NP) {
                     if (c + 2 < NP) {
-                        ta = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 2) * 64, lane);
+                        ta = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 2) * 64, lane_x);
                     }
-                    panel_store(panel, lane, tb);
+                    panel_store(panel, lane_x, tb);
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
-                        xf[4 * (c + 1) + k] = as_bf16x8(panel[panel_slot(prow, 2 * k + g)]);
+                        xf[4 * (c + 1) + k] = as_bf16x8(panel[panel_slot(prow_x, 2 * k + g_x)]);
                     }
                 }
             }
@@ -1077,7 +1084,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         bf16x8 q0, q1;
         uint4 kfrag0, kfrag1, vfrag0, vfrag1; // this block's K and V fragments, parked until the LDS arrays are free
         {
-            const uint4 *wsrc = lds_w + lane;
+            uint4 *gate_park_x = gate_park_base + lane_x;
+            const uint4 *wsrc = lds_w + lane_x;
             f32x16 acc = zero16();
 #pragma unroll
             for (int ks = 0; ks < CK; ++ks) {
@@ -1108,7 +1116,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             for (int ks = 0; ks < CK; ++ks) {
                 acc = mfma(as_bf16x8(wsrc[(PROJ_G * CK + ks) * 64]), xf[ks], acc);
             }
-            const float *bgp = p.bg + h * HEAD + 4 * g;
+            const float *bgp = p.bg + h * HEAD + 4 * g_x;
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 const f32x4 bv = *reinterpret_cast<const f32x4 *>(bgp + 8 * a);
@@ -1117,8 +1125,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                     acc[4 * a + c] = sigmoid_fast(acc[4 * a + c] + bv[c]);
                 }
             }
-            gate_park[0] = as_uint4(pack8(acc, 0));
-            gate_park[64] = as_uint4(pack8(acc, 8));
+            gate_park_x[0] = as_uint4(pack8(acc, 0));
+            gate_park_x[64] = as_uint4(pack8(acc, 8));
         }
         if (n == 2) {
             TL(2);
@@ -1163,15 +1171,19 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, nb_head, p.nb_sq, j * 32, p.nb_vec != 0, panel, q0, q1, sel0,
                                  sel1, NB, S, lane, o, l);
         }
+        int lane_o = lane; // as above: the addresses of the epilogue are not worth a register during the attention loop
+        asm volatile("" : "+v"(lane_o));
+        const int qpos = j * 32 + pi_row(lane_o & 31);
         if (qpos < S) {
-            const bf16x8 gate0 = as_bf16x8(gate_park[0]), gate1 = as_bf16x8(gate_park[64]);
+            const uint4 *gate_park_o = gate_park_base + lane_o;
+            const bf16x8 gate0 = as_bf16x8(gate_park_o[0]), gate1 = as_bf16x8(gate_park_o[64]);
             f32x16 gv;
 #pragma unroll
             for (int v = 0; v < 8; ++v) {
                 gv[v] = to_f32(gate0[v]);
                 gv[8 + v] = to_f32(gate1[v]);
             }
-            store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * g, o,
+            store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * (lane_o >> 5), o,
                         __builtin_amdgcn_rcpf(l), gv);
         }
         if (n == 2) {
