@@ -1230,7 +1230,6 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
     const int r = lane & 31, g = lane >> 5;
     const int n0 = blockIdx.y * 128;
     uint4 *panel = lds + 4 * CK * 64 + wave * 256;
-    const float *bias = bo + n0 + 4 * g; // read per use: 16 cached loads per tile instead of 64 live registers
     // Every wave owns a contiguous range of rows_per_wave rows (a multiple of 8), walked 32 rows at a
     // time; the last step of a range may be partial.  Equal ranges rather than whole 32-row tiles dealt
     // round robin: the kernel is short, and a wave with one tile more than its neighbours would set its
@@ -1263,31 +1262,40 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
     __syncthreads();
     for (int64_t rbase = start; rbase < stop; rbase += 32) {
         const int row0 = (int)rbase;
-        bf16x8 af[CK];
-        panel_store(panel, lane, ta);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            af[k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+        // With 256 input features the lane index is opaque to the optimiser, so that addresses and panel offsets are
+        // formed per step instead of being kept (and partly spilled) across the loop.  With 128 the kernel fits either
+        // way, and the smaller footprint would let a third workgroup onto some CUs of a grid sized for two.
+        int lv = lane;
+        if constexpr (C > 128) {
+            asm volatile("" : "+v"(lv));
         }
-        panel_store(panel, lane, tb);
+        const int rv = lv & 31, gv = lv >> 5;
+        const float *bias = bo + n0 + 4 * gv; // read per use: 16 cached loads per tile instead of 64 live registers
+        bf16x8 af[CK];
+        panel_store(panel, lv, ta);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            af[4 + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+            af[k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+        }
+        panel_store(panel, lv, tb);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            af[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
         }
 #pragma unroll
         for (int c = 2; c < NP; ++c) {
-            ta = panel_load(avg, avg_ld, row0, last_row, c * 64, lane);
-            panel_store(panel, lane, ta);
+            ta = panel_load(avg, avg_ld, row0, last_row, c * 64, lv);
+            panel_store(panel, lv, ta);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                af[4 * c + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+                af[4 * c + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
             }
         }
         {
             // clamped to the last step instead of a branch: one harmless re-read at the end
             const int rnext = rbase + 32 < stop ? row0 + 32 : row0;
-            ta = panel_load(avg, avg_ld, rnext, last_row, 0, lane);
-            tb = panel_load(avg, avg_ld, rnext, last_row, 64, lane);
+            ta = panel_load(avg, avg_ld, rnext, last_row, 0, lv);
+            tb = panel_load(avg, avg_ld, rnext, last_row, 64, lv);
         }
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
@@ -1295,9 +1303,9 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
             if constexpr (EPILOGUE != EPILOGUE_STORE) { // requested before the MFMAs, used after them
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    int64_t row = (int64_t)row0 + 8 * i + (lane >> 3);
+                    int64_t row = (int64_t)row0 + 8 * i + (lv >> 3);
                     row = row < stop ? row : stop - 1;
-                    const int64_t col = n0 + half * 64 + (lane & 7) * 8;
+                    const int64_t col = n0 + half * 64 + (lv & 7) * 8;
                     if constexpr (EPILOGUE == EPILOGUE_GATED_RESIDUAL) {
                         gq[i] = *reinterpret_cast<const uint4 *>(gate + row * gate_ld + col);
                     }
@@ -1310,7 +1318,7 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
             for (int ks = 0; ks < CK; ++ks) {
 #pragma unroll
                 for (int n = 0; n < 2; ++n) {
-                    acc[n] = mfma(as_bf16x8(lds[((2 * half + n) * CK + ks) * 64 + lane]), af[ks], acc[n]);
+                    acc[n] = mfma(as_bf16x8(lds[((2 * half + n) * CK + ks) * 64 + lv]), af[ks], acc[n]);
                 }
             }
             // accumulators -> panel as bf16 [row][64 features], then whole-line stores
@@ -1324,14 +1332,14 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
                     for (int c = 0; c < 4; ++c) {
                         ov[c] = (bf16_t)(acc[n][4 * a + c] + bv[c]);
                     }
-                    bf16x4 *dst = reinterpret_cast<bf16x4 *>(panel + panel_slot(r, n * 4 + a)) + g;
+                    bf16x4 *dst = reinterpret_cast<bf16x4 *>(panel + panel_slot(rv, n * 4 + a)) + gv;
                     *dst = ov;
                 }
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int prow_ = 8 * i + (lane >> 3);
-                uint4 v = panel[panel_slot(prow_, lane & 7)];
+                const int prow_ = 8 * i + (lv >> 3);
+                uint4 v = panel[panel_slot(prow_, lv & 7)];
                 const int64_t row = (int64_t)row0 + prow_;
                 if constexpr (EPILOGUE == EPILOGUE_GATED_RESIDUAL) {
                     const bf16x8 o = as_bf16x8(v), gt = as_bf16x8(gq[i]), z = as_bf16x8(zq[i]);
@@ -1353,7 +1361,7 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
                     v = as_uint4(res);
                 }
                 if (row < stop) {
-                    *reinterpret_cast<uint4 *>(out + target_row(row) * out_ld + n0 + half * 64 + (lane & 7) * 8) = v;
+                    *reinterpret_cast<uint4 *>(out + target_row(row) * out_ld + n0 + half * 64 + (lv & 7) * 8) = v;
                 }
             }
         }
@@ -1580,7 +1588,8 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
         return rc;
     }
     const int64_t tiles = (M + 31) / 32;
-    // two resident workgroups per CU, each wave with an equal share of the rows
+    // two workgroups per CU, each wave with an equal share of the rows (a third resident workgroup, where the registers
+    // allow one, measured slower: the weight slab is staged per workgroup)
     int64_t gx = (tiles + 3) / 4;
     const int64_t cap = (int64_t)num_cus() * 2;
     gx = gx > cap ? cap : gx;
