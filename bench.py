@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # (two runs, scaled against a 256 MiB copy: FETCH x2.000, WRITE x1.000; see
 # profiles/gating_attention_cfg3_hbm_traffic.txt).  Not re-measured live; configurations without an entry report null.
 MEASURED_TRAFFIC_BYTES = {
-    (3, "persistent_head_kernel"): int((26682.4 * 2.0 + 55296.0) * 1024),
+    (3, "persistent_head_kernel"): int((23782.8 * 2.0 + 41472.0) * 1024),
 }
 
 
