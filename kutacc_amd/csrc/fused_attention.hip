@@ -740,7 +740,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     const int tid = threadIdx.x;
     TL(0);
     const int nthreads = p.NW * 64;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, kept in a scalar register
     const int r = lane & 31, g = lane >> 5;
     const int S = p.S, NB = p.NB, NT = p.NT, NW = p.NW, GW = p.GW;
 
@@ -805,7 +805,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             // Opaque to the optimiser: otherwise the row addresses of every block of the wave are computed once, ahead
             // of the loop over the groups, and with three or four blocks of 256-channel rows they no longer fit the
             // registers -- each spilled address then costs a scratch round trip in front of the load it feeds.
-            asm volatile("" : "+v"(j));
+            asm volatile("" : "+s"(j));
             bf16x8 xf[CK];
             if (staged_input) {
                 const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
