@@ -612,10 +612,12 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
     const int64_t stop = start + pos_per_wave < n_pos ? start + pos_per_wave : n_pos;
     const int last = (int)(stop - start) - 1; // last valid position of the range, relative to start
     const bf16_t *xb = x + start * C;
-    PanelRegs t[4]; // two 32-row blocks x two 64-column halves of the current step
+    // two 32-row blocks x two 64-column halves per step; the first three are asked for a step ahead, the fourth at the
+    // top of its own step (a fourth set of registers held across the channel loop does not fit)
+    PanelRegs t[4];
     if (start < stop) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < 3; ++q) {
             t[q] = panel_load(xb, C, (q >> 1) * 32, last, (q & 1) * 64, lane);
         }
     }
@@ -637,26 +639,32 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
     __syncthreads();
     for (int64_t base = start; base < stop; base += 64) {
         const int rel = (int)(base - start);
+        // the lane index is opaque to the optimiser inside a step, so that panel offsets and store addresses are formed
+        // where they are used instead of being kept (and spilled) across the loop
+        int lv = lane;
+        asm volatile("" : "+v"(lv));
+        const int rv = lv & 31, gv = lv >> 5;
         bf16x8 af[2][CK];
+        t[3] = panel_load(xb, C, rel + 32, last, 64, lv);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            panel_store(panel, lane, t[q]);
+            panel_store(panel, lv, t[q]);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                af[q >> 1][(q & 1) * 4 + k] = as_bf16x8(panel[panel_slot(r, 2 * k + g)]);
+                af[q >> 1][(q & 1) * 4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
             }
         }
         {
             const int nrel = base + 64 < stop ? rel + 64 : rel; // clamped: one harmless re-read at the end
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                t[q] = panel_load(xb, C, nrel + (q >> 1) * 32, last, (q & 1) * 64, lane);
+            for (int q = 0; q < 3; ++q) {
+                t[q] = panel_load(xb, C, nrel + (q >> 1) * 32, last, (q & 1) * 64, lv);
             }
         }
 #pragma unroll 1
         for (int n = 0; n < 4; ++n) { // 32 channels at a time
             // projection first, rounded to bf16 and parked as packed pairs, then the gate: half the accumulators live
-            const float pbias = bp[n * 32 + r], gneg = -LOG2E * bg[n * 32 + r];
+            const float pbias = bp[n * 32 + rv], gneg = -LOG2E * bg[n * 32 + rv];
             bf16x8 pp[2][2];
             {
                 f32x16 pa[2];
@@ -666,7 +674,7 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
                 }
 #pragma unroll
                 for (int ks = 0; ks < CK; ++ks) {
-                    const bf16x8 wpf = as_bf16x8(lds[(n * CK + ks) * 64 + lane]);
+                    const bf16x8 wpf = as_bf16x8(lds[(n * CK + ks) * 64 + lv]);
 #pragma unroll
                     for (int rb = 0; rb < 2; ++rb) {
                         pa[rb] = mfma(af[rb][ks], wpf, pa[rb]);
@@ -688,7 +696,7 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
             }
 #pragma unroll
             for (int ks = 0; ks < CK; ++ks) {
-                const bf16x8 wgf = as_bf16x8(lds[((4 + n) * CK + ks) * 64 + lane]);
+                const bf16x8 wgf = as_bf16x8(lds[((4 + n) * CK + ks) * 64 + lv]);
 #pragma unroll
                 for (int rb = 0; rb < 2; ++rb) {
                     ga[rb] = mfma(af[rb][ks], wgf, ga[rb]);
@@ -698,8 +706,8 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
             for (int rb = 0; rb < 2; ++rb) {
 #pragma unroll
                 for (int a = 0; a < 4; ++a) {
-                    // mask of the lane's four consecutive positions (re-read per channel block: it stays in the L1)
-                    int64_t p0 = base + rb * 32 + 8 * a + 4 * g;
+                    // mask of the lv's four consecutive positions (re-read per channel block: it stays in the L1)
+                    int64_t p0 = base + rb * 32 + 8 * a + 4 * gv;
                     p0 = p0 + 4 <= n_pos ? p0 : n_pos - 4; // positions past the end are never stored
                     const bf16x4 mk = *reinterpret_cast<const bf16x4 *>(mask + p0);
                     bf16x4 ov;
@@ -710,14 +718,14 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
                         const float e = __builtin_amdgcn_exp2f(fmaf(ga[rb][4 * a + c], -LOG2E, gneg));
                         ov[c] = (bf16_t)(pv * __builtin_amdgcn_rcpf(1.0f + e));
                     }
-                    *(reinterpret_cast<bf16x4 *>(panel + panel_slot(r, rb * 4 + a)) + g) = ov;
+                    *(reinterpret_cast<bf16x4 *>(panel + panel_slot(rv, rb * 4 + a)) + gv) = ov;
                 }
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int ch = 8 * i + (lane >> 3);
-                const uint4 v = panel[panel_slot(ch, lane & 7)];
-                const int64_t p0 = base + (lane & 7) * 8;
+                const int ch = 8 * i + (lv >> 3);
+                const uint4 v = panel[panel_slot(ch, lv & 7)];
+                const int64_t p0 = base + (lv & 7) * 8;
                 if (p0 < stop) {
                     *reinterpret_cast<uint4 *>(out + (int64_t)(n * 32 + ch) * out_ld + p0) = v;
                 }
