@@ -977,8 +977,8 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
         return KUTACC_HIP_EUNSUPPORTED;
     }
     // The streaming kernel pays a 64 KB weight load per workgroup and works in steps of 64 positions per wave: it
-    // wins once every wave has several steps (measured: 182 us against 225 us at 1024 x 1024 positions, but 44 us
-    // against 32 us at 384 x 384), so small pair tensors stay on the tiled kernel.
+    // wins once every wave has several steps (measured: 141 us against 225 us at 1024 x 1024 positions, but 36 us
+    // against 31 us at 384 x 384), so small pair tensors stay on the tiled kernel.
     if (g.path != KUTACC_HIP_PATH_GENERIC && gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 &&
         g.n >= GATED_STREAMING_MIN_POSITIONS) {
         kutacc_prof::KernelTimer t("gated_projection_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);

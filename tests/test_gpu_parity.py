@@ -80,6 +80,9 @@ SMALL = [
     (2, 3, 70), (3, 2, 33), (2, 2, 1), (3, 2, 200), (4, 2, 97),
     # ragged lengths with enough batch rows for the fragment-major pair-bias copy to fit the q scratch tensor
     (3, 24, 200), (2, 16, 70), (3, 8, 33), (5, 12, 321),
+    # between the persistent kernel's reach and 1024 keys: two and three query blocks per wave of the long-sequence
+    # kernel, an odd number of key tiles, with and without the fragment-major pair bias (it needs batch rows enough)
+    (5, 3, 512), (5, 20, 450), (5, 2, 650), (4, 2, 768), (4, 3, 400), (3, 16, 736),
 ]
 
 
