@@ -73,8 +73,19 @@ __device__ __forceinline__ PanelRegs load_kmajor(const bf16_t *base, int64_t ld,
     return p;
 }
 
-// M-major operand (element (m, k) at base + k*ld + m): 64 rows m from m0, 32 k from k0.  Lane (kk, mc)
-// takes 8 consecutive m of row k0 + kk + 8i; a load instruction covers 8 k x 128 contiguous bytes.
+// M-major operand (element (m, k) at base + k*ld + m).  Its tile goes to LDS the way it lies in memory, 64 rows k of
+// 128 m (256 bytes), and the MFMA fragments -- 8 consecutive k of one m per lane -- come out of the LDS transposing
+// read of gfx950, ds_read_b64_tr_b16: within 16 lanes, lane i receives element (i & 3) of the 8-byte chunks that lanes
+// 4j + (i >> 2), j = 0..3, point at.  With lane s of the group pointing at row k0 + (s >> 2), m = m0 + 4 (s & 3), lane
+// i ends up with k0..k0+3 of m0 + i: a 4 x 16 block transposed per group and instruction, two instructions per
+// fragment.  The 8-byte chunk index of a row is XOR-ed with 8 (k & 3), which spreads the four rows a group reads over
+// all banks; writes are whole 16-byte pieces of a row.
+//
+// Loading: 64 m from m0, 32 k from k0 per wave.  Lane (kk, mc) takes 8 consecutive m of row k0 + 8i + mm_row(kk); a
+// load instruction covers 8 k x 128 contiguous bytes.  mm_row orders the rows so that the 16 lanes that store together
+// hold rows with different k & 3 (different bank halves after the swizzle).
+__device__ __forceinline__ int mm_row(int kk) { return (kk & 4) | ((kk & 1) << 1) | ((kk >> 1) & 1); }
+
 __device__ __forceinline__ PanelRegs load_mmajor(const bf16_t *base, int64_t ld, int m0, int rows, int k0, int K, int lane)
 {
     int m = m0 + (lane & 7) * 8;
@@ -83,7 +94,7 @@ __device__ __forceinline__ PanelRegs load_mmajor(const bf16_t *base, int64_t ld,
     uint4 *dst[4] = {&p.r0, &p.r1, &p.r2, &p.r3};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int k = k0 + 8 * i + (lane >> 3);
+        const int k = k0 + 8 * i + mm_row(lane >> 3);
         const bool ok = k < K;
         uint4 v = *reinterpret_cast<const uint4 *>(base + (int64_t)(ok ? k : 0) * ld + m);
         if (!ok) {
@@ -94,19 +105,43 @@ __device__ __forceinline__ PanelRegs load_mmajor(const bf16_t *base, int64_t ld,
     return p;
 }
 
-// Transposing store of what load_mmajor fetched: operand tile rows mrow0.., k columns kcol0...
-// Register i of lane (kk, mc) holds 8 consecutive m (8mc..8mc+7) of row k = 8i + kk; after transpose8x8_lanes the
-// lane holds k = 8i..8i+7 of m = 8mc + kk, one 16-byte fragment slot.
-__device__ __forceinline__ void store_mmajor(uint4 *operand, int mrow0, int kcol0, int lane, const PanelRegs &p)
+// what load_mmajor fetched -> operand tile [64 k][128 m], m columns mcol0.., rows krow0..
+__device__ __forceinline__ void store_mmajor(uint4 *operand, int mcol0, int krow0, int lane, const PanelRegs &p)
 {
-    const uint32_t sel = transpose8x8_selector(lane);
-    const int row = mrow0 + (lane & 7) * 8 + (lane >> 3);
-    uint4 *dst = operand + (row >> 5) * 256;
+    const int chunk = (mcol0 >> 2) + 2 * (lane & 7); // 8-byte chunk of the row: 4 m each
     const uint4 regs[4] = {p.r0, p.r1, p.r2, p.r3};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        dst[panel_slot(row & 31, (kcol0 >> 3) + i)] = transpose8x8_lanes(regs[i], sel);
+        const int k = krow0 + 8 * i + mm_row(lane >> 3);
+        operand[k * 16 + ((chunk ^ (8 * (k & 3))) >> 1)] = regs[i];
     }
+}
+
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) char lds_char;
+
+// byte offset, inside an m-major operand tile, of the chunk a lane points ds_read_b64_tr_b16 at for the 32-row block
+// mblk of the tile: row (lane >> 5) * 8 + ((lane & 15) >> 2) of a 16-k step, m = 32 mblk + 16 ((lane >> 4) & 1) + 4 (lane & 3)
+__device__ __forceinline__ int mm_fragment_offset(int mblk, int lane)
+{
+    const int a = (lane & 15) >> 2;
+    const int chunk = 8 * mblk + 4 * ((lane >> 4) & 1) + (lane & 3);
+    return ((lane >> 5) * 8 + a) * 256 + ((chunk ^ (8 * a)) * 8);
+}
+
+// fragment of k-step s (16 k) from an m-major operand tile: k = 16 s + 8 (lane >> 5) + 0..7 of the lane's m
+__device__ __forceinline__ bf16x8 mm_fragment(const lds_char *operand, int lane_off, int s)
+{
+    const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        reinterpret_cast<__attribute__((address_space(3))) v4i16 *>(const_cast<lds_char *>(operand + lane_off + s * 4096)));
+    const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        reinterpret_cast<__attribute__((address_space(3))) v4i16 *>(const_cast<lds_char *>(operand + lane_off + s * 4096 + 1024)));
+    union {
+        v4i16 h[2];
+        bf16x8 b;
+    } u;
+    u.h[0] = lo, u.h[1] = hi;
+    return u.b;
 }
 
 template <bool A_MMAJOR, bool B_MMAJOR, bool GATED>
@@ -181,6 +216,10 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
         }
     }
 
+    // m-major operands: where this lane points the transposing reads for the wave's two row blocks and two column blocks
+    const int mm_a0 = mm_fragment_offset(2 * wm, lane), mm_a1 = mm_fragment_offset(2 * wm + 1, lane);
+    const int mm_b0 = mm_fragment_offset(2 * wn, lane), mm_b1 = mm_fragment_offset(2 * wn + 1, lane);
+
     const int KT = (p.K + KSTEP - 1) / KSTEP;
     PanelRegs ra = fetch_a(0), rb = fetch_b(0);
     for (int kt = 0; kt < KT; ++kt) {
@@ -193,11 +232,21 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
         }
         const uint4 *oa = stage + (2 * wm) * 256;
         const uint4 *ob = stage + OPERAND_SLOTS + (2 * wn) * 256;
+        const lds_char *ta = (const lds_char *)stage, *tb = (const lds_char *)(stage + OPERAND_SLOTS);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const int slot = panel_slot(r, 2 * s + g);
-            const bf16x8 a0 = as_bf16x8(oa[slot]), a1 = as_bf16x8(oa[256 + slot]);
-            const bf16x8 b0 = as_bf16x8(ob[slot]), b1 = as_bf16x8(ob[256 + slot]);
+            bf16x8 a0, a1, b0, b1;
+            if constexpr (A_MMAJOR) {
+                a0 = mm_fragment(ta, mm_a0, s), a1 = mm_fragment(ta, mm_a1, s);
+            } else {
+                a0 = as_bf16x8(oa[slot]), a1 = as_bf16x8(oa[256 + slot]);
+            }
+            if constexpr (B_MMAJOR) {
+                b0 = mm_fragment(tb, mm_b0, s), b1 = mm_fragment(tb, mm_b1, s);
+            } else {
+                b0 = as_bf16x8(ob[slot]), b1 = as_bf16x8(ob[256 + slot]);
+            }
             acc[0][0] = mfma(b0, a0, acc[0][0]);
             acc[0][1] = mfma(b1, a0, acc[0][1]);
             acc[1][0] = mfma(b0, a1, acc[1][0]);
