@@ -1420,26 +1420,16 @@ struct Plan {
     size_t lds_bytes;
 };
 
-int device_attribute(hipDeviceAttribute_t attr, int fallback)
-{
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, attr, dev) != hipSuccess) {
-        (void)hipGetLastError();
-        return fallback;
-    }
-    return v;
-}
-
 int max_lds_bytes()
 {
-    static const int cached = device_attribute(hipDeviceAttributeMaxSharedMemoryPerBlock, 64 * 1024);
-    return cached;
+    static int table[KUTACC_DEVICE_SLOTS] = {};
+    return kutacc_device_attribute(hipDeviceAttributeMaxSharedMemoryPerBlock, 64 * 1024, table);
 }
 
 int num_cus()
 {
-    static const int cached = device_attribute(hipDeviceAttributeMultiprocessorCount, 256);
-    return cached;
+    static int table[KUTACC_DEVICE_SLOTS] = {};
+    return kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, table);
 }
 
 size_t head_kernel_lds(int C, int NB, int GW)
@@ -1514,24 +1504,16 @@ bool make_plan(int64_t S, int C, Plan &pl)
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 template <typename K>
-int opt_in_lds(K kern, size_t bytes, size_t &configured)
+int opt_in_lds(K kern, size_t bytes, size_t *table)
 {
-    if (bytes > configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-        if (e != hipSuccess) {
-            return (int)e;
-        }
-        configured = bytes;
-    }
-    return 0;
+    return (int)kutacc_opt_in_lds(reinterpret_cast<const void *>(kern), bytes, table);
 }
 
 template <int C, int BPW, bool HAS_NB>
 int launch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t stream)
 {
     auto kern = fused_head_kernel<C, BPW, HAS_NB>;
-    static size_t configured = 0; // per instantiation: largest dynamic LDS size opted into so far
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {}; // per instantiation and device: dynamic LDS opted into so far
     if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
         return rc;
     }
@@ -1544,7 +1526,7 @@ template <int C, bool HAS_NB>
 int launch_persistent_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
 {
     auto kern = persistent_head_kernel<C, HAS_NB>;
-    static size_t configured = 0;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
     if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
         return rc;
     }
@@ -1583,7 +1565,7 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
 {
     auto kern = output_projection_kernel<C, EPILOGUE>;
     const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16 + 4 * 4096;
-    static size_t configured = 0;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
         return rc;
     }

@@ -434,15 +434,14 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
     const size_t lds_bytes = (size_t)(256 + 256 + 512 + 512 + 4 * 256) * 16 +
                              (size_t)(2 * p.NT * 32 + 4 * 68 + 3 * GC + 4 * 64 * MERGE_LD) * 4;
     const bool cached = p.NT <= 32;
-    static size_t configured[2] = {0, 0};
-    if (lds_bytes > configured[cached]) {
+    static size_t configured[2][KUTACC_DEVICE_SLOTS] = {};
+    {
         const void *fn = cached ? reinterpret_cast<const void *>(global_attention_kernel<true>)
                                 : reinterpret_cast<const void *>(global_attention_kernel<false>);
-        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        const hipError_t e = kutacc_opt_in_lds(fn, lds_bytes, configured[cached]);
         if (e != hipSuccess) {
             return (int)e;
         }
-        configured[cached] = lds_bytes;
     }
     const double BS = (double)a.batch * (double)a.seq_len;
     kutacc_prof::KernelTimer t("global_attention_kernel", BS * (4.0 * GC * a.head_size + 4.0 * GC * GC + 4.0 * GC), stream);

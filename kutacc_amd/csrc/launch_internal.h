@@ -12,6 +12,56 @@ static inline int kutacc_hip_status(hipError_t e) { return e == hipSuccess ? 0 :
 // 16-byte alignment of a pointer: what the vector loads and stores of the fast kernels need
 static inline bool kutacc_hip_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// One-time kernel set-up and device properties are per device (hipFuncSetAttribute applies to the current device only),
+// and a process may drive several: the launchers keep what they have done in small tables indexed by the device ordinal.
+constexpr int KUTACC_DEVICE_SLOTS = 64;
+
+// ordinal of the current device, or -1 when it cannot be had or does not fit the tables (then nothing is remembered)
+static inline int kutacc_device_slot()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return (dev >= 0 && dev < KUTACC_DEVICE_SLOTS) ? dev : -1;
+}
+
+// Opt a kernel into `bytes` of dynamic LDS on the current device unless the table says it already has that much.
+// `table` is a zero-initialised array of KUTACC_DEVICE_SLOTS entries owned by the caller, one per kernel instantiation.
+static inline hipError_t kutacc_opt_in_lds(const void *kernel, size_t bytes, size_t *table)
+{
+    const int slot = kutacc_device_slot();
+    if (slot < 0 || bytes > table[slot]) {
+        const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) {
+            return e;
+        }
+        if (slot >= 0) {
+            table[slot] = bytes;
+        }
+    }
+    return hipSuccess;
+}
+
+// an integer attribute of the current device, remembered per device in `table` (zero-initialised, values are positive)
+static inline int kutacc_device_attribute(hipDeviceAttribute_t attr, int fallback, int *table)
+{
+    const int slot = kutacc_device_slot();
+    if (slot >= 0 && table[slot] > 0) {
+        return table[slot];
+    }
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, attr, dev) != hipSuccess || v <= 0) {
+        (void)hipGetLastError();
+        return fallback;
+    }
+    if (slot >= 0) {
+        table[slot] = v;
+    }
+    return v;
+}
+
 namespace kutacc_launch {
 
 // generic_kernels.hip

@@ -872,14 +872,9 @@ bool operand_ok(const void *ptr, int64_t s_row, int64_t s_k, int64_t s_batch, in
 template <bool AM, bool BM, bool G>
 hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
 {
-    static bool configured = false; // per instantiation: 64 KB of dynamic LDS needs the opt-in once
-    if (!configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_gemm_kernel<AM, BM, G>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_LDS);
-        if (e != hipSuccess) {
-            return e;
-        }
-        configured = true;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {}; // per instantiation and device: 64 KB of dynamic LDS needs the opt-in
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&pair_gemm_kernel<AM, BM, G>), GEMM_LDS, configured)) {
+        return e;
     }
     pair_gemm_kernel<AM, BM, G><<<dim3((unsigned)blocks), 256, GEMM_LDS, stream>>>(p);
     return hipGetLastError();
@@ -898,28 +893,17 @@ bool gated_projection_fits(const kutacc_hip_gemm_args_t &g)
 hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
 {
     constexpr size_t lds_bytes = (size_t)2 * 4 * 8 * 64 * 16 + 4 * 4096;
-    static bool configured = false;
-    static int cus = 0;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gated_projection_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        int dev = 0;
-        if (e == hipSuccess) {
-            e = hipGetDevice(&dev);
-        }
-        if (e == hipSuccess) {
-            e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        }
-        if (e != hipSuccess) {
-            return e;
-        }
-        configured = true;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    static int cu_table[KUTACC_DEVICE_SLOTS] = {};
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&gated_projection_kernel), lds_bytes, configured)) {
+        return e;
     }
+    const int cus = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
     // two resident workgroups per CU, every wave an equal range of positions (a multiple of 8; the last step of a
     // range may be partial)
     const int64_t tiles = (g.n + 63) / 64;
     int64_t gx = (tiles + 3) / 4;
-    const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * 2;
+    const int64_t cap = (int64_t)cus * 2;
     gx = gx > cap ? cap : gx;
     const int64_t ppw = ((g.n + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
     gated_projection_kernel<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>(
@@ -937,15 +921,10 @@ hipError_t launch_transition(const void *x, const void *w1, const float *b1, con
 {
     constexpr int STAGE_PANELS = 2 * (CO / 64) + CO / 32;
     const size_t lds_bytes = (size_t)(2 * STAGE_PANELS + 4) * 4096 + (size_t)c_i * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB, BLOCK>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 (2 * STAGE_PANELS + 4) * 4096 + MAX_HIDDEN * (int)sizeof(float));
-        if (e != hipSuccess) {
-            return e;
-        }
-        configured = true;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB, BLOCK>),
+                                               (size_t)(2 * STAGE_PANELS + 4) * 4096 + MAX_HIDDEN * sizeof(float), configured)) {
+        return e;
     }
     const int64_t blocks = (rows + 128 * RB - 1) / (128 * RB);
     transition_fused_kernel<CO, RB, BLOCK><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(
