@@ -943,6 +943,33 @@ bool transition_fused_supports(int64_t rows, int64_t c_o, int64_t c_i, const voi
            kutacc_hip_aligned16(b2) && kutacc_hip_aligned16(out);
 }
 
+// 128 channels: a workgroup of the main kernel takes 256 rows (64 per wave) and a CU holds one workgroup, so a grid
+// that is not a whole number of rounds ends with a round in which most CUs idle for a full workgroup's time (n = 384:
+// 576 workgroups on 256 CUs, the third round a quarter full).  The rows of whole rounds go to the main kernel; the rest
+// to the 32-rows-per-wave variant, whose workgroups are half as big and finish in about two thirds of the time.
+template <bool BLOCK>
+static hipError_t launch_transition_128(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
+                                        int64_t rows, int c_i, const float *ln_gamma, const float *ln_beta, float ln_eps,
+                                        hipStream_t stream)
+{
+    static int cu_table[KUTACC_DEVICE_SLOTS] = {};
+    const int64_t cus = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
+    const int64_t groups = (rows + 255) / 256;
+    const int64_t whole = groups / cus * cus; // workgroups in whole rounds
+    const int64_t rest = groups - whole;
+    if (whole == 0 || rest == 0 || rest * 2 > cus) {
+        return launch_transition<128, 2, BLOCK>(x, w1, b1, w2, b2, out, rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
+    }
+    const int64_t main_rows = whole * 256;
+    hipError_t e = launch_transition<128, 2, BLOCK>(x, w1, b1, w2, b2, out, main_rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
+    if (e != hipSuccess) {
+        return e;
+    }
+    const bf16_t *xt = static_cast<const bf16_t *>(x) + main_rows * 128;
+    bf16_t *ot = static_cast<bf16_t *>(out) + main_rows * 128;
+    return launch_transition<128, 1, BLOCK>(xt, w1, b1, w2, b2, ot, rows - main_rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
+}
+
 int transition_fused(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
                      int64_t rows, int64_t c_o, int64_t c_i, hipStream_t stream)
 {
@@ -950,7 +977,7 @@ int transition_fused(const void *x, const void *w1, const float *b1, const void 
         return KUTACC_HIP_EUNSUPPORTED;
     }
     kutacc_prof::KernelTimer t("transition_fused_kernel", 4.0 * (double)rows * (double)c_o * (double)c_i, stream);
-    const hipError_t e = c_o == 128 ? launch_transition<128, 2, false>(x, w1, b1, w2, b2, out, rows, (int)c_i, nullptr, nullptr, 0.f, stream)
+    const hipError_t e = c_o == 128 ? launch_transition_128<false>(x, w1, b1, w2, b2, out, rows, (int)c_i, nullptr, nullptr, 0.f, stream)
                                     : launch_transition<256, 1, false>(x, w1, b1, w2, b2, out, rows, (int)c_i, nullptr, nullptr, 0.f, stream);
     return kutacc_hip_status(e);
 }
@@ -964,7 +991,7 @@ int transition_block_fused(void *act, const float *ln_gamma, const float *ln_bet
     }
     kutacc_prof::KernelTimer t("transition_fused_kernel<block>", 4.0 * (double)rows * (double)c_o * (double)c_i, stream);
     const hipError_t e =
-        c_o == 128 ? launch_transition<128, 2, true>(act, w1, b1, w2, b2, act, rows, (int)c_i, ln_gamma, ln_beta, ln_eps, stream)
+        c_o == 128 ? launch_transition_128<true>(act, w1, b1, w2, b2, act, rows, (int)c_i, ln_gamma, ln_beta, ln_eps, stream)
                    : launch_transition<256, 1, true>(act, w1, b1, w2, b2, act, rows, (int)c_i, ln_gamma, ln_beta, ln_eps, stream);
     return kutacc_hip_status(e);
 }
