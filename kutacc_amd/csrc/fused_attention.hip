@@ -1210,11 +1210,14 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 // transposed back for the ending node.
 constexpr int EPILOGUE_STORE = 0, EPILOGUE_GATED_RESIDUAL = 1, EPILOGUE_RESIDUAL = 2;
 
+// With 256 input features a workgroup has eight waves and keeps two 128-feature slabs of Wo (128 KB, the whole matrix of
+// the attention's output projection), so a row is read once for all 256 output features; with 128 it has four waves,
+// one slab, and two workgroups share a CU.
 template <int C, int EPILOGUE>
-__global__ __launch_bounds__(256, 2) void output_projection_kernel(
+__global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output_projection_kernel(
     const bf16_t *__restrict__ avg, int64_t avg_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
-    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave, const bf16_t *__restrict__ gate, int64_t gate_ld,
-    int64_t swap_n)
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int N, int rows_per_wave, const bf16_t *__restrict__ gate,
+    int64_t gate_ld, int64_t swap_n)
 {
     // row of `out` that receives row `row` of the result
     auto target_row = [&](int64_t row) -> int64_t {
@@ -1225,17 +1228,20 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
     };
     constexpr int CK = C / 16;
     constexpr int NP = CK / 4;
-    extern __shared__ uint4 lds[]; // W slab [4 feature blocks][CK][64 lanes], then 4 panels of 256
+    constexpr int SLABS = C / 128, WAVES = 4 * SLABS, THREADS = 64 * WAVES;
+    extern __shared__ uint4 lds[]; // W slabs [SLABS][4 feature blocks][CK][64 lanes], then one panel of 256 per wave
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
-    const int n0 = blockIdx.y * 128;
-    uint4 *panel = lds + 4 * CK * 64 + wave * 256;
+    const int nbase = blockIdx.y * (128 * SLABS);               // first output feature of this workgroup
+    // slabs it has: with two per workgroup the last workgroup of a row of them may have one
+    const int nslab = (SLABS == 1 || N - nbase >= 128 * SLABS) ? SLABS : (N - nbase) / 128;
+    uint4 *panel = lds + SLABS * 4 * CK * 64 + wave * 256;
     // Every wave owns a contiguous range of rows_per_wave rows (a multiple of 8), walked 32 rows at a
     // time; the last step of a range may be partial.  Equal ranges rather than whole 32-row tiles dealt
     // round robin: the kernel is short, and a wave with one tile more than its neighbours would set its
     // duration.  The first two panels of a step are fetched while the previous step is multiplied and
     // stored; those of the first step while the weight slab is staged.
-    const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
+    const int64_t start = ((int64_t)blockIdx.x * WAVES + wave) * rows_per_wave;
     const int64_t stop = start + rows_per_wave < M ? start + rows_per_wave : M;
     const int last_row = (int)(stop - 1);
     PanelRegs ta, tb;
@@ -1244,19 +1250,20 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
         tb = panel_load(avg, avg_ld, (int)start, last_row, 64, lane);
     }
     {
-        constexpr int PER = 4 * CK * 64 / 256; // weight fragments per thread, all loads issued before the first store
+        constexpr int PER = SLABS * 4 * CK * 64 / THREADS; // weight fragments per thread, all loads issued before the first store
         uint4 wreg[PER];
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int idx = tid + i * 256;
-            const int nb_ = idx / (CK * 64);
+            const int idx = tid + i * THREADS;
+            int nb_ = idx / (CK * 64);
+            nb_ = nb_ < 4 * nslab ? nb_ : 0; // a slab this workgroup does not have: any valid rows, never used
             const int ks = (idx >> 6) % CK;
             const int ln = idx & 63;
-            wreg[i] = *reinterpret_cast<const uint4 *>(wo + (int64_t)(n0 + nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8);
+            wreg[i] = *reinterpret_cast<const uint4 *>(wo + (int64_t)(nbase + nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8);
         }
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            lds[tid + i * 256] = wreg[i];
+            lds[tid + i * THREADS] = wreg[i];
         }
     }
     __syncthreads();
@@ -1270,7 +1277,6 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
             asm volatile("" : "+v"(lv));
         }
         const int rv = lv & 31, gv = lv >> 5;
-        const float *bias = bo + n0 + 4 * gv; // read per use: 16 cached loads per tile instead of 64 live registers
         bf16x8 af[CK];
         panel_store(panel, lv, ta);
 #pragma unroll
@@ -1297,6 +1303,11 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
             ta = panel_load(avg, avg_ld, rnext, last_row, 0, lv);
             tb = panel_load(avg, avg_ld, rnext, last_row, 64, lv);
         }
+#pragma unroll 1
+        for (int slab = 0; slab < nslab; ++slab) {
+        const int n0 = nbase + slab * 128;
+        const uint4 *wslab = lds + slab * 4 * CK * 64;
+        const float *bias = bo + n0 + 4 * gv; // read per use: 16 cached loads per tile instead of 64 live registers
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
             uint4 gq[4], zq[4];
@@ -1318,7 +1329,7 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
             for (int ks = 0; ks < CK; ++ks) {
 #pragma unroll
                 for (int n = 0; n < 2; ++n) {
-                    acc[n] = mfma(as_bf16x8(lds[((2 * half + n) * CK + ks) * 64 + lv]), af[ks], acc[n]);
+                    acc[n] = mfma(as_bf16x8(wslab[((2 * half + n) * CK + ks) * 64 + lv]), af[ks], acc[n]);
                 }
             }
             // accumulators -> panel as bf16 [row][64 features], then whole-line stores
@@ -1365,6 +1376,7 @@ __global__ __launch_bounds__(256, 2) void output_projection_kernel(
                 }
             }
         }
+        } // slabs
     }
 }
 
@@ -1564,21 +1576,23 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
                              int64_t swap_n = 0)
 {
     auto kern = output_projection_kernel<C, EPILOGUE>;
-    const size_t lds_bytes = (size_t)4 * (C / 16) * 64 * 16 + 4 * 4096;
+    constexpr int SLABS = C / 128, WAVES = 4 * SLABS;
+    const size_t lds_bytes = (size_t)SLABS * 4 * (C / 16) * 64 * 16 + WAVES * 4096;
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
         return rc;
     }
     const int64_t tiles = (M + 31) / 32;
-    // two workgroups per CU, each wave with an equal share of the rows (a third resident workgroup, where the registers
-    // allow one, measured slower: the weight slab is staged per workgroup)
-    int64_t gx = (tiles + 3) / 4;
-    const int64_t cap = (int64_t)num_cus() * 2;
+    // two workgroups of four waves per CU, or one of eight: each wave with an equal share of the rows (a third resident
+    // workgroup, where the registers allow one, measured slower: the weight slab is staged per workgroup)
+    int64_t gx = (tiles + WAVES - 1) / WAVES;
+    const int64_t cap = (int64_t)num_cus() * (C == 128 ? 2 : 1);
     gx = gx > cap ? cap : gx;
-    const int64_t rpw = ((M + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
-    kern<<<dim3((unsigned)gx, (unsigned)(N / 128)), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)rpw, (const bf16_t *)gate, gate_ld,
-        swap_n);
+    const int64_t rpw = ((M + gx * WAVES - 1) / (gx * WAVES) + 7) / 8 * 8;
+    const int64_t gy = (N / 128 + SLABS - 1) / SLABS;
+    kern<<<dim3((unsigned)gx, (unsigned)gy), 64 * WAVES, lds_bytes, stream>>>(
+        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)N, (int)rpw, (const bf16_t *)gate,
+        gate_ld, swap_n);
     return kutacc_hip_status(hipGetLastError());
 }
 
