@@ -205,8 +205,11 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
         rc = kutacc_launch::layernorm_channel_first(center_cf, rows, a->ln_center_gamma, a->ln_center_beta, center, ci, ci, rows,
                                                     a->ln_eps, KUTACC_DTYPE_BF16, s);
     }
-    // 5. gate from the normalised input
-    if (rc == 0) {
+    // 5. gate from the normalised input -- unless the last kernel can form it itself (128 channels in and out): then the
+    //    gate tensor is never written
+    const bool gate_inside = kutacc_launch::row_projection_projected_gate_supports(
+        center, ci, a->output_w, a->output_b, act, cz, a->gating_w, a->gating_b, a->pair_act, cz, rows, cz, ci, cz);
+    if (rc == 0 && !gate_inside) {
         kutacc_hip_gemm_args_t g;
         std::memset(&g, 0, sizeof(g));
         g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO, g.batches = 1;
@@ -219,7 +222,10 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
     }
     // 6. output projection of the normalised centre, times sigmoid(gate), added to the pair activation: one kernel
     //    when the shape allows, else projection, gating and residual as three passes
-    if (rc == 0) {
+    if (rc == 0 && gate_inside) {
+        rc = kutacc_launch::row_projection_projected_gate_residual(center, ci, a->output_w, a->output_b, act, cz, a->gating_w,
+                                                                   a->gating_b, a->pair_act, cz, rows, s);
+    } else if (rc == 0) {
         rc = kutacc_launch::row_projection_gated_residual(center, ci, a->output_w, a->output_b, gate, cz, a->pair_act, cz, rows,
                                                           cz, ci, s);
         if (rc == KUTACC_HIP_EUNSUPPORTED) {

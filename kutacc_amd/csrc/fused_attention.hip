@@ -1380,6 +1380,157 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
     }
 }
 
+// out[t][:] += bf16( bf16(x[t] . Wo^T + bo) * sigmoid(bf16(y[t] . Wg^T + bg)) ) for rows of 128 features in and out: the last
+// three steps of the triangle multiplication with the gate projection folded in (reference
+// src/attention/triangle_multiplication.cpp:106-150: gate = Linear(normalised input), out = Linear(normalised centre),
+// out * sigmoid(gate), residual).  The gate tensor never exists in memory: against the separate gate projection this
+// saves its write, its read and a launch.  Same structure as output_projection_kernel: both weight slabs stay in LDS
+// (64 KB), every wave streams an equal range of rows 32 at a time, rows in and out as whole cache lines through its
+// panel, the next step's rows requested while the current one is multiplied.  The gate goes first: its accumulators,
+// rounded to bf16 as the reference stores them, wait as 32 packed registers for the projection of the same rows.
+__global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
+    const bf16_t *__restrict__ x, int64_t x_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
+    const bf16_t *__restrict__ y, int64_t y_ld, const bf16_t *__restrict__ wg, const float *__restrict__ bg,
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave)
+{
+    constexpr int C = 128, CK = C / 16;
+    extern __shared__ uint4 lds[]; // [Wo, Wg][4 feature blocks][CK][64 lanes], then 4 panels of 256
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint4 *panel = lds + 2 * 4 * CK * 64 + wave * 256;
+    const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
+    const int64_t stop = start + rows_per_wave < M ? start + rows_per_wave : M;
+    const int last_row = (int)(stop - 1);
+    // the first 64 features of the next step's rows of y and x are requested a step ahead; the second 64 at the top of
+    // their own step, behind the first (four sets of registers held across a step do not fit)
+    PanelRegs ya, xa;
+    if (start < stop) {
+        ya = panel_load(y, y_ld, (int)start, last_row, 0, lane);
+        xa = panel_load(x, x_ld, (int)start, last_row, 0, lane);
+    }
+    {
+        constexpr int PER = 2 * 4 * CK * 64 / 256;
+        uint4 wreg[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = tid + i * 256;
+            const int mat = idx / (4 * CK * 64), nb_ = (idx / (CK * 64)) % 4, ks = (idx >> 6) % CK, ln = idx & 63;
+            const bf16_t *w = mat ? wg : wo;
+            wreg[i] = *reinterpret_cast<const uint4 *>(w + (int64_t)(nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            lds[tid + i * 256] = wreg[i];
+        }
+    }
+    __syncthreads();
+    const uint4 *wo_s = lds, *wg_s = lds + 4 * CK * 64;
+    for (int64_t rbase = start; rbase < stop; rbase += 32) {
+        const int row0 = (int)rbase;
+        int lv = lane; // opaque: addresses and panel offsets are formed per step, not kept across the loop
+        asm volatile("" : "+v"(lv));
+        const int rv = lv & 31, gv = lv >> 5;
+        const int rnext = rbase + 32 < stop ? row0 + 32 : row0; // clamped: one harmless re-read at the end
+        // ---- gate: 128 features of the 32 rows, rounded to bf16, kept in accumulator order ----
+        bf16x8 gate[4][2];
+        {
+            bf16x8 yf[CK];
+            const PanelRegs yb = panel_load(y, y_ld, row0, last_row, 64, lv);
+            panel_store(panel, lv, ya);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                yf[k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+            }
+            panel_store(panel, lv, yb);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                yf[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+            }
+            ya = panel_load(y, y_ld, rnext, last_row, 0, lv);
+            const float *gbias = bg + 4 * gv;
+#pragma unroll
+            for (int nb_ = 0; nb_ < 4; ++nb_) {
+                f32x16 acc = zero16();
+#pragma unroll
+                for (int ks = 0; ks < CK; ++ks) {
+                    acc = mfma(as_bf16x8(wg_s[(nb_ * CK + ks) * 64 + lv]), yf[ks], acc);
+                }
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(gbias + nb_ * 32 + 8 * a);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        gate[nb_][a >> 1][4 * (a & 1) + c] = (bf16_t)(acc[4 * a + c] + bv[c]);
+                    }
+                }
+            }
+        }
+        // ---- projection of the same rows, gating, residual ----
+        bf16x8 xf[CK];
+        const PanelRegs xb = panel_load(x, x_ld, row0, last_row, 64, lv);
+        panel_store(panel, lv, xa);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            xf[k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+        }
+        panel_store(panel, lv, xb);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            xf[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+        }
+        xa = panel_load(x, x_ld, rnext, last_row, 0, lv);
+        const float *bias = bo + 4 * gv;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) { // 64 output features per panel
+            uint4 zq[4]; // the rows of `out` to add to, requested before the MFMAs
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int64_t row = (int64_t)row0 + 8 * i + (lv >> 3);
+                row = row < stop ? row : stop - 1;
+                zq[i] = *reinterpret_cast<const uint4 *>(out + row * out_ld + half * 64 + (lv & 7) * 8);
+            }
+            f32x16 acc[2];
+            acc[0] = zero16(), acc[1] = zero16();
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+#pragma unroll
+                for (int n = 0; n < 2; ++n) {
+                    acc[n] = mfma(as_bf16x8(wo_s[((2 * half + n) * CK + ks) * 64 + lv]), xf[ks], acc[n]);
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(bias + (2 * half + n) * 32 + 8 * a);
+                    bf16x4 ov;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        // bf16(out) * sigmoid(bf16(gate)), rounded to bf16: the reference's rounding points
+                        const float o = to_f32((bf16_t)(acc[n][4 * a + c] + bv[c]));
+                        const float gt = to_f32(gate[2 * half + n][a >> 1][4 * (a & 1) + c]);
+                        ov[c] = (bf16_t)(o * sigmoid_fast(gt));
+                    }
+                    *(reinterpret_cast<bf16x4 *>(panel + panel_slot(rv, n * 4 + a)) + gv) = ov;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int prow_ = 8 * i + (lv >> 3);
+                const bf16x8 u = as_bf16x8(panel[panel_slot(prow_, lv & 7)]), z = as_bf16x8(zq[i]);
+                bf16x8 res;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    res[e] = (bf16_t)(to_f32(z[e]) + to_f32(u[e]));
+                }
+                const int64_t row = (int64_t)row0 + prow_;
+                if (row < stop) {
+                    *reinterpret_cast<uint4 *>(out + row * out_ld + half * 64 + (lv & 7) * 8) = as_uint4(res);
+                }
+            }
+        }
+    }
+}
+
 // Pair bias [H, S, S] -> fragment-major order: for head h, query block j and key tile t the two B
 // operands of the selector MFMAs, [h][j][t][2][64 lanes] x 16 bytes, so that a wave of the attention
 // kernels fetches the pair bias of a tile with two contiguous 1 KB loads straight into registers.
@@ -1741,6 +1892,41 @@ int row_projection_gated_residual(const void *a, int64_t a_ld, const void *w, co
     kutacc_prof::KernelTimer t("output_projection_kernel<gated residual>", 2.0 * (double)m * (double)n * (double)k, stream);
     return k == 128 ? launch_output_projection<128, EPILOGUE_GATED_RESIDUAL>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld)
                     : launch_output_projection<256, EPILOGUE_GATED_RESIDUAL>(a, a_ld, w, bias, acc, acc_ld, m, n, stream, gate, gate_ld);
+}
+
+// acc[m, 128] += bf16(bf16(a . w^T + bias) * sigmoid(bf16(y . wg^T + bg))), a and y rows of 128 features: the gate
+// projection inside the kernel (no gate tensor)
+bool row_projection_projected_gate_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
+                                            int64_t y_ld, const void *wg, const float *bg, const void *acc, int64_t acc_ld,
+                                            int64_t m, int64_t n, int64_t k, int64_t ky)
+{
+    return k == 128 && ky == 128 && n == 128 && m > 0 && m <= INT32_MAX - 64 && bias && bg && y && wg && a_ld % 8 == 0 &&
+           y_ld % 8 == 0 && acc_ld % 8 == 0 && aligned(a, 16) && aligned(w, 16) && aligned(bias, 16) && aligned(y, 16) &&
+           aligned(wg, 16) && aligned(bg, 16) && aligned(acc, 16);
+}
+
+int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
+                                           int64_t y_ld, const void *wg, const float *bg, void *acc, int64_t acc_ld, int64_t m,
+                                           hipStream_t stream)
+{
+    if (!row_projection_projected_gate_supports(a, a_ld, w, bias, y, y_ld, wg, bg, acc, acc_ld, m, 128, 128, 128)) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    constexpr size_t lds_bytes = (size_t)2 * 4 * 8 * 64 * 16 + 4 * 4096;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    if (const int rc = opt_in_lds(projected_gate_residual_kernel, lds_bytes, configured)) {
+        return rc;
+    }
+    kutacc_prof::KernelTimer t("projected_gate_residual_kernel", 4.0 * (double)m * 128.0 * 128.0, stream);
+    const int64_t tiles = (m + 31) / 32;
+    int64_t gx = (tiles + 3) / 4;
+    const int64_t cap = (int64_t)num_cus() * 2; // two workgroups per CU, each wave with an equal share of the rows
+    gx = gx > cap ? cap : gx;
+    const int64_t rpw = ((m + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
+    projected_gate_residual_kernel<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>(
+        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (const bf16_t *)y, y_ld, (const bf16_t *)wg, bg, (bf16_t *)acc, acc_ld,
+        m, (int)rpw);
+    return kutacc_hip_status(hipGetLastError());
 }
 
 } // namespace kutacc_launch

@@ -92,6 +92,13 @@ int row_projection(const void *a, int64_t a_ld, const void *w, const float *bias
 int row_projection_gated_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *gate,
                                   int64_t gate_ld, void *acc, int64_t acc_ld, int64_t m, int64_t n, int64_t k,
                                   hipStream_t stream);
+// the same with the gate projected inside the kernel from rows y of 128 features (no gate tensor); 128 features in and out
+bool row_projection_projected_gate_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
+                                            int64_t y_ld, const void *wg, const float *bg, const void *acc, int64_t acc_ld,
+                                            int64_t m, int64_t n, int64_t k, int64_t ky);
+int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
+                                           int64_t y_ld, const void *wg, const float *bg, void *acc, int64_t acc_ld, int64_t m,
+                                           hipStream_t stream);
 
 // global_attention.hip
 int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);
