@@ -200,15 +200,18 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
         g.c = center_cf, g.c_stride_m = n;
         rc = kutacc_launch::pair_gemm(g, s);
     }
+    // The last kernel can form the gate itself (128 channels in and out: the gate tensor is then never written), and with
+    // positions in whole 16-byte runs it also reads the centre channel-first and normalises it on the way in
+    const bool gate_inside = kutacc_launch::row_projection_projected_gate_supports(
+        center, ci, a->output_w, a->output_b, act, cz, a->gating_w, a->gating_b, a->pair_act, cz, rows, cz, ci, cz);
+    const bool norm_inside = gate_inside && rows % 8 == 0 && kutacc_hip_aligned16(a->ln_center_gamma) &&
+                             kutacc_hip_aligned16(a->ln_center_beta);
     // 4. center_layer_norm, channel-first in, channel-last out
-    if (rc == 0) {
+    if (rc == 0 && !norm_inside) {
         rc = kutacc_launch::layernorm_channel_first(center_cf, rows, a->ln_center_gamma, a->ln_center_beta, center, ci, ci, rows,
                                                     a->ln_eps, KUTACC_DTYPE_BF16, s);
     }
-    // 5. gate from the normalised input -- unless the last kernel can form it itself (128 channels in and out): then the
-    //    gate tensor is never written
-    const bool gate_inside = kutacc_launch::row_projection_projected_gate_supports(
-        center, ci, a->output_w, a->output_b, act, cz, a->gating_w, a->gating_b, a->pair_act, cz, rows, cz, ci, cz);
+    // 5. gate from the normalised input
     if (rc == 0 && !gate_inside) {
         kutacc_hip_gemm_args_t g;
         std::memset(&g, 0, sizeof(g));
@@ -222,7 +225,11 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
     }
     // 6. output projection of the normalised centre, times sigmoid(gate), added to the pair activation: one kernel
     //    when the shape allows, else projection, gating and residual as three passes
-    if (rc == 0 && gate_inside) {
+    if (rc == 0 && norm_inside) {
+        rc = kutacc_launch::row_projection_projected_gate_residual(center_cf, rows, a->output_w, a->output_b, act, cz,
+                                                                   a->gating_w, a->gating_b, a->pair_act, cz, rows, s,
+                                                                   a->ln_center_gamma, a->ln_center_beta, a->ln_eps);
+    } else if (rc == 0 && gate_inside) {
         rc = kutacc_launch::row_projection_projected_gate_residual(center, ci, a->output_w, a->output_b, act, cz, a->gating_w,
                                                                    a->gating_b, a->pair_act, cz, rows, s);
     } else if (rc == 0) {

@@ -1388,10 +1388,19 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
 // (64 KB), every wave streams an equal range of rows 32 at a time, rows in and out as whole cache lines through its
 // panel, the next step's rows requested while the current one is multiplied.  The gate goes first: its accumulators,
 // rounded to bf16 as the reference stores them, wait as 32 packed registers for the projection of the same rows.
+//
+// X_CHANNEL_FIRST: x is the centre of the triangle multiplication as the equation leaves it, channel-first ([128, M],
+// channel stride x_ld) and not yet normalised.  The kernel then takes the place of the channel-first LayerNorm too: a
+// wave loads 64 channels x 32 positions (64 contiguous bytes per channel), stores them in its panel as they lie, gets
+// its MFMA fragments -- 8 consecutive channels of one position per lane -- with the LDS transposing read, and normalises
+// them in registers (a position's 128 channels sit in two lanes; the arithmetic is that of the LayerNorm kernels,
+// reference src/normalization/layernorm_kernel.h:21-53, the result rounded to bf16 as the tensor it replaces was).
+template <bool X_CHANNEL_FIRST>
 __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
     const bf16_t *__restrict__ x, int64_t x_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
     const bf16_t *__restrict__ y, int64_t y_ld, const bf16_t *__restrict__ wg, const float *__restrict__ bg,
-    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave)
+    bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int rows_per_wave, const float *__restrict__ ln_gamma,
+    const float *__restrict__ ln_beta, float ln_eps)
 {
     constexpr int C = 128, CK = C / 16;
     extern __shared__ uint4 lds[]; // [Wo, Wg][4 feature blocks][CK][64 lanes], then 4 panels of 256
@@ -1402,10 +1411,27 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
     const int last_row = (int)(stop - 1);
     // the first 64 features of the next step's rows of y and x are requested a step ahead; the second 64 at the top of
     // their own step, behind the first (four sets of registers held across a step do not fit)
+    // channel-first x: 64 channels (from c0) x 32 positions (from p0), lane -> channel c0 + 16 i + lane / 4, positions
+    // p0 + 8 (lane & 3) .. +7; a chunk past the end of the tensor repeats the last one (M is a multiple of 8)
+    auto load_cf = [&](int c0, int64_t p0, int ln) {
+        int64_t pos = p0 + 8 * (ln & 3);
+        pos = pos + 8 <= M ? pos : M - 8;
+        PanelRegs t;
+        const bf16_t *src = x + (int64_t)(c0 + (ln >> 2)) * x_ld + pos;
+        t.r0 = *reinterpret_cast<const uint4 *>(src);
+        t.r1 = *reinterpret_cast<const uint4 *>(src + 16 * x_ld);
+        t.r2 = *reinterpret_cast<const uint4 *>(src + 32 * x_ld);
+        t.r3 = *reinterpret_cast<const uint4 *>(src + 48 * x_ld);
+        return t;
+    };
     PanelRegs ya, xa;
     if (start < stop) {
         ya = panel_load(y, y_ld, (int)start, last_row, 0, lane);
-        xa = panel_load(x, x_ld, (int)start, last_row, 0, lane);
+        if constexpr (X_CHANNEL_FIRST) {
+            xa = load_cf(0, start, lane);
+        } else {
+            xa = panel_load(x, x_ld, (int)start, last_row, 0, lane);
+        }
     }
     {
         constexpr int PER = 2 * 4 * CK * 64 / 256;
@@ -1466,18 +1492,68 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
         }
         // ---- projection of the same rows, gating, residual ----
         bf16x8 xf[CK];
-        const PanelRegs xb = panel_load(x, x_ld, row0, last_row, 64, lv);
-        panel_store(panel, lv, xa);
+        if constexpr (X_CHANNEL_FIRST) {
+            const PanelRegs xb = load_cf(64, rbase, lv);
+            // the panel holds [64 channels][32 positions], 64 bytes per channel, lane ln's pieces at slots ln + 64 i
+            const lds_char *tile = (const lds_char *)panel;
+            const int tr_off = ((lv >> 5) * 8 + ((lv & 15) >> 2)) * 64 + (4 * ((lv >> 4) & 1) + (lv & 3)) * 8;
+            panel[lv] = xa.r0, panel[64 + lv] = xa.r1, panel[128 + lv] = xa.r2, panel[192 + lv] = xa.r3;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            xf[k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
-        }
-        panel_store(panel, lv, xb);
+            for (int k = 0; k < 4; ++k) {
+                xf[k] = lds_transposed_fragment(tile + tr_off + k * 1024, tile + tr_off + k * 1024 + 256);
+            }
+            panel[lv] = xb.r0, panel[64 + lv] = xb.r1, panel[128 + lv] = xb.r2, panel[192 + lv] = xb.r3;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            xf[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+            for (int k = 0; k < 4; ++k) {
+                xf[4 + k] = lds_transposed_fragment(tile + tr_off + k * 1024, tile + tr_off + k * 1024 + 256);
+            }
+            xa = load_cf(0, rbase + 32 < stop ? rbase + 32 : rbase, lv);
+            // LayerNorm over the 128 channels of the lane's position: this lane holds channels 16 k + 8 g + 0..7
+            float x0 = to_f32(xf[0][0]);
+            x0 = __shfl(x0, lv & 31, 64); // channel 0 sits in the lane of the lower half
+            float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int k = 0; k < CK; ++k) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float d = to_f32(xf[k][e]) - x0;
+                    s1 += d;
+                    s2 = fmaf(d, d, s2);
+                }
+            }
+            s1 = half_swap_sum(s1), s2 = half_swap_sum(s2);
+            const float nch = (float)C;
+            const float mean = s1 / nch + x0;
+            const float var = fmaxf((s2 - s1 * s1 / nch) / nch, 0.f);
+            const float rstd = 1.0f / sqrtf(var + ln_eps);
+            const float shift = -rstd * mean;
+#pragma unroll
+            for (int k = 0; k < CK; ++k) {
+                const float *gm = ln_gamma + 16 * k + 8 * gv, *bt = ln_beta + 16 * k + 8 * gv;
+                const f32x4 g0 = *reinterpret_cast<const f32x4 *>(gm), g1 = *reinterpret_cast<const f32x4 *>(gm + 4);
+                const f32x4 b0 = *reinterpret_cast<const f32x4 *>(bt), b1 = *reinterpret_cast<const f32x4 *>(bt + 4);
+                bf16x8 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o[e] = (bf16_t)fmaf(fmaf(to_f32(xf[k][e]), rstd, shift), g0[e], b0[e]);
+                    o[4 + e] = (bf16_t)fmaf(fmaf(to_f32(xf[k][4 + e]), rstd, shift), g1[e], b1[e]);
+                }
+                xf[k] = o;
+            }
+        } else {
+            const PanelRegs xb = panel_load(x, x_ld, row0, last_row, 64, lv);
+            panel_store(panel, lv, xa);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                xf[k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+            }
+            panel_store(panel, lv, xb);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                xf[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
+            }
+            xa = panel_load(x, x_ld, rnext, last_row, 0, lv);
         }
-        xa = panel_load(x, x_ld, rnext, last_row, 0, lv);
         const float *bias = bo + 4 * gv;
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
@@ -1905,27 +1981,36 @@ bool row_projection_projected_gate_supports(const void *a, int64_t a_ld, const v
            aligned(wg, 16) && aligned(bg, 16) && aligned(acc, 16);
 }
 
+// ln_gamma != nullptr: `a` is channel-first ([128, m], channel stride a_ld, m a multiple of 8) and not yet normalised;
+// the kernel applies LayerNorm(ln_gamma, ln_beta, ln_eps) over its 128 channels on the way in
 int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
                                            int64_t y_ld, const void *wg, const float *bg, void *acc, int64_t acc_ld, int64_t m,
-                                           hipStream_t stream)
+                                           hipStream_t stream, const float *ln_gamma, const float *ln_beta, float ln_eps)
 {
     if (!row_projection_projected_gate_supports(a, a_ld, w, bias, y, y_ld, wg, bg, acc, acc_ld, m, 128, 128, 128)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
+    const bool cf = ln_gamma != nullptr;
+    if (cf && (!ln_beta || m % 8 != 0 || m < 8 || !aligned(ln_gamma, 16) || !aligned(ln_beta, 16))) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
     constexpr size_t lds_bytes = (size_t)2 * 4 * 8 * 64 * 16 + 4 * 4096;
-    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
-    if (const int rc = opt_in_lds(projected_gate_residual_kernel, lds_bytes, configured)) {
+    static size_t configured[2][KUTACC_DEVICE_SLOTS] = {};
+    if (const int rc = cf ? opt_in_lds(projected_gate_residual_kernel<true>, lds_bytes, configured[1])
+                          : opt_in_lds(projected_gate_residual_kernel<false>, lds_bytes, configured[0])) {
         return rc;
     }
-    kutacc_prof::KernelTimer t("projected_gate_residual_kernel", 4.0 * (double)m * 128.0 * 128.0, stream);
+    kutacc_prof::KernelTimer t(cf ? "projected_gate_residual_kernel<channel-first>" : "projected_gate_residual_kernel",
+                               4.0 * (double)m * 128.0 * 128.0, stream);
     const int64_t tiles = (m + 31) / 32;
     int64_t gx = (tiles + 3) / 4;
     const int64_t cap = (int64_t)num_cus() * 2; // two workgroups per CU, each wave with an equal share of the rows
     gx = gx > cap ? cap : gx;
     const int64_t rpw = ((m + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
-    projected_gate_residual_kernel<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>(
-        (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (const bf16_t *)y, y_ld, (const bf16_t *)wg, bg, (bf16_t *)acc, acc_ld,
-        m, (int)rpw);
+    auto kern = cf ? projected_gate_residual_kernel<true> : projected_gate_residual_kernel<false>;
+    kern<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>((const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (const bf16_t *)y, y_ld,
+                                                         (const bf16_t *)wg, bg, (bf16_t *)acc, acc_ld, m, (int)rpw, ln_gamma,
+                                                         ln_beta, ln_eps);
     return kutacc_hip_status(hipGetLastError());
 }
 

@@ -96,9 +96,11 @@ int row_projection_gated_residual(const void *a, int64_t a_ld, const void *w, co
 bool row_projection_projected_gate_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
                                             int64_t y_ld, const void *wg, const float *bg, const void *acc, int64_t acc_ld,
                                             int64_t m, int64_t n, int64_t k, int64_t ky);
+// ln_gamma != nullptr: `a` is channel-first ([128, m], channel stride a_ld) and is normalised over its channels on the way in
 int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const void *w, const float *bias, const void *y,
                                            int64_t y_ld, const void *wg, const float *bg, void *acc, int64_t acc_ld, int64_t m,
-                                           hipStream_t stream);
+                                           hipStream_t stream, const float *ln_gamma = nullptr, const float *ln_beta = nullptr,
+                                           float ln_eps = 0.f);
 
 // global_attention.hip
 int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);

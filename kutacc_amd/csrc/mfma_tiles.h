@@ -152,6 +152,27 @@ __device__ __forceinline__ uint4 transpose8x8_lanes(uint4 v, uint32_t sel)
     return make_uint4(d[0], d[1], d[2], d[3]);
 }
 
+// LDS transposing read of gfx950 (ds_read_b64_tr_b16).  Within 16 lanes, lane i receives element (i & 3) of the 8-byte
+// chunks that lanes 4j + (i >> 2), j = 0..3, point at.  With lane s of a group pointing at row k0 + (s >> 2), columns
+// m0 + 4 (s & 3) .. +3 of a tile stored [k][m], lane i ends up with k0..k0+3 of column m0 + i: a 4 x 16 block
+// transposed per group and instruction.  Two of them (k0 and k0 + 4) make the 8 consecutive k of an MFMA fragment.
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) char lds_char;
+
+__device__ __forceinline__ bf16x8 lds_transposed_fragment(const lds_char *lo, const lds_char *hi)
+{
+    const v4i16 a =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<__attribute__((address_space(3))) v4i16 *>(const_cast<lds_char *>(lo)));
+    const v4i16 b =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<__attribute__((address_space(3))) v4i16 *>(const_cast<lds_char *>(hi)));
+    union {
+        v4i16 h[2];
+        bf16x8 f;
+    } u;
+    u.h[0] = a, u.h[1] = b;
+    return u.f;
+}
+
 __device__ __forceinline__ float sigmoid_fast(float x)
 {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));

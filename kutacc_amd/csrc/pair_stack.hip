@@ -117,9 +117,6 @@ __device__ __forceinline__ void store_mmajor(uint4 *operand, int mcol0, int krow
     }
 }
 
-typedef short v4i16 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) char lds_char;
-
 // byte offset, inside an m-major operand tile, of the chunk a lane points ds_read_b64_tr_b16 at for the 32-row block
 // mblk of the tile: row (lane >> 5) * 8 + ((lane & 15) >> 2) of a 16-k step, m = 32 mblk + 16 ((lane >> 4) & 1) + 4 (lane & 3)
 __device__ __forceinline__ int mm_fragment_offset(int mblk, int lane)
@@ -132,16 +129,7 @@ __device__ __forceinline__ int mm_fragment_offset(int mblk, int lane)
 // fragment of k-step s (16 k) from an m-major operand tile: k = 16 s + 8 (lane >> 5) + 0..7 of the lane's m
 __device__ __forceinline__ bf16x8 mm_fragment(const lds_char *operand, int lane_off, int s)
 {
-    const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        reinterpret_cast<__attribute__((address_space(3))) v4i16 *>(const_cast<lds_char *>(operand + lane_off + s * 4096)));
-    const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        reinterpret_cast<__attribute__((address_space(3))) v4i16 *>(const_cast<lds_char *>(operand + lane_off + s * 4096 + 1024)));
-    union {
-        v4i16 h[2];
-        bf16x8 b;
-    } u;
-    u.h[0] = lo, u.h[1] = hi;
-    return u.b;
+    return lds_transposed_fragment(operand + lane_off + s * 4096, operand + lane_off + s * 4096 + 1024);
 }
 
 template <bool A_MMAJOR, bool B_MMAJOR, bool GATED>

@@ -240,7 +240,9 @@ def tm_block_oracle(c, incoming):
 
 
 @pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
-@pytest.mark.parametrize("n,c_z,c_i", [(48, 128, 128), (40, 64, 32), (9, 12, 6)])
+# 48: the last kernel takes the centre channel-first, normalises it and projects the gate itself; 46 (positions not in
+# whole 16-byte runs): it still projects the gate, behind the stand-alone channel-first LayerNorm; the others: separate passes
+@pytest.mark.parametrize("n,c_z,c_i", [(48, 128, 128), (46, 128, 128), (40, 64, 32), (9, 12, 6)])
 def test_triangle_multiplication_block_against_the_oracle(torch_cuda, n, c_z, c_i, incoming):
     torch = torch_cuda
     c = tm_block_case(800 + n, n, c_z, c_i)
