@@ -171,19 +171,28 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
     // 1. layer_norm_input
     int rc = kutacc_launch::layernorm_rows(a->pair_act, cz, a->ln_in_gamma, a->ln_in_beta, act, cz, rows, cz, a->ln_eps,
                                            KUTACC_DTYPE_BF16, s);
-    // 2. gated projections, channel-first
-    for (int side = 0; side < 2 && rc == 0; ++side) {
-        kutacc_hip_gemm_args_t g;
-        std::memset(&g, 0, sizeof(g));
-        g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_AUTO, g.batches = 1;
-        g.m = ci, g.n = rows, g.k = cz;
-        g.a = side ? a->right_proj_w : a->left_proj_w, g.a_gate = side ? a->right_gate_w : a->left_gate_w;
-        g.a_stride_m = cz, g.a_stride_k = 1;
-        g.b = act, g.b_stride_n = cz, g.b_stride_k = 1;
-        g.c = side ? right : left, g.c_stride_m = rows;
-        g.bias = side ? a->right_proj_b : a->left_proj_b, g.bias_gate = side ? a->right_gate_b : a->left_gate_b;
-        g.bias_axis = 2, g.mask = a->pair_mask;
-        rc = kutacc_launch::pair_gemm(g, s);
+    // 2. gated projections, channel-first: both sides in one launch where the tiled kernel takes them, else one after
+    //    the other
+    if (rc == 0) {
+        kutacc_hip_gemm_args_t g[2];
+        for (int side = 0; side < 2; ++side) {
+            std::memset(&g[side], 0, sizeof(g[side]));
+            g[side].dtype = KUTACC_DTYPE_BF16, g[side].path = KUTACC_HIP_PATH_AUTO, g[side].batches = 1;
+            g[side].m = ci, g[side].n = rows, g[side].k = cz;
+            g[side].a = side ? a->right_proj_w : a->left_proj_w, g[side].a_gate = side ? a->right_gate_w : a->left_gate_w;
+            g[side].a_stride_m = cz, g[side].a_stride_k = 1;
+            g[side].b = act, g[side].b_stride_n = cz, g[side].b_stride_k = 1;
+            g[side].c = side ? right : left, g[side].c_stride_m = rows;
+            g[side].bias = side ? a->right_proj_b : a->left_proj_b, g[side].bias_gate = side ? a->right_gate_b : a->left_gate_b;
+            g[side].bias_axis = 2, g[side].mask = a->pair_mask;
+        }
+        rc = kutacc_launch::pair_gemm(g[0], s, &g[1]);
+        if (rc == KUTACC_HIP_EUNSUPPORTED) {
+            rc = kutacc_launch::pair_gemm(g[0], s);
+            if (rc == 0) {
+                rc = kutacc_launch::pair_gemm(g[1], s);
+            }
+        }
     }
     // 3. the equation, one n x n product per channel
     if (rc == 0) {

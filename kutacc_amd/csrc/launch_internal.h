@@ -106,7 +106,9 @@ int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const vo
 int global_attention(const kutacc_hip_global_attention_args_t &args, hipStream_t stream);
 
 // pair_stack.hip
-int pair_gemm(const kutacc_hip_gemm_args_t &args, hipStream_t stream);
+// `second`: a second gated projection of the same B and mask to run in the same launch (KUTACC_HIP_EUNSUPPORTED, with
+// nothing launched, when the two cannot share one: the caller then makes two calls)
+int pair_gemm(const kutacc_hip_gemm_args_t &args, hipStream_t stream, const kutacc_hip_gemm_args_t *second = nullptr);
 bool transition_fused_supports(int64_t rows, int64_t c_o, int64_t c_i, const void *x, const void *w1, const float *b1,
                                const void *w2, const float *b2, const void *out);
 int transition_fused(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,

@@ -44,6 +44,11 @@ struct GemmParams {
     int bias_axis; // 0 none, 1 per column n, 2 per row m
     int relu;
     int MT, NT; // tiles along m and n
+    // gated form with two batches that share B and the mask: weights, biases and result of batch 1 (else null).  The two
+    // sides of the triangle multiplication's projections in one launch: the activation tile is fetched from HBM once.
+    const bf16_t *a_alt, *a_gate_alt;
+    const float *bias_alt, *bias_gate_alt;
+    bf16_t *c_alt;
 };
 
 constexpr int TILE = 128, KSTEP = 64;
@@ -150,8 +155,11 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
         }
     }
     const int64_t tiles = (int64_t)p.MT * p.NT;
-    const int batch = (int)(bid / tiles);
-    const int t = (int)(bid % tiles);
+    int batch = (int)(bid / tiles);
+    int t = (int)(bid % tiles);
+    if (GATED && p.a_alt != nullptr) { // two sides of one B: neighbours in the walk, so that they share its tile in the L2
+        batch = (int)(bid & 1), t = (int)(bid >> 1);
+    }
     // the dimension with fewer tiles runs fastest: consecutive workgroups then share the tile of the larger operand
     int mt, nt;
     if (p.MT <= p.NT) {
@@ -162,8 +170,9 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
     constexpr int MROWS = GATED ? 64 : 128; // rows of C per tile
     const int m0 = mt * MROWS, n0 = nt * TILE;
 
-    const bf16_t *a = p.a + (int64_t)batch * p.a_sb;
-    const bf16_t *a_gate = GATED ? p.a_gate + (int64_t)batch * p.a_sb : nullptr;
+    const bool alt = GATED && p.a_alt != nullptr && batch == 1;
+    const bf16_t *a = alt ? p.a_alt : p.a + (int64_t)batch * p.a_sb;
+    const bf16_t *a_gate = GATED ? (alt ? p.a_gate_alt : p.a_gate + (int64_t)batch * p.a_sb) : nullptr;
     const bf16_t *b = p.b + (int64_t)batch * p.b_sb;
 
     auto fetch_a = [&](int k0) -> PanelRegs {
@@ -251,7 +260,7 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
         float row_bias = 0.f;
         if (p.bias_axis == 2) {
             const int gm = GATED ? m0 + 32 * i + r : m0 + trow;
-            const float *bsrc = (GATED && wm == 1) ? p.bias_gate : p.bias;
+            const float *bsrc = (GATED && wm == 1) ? (alt ? p.bias_gate_alt : p.bias_gate) : (alt ? p.bias_alt : p.bias);
             row_bias = gm < p.M ? bsrc[gm] : 0.f;
         }
 #pragma unroll
@@ -278,7 +287,7 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
     }
     __syncthreads();
 
-    bf16_t *c = p.c + (int64_t)batch * p.c_sb;
+    bf16_t *c = alt ? p.c_alt : p.c + (int64_t)batch * p.c_sb;
     if constexpr (GATED) {
         const bf16_t *mask = p.mask + (int64_t)batch * p.mask_sb;
 #pragma unroll
@@ -984,7 +993,7 @@ int transition_block_fused(void *act, const float *ln_gamma, const float *ln_bet
     return kutacc_hip_status(e);
 }
 
-int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
+int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_hip_gemm_args_t *second)
 {
     if (g.m <= 0 || g.n <= 0 || g.k <= 0 || g.batches <= 0 || !g.a || !g.b || !g.c || g.dtype != KUTACC_DTYPE_BF16) {
         return KUTACC_HIP_EINVAL;
@@ -1005,6 +1014,7 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
     p.bias = g.bias, p.bias_gate = g.bias_gate, p.mask = (const bf16_t *)g.mask, p.mask_sb = g.mask_stride_batch;
     p.M = (int)g.m, p.N = (int)g.n, p.K = (int)g.k, p.batches = (int)g.batches;
     p.bias_axis = g.bias_axis, p.relu = g.relu ? 1 : 0;
+    p.a_alt = p.a_gate_alt = nullptr, p.bias_alt = p.bias_gate_alt = nullptr, p.c_alt = nullptr;
 
     bool am = false, bm = false;
     bool mfma_ok = operand_ok(g.a, g.a_stride_m, g.a_stride_k, g.a_stride_batch, g.m, g.k, am) &&
@@ -1022,6 +1032,25 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
     // The streaming kernel pays a 64 KB weight load per workgroup and works in steps of 64 positions per wave: it
     // wins once every wave has several steps (measured: 141 us against 225 us at 1024 x 1024 positions, but 36 us
     // against 31 us at 384 x 384), so small pair tensors stay on the tiled kernel.
+    if (second != nullptr) {
+        // a second gated projection of the same B and mask (other weights, biases and result) rides along as batch 1 of
+        // the tiled kernel, so that the tile of B both need comes from HBM once; any other route: the caller runs the two
+        // separately
+        const kutacc_hip_gemm_args_t &h = *second;
+        const bool same = h.a_gate && h.m == g.m && h.n == g.n && h.k == g.k && h.batches == 1 && g.batches == 1 && h.b == g.b &&
+                          h.mask == g.mask && h.a_stride_m == g.a_stride_m && h.a_stride_k == g.a_stride_k &&
+                          h.b_stride_n == g.b_stride_n && h.b_stride_k == g.b_stride_k && h.c_stride_m == g.c_stride_m &&
+                          h.bias_axis == g.bias_axis && h.relu == g.relu && h.dtype == g.dtype && h.a && h.c &&
+                          (g.bias_axis == 0 || (h.bias && h.bias_gate)) && kutacc_hip_aligned16(h.a) &&
+                          kutacc_hip_aligned16(h.a_gate) && kutacc_hip_aligned16(h.c);
+        const bool streaming = gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 && g.n >= GATED_STREAMING_MIN_POSITIONS;
+        if (!same || !gated || !mfma_ok || streaming || g.path == KUTACC_HIP_PATH_GENERIC) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        p.a_alt = (const bf16_t *)h.a, p.a_gate_alt = (const bf16_t *)h.a_gate, p.bias_alt = h.bias, p.bias_gate_alt = h.bias_gate;
+        p.c_alt = (bf16_t *)h.c;
+        p.batches = 2;
+    }
     if (g.path != KUTACC_HIP_PATH_GENERIC && gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 &&
         g.n >= GATED_STREAMING_MIN_POSITIONS) {
         kutacc_prof::KernelTimer t("gated_projection_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);
@@ -1033,7 +1062,7 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
         kutacc_launch::row_projection_supports(g.a, g.a_stride_m, g.b, g.bias, g.c, g.c_stride_m, g.m, g.n, g.k)) {
         return kutacc_launch::row_projection(g.a, g.a_stride_m, g.b, g.bias, g.c, g.c_stride_m, g.m, g.n, g.k, stream);
     }
-    const double flops = 2.0 * (double)g.m * (double)g.n * (double)g.k * (double)g.batches * (gated ? 2.0 : 1.0);
+    const double flops = 2.0 * (double)g.m * (double)g.n * (double)g.k * (double)p.batches * (gated ? 2.0 : 1.0);
     if (!mfma_ok) {
         const int64_t total = g.m * g.n * g.batches;
         const int64_t blocks = (total + 255) / 256;
@@ -1046,7 +1075,7 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
     }
     p.MT = (int)((g.m + (gated ? 64 : 128) - 1) / (gated ? 64 : 128));
     p.NT = (int)((g.n + 127) / 128);
-    const int64_t blocks = (int64_t)p.MT * p.NT * g.batches;
+    const int64_t blocks = (int64_t)p.MT * p.NT * p.batches;
     if (blocks > INT32_MAX) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
