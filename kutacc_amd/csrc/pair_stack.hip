@@ -643,18 +643,26 @@ __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *
 // rows it fetches as whole cache lines one step ahead, and the products are formed with positions as MFMA rows
 // and channels as columns: a lane then owns one channel and four consecutive positions per accumulator group,
 // which is the order of the channel-first output -- an 8-byte panel write, then 128-byte runs per channel.
-__global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ wp,
-                                                                  const float *__restrict__ bp, const bf16_t *__restrict__ wg,
-                                                                  const float *__restrict__ bg, const bf16_t *__restrict__ mask,
-                                                                  bf16_t *__restrict__ out, int64_t out_ld, int64_t n_pos,
-                                                                  int pos_per_wave)
+// SIDES = 2: the left and the right projection of the triangle multiplication in one pass over the activation (a
+// workgroup of eight waves, all four weight matrices in LDS: 128 KB + eight panels, the whole 160 KB).
+struct GatedSide {
+    const bf16_t *wp, *wg;
+    const float *bp, *bg;
+    bf16_t *out;
+};
+
+template <int SIDES>
+__global__ __launch_bounds__(256 * SIDES, 2 / SIDES) void gated_projection_kernel(const bf16_t *__restrict__ x, GatedSide s0,
+                                                                                 GatedSide s1,
+                                                                                 const bf16_t *__restrict__ mask,
+                                                                                 int64_t out_ld, int64_t n_pos, int pos_per_wave)
 {
-    constexpr int C = 128, CK = C / 16;
-    extern __shared__ uint4 lds[]; // [2 matrices][4 channel blocks][CK][64 lanes], then one panel per wave
+    constexpr int C = 128, CK = C / 16, WAVES = 4 * SIDES, THREADS = 64 * WAVES;
+    extern __shared__ uint4 lds[]; // [SIDES][2 matrices][4 channel blocks][CK][64 lanes], then one panel per wave
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
-    uint4 *panel = lds + 2 * 4 * CK * 64 + wave * 256;
-    const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * pos_per_wave;
+    uint4 *panel = lds + SIDES * 2 * 4 * CK * 64 + wave * 256;
+    const int64_t start = ((int64_t)blockIdx.x * WAVES + wave) * pos_per_wave;
     const int64_t stop = start + pos_per_wave < n_pos ? start + pos_per_wave : n_pos;
     const int last = (int)(stop - start) - 1; // last valid position of the range, relative to start
     const bf16_t *xb = x + start * C;
@@ -668,18 +676,19 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
         }
     }
     {
-        constexpr int PER = 2 * 4 * CK * 64 / 256;
+        constexpr int PER = SIDES * 2 * 4 * CK * 64 / THREADS;
         uint4 wreg[PER];
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int idx = tid + i * 256;
+            const int idx = tid + i * THREADS;
             const int mat = idx / (4 * CK * 64), nb_ = (idx / (CK * 64)) % 4, ks = (idx >> 6) % CK, ln = idx & 63;
-            const bf16_t *w = mat ? wg : wp;
+            const GatedSide &sd = (SIDES == 2 && mat >= 2) ? s1 : s0;
+            const bf16_t *w = (mat & 1) ? sd.wg : sd.wp;
             wreg[i] = *reinterpret_cast<const uint4 *>(w + (int64_t)(nb_ * 32 + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8);
         }
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            lds[tid + i * 256] = wreg[i];
+            lds[tid + i * THREADS] = wreg[i];
         }
     }
     __syncthreads();
@@ -708,9 +717,13 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
             }
         }
 #pragma unroll 1
-        for (int n = 0; n < 4; ++n) { // 32 channels at a time
+        for (int sn = 0; sn < 4 * SIDES; ++sn) { // 32 channels of one side at a time
+            const int n = sn & 3;
+            const GatedSide &sd = (SIDES == 2 && sn >= 4) ? s1 : s0;
+            const uint4 *wside = lds + (sn >> 2) * 2 * 4 * CK * 64;
+            bf16_t *out = sd.out;
             // projection first, rounded to bf16 and parked as packed pairs, then the gate: half the accumulators live
-            const float pbias = bp[n * 32 + rv], gneg = -LOG2E * bg[n * 32 + rv];
+            const float pbias = sd.bp[n * 32 + rv], gneg = -LOG2E * sd.bg[n * 32 + rv];
             bf16x8 pp[2][2];
             {
                 f32x16 pa[2];
@@ -720,7 +733,7 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
                 }
 #pragma unroll
                 for (int ks = 0; ks < CK; ++ks) {
-                    const bf16x8 wpf = as_bf16x8(lds[(n * CK + ks) * 64 + lv]);
+                    const bf16x8 wpf = as_bf16x8(wside[(n * CK + ks) * 64 + lv]);
 #pragma unroll
                     for (int rb = 0; rb < 2; ++rb) {
                         pa[rb] = mfma(af[rb][ks], wpf, pa[rb]);
@@ -742,7 +755,7 @@ __global__ __launch_bounds__(256, 2) void gated_projection_kernel(const bf16_t *
             }
 #pragma unroll
             for (int ks = 0; ks < CK; ++ks) {
-                const bf16x8 wgf = as_bf16x8(lds[((4 + n) * CK + ks) * 64 + lv]);
+                const bf16x8 wgf = as_bf16x8(wside[((4 + n) * CK + ks) * 64 + lv]);
 #pragma unroll
                 for (int rb = 0; rb < 2; ++rb) {
                     ga[rb] = mfma(af[rb][ks], wgf, ga[rb]);
@@ -887,25 +900,31 @@ bool gated_projection_fits(const kutacc_hip_gemm_args_t &g)
            (reinterpret_cast<uintptr_t>(g.mask) & 7u) == 0 && !g.relu;
 }
 
-hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, hipStream_t stream)
+template <int SIDES>
+hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, const kutacc_hip_gemm_args_t *second, hipStream_t stream)
 {
-    constexpr size_t lds_bytes = (size_t)2 * 4 * 8 * 64 * 16 + 4 * 4096;
+    constexpr int WAVES = 4 * SIDES;
+    constexpr size_t lds_bytes = (size_t)SIDES * 2 * 4 * 8 * 64 * 16 + WAVES * 4096;
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
     static int cu_table[KUTACC_DEVICE_SLOTS] = {};
-    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&gated_projection_kernel), lds_bytes, configured)) {
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&gated_projection_kernel<SIDES>), lds_bytes, configured)) {
         return e;
     }
     const int cus = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
-    // two resident workgroups per CU, every wave an equal range of positions (a multiple of 8; the last step of a
-    // range may be partial)
+    // eight resident waves per CU (two workgroups of four, or one of eight), every wave an equal range of positions (a
+    // multiple of 8; the last step of a range may be partial)
     const int64_t tiles = (g.n + 63) / 64;
-    int64_t gx = (tiles + 3) / 4;
-    const int64_t cap = (int64_t)cus * 2;
+    int64_t gx = (tiles + WAVES - 1) / WAVES;
+    const int64_t cap = (int64_t)cus * (2 / SIDES);
     gx = gx > cap ? cap : gx;
-    const int64_t ppw = ((g.n + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
-    gated_projection_kernel<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>(
-        (const bf16_t *)g.b, (const bf16_t *)g.a, g.bias, (const bf16_t *)g.a_gate, g.bias_gate, (const bf16_t *)g.mask,
-        (bf16_t *)g.c, g.c_stride_m, g.n, (int)ppw);
+    const int64_t ppw = ((g.n + gx * WAVES - 1) / (gx * WAVES) + 7) / 8 * 8;
+    const GatedSide s0 = {(const bf16_t *)g.a, (const bf16_t *)g.a_gate, g.bias, g.bias_gate, (bf16_t *)g.c};
+    GatedSide s1 = s0;
+    if (SIDES == 2) {
+        s1 = GatedSide{(const bf16_t *)second->a, (const bf16_t *)second->a_gate, second->bias, second->bias_gate, (bf16_t *)second->c};
+    }
+    gated_projection_kernel<SIDES><<<dim3((unsigned)gx), 64 * WAVES, lds_bytes, stream>>>(
+        (const bf16_t *)g.b, s0, s1, (const bf16_t *)g.mask, g.c_stride_m, g.n, (int)ppw);
     return hipGetLastError();
 }
 
@@ -1043,8 +1062,16 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
                           h.bias_axis == g.bias_axis && h.relu == g.relu && h.dtype == g.dtype && h.a && h.c &&
                           (g.bias_axis == 0 || (h.bias && h.bias_gate)) && kutacc_hip_aligned16(h.a) &&
                           kutacc_hip_aligned16(h.a_gate) && kutacc_hip_aligned16(h.c);
-        const bool streaming = gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 && g.n >= GATED_STREAMING_MIN_POSITIONS;
-        if (!same || !gated || !mfma_ok || streaming || g.path == KUTACC_HIP_PATH_GENERIC) {
+        const bool streaming = gated && gated_projection_fits(g) && gated_projection_fits(h) && g.n <= INT32_MAX / 2 &&
+                               g.n >= GATED_STREAMING_MIN_POSITIONS;
+        if (!same || !gated || g.path == KUTACC_HIP_PATH_GENERIC) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        if (streaming) { // large pair tensors: both sides in one pass of the streaming kernel over the activation
+            kutacc_prof::KernelTimer t("gated_projection_kernel<2>", 8.0 * (double)g.m * (double)g.n * (double)g.k, stream);
+            return kutacc_hip_status(launch_gated_projection<2>(g, second, stream));
+        }
+        if (!mfma_ok || (gated_projection_fits(g) && g.n >= GATED_STREAMING_MIN_POSITIONS)) {
             return KUTACC_HIP_EUNSUPPORTED;
         }
         p.a_alt = (const bf16_t *)h.a, p.a_gate_alt = (const bf16_t *)h.a_gate, p.bias_alt = h.bias, p.bias_gate_alt = h.bias_gate;
@@ -1054,7 +1081,7 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
     if (g.path != KUTACC_HIP_PATH_GENERIC && gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 &&
         g.n >= GATED_STREAMING_MIN_POSITIONS) {
         kutacc_prof::KernelTimer t("gated_projection_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);
-        return kutacc_hip_status(launch_gated_projection(g, stream));
+        return kutacc_hip_status(launch_gated_projection<1>(g, nullptr, stream));
     }
     // rows of 128 or 256 features against a dense weight matrix: the attention's output-projection kernel keeps
     // the weight slab in LDS and streams the rows, which suits these HBM-bound shapes better than square tiles

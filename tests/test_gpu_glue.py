@@ -258,14 +258,16 @@ def test_triangle_multiplication_block_against_the_oracle(torch_cuda, n, c_z, c_
 
 
 @pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
-def test_triangle_multiplication_block_full_size(torch_cuda, incoming):
-    """384 residues, 128 channels, the real shape.  The oracle follows a sample of output positions (i, j) through the
+@pytest.mark.parametrize("n", [384, 512])
+def test_triangle_multiplication_block_full_size(torch_cuda, incoming, n):
+    """384 residues, 128 channels, the real shape, and 512, from where on the gated projections run on the streaming
+    kernel (both sides in one pass).  The oracle follows a sample of output positions (i, j) through the
     whole block: their centre needs the left projections of row i and the right projections of row j (columns for the
     incoming form), which the oracle computes for just those rows."""
     from oracle import oracle
     torch = torch_cuda
-    n, c = 384, 128
-    case = tm_block_case(900, n, c, c)
+    c = 128
+    case = tm_block_case(900 + n, n, c, c)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
         device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
     w = {k: dev(v) for k, v in case.items() if k not in ("z", "mask")}
@@ -273,7 +275,7 @@ def test_triangle_multiplication_block_full_size(torch_cuda, incoming):
     assert capi.TriangleMultiplicationBlock(pair, dev(case["mask"]), w, incoming).run() == 0
     torch.cuda.synchronize()
     got = helpers.to_numpy(pair)
-    I, J = [0, 77, 200, 383], [5, 100, 383]
+    I, J = [0, 77, 200, n - 1], [5, 100, n - 1]
     act = oracle.layernorm_rows_f32(case["z"].reshape(-1, c), case["ln_in_gamma"], case["ln_in_beta"], 1e-5).reshape(n, n, c)
     proj = lambda side, x, m: oracle.tm_calc_proj_f32(x, m, case[side + "_proj_w"], case[side + "_proj_b"],  # noqa: E731
                                                        case[side + "_gate_w"], case[side + "_gate_b"])
@@ -288,7 +290,7 @@ def test_triangle_multiplication_block_full_size(torch_cuda, incoming):
     act_ij = act[np.ix_(I, J)].reshape(-1, c)
     gate, out = oracle.tm_gate_and_out_f32(act_ij, center, case["gating_w"], case["gating_b"], case["output_w"], case["output_b"])
     want = case["z"][np.ix_(I, J)].reshape(-1, c) + oracle.tm_last_f32(out, gate)
-    helpers.check_close(got[np.ix_(I, J)].reshape(-1, c), want, "bf16", f"TM block 384 incoming={incoming}")
+    helpers.check_close(got[np.ix_(I, J)].reshape(-1, c), want, "bf16", f"TM block {n} incoming={incoming}")
     assert not np.array_equal(got, case["z"])
 
 
