@@ -197,8 +197,7 @@ kutacc_export int kutacc_hip_gemm(const kutacc_hip_gemm_args_t *args, void *stre
  * Transition: out = relu(x . w1^T + b1) . w2^T + b2 over `rows` dense rows (x, out [rows, c_o]; w1 [c_i, c_o] and
  * w2 [c_o, c_i] stored [out, in]; b1 fp32 [c_i], b2 fp32 [c_o]).  Replaces kutacc::transition_kernel (reference
  * src/attention/transition.cpp:21-39).  path AUTO: one kernel that keeps the hidden layer on chip when c_o is 128
- * or 256 and c_i a multiple of 64 (`intermediate` is then not touched and may be NULL; at 128 channels the rows of a
- * last, partial round of workgroups go to a second launch of the same kernel with smaller workgroups), else two kutacc_hip_gemm
+ * or 256 and c_i a multiple of 64 (`intermediate` is then not touched and may be NULL), else two kutacc_hip_gemm
  * launches through `intermediate` ([rows, c_i], required); GENERIC: always the two launches; FUSED: the one kernel
  * or KUTACC_HIP_EUNSUPPORTED.
  */

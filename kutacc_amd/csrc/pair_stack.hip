@@ -341,8 +341,8 @@ __device__ __forceinline__ int sigma_row(int r) { return (r & 0x13) | ((r & 4) <
 // lanes that loaded them: sums by DPP adds, arithmetic of reference src/normalization/layernorm_kernel.h:21-53), and
 // the epilogue re-reads the rows in the order it writes them and adds.  One read and one write of the activation
 // for LayerNorm, both linears and the residual.
-template <int CO, int RB, bool BLOCK>
-__global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *__restrict__ x,
+template <int CO, int RB, bool BLOCK, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES, 1) void transition_fused_kernel(const bf16_t *__restrict__ x,
                                                                  const bf16_t *__restrict__ w1,
                                                                  const float *__restrict__ b1,
                                                                  const bf16_t *__restrict__ w2,
@@ -353,17 +353,18 @@ __global__ __launch_bounds__(256, 1) void transition_fused_kernel(const bf16_t *
     constexpr int KS = CO / 16; // k-steps of the first product
     constexpr int CP = CO / 64; // 64-column panels across a row of x or W1
     constexpr int CB = CO / 32; // 32-channel blocks of the output
-    constexpr int W1_PANELS = 2 * CP, STAGE_PANELS = W1_PANELS + CB, PPW = STAGE_PANELS / 4;
+    constexpr int W1_PANELS = 2 * CP, STAGE_PANELS = W1_PANELS + CB, PPW = STAGE_PANELS / WAVES;
+    static_assert(STAGE_PANELS % WAVES == 0, "every wave stages the same number of weight panels");
     extern __shared__ uint4 lds[]; // [2 stages][STAGE_PANELS][256 slots], one private panel per wave, b1 as fp32
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5, sr = sigma_row(r);
     uint4 *xpanel = lds + 2 * STAGE_PANELS * 256 + wave * 256;
-    float *b1s = reinterpret_cast<float *>(lds + 2 * STAGE_PANELS * 256 + 4 * 256);
-    for (int i = tid; i < c_i; i += 256) {
+    float *b1s = reinterpret_cast<float *>(lds + 2 * STAGE_PANELS * 256 + WAVES * 256);
+    for (int i = tid; i < c_i; i += 64 * WAVES) {
         b1s[i] = b1[i]; // visible after the first barrier of the slice loop
     }
 
-    int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (32 * RB);
+    int64_t row0 = ((int64_t)blockIdx.x * WAVES + wave) * (32 * RB);
     const bool active = row0 < rows;
     if (!active) {
         row0 = rows - 1; // keeps every address valid; nothing is stored
@@ -930,20 +931,21 @@ hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, const kutacc
 
 constexpr int MAX_HIDDEN = 2048; // hidden units whose bias fits next to the weight stages in LDS
 
-template <int CO, int RB, bool BLOCK>
+template <int CO, int RB, bool BLOCK, int WAVES = 4>
 hipError_t launch_transition(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
                              int64_t rows, int c_i, const float *ln_gamma, const float *ln_beta, float ln_eps,
                              hipStream_t stream)
 {
     constexpr int STAGE_PANELS = 2 * (CO / 64) + CO / 32;
-    const size_t lds_bytes = (size_t)(2 * STAGE_PANELS + 4) * 4096 + (size_t)c_i * sizeof(float);
+    const size_t lds_bytes = (size_t)(2 * STAGE_PANELS + WAVES) * 4096 + (size_t)c_i * sizeof(float);
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
-    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB, BLOCK>),
-                                               (size_t)(2 * STAGE_PANELS + 4) * 4096 + MAX_HIDDEN * sizeof(float), configured)) {
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&transition_fused_kernel<CO, RB, BLOCK, WAVES>),
+                                               (size_t)(2 * STAGE_PANELS + WAVES) * 4096 + MAX_HIDDEN * sizeof(float), configured)) {
         return e;
     }
-    const int64_t blocks = (rows + 128 * RB - 1) / (128 * RB);
-    transition_fused_kernel<CO, RB, BLOCK><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(
+    const int64_t per_group = 32 * RB * WAVES;
+    const int64_t blocks = (rows + per_group - 1) / per_group;
+    transition_fused_kernel<CO, RB, BLOCK, WAVES><<<dim3((unsigned)blocks), 64 * WAVES, lds_bytes, stream>>>(
         (const bf16_t *)x, (const bf16_t *)w1, b1, (const bf16_t *)w2, b2, (bf16_t *)out, rows, c_i, ln_gamma, ln_beta, ln_eps);
     return hipGetLastError();
 }
@@ -959,31 +961,17 @@ bool transition_fused_supports(int64_t rows, int64_t c_o, int64_t c_i, const voi
            kutacc_hip_aligned16(b2) && kutacc_hip_aligned16(out);
 }
 
-// 128 channels: a workgroup of the main kernel takes 256 rows (64 per wave) and a CU holds one workgroup, so a grid
-// that is not a whole number of rounds ends with a round in which most CUs idle for a full workgroup's time (n = 384:
-// 576 workgroups on 256 CUs, the third round a quarter full).  The rows of whole rounds go to the main kernel; the rest
-// to the 32-rows-per-wave variant, whose workgroups are half as big and finish in about two thirds of the time.
+// 128 channels: eight waves of 32 rows each per workgroup (one workgroup per CU, two waves per SIMD, which hide each
+// other's LDS round trips and barriers).  Measured against four waves of 64 rows, which reads every weight fragment from
+// LDS half as often but leaves a SIMD to one wave: 12 % faster for the transition at n = 384, 14 % for the block with
+// its LayerNorm and residual, 5 % and 17 % at n = 1024.  (With the four-wave kernel a separate, smaller-workgroup launch
+// for the rows of a last, partial round of workgroups paid off; with this one it no longer does.)
 template <bool BLOCK>
 static hipError_t launch_transition_128(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,
                                         int64_t rows, int c_i, const float *ln_gamma, const float *ln_beta, float ln_eps,
                                         hipStream_t stream)
 {
-    static int cu_table[KUTACC_DEVICE_SLOTS] = {};
-    const int64_t cus = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
-    const int64_t groups = (rows + 255) / 256;
-    const int64_t whole = groups / cus * cus; // workgroups in whole rounds
-    const int64_t rest = groups - whole;
-    if (whole == 0 || rest == 0 || rest * 2 > cus) {
-        return launch_transition<128, 2, BLOCK>(x, w1, b1, w2, b2, out, rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
-    }
-    const int64_t main_rows = whole * 256;
-    hipError_t e = launch_transition<128, 2, BLOCK>(x, w1, b1, w2, b2, out, main_rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
-    if (e != hipSuccess) {
-        return e;
-    }
-    const bf16_t *xt = static_cast<const bf16_t *>(x) + main_rows * 128;
-    bf16_t *ot = static_cast<bf16_t *>(out) + main_rows * 128;
-    return launch_transition<128, 1, BLOCK>(xt, w1, b1, w2, b2, ot, rows - main_rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
+    return launch_transition<128, 1, BLOCK, 8>(x, w1, b1, w2, b2, out, rows, c_i, ln_gamma, ln_beta, ln_eps, stream);
 }
 
 int transition_fused(const void *x, const void *w1, const float *b1, const void *w2, const float *b2, void *out,

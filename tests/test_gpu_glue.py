@@ -319,8 +319,7 @@ def test_gated_residual_projection(torch_cuda, m, n, k):
     assert rc == capi.EUNSUPPORTED
 
 
-# 65536 + 20000 rows: more than one round of workgroups plus a partial one, which the launcher hands to the kernel variant
-# with smaller workgroups (the rows of both parts must come out alike)
+# 65536 + 20000 rows: more than one round of workgroups plus a partial one
 @pytest.mark.parametrize("rows,c_o,c_i", [(300, 128, 512), (200, 256, 1024), (64 * 64, 128, 512), (50, 24, 40),
                                           (65536 + 20000, 128, 256)])
 def test_transition_block(torch_cuda, rows, c_o, c_i):
