@@ -103,6 +103,43 @@ def test_reduced_shapes_both_kernel_families(torch_cuda, config, batch, seq, pat
     helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
 
 
+def _sweep_cases():
+    """24 seeded shapes over the whole range the MFMA kernels take: any sequence length up to 1024 (ragged tails, odd
+    numbers of key tiles, every blocks-per-wave variant of the long-sequence kernel), both channel counts, with and without
+    pair bias, batches small and large enough for the fragment-major pair bias, masks with random holes, masked tails
+    and fully masked rows."""
+    rng = np.random.Generator(np.random.PCG64(20240))
+    cases = []
+    for i in range(24):
+        config = int(rng.choice([2, 3, 4, 5]))
+        seq = int(rng.integers(1, 1025)) if i % 3 else int(rng.choice([31, 32, 33, 383, 385, 511, 513, 767, 1023]))
+        batch = int(rng.integers(1, 5)) if i % 2 else int(rng.integers(8, 20))
+        cases.append((i, config, batch, seq))
+    return cases
+
+
+@pytest.mark.parametrize("index,config,batch,seq", _sweep_cases())
+def test_seeded_shape_sweep_matches_oracle(torch_cuda, index, config, batch, seq):
+    w = make_workload(config, batch=batch, seq_len=seq)
+    rng = np.random.Generator(np.random.PCG64(500 + index))
+    kind = index % 4
+    if kind == 1:    # random holes
+        w.bias[:] = round_to_bf16(np.where(rng.random((batch, seq)) < 0.2, -1e9, 0.0).astype(np.float32))
+    elif kind == 2:  # masked tails of random length, one fully masked row
+        for b in range(batch):
+            w.bias[b, seq - int(rng.integers(0, seq)):] = -1e9
+        w.bias[batch - 1, :] = -1e9
+    elif kind == 3:  # no mask at all
+        w.bias[:] = 0.0
+    print(f"sweep {index}: config {config} B={batch} S={seq} mask kind {kind}", flush=True)
+    ten, scratch = helpers.to_device(w)
+    rc = helpers.run_hip(w, ten, scratch, capi.PATH_FUSED)
+    assert rc == 0, rc
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, f"sweep {index} gated average")
+    helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, f"sweep {index} out")
+
+
 def test_fp32_storage_meets_fp32_tolerance(torch_cuda):
     w = make_workload(1)
     op, ten, scratch = helpers.make_op(w)
