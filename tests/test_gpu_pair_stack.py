@@ -120,6 +120,31 @@ def test_gemm_m_major_operands(torch_cuda, shape, a_mmajor, b_mmajor):
     helpers.assert_within(got, same, 1e-3 + 8e-3 * np.abs(same), "mfma vs scalar kernel")
 
 
+def _gemm_sweep():
+    rng = np.random.Generator(np.random.PCG64(777))
+    cases = []
+    for i in range(20):
+        nb = int(rng.integers(1, 4))
+        M, N, K = (int(8 * rng.integers(1, 60)) for _ in range(3))
+        am, bm = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        bias_axis, relu = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        cases.append((i, nb, M, N, K, am, bm, bias_axis, relu))
+    return cases
+
+
+@pytest.mark.parametrize("index,nb,M,N,K,am,bm,bias_axis,relu", _gemm_sweep())
+def test_gemm_seeded_sweep(torch_cuda, index, nb, M, N, K, am, bm, bias_axis, relu):
+    """20 seeded combinations of sizes (multiples of 8 up to 472), batches, operand orders and epilogues on the MFMA
+    kernel, against float64."""
+    rng = np.random.Generator(np.random.PCG64(900 + index))
+    A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
+    bias = rng.standard_normal(N if bias_axis == 1 else M).astype(np.float32) if bias_axis else None
+    got = run_gemm(torch_cuda, A, B, a_mmajor=am, b_mmajor=bm, bias=bias, bias_axis=bias_axis, relu=relu,
+                   path=capi.PATH_FUSED, c_pad=8)
+    ref = gemm_ref(A, B, bias, bias_axis, relu)
+    helpers.assert_within(got, ref, GEMM_TOL(ref), f"gemm sweep {index}: {nb}x{M}x{N}x{K} am={am} bm={bm}")
+
+
 def test_gemm_rejects_what_it_cannot_run(torch_cuda):
     torch = torch_cuda
     t = torch.zeros(64 * 64, dtype=torch.bfloat16, device="cuda")
