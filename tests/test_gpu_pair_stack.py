@@ -206,6 +206,23 @@ def test_transition_small(torch_cuda, shape, path):
     helpers.check_close(helpers.to_numpy(out).reshape(ref.shape), ref, "bf16", f"transition {shape}")
 
 
+def _transition_sweep():
+    rng = np.random.Generator(np.random.PCG64(4242))
+    return [(i, int(rng.integers(1, 4)), int(rng.integers(1, 900)), int(rng.choice([128, 256])), int(64 * rng.integers(1, 17)))
+            for i in range(12)]
+
+
+@pytest.mark.parametrize("index,batch,n_res,c_o,c_i", _transition_sweep())
+def test_transition_seeded_sweep(torch_cuda, index, batch, n_res, c_o, c_i):
+    """12 seeded row counts (1 to 2700) and hidden widths (64 to 1024) of the one-kernel transition against the oracle."""
+    from oracle import oracle
+    c = transition_case(1300 + index, batch, n_res, c_o, c_i)
+    out, mid = run_transition(torch_cuda, c)
+    assert bool((mid == -5.0).all())
+    ref = oracle.transition_f32(c["x"].reshape(-1, c_o), c["w1"], c["b1"], c["w2"], c["b2"])
+    helpers.check_close(helpers.to_numpy(out).reshape(ref.shape), ref, "bf16", f"transition sweep {index}: {batch}x{n_res}x{c_o}->{c_i}")
+
+
 def test_transition_forced_paths(torch_cuda):
     c = transition_case(305, 1, 70, 128, 256)
     a, _ = run_transition(torch_cuda, c, capi.PATH_FUSED)
