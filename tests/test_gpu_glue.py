@@ -257,6 +257,22 @@ def test_triangle_multiplication_block_against_the_oracle(torch_cuda, n, c_z, c_
     helpers.check_close(helpers.to_numpy(pair), tm_block_oracle(c, incoming), "bf16", f"TM block n={n} incoming={incoming}")
 
 
+@pytest.mark.parametrize("index,n", [(i, int(n)) for i, n in enumerate(np.random.Generator(np.random.PCG64(31)).integers(8, 90, size=8))])
+def test_triangle_multiplication_block_seeded_sweep(torch_cuda, index, n):
+    """Eight seeded pair sizes between 8 and 89 at 128 channels (positions in and out of whole 16-byte runs, so both forms of
+    the block's last kernel and the stand-alone centre LayerNorm), orientation alternating, against the oracle."""
+    torch = torch_cuda
+    incoming = bool(index & 1)
+    c = tm_block_case(2000 + index, n, 128, 128)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    pair = dev(c["z"])
+    w = {k: dev(v) for k, v in c.items() if k not in ("z", "mask")}
+    assert capi.TriangleMultiplicationBlock(pair, dev(c["mask"]), w, incoming).run() == 0
+    torch.cuda.synchronize()
+    helpers.check_close(helpers.to_numpy(pair), tm_block_oracle(c, incoming), "bf16", f"TM block sweep {index}: n={n} incoming={incoming}")
+
+
 @pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
 @pytest.mark.parametrize("n", [384, 512])
 def test_triangle_multiplication_block_full_size(torch_cuda, incoming, n):
