@@ -153,6 +153,15 @@ def test_triangle_attention_block_against_the_oracle(torch_cuda, n, heads, endin
     helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block n={n} ending={ending}")
 
 
+@pytest.mark.parametrize("index,n", [(i, int(n)) for i, n in enumerate(np.random.Generator(np.random.PCG64(57)).integers(8, 200, size=8))])
+def test_triangle_attention_block_seeded_sweep(torch_cuda, index, n):
+    """Eight seeded pair sizes between 8 and 199 (ragged key tiles, odd tile counts), four heads, node alternating."""
+    ending = bool(index & 1)
+    c = block_case(3000 + index, n, 4)
+    got = run_block(torch_cuda, c, ending)
+    helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block sweep {index}: n={n} ending={ending}")
+
+
 def test_triangle_attention_block_full_size_orientation_identity(torch_cuda):
     """384 residues: the ending-node block equals the starting-node block on the transposed pair tensor and mask,
     transposed back -- the two orientations differ only in which element is read or written where."""
