@@ -725,6 +725,7 @@ template <int C, int BPW, bool HAS_NB>
 __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(FusedParams p)
 {
     constexpr int CK = C / 16;
+    constexpr bool V_ALIAS = C == 256 && BPW == 4; // second LDS layout, below
     extern __shared__ uint4 lds[];
 
     // XCD-aware unit mapping: consecutive workgroup ids land on different XCDs (8 of them), so the H
@@ -742,19 +743,32 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     const int nthreads = p.NW * 64;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, kept in a scalar register
     const int r = lane & 31, g = lane >> 5;
-    const int S = p.S, NB = p.NB, NT = p.NT, NW = p.NW, GW = p.GW;
+    const int S = p.S, NB = p.NB, NT = p.NT, NW = p.NW, GW = V_ALIAS ? 4 : p.GW;
 
+    // Second layout (256 channels at the longest sequences, NT == NB): all four weight matrices (64 KB) lie on the V array,
+    // whose fragments wait in registers until the projections are done; K, then V / weights, then one 4 KB input panel
+    // per wave (the mask's place afterwards).  The input rows are then staged once for all four projections.
     uint4 *lds_w = lds;
     uint4 *lds_k = lds_w + GW * CK * 64;
     uint4 *lds_v = lds_k + NT * 2 * 64;
+    uint4 *own_panel = nullptr;
     float *mask = reinterpret_cast<float *>(lds_w);
+    if constexpr (V_ALIAS) {
+        lds_k = lds, lds_v = lds_k + NT * 2 * 64, lds_w = lds_v;
+        uint4 *panels = lds_v + (NT * 2 * 64 > 4 * CK * 64 ? NT * 2 * 64 : 4 * CK * 64); // past the longer of V and weights
+        own_panel = panels + wave * 256;
+        mask = reinterpret_cast<float *>(panels);
+    }
     uint32_t *part_flags = reinterpret_cast<uint32_t *>(mask + NT * 32); // two flag bits per 64 keys, one word each
+    uint4 vpark[V_ALIAS ? BPW : 1][2];
 
-    if (NT > NB) { // phantom key tile: zero K and V fragments
+    if (NT > NB) { // phantom key tile: zero K and V fragments (V after the projections when the weights lie there)
         const uint4 z4 = {0u, 0u, 0u, 0u};
         for (int idx = tid; idx < 128; idx += nthreads) {
             lds_k[NB * 2 * 64 + idx] = z4;
-            lds_v[NB * 2 * 64 + idx] = z4;
+            if constexpr (!V_ALIAS) {
+                lds_v[NB * 2 * 64 + idx] = z4;
+            }
         }
     }
     // wave w holds the mask of keys [64(w + q NW), +64): NT <= 4 NW + 1 tiles are at most 2 NW such parts
@@ -777,7 +791,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     // the block's K slot (rows 0-15) and V slot (rows 16-31), private to the wave that owns the block.  With one matrix
     // per group there is no such free space (LDS is full at that sequence length) and the fragments are loaded from
     // global memory directly.
-    const bool staged_input = GW >= 2;
+    const bool staged_input = V_ALIAS || GW >= 2;
     const int prow = pi_row(r);
     for (int pi = 0; pi < npass; ++pi) {
         const int pass = staged_input ? npass - 1 - pi : pi;
@@ -810,6 +824,9 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             if (staged_input) {
                 const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
                 uint4 *kslot = lds_k + j * 128, *vslot = lds_v + j * 128 - 128; // panel slots 0-127 and 128-255
+                if constexpr (V_ALIAS) {
+                    kslot = vslot = own_panel;
+                }
                 const uint4 *fsrc = prow < 16 ? kslot : vslot;
                 const int srow8 = lane >> 3, chunk = lane & 7;
                 PanelRegs t = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane);
@@ -846,8 +863,13 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
                     for (int ks = 0; ks < CK; ++ks) {
                         acc = mfma(xf[ks], as_bf16x8(wsrc[ks * 64]), acc);
                     }
-                    lds_v[(j * 2 + 0) * 64 + lane] = as_uint4(pack8(acc, 0));
-                    lds_v[(j * 2 + 1) * 64 + lane] = as_uint4(pack8(acc, 8));
+                    if constexpr (V_ALIAS) {
+                        vpark[i][0] = as_uint4(pack8(acc, 0));
+                        vpark[i][1] = as_uint4(pack8(acc, 8));
+                    } else {
+                        lds_v[(j * 2 + 0) * 64 + lane] = as_uint4(pack8(acc, 0));
+                        lds_v[(j * 2 + 1) * 64 + lane] = as_uint4(pack8(acc, 8));
+                    }
                 } else {
                     // W_h . x^T: rows = head-dim, columns = sequence positions
 #pragma unroll
@@ -883,6 +905,19 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     }
     TL(3);
     __syncthreads(); // K and V of the whole sequence are in LDS; the weight fragments are no longer read
+    if constexpr (V_ALIAS) {
+#pragma unroll
+        for (int i = 0; i < BPW; ++i) {
+            const int j = wave + i * NW;
+            if (j < NB) {
+                lds_v[(j * 2 + 0) * 64 + lane] = vpark[i][0];
+                lds_v[(j * 2 + 1) * 64 + lane] = vpark[i][1];
+            }
+        }
+        if (NT > NB && tid < 128) {
+            lds_v[NB * 2 * 64 + tid] = uint4{0u, 0u, 0u, 0u};
+        }
+    }
 #pragma unroll
     for (int q = 0; q < MASK_PARTS; ++q) {
         const int part = wave + q * NW;
@@ -1671,9 +1706,15 @@ int num_cus()
     return kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, table);
 }
 
-size_t head_kernel_lds(int C, int NB, int GW)
+size_t head_kernel_lds(int C, int NB, int GW, int NW, int BPW)
 {
     const int NT = (NB + 1) & ~1; // key tiles, padded to a pair
+    if (C == 256 && BPW == 4) {
+        // second layout of fused_head_kernel: K, then V with all four weight matrices lying on it, then a 4 KB input
+        // panel per wave (the mask's place later: 128 NT + 64 bytes always fit under 4 NW + 1 >= NT)
+        const size_t kv = (size_t)NT * 2 * 64 * 16, wbytes = (size_t)4 * (C / 16) * 64 * 16;
+        return kv + (kv > wbytes ? kv : wbytes) + (size_t)NW * 4096;
+    }
     // weight fragments (the mask, 4 bytes per key, and 16 flag words take their place later), K and V
     return (size_t)GW * (C / 16) * 64 * 16 + (size_t)NT * 2 * 64 * 16 * 2;
 }
@@ -1708,8 +1749,11 @@ bool make_plan(int64_t S, int C, Plan &pl)
         int bpw = 0, gw = 0;
         if (sscanf(env, "%d,%d", &bpw, &gw) == 2 && bpw >= 1 && bpw <= 4 && (gw == 1 || gw == 2 || gw == 4)) {
             const int nw = (int)((NB + bpw - 1) / bpw);
-            if (nw <= max_waves(C, bpw) && head_kernel_lds(C, pl.NB, gw) <= cap) {
-                pl.BPW = bpw, pl.NW = nw, pl.GW = gw, pl.lds_bytes = head_kernel_lds(C, pl.NB, gw);
+            if (C == 256 && bpw == 4) {
+                gw = 4;
+            }
+            if (nw <= max_waves(C, bpw) && head_kernel_lds(C, pl.NB, gw, nw, bpw) <= cap) {
+                pl.BPW = bpw, pl.NW = nw, pl.GW = gw, pl.lds_bytes = head_kernel_lds(C, pl.NB, gw, nw, bpw);
                 return true;
             }
         }
@@ -1731,7 +1775,7 @@ bool make_plan(int64_t S, int C, Plan &pl)
         return false;
     }
     for (int gw = 4; gw >= 1; gw >>= 1) {
-        const size_t need = head_kernel_lds(C, pl.NB, gw);
+        const size_t need = head_kernel_lds(C, pl.NB, gw, pl.NW, pl.BPW);
         if (need <= cap) {
             pl.GW = gw, pl.lds_bytes = need;
             return true;

@@ -83,6 +83,9 @@ SMALL = [
     # between the persistent kernel's reach and 1024 keys: two and three query blocks per wave of the long-sequence
     # kernel, an odd number of key tiles, with and without the fragment-major pair bias (it needs batch rows enough)
     (5, 3, 512), (5, 20, 450), (5, 2, 650), (4, 2, 768), (4, 3, 400), (3, 16, 736),
+    # 256 channels, four query blocks per wave: the weights lie on the V array there; an odd tile count with seven waves,
+    # a V array shorter than the weights with five waves, a ragged last block at eight waves
+    (4, 2, 800), (4, 3, 640), (4, 2, 1000),
 ]
 
 
