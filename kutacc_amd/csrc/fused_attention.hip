@@ -68,6 +68,7 @@ extern "C" __attribute__((visibility("default"))) int kutacc_debug_timeline(unsi
 namespace {
 
 constexpr int HEAD = 32;            // head_size the MFMA kernels are written for
+constexpr int WEIGHT_LOADS_IN_FLIGHT = 8; // per wave, while the weight fragments of a head are copied into LDS
 constexpr int MAX_WAVES = 12;       // fused_head_kernel: 768 threads, 3 waves per SIMD, 168 VGPRs each
 constexpr float RESCALE_GAP = 5.5f; // running max may lag the true max by this much (natural log units, ~8 octaves)
 
@@ -142,19 +143,21 @@ __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *m
     }
 }
 
-// The value stage_mask_part would store for key k, for kernels that fetch the mask early and store it later.
-__device__ __forceinline__ float mask_bias_value(const bf16_t *bias_row, int S, int k, float scale, int64_t stride_k,
-                                                 bool from_mask)
+// The value stage_mask_part would store for key k, in two steps for kernels that fetch the mask early and store it
+// later, so that nothing waits for the load where it is issued: the raw element of key min(k, S - 1) ...
+__device__ __forceinline__ bf16_t mask_bias_fetch(const bf16_t *bias_row, int S, int k, int64_t stride_k)
 {
-    float mv = -INFINITY;
-    if (k < S) {
-        mv = to_f32(bias_row[k * stride_k]);
-        if (from_mask) {
-            mv = to_f32((bf16_t)fmaf(mv, 1e9f, -1e9f));
-        }
-        mv *= scale;
+    return bias_row[(k < S ? k : S - 1) * stride_k];
+}
+
+// ... and the value made of it where it is stored.
+__device__ __forceinline__ float mask_bias_finish(bf16_t raw, bool in_range, float scale, bool from_mask)
+{
+    float mv = to_f32(raw);
+    if (from_mask) {
+        mv = to_f32((bf16_t)fmaf(mv, 1e9f, -1e9f));
     }
-    return mv;
+    return in_range ? mv * scale : -INFINITY;
 }
 
 // Flash-style attention of one 32-query block against all keys of the unit.
@@ -710,6 +713,40 @@ __device__ __forceinline__ void store_gated(bf16_t *dst, const f32x16 &o, float 
     }
 }
 
+// Copies head h's rows of `count` weight matrices (first, first + 1, ...) into LDS in MFMA fragment order.  One
+// fragment -- a matrix's 32 rows by 16 channels, 1 KB -- is one wave-wide copy, so the fragment index is wave-uniform
+// and the matrix pointer is picked with scalar selects (indexing the pointer array per lane made every copy wait for a
+// load of the pointer first).  Whole batches of eight fragments per wave go without a branch between the loads and the
+// stores: eight L2 round trips overlap instead of queueing (one at a time they were 9 % of the long-sequence kernel).
+// ------------------------------------------------------------------------------------------------
+template <int C>
+__device__ inline void stage_weight_fragments(uint4 *lds_w, const FusedParams &p, int first, int count, int h, int wave,
+                                              int nwaves, int lane)
+{
+    constexpr int CK = C / 16;
+    const int nfrag = count * CK;
+    auto fragment = [&](int f) {
+        const int m = first + f / CK, ks = f % CK;
+        const bf16_t *w = m == 0 ? p.w[0] : m == 1 ? p.w[1] : m == 2 ? p.w[2] : p.w[3];
+        return *reinterpret_cast<const uint4 *>(w + (int64_t)(h * HEAD + (lane & 31)) * C + ks * 16 + (lane >> 5) * 8);
+    };
+    int f = wave;
+    for (; f + (WEIGHT_LOADS_IN_FLIGHT - 1) * nwaves < nfrag; f += WEIGHT_LOADS_IN_FLIGHT * nwaves) {
+        uint4 t[WEIGHT_LOADS_IN_FLIGHT];
+#pragma unroll
+        for (int k = 0; k < WEIGHT_LOADS_IN_FLIGHT; ++k) {
+            t[k] = fragment(f + k * nwaves);
+        }
+#pragma unroll
+        for (int k = 0; k < WEIGHT_LOADS_IN_FLIGHT; ++k) {
+            lds_w[(f + k * nwaves) * 64 + lane] = t[k];
+        }
+    }
+    for (; f < nfrag; f += nwaves) {
+        lds_w[f * 64 + lane] = fragment(f);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // fused_head_kernel: one workgroup per (b, h) unit
 // LDS carve-up, in 16-byte units unless noted:
@@ -726,6 +763,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
 {
     constexpr int CK = C / 16;
     constexpr bool V_ALIAS = C == 256 && BPW == 4; // second LDS layout, below
+    constexpr bool ONE_GROUP = V_ALIAS || C == 128; // all four weight matrices staged at once, always (see make_plan)
     extern __shared__ uint4 lds[];
 
     // XCD-aware unit mapping: consecutive workgroup ids land on different XCDs (8 of them), so the H
@@ -743,7 +781,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     const int nthreads = p.NW * 64;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, kept in a scalar register
     const int r = lane & 31, g = lane >> 5;
-    const int S = p.S, NB = p.NB, NT = p.NT, NW = p.NW, GW = V_ALIAS ? 4 : p.GW;
+    const int S = p.S, NB = p.NB, NT = p.NT, NW = p.NW, GW = ONE_GROUP ? 4 : p.GW;
 
     // Second layout (256 channels at the longest sequences, NT == NB): all four weight matrices (64 KB) lie on the V array,
     // whose fragments wait in registers until the projections are done; K, then V / weights, then one 4 KB input panel
@@ -773,39 +811,33 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     }
     // wave w holds the mask of keys [64(w + q NW), +64): NT <= 4 NW + 1 tiles are at most 2 NW such parts
     constexpr int MASK_PARTS = (BPW + 1) / 2;
-    float mask_value[MASK_PARTS];
+    bf16_t mask_raw[MASK_PARTS];
 #pragma unroll
     for (int q = 0; q < MASK_PARTS; ++q) {
-        mask_value[q] = mask_bias_value(p.bias + (int64_t)b * p.bias_sb, S, (wave + q * NW) * 64 + lane,
-                                        p.l2mode ? LOG2E : 1.0f, p.bias_sk, p.bias_is_mask != 0);
+        mask_raw[q] = mask_bias_fetch(p.bias + (int64_t)b * p.bias_sb, S, (wave + q * NW) * 64 + lane, p.bias_sk);
     }
 
     const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
     // ---- projections, in groups of GW weight matrices staged through LDS ----
     bf16x8 qf[BPW][2];   // Q^T fragments (B operand of the logits MFMA), scaled by 1/sqrt(d)
     bf16x8 gate[BPW][2]; // sigmoid(gate) in accumulator order, packed
-    const int npass = 4 / GW;
+    const int npass = ONE_GROUP ? 1 : 4 / GW;
     // With at least two matrices per group K and V (matrices 0 and 1) share a group; the groups are then walked from the
     // last to the first, so that K and V come last and the K/V fragment slots of a block stay free until that block's
     // own results land in them.  That lets the input rows take the coalesced route: a 4 KB staging panel aliased onto
     // the block's K slot (rows 0-15) and V slot (rows 16-31), private to the wave that owns the block.  With one matrix
     // per group there is no such free space (LDS is full at that sequence length) and the fragments are loaded from
     // global memory directly.
-    const bool staged_input = V_ALIAS || GW >= 2;
+    const bool staged_input = ONE_GROUP || GW >= 2;
     const int prow = pi_row(r);
     for (int pi = 0; pi < npass; ++pi) {
         const int pass = staged_input ? npass - 1 - pi : pi;
-        __syncthreads(); // previous group's fragments are no longer being read
-        if (pi == 0) {
+        if (pi > 0) {
+            __syncthreads(); // previous group's fragments are no longer being read
+        } else {
             TL(1);
         }
-        for (int idx = tid; idx < GW * CK * 64; idx += nthreads) {
-            const int mm = idx / (CK * 64);
-            const int ks = (idx >> 6) % CK;
-            const int ln = idx & 63;
-            const bf16_t *src = p.w[pass * GW + mm] + (int64_t)(h * HEAD + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8;
-            lds_w[idx] = *reinterpret_cast<const uint4 *>(src);
-        }
+        stage_weight_fragments<C>(lds_w, p, pass * GW, GW, h, wave, NW, lane);
         __syncthreads();
         if (pi == 0) {
             TL(2);
@@ -922,7 +954,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
     for (int q = 0; q < MASK_PARTS; ++q) {
         const int part = wave + q * NW;
         if (part * 64 < NT * 32) {
-            const float mv = mask_value[q];
+            const float mv = mask_bias_finish(mask_raw[q], part * 64 + lane < S, p.l2mode ? LOG2E : 1.0f, p.bias_is_mask != 0);
             mask[part * 64 + lane] = mv;
             const unsigned long long nz = __ballot(mv != 0.f);
             if (lane == 0) {
@@ -1034,13 +1066,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 2 * NT * 32);            // two, alternating by batch row
 
     // the head's rows of the four weight matrices, in fragment order, for the whole kernel
-    for (int idx = tid; idx < 4 * CK * 64; idx += nthreads) {
-        const int mm = idx / (CK * 64);
-        const int ks = (idx >> 6) % CK;
-        const int ln = idx & 63;
-        const bf16_t *src = p.w[mm] + (int64_t)(h * HEAD + (ln & 31)) * C + ks * 16 + (ln >> 5) * 8;
-        lds_w[idx] = *reinterpret_cast<const uint4 *>(src);
-    }
+    stage_weight_fragments<C>(lds_w, p, 0, 4, h, wave, nthreads >> 6, lane);
     if (tid == 0) {
         flag_words[0] = 0;
         flag_words[1] = 0;
@@ -1749,8 +1775,8 @@ bool make_plan(int64_t S, int C, Plan &pl)
         int bpw = 0, gw = 0;
         if (sscanf(env, "%d,%d", &bpw, &gw) == 2 && bpw >= 1 && bpw <= 4 && (gw == 1 || gw == 2 || gw == 4)) {
             const int nw = (int)((NB + bpw - 1) / bpw);
-            if (C == 256 && bpw == 4) {
-                gw = 4;
+            if (C == 128 || bpw == 4) {
+                gw = 4; // what those kernels are compiled for
             }
             if (nw <= max_waves(C, bpw) && head_kernel_lds(C, pl.NB, gw, nw, bpw) <= cap) {
                 pl.BPW = bpw, pl.NW = nw, pl.GW = gw, pl.lds_bytes = head_kernel_lds(C, pl.NB, gw, nw, bpw);
@@ -1774,7 +1800,9 @@ bool make_plan(int64_t S, int C, Plan &pl)
     if (pl.BPW == 0) {
         return false;
     }
-    for (int gw = 4; gw >= 1; gw >>= 1) {
+    // The 128-channel kernels and the 256-channel one with four blocks per wave are compiled for one group of four.
+    const int gw_min = (C == 128 || pl.BPW == 4) ? 4 : 1;
+    for (int gw = 4; gw >= gw_min; gw >>= 1) {
         const size_t need = head_kernel_lds(C, pl.NB, gw, pl.NW, pl.BPW);
         if (need <= cap) {
             pl.GW = gw, pl.lds_bytes = need;
