@@ -55,7 +55,10 @@ constexpr int TILE = 128, KSTEP = 64;
 constexpr int OPERAND_SLOTS = 4 * 256;          // four 32-row panels of 256 16-byte slots
 constexpr int STAGE_SLOTS = 2 * OPERAND_SLOTS;  // A and B
 constexpr int CT_LD = 136;                      // bf16 elements per row of the C tile in LDS (272 bytes)
-constexpr size_t GEMM_LDS = 2 * STAGE_SLOTS * 16;
+// One operand stage (two barriers per k-step) that the C tile takes over at the end: 34 KB, three workgroups per CU.
+// With a second stage only two fit, and the third workgroup hides more of a short tile's prologue and epilogue than
+// the second stage did (triangle-multiplication products at 384 residues: 30.7 -> 26.6 us, gated projection 32 -> 27).
+constexpr size_t GEMM_LDS = TILE * CT_LD * 2 > STAGE_SLOTS * 16 ? TILE * CT_LD * 2 : STAGE_SLOTS * 16;
 
 // K-major operand: rows row0..row0+31 (clamped), 64 k from k0; chunks past K read as zero
 __device__ __forceinline__ PanelRegs load_kmajor(const bf16_t *base, int64_t ld, int row0, int last_row, int k0, int K, int lane)
@@ -138,7 +141,7 @@ __device__ __forceinline__ bf16x8 mm_fragment(const lds_char *operand, int lane_
 }
 
 template <bool A_MMAJOR, bool B_MMAJOR, bool GATED>
-__global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
+__global__ __launch_bounds__(256, 3) void pair_gemm_kernel(const GemmParams p)
 {
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -220,7 +223,10 @@ __global__ __launch_bounds__(256, 2) void pair_gemm_kernel(const GemmParams p)
     const int KT = (p.K + KSTEP - 1) / KSTEP;
     PanelRegs ra = fetch_a(0), rb = fetch_b(0);
     for (int kt = 0; kt < KT; ++kt) {
-        uint4 *stage = lds + (kt & 1) * STAGE_SLOTS;
+        uint4 *stage = lds;
+        if (kt > 0) {
+            __syncthreads(); // the stage is no longer being read
+        }
         park(stage, ra, rb);
         __syncthreads();
         if (kt + 1 < KT) {
@@ -883,7 +889,7 @@ bool operand_ok(const void *ptr, int64_t s_row, int64_t s_k, int64_t s_batch, in
 template <bool AM, bool BM, bool G>
 hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
 {
-    static size_t configured[KUTACC_DEVICE_SLOTS] = {}; // per instantiation and device: 64 KB of dynamic LDS needs the opt-in
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {}; // per instantiation and device: dynamic LDS is set through the opt-in
     if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&pair_gemm_kernel<AM, BM, G>), GEMM_LDS, configured)) {
         return e;
     }
