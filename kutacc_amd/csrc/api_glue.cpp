@@ -108,8 +108,13 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
         return KUTACC_HIP_EUNSUPPORTED;
     }
     // 1. LayerNorm + pair-bias projection in one pass over the pair tensor; the ending node reads it transposed
+    //    -- and, where the grid allows it, writes the fragment-major copy the attention kernels read as well
+    int frag_nb = 0, frag_nt = 0;
+    const bool fragments = kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt) &&
+                           kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, ws + w.z_norm, n, n, c, heads,
+                                                                     KUTACC_DTYPE_BF16);
     int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, ws + w.z_norm, n, n, c, heads,
-                                      a->ln_eps, KUTACC_DTYPE_BF16, ending, s);
+                                      a->ln_eps, KUTACC_DTYPE_BF16, ending, s, fragments ? g.q : nullptr, frag_nb, frag_nt);
     if (rc != 0) {
         return rc;
     }
@@ -119,6 +124,7 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     opt.out_mode = ending ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
     opt.bias_is_mask = true; // element (b, k) of the mask bias comes from mask[b, k], or mask[k, b] for the ending node
     opt.bias_stride_k = ending ? n : 1;
+    opt.nb_fragments_ready = fragments;
     return kutacc_launch::gating_attention_fused(g, s, opt);
 }
 
@@ -388,9 +394,16 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
     int rc = kutacc_launch::layernorm_rows(a->msa_act, c, a->ln_gamma, a->ln_beta, ws + w.m_norm, c, n_seq * n_res, c, a->ln_eps,
                                            KUTACC_DTYPE_BF16, s, column ? n_seq : 0);
     // 2. pair bias from the pair activation (row-wise form only)
+    //    -- with the fragment-major copy the attention kernels read, where the grid allows it
+    bool fragments = false;
     if (rc == 0 && !column) {
+        int frag_nb = 0, frag_nt = 0;
+        fragments = kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt) &&
+                    kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, nullptr, n_res, n_res, a->c_z, heads,
+                                                              KUTACC_DTYPE_BF16);
         rc = kutacc_launch::pair_bias(a->pair_act, a->pair_ln_gamma, a->pair_ln_beta, a->bias_w, ws + w.nb, nullptr, n_res, n_res,
-                                      a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s);
+                                      a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s, fragments ? g.q : nullptr, frag_nb,
+                                      frag_nt);
     }
     // 3. the operator: mask bias formed from the msa mask on the fly, output projection adding into the msa (transposed
     //    back for the column-wise form)
@@ -399,6 +412,7 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
         opt.out_mode = column ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
         opt.bias_is_mask = true; // msa_mask[s, r] is element (b = s, k = r) row-wise and (b = r, k = s) column-wise
         opt.bias_stride_k = column ? n_res : 1;
+        opt.nb_fragments_ready = fragments;
         rc = kutacc_launch::gating_attention_fused(g, s, opt);
     }
     return rc;

@@ -1814,6 +1814,18 @@ bool make_plan(int64_t S, int C, Plan &pl)
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// Whether the fast attention loop gets a fragment-major copy of the pair bias: it lives in the caller's q scratch tensor,
+// when that is dense, aligned and large enough.
+bool wants_fragments(const kutacc_hip_attention_args_t &a, int NB)
+{
+    const int64_t C = a.nheads * a.head_size;
+    const int64_t nbf_bytes = (int64_t)a.nheads * NB * ((NB + 1) & ~1) * 2048;
+    const bool q_dense = a.q != nullptr && aligned(a.q, 16) && a.q_stride_h == a.head_size && a.q_stride_s == C &&
+                         a.q_stride_b == a.seq_len * C;
+    return a.nonbatched_bias != nullptr && q_dense && nbf_bytes <= a.batch * a.seq_len * C * 2 &&
+           !getenv("KUTACC_HIP_NO_FRAGMENTS");
+}
+
 template <typename K>
 int opt_in_lds(K kern, size_t bytes, size_t *table)
 {
@@ -1899,6 +1911,16 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
 
 namespace kutacc_launch {
 
+bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &a, int *nb, int *nt)
+{
+    Plan pl;
+    if (!fused_attention_supports(a) || !make_plan(a.seq_len, (int)(a.nheads * a.head_size), pl) || !wants_fragments(a, pl.NB)) {
+        return false;
+    }
+    *nb = pl.NB, *nt = (pl.NB + 1) & ~1;
+    return true;
+}
+
 bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
 {
     if (a.dtype != KUTACC_DTYPE_BF16 || a.head_size != HEAD) {
@@ -1956,15 +1978,13 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     // scratch tensor (which this path does not otherwise use; its contents are unspecified after any
     // call) when that is dense, aligned and large enough; otherwise the kernels read the pair bias in
     // place through the staging panels.
-    const int64_t nbf_bytes = (int64_t)a.nheads * pl.NB * p.NT * 2048;
-    const bool q_dense = a.q != nullptr && aligned(a.q, 16) && a.q_stride_h == a.head_size && a.q_stride_s == C &&
-                         a.q_stride_b == a.seq_len * C;
-    const bool want_fragments = p.nb != nullptr && q_dense &&
-                                nbf_bytes <= a.batch * a.seq_len * C * 2 && !getenv("KUTACC_HIP_NO_FRAGMENTS");
+    const bool want_fragments = wants_fragments(a, pl.NB);
 
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
-    if (want_fragments) {
+    if (want_fragments && opt.nb_fragments_ready) {
+        p.nbf = (const uint4 *)a.q; // the producer of the pair bias wrote the copy
+    } else if (want_fragments) {
         kutacc_prof::KernelTimer t("pair_bias_fragments_kernel", 0.0, stream);
         pair_bias_fragments_kernel<<<dim3((unsigned)(pl.NB * p.NT), (unsigned)a.nheads), 64, 0, stream>>>(
             p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.NT, p.nb_vec, (uint4 *)a.q);

@@ -80,7 +80,13 @@ struct FusedAttentionOptions {
     int out_mode = FUSED_OUT_STORE;
     bool bias_is_mask = false;
     int64_t bias_stride_k = 1;
+    // the fragment-major copy of the pair bias already lies in args.q (written by pair_bias with the layout
+    // fused_attention_fragment_layout reports): the pass that makes it is skipped
+    bool nb_fragments_ready = false;
 };
+// Whether gating_attention_fused would keep a fragment-major copy of the pair bias in args.q, and the copy's extent:
+// [nheads][*nb query blocks][*nt key tiles][2][64 lanes] x 16 bytes.
+bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &args, int *nb, int *nt);
 int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream,
                            const FusedAttentionOptions &opt = FusedAttentionOptions());
 
@@ -132,8 +138,12 @@ int layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, con
 // row (j, i) of the transposed grid
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                    int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream, int64_t swap_j = 0);
+// fragments != nullptr: the fragment-major copy the attention kernels read ([nheads][frag_nb][frag_nt][2][64] x 16 bytes,
+// values times log2(e)) is written as well; only where pair_bias_writes_fragments says so, else KUTACC_HIP_EINVAL
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
               int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
-              hipStream_t stream);
+              hipStream_t stream, void *fragments = nullptr, int frag_nb = 0, int frag_nt = 0);
+bool pair_bias_writes_fragments(const void *z, const void *w, const void *z_norm, int64_t rows_i, int64_t rows_j, int64_t c_z,
+                                int64_t nheads, int32_t dtype);
 
 } // namespace kutacc_launch

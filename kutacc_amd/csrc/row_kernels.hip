@@ -208,7 +208,8 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
                                                              const float *__restrict__ beta, const bf16_t *__restrict__ w,
                                                              bf16_t *__restrict__ nb, bf16_t *__restrict__ z_norm,
                                                              int64_t rows, float eps, int64_t rows_i, int64_t rows_j,
-                                                             int transposed)
+                                                             int transposed, uint4 *__restrict__ nbf, int frag_nb,
+                                                             int frag_nt)
 {
     constexpr int LPR = 16, CZ = 128, STEPS = PAIR_BIAS_ROWS_PER_WAVE / 4, RB = PAIR_BIAS_ROWS_PER_WAVE / 32;
     __shared__ uint4 tiles[4][RB * 2 * 256]; // per wave: its rows x 128 channels as 32 x 64 panels
@@ -297,6 +298,33 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
                 }
             }
         }
+        if (nbf != nullptr) {
+            // The copy the attention kernels read (rows_j a multiple of 32: the wave's rows are key tile t of one query
+            // q): for head h, query block j, key tile t, 16-key half g' and 8-key half e the 16 bytes of lane
+            // (pi^-1(q mod 32), g'), pi being the row order of the attention's accumulators; values in log2 units,
+            // rounded to bf16 a second time.  Through the wave's tile, which nobody reads any more: [head][32 keys].
+            static_assert(RB == 1, "the transposing buffer lies on the first row block of the tile");
+            bf16_t *t16 = reinterpret_cast<bf16_t *>(tile);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if (4 * g + v < H) {
+                    t16[(4 * g + v) * 32 + col] = (bf16_t)((float)(bf16_t)acc[v] * kutacc_dev::LOG2E);
+                }
+            }
+            __builtin_amdgcn_wave_barrier(); // other lanes' stores: keep the loads below behind them
+            if (lane < 4 * H) {
+                const int h = lane >> 2, c = lane & 3;
+                const uint4 val = *reinterpret_cast<const uint4 *>(t16 + h * 32 + c * 8);
+                const int64_t r0b = r0 + rb * 32;
+                const int q = (int)(r0b / rows_j), t = (int)(r0b % rows_j) >> 5, qr = q & 31;
+                const int qlane = (qr & 3) | (((qr >> 4) & 1) << 2) | (((qr >> 2) & 3) << 3);
+                uint4 *dst = nbf + ((((int64_t)h * frag_nb + (q >> 5)) * frag_nt + t) * 2 + (c & 1)) * 64 + qlane + 32 * (c >> 1);
+                *dst = val;
+                if (t + 1 == frag_nb && frag_nt > frag_nb) { // the phantom tile that pads the key tiles to a pair
+                    dst[128] = make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+        }
     }
 }
 
@@ -334,9 +362,15 @@ int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const floa
 template <typename T>
 int launch_pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
                      int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int transposed,
-                     hipStream_t stream)
+                     hipStream_t stream, void *fragments, int frag_nb, int frag_nt)
 {
     const int64_t rows = rows_i * rows_j;
+    if (fragments != nullptr &&
+        (!kutacc_launch::pair_bias_writes_fragments(z, w, z_norm, rows_i, rows_j, c_z, nheads,
+                                                    sizeof(T) == 2 ? KUTACC_DTYPE_BF16 : KUTACC_DTYPE_FP32) ||
+         frag_nb != rows_j / 32 || frag_nt != ((frag_nb + 1) & ~1))) {
+        return KUTACC_HIP_EINVAL;
+    }
     if (sizeof(T) == 2 && c_z == 128 && (nheads == 4 || nheads == 8) &&
         (reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(z_norm)) % 16 == 0) {
         const int64_t nblk = (rows + 4 * PAIR_BIAS_ROWS_PER_WAVE - 1) / (4 * PAIR_BIAS_ROWS_PER_WAVE);
@@ -346,11 +380,11 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
         if (nheads == 4) {
             pair_bias_bf16_kernel<4><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
                                                                         (bf16_t *)nb, (bf16_t *)z_norm, rows, eps, rows_i, rows_j,
-                                                                        transposed);
+                                                                        transposed, (uint4 *)fragments, frag_nb, frag_nt);
         } else {
             pair_bias_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
                                                                         (bf16_t *)nb, (bf16_t *)z_norm, rows, eps, rows_i, rows_j,
-                                                                        transposed);
+                                                                        transposed, (uint4 *)fragments, frag_nb, frag_nt);
         }
         return kutacc_hip_status(hipGetLastError());
     }
@@ -383,18 +417,29 @@ int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float 
     return KUTACC_HIP_EINVAL;
 }
 
+bool pair_bias_writes_fragments(const void *z, const void *w, const void *z_norm, int64_t rows_i, int64_t rows_j, int64_t c_z,
+                                int64_t nheads, int32_t dtype)
+{
+    // the MFMA producer, whose waves own 32 consecutive rows: whole key tiles of one query when the grid is square
+    // and its side a multiple of 32
+    return dtype == KUTACC_DTYPE_BF16 && c_z == 128 && (nheads == 4 || nheads == 8) && rows_i == rows_j && rows_j % 32 == 0 &&
+           (reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(z_norm)) % 16 == 0;
+}
+
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
               int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
-              hipStream_t stream)
+              hipStream_t stream, void *fragments, int frag_nb, int frag_nt)
 {
     if (!z || !gamma || !beta || !w || !nb || rows_i <= 0 || rows_j <= 0 || c_z <= 0 || nheads <= 0) {
         return KUTACC_HIP_EINVAL;
     }
     if (dtype == KUTACC_DTYPE_BF16) {
-        return launch_pair_bias<bf16_t>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream);
+        return launch_pair_bias<bf16_t>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream,
+                                        fragments, frag_nb, frag_nt);
     }
     if (dtype == KUTACC_DTYPE_FP32) {
-        return launch_pair_bias<float>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream);
+        return launch_pair_bias<float>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream,
+                                       fragments, frag_nb, frag_nt);
     }
     return KUTACC_HIP_EINVAL;
 }

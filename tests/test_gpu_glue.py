@@ -146,7 +146,9 @@ def run_block(torch, c, ending, z=None, mask=None):
 
 
 @pytest.mark.parametrize("ending", [False, True], ids=["starting node", "ending node"])
-@pytest.mark.parametrize("n,heads", [(48, 4), (70, 4), (40, 8)])
+# 64, 96 and 160: whole key tiles, where the producer of the pair bias also writes the copy the attention kernels read
+# (96 and 160: an odd tile count, padded with a zero tile)
+@pytest.mark.parametrize("n,heads", [(48, 4), (70, 4), (40, 8), (64, 4), (96, 4), (160, 4), (64, 8)])
 def test_triangle_attention_block_against_the_oracle(torch_cuda, n, heads, ending):
     c = block_case(600 + n, n, heads)
     got = run_block(torch_cuda, c, ending)
@@ -417,7 +419,8 @@ def msa_oracle(c, column):
 
 
 @pytest.mark.parametrize("column", [False, True], ids=["row-wise with pair bias", "column-wise"])
-@pytest.mark.parametrize("n_seq,n_res,heads,c_z", [(24, 40, 8, 128), (50, 20, 8, 128), (33, 33, 4, 64)])
+@pytest.mark.parametrize("n_seq,n_res,heads,c_z", [(24, 40, 8, 128), (50, 20, 8, 128), (33, 33, 4, 64), (24, 64, 8, 128),
+                                                   (20, 96, 8, 128)])
 def test_msa_attention_block_against_the_oracle(torch_cuda, n_seq, n_res, heads, c_z, column):
     torch = torch_cuda
     c = msa_case(1000 + n_seq, n_seq, n_res, heads, c_z)
