@@ -141,7 +141,7 @@ __device__ __forceinline__ bf16x8 mm_fragment(const lds_char *operand, int lane_
 }
 
 template <bool A_MMAJOR, bool B_MMAJOR, bool GATED>
-__global__ __launch_bounds__(256, 3) void pair_gemm_kernel(const GemmParams p)
+__global__ __launch_bounds__(256, (A_MMAJOR && B_MMAJOR) ? 4 : 3) void pair_gemm_kernel(const GemmParams p)
 {
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
