@@ -292,7 +292,7 @@ kutacc_export int kutacc_hip_gated_residual_projection(const void *a, int64_t a_
  * with the two LayerNorms, the layout change and the residual a caller of the reference adds around them; seven
  * launches on `stream` (the output projection, its gating and the residual are one kernel when c_i is 128 or 256
  * and c_z a multiple of 128; with c_i = c_z = 128 that kernel projects the gate as well and, when n_res^2 is a multiple
- * of 8, normalises the centre on its way in: five launches).  bf16; weights stored [out, in]: *_proj_w, *_gate_w [c_i, c_z], output_w [c_z, c_i], gating_w
+ * of 8, normalises the centre on its way in: five launches, four when both gated projections share one).  bf16; weights stored [out, in]: *_proj_w, *_gate_w [c_i, c_z], output_w [c_z, c_i], gating_w
  * [c_z, c_z]; all biases and LayerNorm parameters fp32.  `workspace`: device memory, 256-byte aligned, at least
  * kutacc_hip_triangle_multiplication_workspace(n_res, c_z, c_i) bytes.
  */
