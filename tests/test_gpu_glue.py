@@ -148,7 +148,7 @@ def run_block(torch, c, ending, z=None, mask=None):
 @pytest.mark.parametrize("ending", [False, True], ids=["starting node", "ending node"])
 # 64, 96 and 160: whole key tiles, where the producer of the pair bias also writes the copy the attention kernels read
 # (96 and 160: an odd tile count, padded with a zero tile)
-@pytest.mark.parametrize("n,heads", [(48, 4), (70, 4), (40, 8), (64, 4), (96, 4), (160, 4), (64, 8)])
+@pytest.mark.parametrize("n,heads", [(48, 4), (70, 4), (40, 8), (64, 4), (96, 4), (160, 4), (64, 8), (32, 4), (128, 8)])
 def test_triangle_attention_block_against_the_oracle(torch_cuda, n, heads, ending):
     c = block_case(600 + n, n, heads)
     got = run_block(torch_cuda, c, ending)
