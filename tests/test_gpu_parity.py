@@ -106,6 +106,27 @@ def test_reduced_shapes_both_kernel_families(torch_cuda, config, batch, seq, pat
     helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
 
 
+@pytest.mark.parametrize("config,batch,seq,plan", [
+    # 256 channels: two matrices per group (rows staged through the block's own K/V slots, groups walked backwards), one
+    # per group (fragments loaded straight from global memory), and four blocks per wave well below the lengths that pick it
+    (4, 2, 512, "2,2"), (4, 2, 500, "3,1"), (4, 2, 512, "4,4"), (4, 3, 300, "2,1"),
+    # 128 channels with more blocks per wave than the planner would take
+    (5, 3, 384, "2,4"), (5, 2, 330, "4,4"),
+])
+def test_forced_kernel_plans_match_the_oracle(torch_cuda, monkeypatch, config, batch, seq, plan):
+    """Routes of the long-sequence kernel that the planner only takes on a device with less LDS, forced through the
+    library's tuning hook."""
+    monkeypatch.setenv("KUTACC_HIP_PLAN", plan)
+    w = make_workload(config, batch=batch, seq_len=seq)
+    print(f"config {config} B={batch} S={seq} plan={plan}", flush=True)
+    ten, scratch = helpers.to_device(w)
+    rc = helpers.run_hip(w, ten, scratch, capi.PATH_FUSED)
+    assert rc == 0, rc
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, "gated average")
+    helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
+
+
 def _sweep_cases():
     """24 seeded shapes over the whole range the MFMA kernels take: any sequence length up to 1024 (ragged tails, odd
     numbers of key tiles, every blocks-per-wave variant of the long-sequence kernel), both channel counts, with and without
