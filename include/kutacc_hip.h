@@ -402,6 +402,13 @@ kutacc_export void kutacc_hip_profile_enable(int on);
 kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, double *total_ms, int64_t *launches,
                                           double *flops_per_launch);
 
+/* Tuning hooks for tests and experiments; name/value strings, 0 on success, KUTACC_HIP_EINVAL for an unknown name.
+ *   "plan"      "bpw,gw": force the long-sequence attention kernel with bpw (1-4) query blocks per wave and gw (1, 2, 4)
+ *               weight matrices per LDS group where that fits the device; anything else: the planner decides (default)
+ *   "fragments" "0": keep the attention kernels off the fragment-major pair bias (general softmax blocks); "1": default
+ *   "debug"     "1": one line per fused call on stderr with the plan taken; "0": default */
+kutacc_export int kutacc_hip_set_tuning(const char *name, const char *value);
+
 /* The process-wide sticky error flag behind KUTACC_CHECK (reference src/utils/check.cpp:16 keeps it
  * hidden and never resets it).  Reading/clearing it is an addition for tests and long-lived hosts. */
 kutacc_export int kutacc_hip_error_flag(void);

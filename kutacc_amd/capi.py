@@ -167,7 +167,7 @@ DECLARED_SYMBOLS = [
     "kutacc_hip_gating_attention", "kutacc_hip_global_attention", "kutacc_hip_last_path", "kutacc_hip_layernorm_rows", "kutacc_hip_linear",
     "kutacc_hip_pair_bias", "kutacc_hip_set_stream", "kutacc_hip_get_stream", "kutacc_hip_set_blocking",
     "kutacc_hip_error_flag", "kutacc_hip_clear_error", "kutacc_hip_tensor_create", "kutacc_hip_tensor_destroy",
-    "kutacc_hip_profile_enable", "kutacc_hip_profile_read",
+    "kutacc_hip_profile_enable", "kutacc_hip_profile_read", "kutacc_hip_set_tuning",
 ]
 
 _lib = None
@@ -181,6 +181,13 @@ def lib() -> ctypes.CDLL:
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m kutacc_amd.build` "
                            "(the HIP library is the only implementation; there is no CPU path)")
+    # One HIP runtime per process: PyTorch ships its own libamdhip64, and a library loaded before it would bind the
+    # system copy instead -- a second runtime, which on a GPU box reports "no device" for every call made through it.
+    # Loading torch first makes the dynamic loader hand this library the runtime torch already mapped.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = ctypes.CDLL(LIB_PATH)
     L.kutacc_get_version.argtypes = [ctypes.POINTER(Version)]
     L.kutacc_get_version.restype = ctypes.c_int
@@ -270,6 +277,8 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_profile_read.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(_i64), ctypes.POINTER(ctypes.c_double)]
     L.kutacc_hip_profile_read.restype = ctypes.c_int
+    L.kutacc_hip_set_tuning.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
+    L.kutacc_hip_set_tuning.restype = ctypes.c_int
     _lib = L
     return L
 
@@ -299,6 +308,11 @@ def set_stream(stream_ptr: int | None) -> None:
 
 def set_blocking(blocking: bool) -> None:
     lib().kutacc_hip_set_blocking(1 if blocking else 0)
+
+
+def set_tuning(name: str, value: str | None) -> int:
+    """kutacc_hip_set_tuning: "plan" / "fragments" / "debug" hooks of the attention launcher (None = default)."""
+    return lib().kutacc_hip_set_tuning(name.encode(), None if value is None else value.encode())
 
 
 class TensorHandle:

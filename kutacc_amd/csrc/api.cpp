@@ -355,6 +355,11 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
     a.avg_stride_b = av.stride(0), a.avg_stride_s = av.stride(1), a.avg_stride_h = av.stride(2);
     a.v_stride_h = v.stride(0), a.v_stride_e = v.stride(1), a.v_stride_b = v.stride(2);
     a.out = ot.data, a.out_ld = ot.stride(ot.dim >= 3 ? 1 : 0);
+    // The MFMA kernels may use q as workspace for a copy of the pair bias and take its extent from batch, seq_len and
+    // the strides: a handle that describes fewer elements than that must not be written through.
+    if (q.numel() < batch * seq_len * nchannels && kutacc_launch::fused_attention_supports(a)) {
+        a.q = nullptr;
+    }
 
     hipStream_t s = g_stream;
     const Space sp = space_of(in.data);

@@ -28,10 +28,14 @@
 //     keys (pair-bias row loads become two 16-byte loads).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <climits>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
+#include "api_internal.h"
 #include "device_util.h"
 #include "launch_internal.h"
 #include "mfma_tiles.h"
@@ -1714,6 +1718,12 @@ __global__ __launch_bounds__(64) void pair_bias_fragments_kernel(const bf16_t *_
     dst[64] = as_uint4(d1);
 }
 
+// Tuning hooks (kutacc_hip_set_tuning): a forced plan of the long-sequence kernel, the fragment-major pair bias switched
+// off, one line per call on stderr.  Plain atomics: set from a test or an experiment, read on every launch.
+std::atomic<int> g_forced_bpw{0}, g_forced_gw{0}, g_no_fragments{0}, g_debug{0};
+
+bool fragments_disabled() { return g_no_fragments.load(std::memory_order_relaxed) != 0; }
+
 struct Plan {
     bool persistent;
     int NB, NW, BPW, GW;
@@ -1763,25 +1773,21 @@ bool make_plan(int64_t S, int C, Plan &pl)
     pl.NB = (int)NB;
     pl.persistent = false;
     const size_t cap = (size_t)max_lds_bytes();
-    const char *env = getenv("KUTACC_HIP_PLAN"); // experiment hook: "p" | "bpw,gw"
+    const int forced_bpw = g_forced_bpw.load(std::memory_order_relaxed), forced_gw = g_forced_gw.load(std::memory_order_relaxed);
     // persistent kernel: one wave per sequence block, everything of one head resident in LDS
     const bool fits_persistent = NB <= max_waves(C, 1) && persistent_kernel_lds(C, (int)NB) <= cap;
-    if (fits_persistent && !(env && env[0] != 'p')) {
+    if (fits_persistent && forced_bpw == 0) {
         pl.persistent = true;
         pl.NW = (int)NB, pl.BPW = 1, pl.GW = 4, pl.lds_bytes = persistent_kernel_lds(C, (int)NB);
         return true;
     }
-    if (env && env[0] != 'p') {
-        int bpw = 0, gw = 0;
-        if (sscanf(env, "%d,%d", &bpw, &gw) == 2 && bpw >= 1 && bpw <= 4 && (gw == 1 || gw == 2 || gw == 4)) {
-            const int nw = (int)((NB + bpw - 1) / bpw);
-            if (C == 128 || bpw == 4) {
-                gw = 4; // what those kernels are compiled for
-            }
-            if (nw <= max_waves(C, bpw) && head_kernel_lds(C, pl.NB, gw, nw, bpw) <= cap) {
-                pl.BPW = bpw, pl.NW = nw, pl.GW = gw, pl.lds_bytes = head_kernel_lds(C, pl.NB, gw, nw, bpw);
-                return true;
-            }
+    if (forced_bpw != 0) {
+        const int bpw = forced_bpw;
+        const int gw = (C == 128 || bpw == 4) ? 4 : forced_gw; // those kernels are compiled for one group of four
+        const int nw = (int)((NB + bpw - 1) / bpw);
+        if (nw <= max_waves(C, bpw) && head_kernel_lds(C, pl.NB, gw, nw, bpw) <= cap) {
+            pl.BPW = bpw, pl.NW = nw, pl.GW = gw, pl.lds_bytes = head_kernel_lds(C, pl.NB, gw, nw, bpw);
+            return true;
         }
     }
     // fewest idle wave slots first, then fewest blocks per wave (more waves to overlap MFMA and VALU)
@@ -1814,16 +1820,26 @@ bool make_plan(int64_t S, int C, Plan &pl)
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// Whether the fast attention loop gets a fragment-major copy of the pair bias: it lives in the caller's q scratch tensor,
-// when that is dense, aligned and large enough.
-bool wants_fragments(const kutacc_hip_attention_args_t &a, int NB)
+// Bytes of the fragment-major copy of the pair bias: [nheads][NB query blocks][NB rounded up to even key tiles][2][64] x 16
+int64_t fragment_bytes(int64_t nheads, int NB) { return nheads * NB * ((NB + 1) & ~1) * 2048; }
+
+// Where the fast attention loop keeps its fragment-major copy of the pair bias, or nullptr when the call gets none: the
+// workspace the options bring, else the caller's q scratch tensor when that is dense, aligned and large enough.
+void *fragment_home(const kutacc_hip_attention_args_t &a, int NB, const kutacc_launch::FusedAttentionOptions &opt)
 {
+    if (a.nonbatched_bias == nullptr || fragments_disabled()) {
+        return nullptr;
+    }
+    const int64_t nbf_bytes = fragment_bytes(a.nheads, NB);
+    if (opt.fragment_workspace != nullptr) {
+        return (aligned(opt.fragment_workspace, 16) && (uint64_t)nbf_bytes <= opt.fragment_workspace_bytes)
+                   ? opt.fragment_workspace
+                   : nullptr;
+    }
     const int64_t C = a.nheads * a.head_size;
-    const int64_t nbf_bytes = (int64_t)a.nheads * NB * ((NB + 1) & ~1) * 2048;
     const bool q_dense = a.q != nullptr && aligned(a.q, 16) && a.q_stride_h == a.head_size && a.q_stride_s == C &&
                          a.q_stride_b == a.seq_len * C;
-    return a.nonbatched_bias != nullptr && q_dense && nbf_bytes <= a.batch * a.seq_len * C * 2 &&
-           !getenv("KUTACC_HIP_NO_FRAGMENTS");
+    return (q_dense && nbf_bytes <= a.batch * a.seq_len * C * 2) ? a.q : nullptr;
 }
 
 template <typename K>
@@ -1914,7 +1930,8 @@ namespace kutacc_launch {
 bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &a, int *nb, int *nt)
 {
     Plan pl;
-    if (!fused_attention_supports(a) || !make_plan(a.seq_len, (int)(a.nheads * a.head_size), pl) || !wants_fragments(a, pl.NB)) {
+    if (!fused_attention_supports(a) || !make_plan(a.seq_len, (int)(a.nheads * a.head_size), pl) ||
+        fragment_home(a, pl.NB, FusedAttentionOptions()) == nullptr) {
         return false;
     }
     *nb = pl.NB, *nt = (pl.NB + 1) & ~1;
@@ -1974,31 +1991,31 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     p.ngrp = 1;
     p.nbf = nullptr;
     p.l2mode = 0;
-    // Fragment-major copy of the pair bias for the fast attention loop.  It lives in the caller's q
-    // scratch tensor (which this path does not otherwise use; its contents are unspecified after any
-    // call) when that is dense, aligned and large enough; otherwise the kernels read the pair bias in
-    // place through the staging panels.
-    const bool want_fragments = wants_fragments(a, pl.NB);
+    // Fragment-major copy of the pair bias for the fast attention loop.  It lives in the workspace the options bring or in
+    // the caller's q scratch tensor (which this path does not otherwise use; its contents are unspecified after any
+    // call) when that is dense, aligned and large enough; otherwise the kernels read the pair bias in place through the
+    // staging panels.
+    void *const fragments = fragment_home(a, pl.NB, opt);
+    if (opt.fragment_workspace != nullptr && p.nb != nullptr && fragments == nullptr && !fragments_disabled()) {
+        return KUTACC_HIP_EINVAL; // the caller's workspace cannot hold the copy
+    }
 
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
-    if (want_fragments && opt.nb_fragments_ready) {
-        p.nbf = (const uint4 *)a.q; // the producer of the pair bias wrote the copy
-    } else if (want_fragments) {
+    if (fragments != nullptr && opt.nb_fragments_ready) {
+        p.nbf = (const uint4 *)fragments; // the producer of the pair bias wrote the copy
+    } else if (fragments != nullptr) {
         kutacc_prof::KernelTimer t("pair_bias_fragments_kernel", 0.0, stream);
         pair_bias_fragments_kernel<<<dim3((unsigned)(pl.NB * p.NT), (unsigned)a.nheads), 64, 0, stream>>>(
-            p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.NT, p.nb_vec, (uint4 *)a.q);
+            p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.NT, p.nb_vec, (uint4 *)fragments);
         rc = kutacc_hip_status(hipGetLastError());
         if (rc != 0) {
             return rc;
         }
-        p.nbf = (const uint4 *)a.q;
+        p.nbf = (const uint4 *)fragments;
     }
-    p.l2mode = ((p.nb == nullptr || p.nbf != nullptr) &&
-                !getenv("KUTACC_HIP_NO_FRAGMENTS"))
-                   ? 1
-                   : 0;
-    if (getenv("KUTACC_HIP_DEBUG")) {
+    p.l2mode = ((p.nb == nullptr || p.nbf != nullptr) && !fragments_disabled()) ? 1 : 0;
+    if (g_debug.load(std::memory_order_relaxed)) {
         fprintf(stderr,
                 "[kutacc] fused plan: persistent=%d C=%d NB=%d NT=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d log2_units=%d "
                 "fragments=%d\n",
@@ -2107,3 +2124,32 @@ int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const vo
 }
 
 } // namespace kutacc_launch
+
+// Tuning hooks for tests and experiments: "plan" = "bpw,gw" forces the long-sequence kernel with that many query blocks
+// per wave and weight matrices per group where it fits (anything else: the planner decides), "fragments" = "0" keeps the
+// kernels off the fragment-major pair bias (general attention blocks), "debug" = "1" prints the plan of every call.
+extern "C" kutacc_export int kutacc_hip_set_tuning(const char *name, const char *value)
+{
+    if (!name) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const bool on = value && value[0] != '\0' && value[0] != '0';
+    if (!strcmp(name, "plan")) {
+        int bpw = 0, gw = 0;
+        if (value && sscanf(value, "%d,%d", &bpw, &gw) == 2 && bpw >= 1 && bpw <= 4 && (gw == 1 || gw == 2 || gw == 4)) {
+            g_forced_gw.store(gw), g_forced_bpw.store(bpw);
+        } else {
+            g_forced_bpw.store(0), g_forced_gw.store(0);
+        }
+        return 0;
+    }
+    if (!strcmp(name, "fragments")) {
+        g_no_fragments.store((value && value[0] == '0') ? 1 : 0);
+        return 0;
+    }
+    if (!strcmp(name, "debug")) {
+        g_debug.store(on ? 1 : 0);
+        return 0;
+    }
+    return KUTACC_HIP_EINVAL;
+}

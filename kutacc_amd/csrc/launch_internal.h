@@ -83,6 +83,10 @@ struct FusedAttentionOptions {
     // the fragment-major copy of the pair bias already lies in args.q (written by pair_bias with the layout
     // fused_attention_fragment_layout reports): the pass that makes it is skipped
     bool nb_fragments_ready = false;
+    // device memory (16-byte aligned) that takes the fragment-major copy of the pair bias instead of args.q, which is then
+    // neither read nor written; a call whose copy does not fit is rejected with KUTACC_HIP_EINVAL
+    void *fragment_workspace = nullptr;
+    size_t fragment_workspace_bytes = 0;
 };
 // Whether gating_attention_fused would keep a fragment-major copy of the pair bias in args.q, and the copy's extent:
 // [nheads][*nb query blocks][*nt key tiles][2][64 lanes] x 16 bytes.

@@ -54,9 +54,13 @@ void resolve_locked()
 namespace kutacc_prof {
 bool enabled() { return g_enabled; }
 
+static thread_local int t_suppressed = 0;
+Suppress::Suppress() { ++t_suppressed; }
+Suppress::~Suppress() { --t_suppressed; }
+
 KernelTimer::KernelTimer(const char *name, double flops, hipStream_t stream) : name_(name), flops_(flops), stream_(stream)
 {
-    if (g_enabled && hipEventCreate(&start_) == hipSuccess) {
+    if (g_enabled && t_suppressed == 0 && hipEventCreate(&start_) == hipSuccess) {
         (void)hipEventRecord(start_, stream_);
     }
 }

@@ -7,6 +7,16 @@
 namespace kutacc_prof {
 bool enabled();
 
+// While one of these lives on a thread, KernelTimer records nothing there (event creation allocates, which the entry
+// points that promise not to allocate must not do even when a benchmark has switched timing on).
+class Suppress {
+public:
+    Suppress();
+    ~Suppress();
+    Suppress(const Suppress &) = delete;
+    Suppress &operator=(const Suppress &) = delete;
+};
+
 // Brackets the launches issued during its lifetime.  `flops` is the algorithmic work of one launch,
 // reported back next to the measured time.
 class KernelTimer {

@@ -113,14 +113,17 @@ def test_reduced_shapes_both_kernel_families(torch_cuda, config, batch, seq, pat
     # 128 channels with more blocks per wave than the planner would take
     (5, 3, 384, "2,4"), (5, 2, 330, "4,4"),
 ])
-def test_forced_kernel_plans_match_the_oracle(torch_cuda, monkeypatch, config, batch, seq, plan):
+def test_forced_kernel_plans_match_the_oracle(torch_cuda, config, batch, seq, plan):
     """Routes of the long-sequence kernel that the planner only takes on a device with less LDS, forced through the
     library's tuning hook."""
-    monkeypatch.setenv("KUTACC_HIP_PLAN", plan)
     w = make_workload(config, batch=batch, seq_len=seq)
     print(f"config {config} B={batch} S={seq} plan={plan}", flush=True)
     ten, scratch = helpers.to_device(w)
-    rc = helpers.run_hip(w, ten, scratch, capi.PATH_FUSED)
+    assert capi.set_tuning("plan", plan) == 0
+    try:
+        rc = helpers.run_hip(w, ten, scratch, capi.PATH_FUSED)
+    finally:
+        capi.set_tuning("plan", None)
     assert rc == 0, rc
     ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
     helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, "gated average")
