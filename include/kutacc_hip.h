@@ -89,6 +89,21 @@ typedef struct kutacc_hip_attention_args {
  * (reference src/attention/gating_attention.cpp:33-158). */
 kutacc_export int kutacc_hip_gating_attention(const kutacc_hip_attention_args_t *args, void *stream);
 
+/*
+ * kutacc_hip_gating_attention for callers that cannot allocate device memory or lend scratch: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The one
+ * scratch buffer of the MFMA kernels, a fragment-major copy of the pair bias, lives in a device array inside the
+ * library image (KUTACC_HIP_STATIC_SCRATCH_BYTES; each GPU the library runs on holds it until the process ends), so
+ * args->q, k, v and gate are neither read nor written and may be NULL.  Nothing on this path calls hipMalloc, hipFree
+ * or any allocating routine; per-kernel profiling events are not recorded for it.  Only shapes the MFMA kernels take
+ * (bf16, head_size 32, nheads*32 in {128, 256}, seq_len <= 1024): others return KUTACC_HIP_EUNSUPPORTED.  A pair bias
+ * whose copy, nheads * ceil(S/32) * 2*ceil(S/64) * 2048 bytes, exceeds the array is rejected with KUTACC_HIP_EINVAL
+ * and a line on stderr (16 MiB holds 8 heads at 1024 positions).  All calls on one GPU share the array, which keeps
+ * the last call's contents: every call rewrites the part it reads, and calls that overlap in time on one GPU race.
+ */
+#define KUTACC_HIP_STATIC_SCRATCH_BYTES (16u << 20)
+kutacc_export int kutacc_hip_gating_attention_static(const kutacc_hip_attention_args_t *args, void *stream);
+
 /* Global (extra-MSA column) attention, reference src/attention/global_attention.cpp:30-164 (kernel) and
  * :167-205 (entry).  One query per batch row and head (the masked mean of the row), one key/value head
  * shared by all heads.  bf16 storage, nheads*head_size == 64 (the reference hard-wires nchannels == 64,

@@ -2125,6 +2125,78 @@ int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const vo
 
 } // namespace kutacc_launch
 
+// ------------------------------------------------------------------------------------------------
+// Entry point that allocates nothing: the fragment-major copy of the pair bias -- the one scratch buffer of the fused
+// path, which kutacc_hip_gating_attention keeps in the caller's q tensor -- lives in a device array that is part of the
+// library image.  Every GPU the library runs on holds its own copy of the array, at its own address, until the process
+// ends; the address is asked for once per device and kept.
+// ------------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)KUTACC_HIP_STATIC_SCRATCH_BYTES;
+}
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+namespace {
+std::atomic<void *> g_scratch_ptr[KUTACC_DEVICE_SLOTS];
+
+// device address of `scratch` on the current device (the array's name is a host-side stand-in, never a device address)
+int static_scratch_address(void **out)
+{
+    const int slot = kutacc_device_slot();
+    if (slot < 0) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    void *ptr = g_scratch_ptr[slot].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            return e != hipSuccess ? (int)e : KUTACC_HIP_EUNSUPPORTED;
+        }
+        g_scratch_ptr[slot].store(ptr, std::memory_order_release); // every thread gets the same answer for a device
+    }
+    *out = ptr;
+    return 0;
+}
+} // namespace
+
+extern "C" kutacc_export int kutacc_hip_gating_attention_static(const kutacc_hip_attention_args_t *a, void *stream)
+{
+    if (!a || !a->input || !a->query_w || !a->key_w || !a->value_w || !a->gating_w || !a->output_w || !a->gating_b ||
+        !a->output_b || !a->bias || !a->out || !a->avg) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (a->batch <= 0 || a->seq_len <= 0 || a->nheads <= 0 || a->head_size <= 0 || a->batch > INT32_MAX / a->seq_len ||
+        a->nheads > INT32_MAX / a->head_size) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int64_t C = a->nheads * a->head_size;
+    if (a->input_ld < C || a->out_ld < C) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (!kutacc_launch::fused_attention_supports(*a)) {
+        return KUTACC_HIP_EUNSUPPORTED; // the shape-agnostic kernels need the caller's q, k, v and gate tensors
+    }
+    kutacc_launch::FusedAttentionOptions opt;
+    if (a->nonbatched_bias != nullptr) {
+        const int64_t need = fragment_bytes(a->nheads, (int)((a->seq_len + 31) / 32));
+        if ((uint64_t)need > STATIC_SCRATCH_BYTES) {
+            fprintf(stderr,
+                    "kutacc_hip_gating_attention_static: the pair bias of %lld heads x %lld positions needs %lld bytes of "
+                    "scratch, the library's static array holds %zu\n",
+                    (long long)a->nheads, (long long)a->seq_len, (long long)need, STATIC_SCRATCH_BYTES);
+            return KUTACC_HIP_EINVAL;
+        }
+        void *ptr = nullptr;
+        if (const int rc = static_scratch_address(&ptr)) {
+            return rc;
+        }
+        opt.fragment_workspace = ptr;
+        opt.fragment_workspace_bytes = STATIC_SCRATCH_BYTES;
+    }
+    kutacc_prof::Suppress no_events;
+    return kutacc_launch::gating_attention_fused(*a, stream ? (hipStream_t)stream : kutacc_api::default_stream(), opt);
+}
+
 // Tuning hooks for tests and experiments: "plan" = "bpw,gw" forces the long-sequence kernel with that many query blocks
 // per wave and weight matrices per group where it fits (anything else: the planner decides), "fragments" = "0" keeps the
 // kernels off the fragment-major pair bias (general attention blocks), "debug" = "1" prints the plan of every call.
