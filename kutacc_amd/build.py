@@ -63,5 +63,37 @@ def build(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+def host_cxx() -> str:
+    """ROCm's clang++: the public header uses __bf16, which g++ 11 does not know on x86."""
+    for exe in ("/opt/rocm/llvm/bin/clang++", shutil.which("amdclang++"), shutil.which("clang++")):
+        if exe and os.path.exists(exe):
+            return exe
+    raise RuntimeError("no clang++ found for the host-side test caller")
+
+
+REFERENCE_INCLUDE = "/root/reference/include"
+
+
+def build_dropin_callers() -> list:
+    """tests/cxx/dropin_caller.cpp as a small shared object linked against libkutacc.so, once per public header: this
+    repository's (libdropin_caller.so) and, where the reference tree is present, the reference's own include/kutacc.h
+    (libdropin_caller_ref.so) -- a caller compiled with the Kunpeng header, run against this library."""
+    src = os.path.join(ROOT, "tests", "cxx", "dropin_caller.cpp")
+    out_dir = os.path.dirname(src)
+    built = []
+    variants = [("libdropin_caller.so", os.path.join(ROOT, "include"))]
+    if os.path.exists(os.path.join(REFERENCE_INCLUDE, "kutacc.h")):
+        variants.append(("libdropin_caller_ref.so", REFERENCE_INCLUDE))
+    for name, inc in variants:
+        out = os.path.join(out_dir, name)
+        cmd = [host_cxx(), "-std=c++17", "-O1", "-fPIC", "-shared", "-Wall", "-D_GLIBCXX_USE_CXX11_ABI=1", "-I", inc, src,
+               "-o", out + ".tmp", "-L", LIB_DIR, "-lkutacc", "-Wl,-rpath,$ORIGIN/../../kutacc_amd/lib"]
+        subprocess.check_call(cmd)
+        os.replace(out + ".tmp", out)
+        built.append(out)
+    return built
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    print("\n".join(build_dropin_callers()))

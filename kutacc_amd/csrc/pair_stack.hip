@@ -263,10 +263,12 @@ __global__ __launch_bounds__(256, (A_MMAJOR && B_MMAJOR) ? 4 : 3) void pair_gemm
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int trow = 64 * wm + 32 * i + r; // row of the LDS tile
+        // gated form: rows 64-127 of the tile are the gate product, with its own bias and no ReLU
+        const bool gate_rows = GATED && wm == 1;
+        const float *bsrc = gate_rows ? (alt ? p.bias_gate_alt : p.bias_gate) : (alt ? p.bias_alt : p.bias);
         float row_bias = 0.f;
         if (p.bias_axis == 2) {
             const int gm = GATED ? m0 + 32 * i + r : m0 + trow;
-            const float *bsrc = (GATED && wm == 1) ? (alt ? p.bias_gate_alt : p.bias_gate) : (alt ? p.bias_alt : p.bias);
             row_bias = gm < p.M ? bsrc[gm] : 0.f;
         }
 #pragma unroll
@@ -276,13 +278,13 @@ __global__ __launch_bounds__(256, (A_MMAJOR && B_MMAJOR) ? 4 : 3) void pair_gemm
                 const int tcol = 64 * wn + 32 * j + 8 * q + 4 * g;
                 f32x4 bv = {row_bias, row_bias, row_bias, row_bias};
                 if (p.bias_axis == 1 && n0 + tcol + 4 <= p.N) {
-                    bv = *reinterpret_cast<const f32x4 *>(p.bias + n0 + tcol);
+                    bv = *reinterpret_cast<const f32x4 *>(bsrc + n0 + tcol);
                 }
                 bf16x4 ov;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     float x = acc[i][j][4 * q + c] + bv[c];
-                    if (p.relu) {
+                    if (p.relu && !gate_rows) {
                         x = fmaxf(x, 0.f);
                     }
                     ov[c] = (bf16_t)x;
@@ -1035,7 +1037,8 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
                    g.c_stride_m % 8 == 0 && g.c_stride_batch % 8 == 0 && g.n % 8 == 0 &&
                    (g.bias_axis != 1 || kutacc_hip_aligned16(g.bias));
     if (gated) {
-        mfma_ok = mfma_ok && !am && !bm && kutacc_hip_aligned16(g.a_gate) && kutacc_hip_aligned16(g.mask) && g.mask_stride_batch % 8 == 0;
+        mfma_ok = mfma_ok && !am && !bm && kutacc_hip_aligned16(g.a_gate) && kutacc_hip_aligned16(g.mask) && g.mask_stride_batch % 8 == 0 &&
+                  (g.bias_axis != 1 || kutacc_hip_aligned16(g.bias_gate));
     }
     if (g.path == KUTACC_HIP_PATH_GENERIC) {
         mfma_ok = false;
@@ -1054,7 +1057,8 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
                           h.mask == g.mask && h.a_stride_m == g.a_stride_m && h.a_stride_k == g.a_stride_k &&
                           h.b_stride_n == g.b_stride_n && h.b_stride_k == g.b_stride_k && h.c_stride_m == g.c_stride_m &&
                           h.bias_axis == g.bias_axis && h.relu == g.relu && h.dtype == g.dtype && h.a && h.c &&
-                          (g.bias_axis == 0 || (h.bias && h.bias_gate)) && kutacc_hip_aligned16(h.a) &&
+                          (g.bias_axis == 0 || (h.bias && h.bias_gate)) &&
+                          (g.bias_axis != 1 || (kutacc_hip_aligned16(h.bias) && kutacc_hip_aligned16(h.bias_gate))) && kutacc_hip_aligned16(h.a) &&
                           kutacc_hip_aligned16(h.a_gate) && kutacc_hip_aligned16(h.c);
         const bool streaming = gated && gated_projection_fits(g) && gated_projection_fits(h) && g.n <= INT32_MAX / 2 &&
                                g.n >= GATED_STREAMING_MIN_POSITIONS;

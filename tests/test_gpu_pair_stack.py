@@ -120,6 +120,45 @@ def test_gemm_m_major_operands(torch_cuda, shape, a_mmajor, b_mmajor):
     helpers.assert_within(got, same, 1e-3 + 8e-3 * np.abs(same), "mfma vs scalar kernel")
 
 
+@pytest.mark.parametrize("bias_axis,relu", [(1, False), (1, True), (2, False), (2, True), (0, False)])
+@pytest.mark.parametrize("path", [capi.PATH_FUSED, capi.PATH_GENERIC], ids=["mfma", "scalar"])
+def test_gemm_gated_form_bias_axes(torch_cuda, path, bias_axis, relu):
+    """The gated form C = bf16(bf16(relu?(A.B^T + bias)) * mask[n] * sigmoid(bf16(A_gate.B^T + bias_gate))) with the biases
+    along either axis: each product takes its own bias, and ReLU applies to the projection only.  Against float64 with the
+    same two intermediate roundings."""
+    torch = torch_cuda
+    nb, M, N, K = 2, 136, 200, 96
+    rng = np.random.Generator(np.random.PCG64(31 + bias_axis))
+    A, G = draw(rng, nb, M, K), draw(rng, nb, M, K)
+    B = draw(rng, nb, N, K, scale=1 / math.sqrt(K))
+    mask = (rng.random((nb, N)) > 0.2).astype(np.float32)
+    blen = N if bias_axis == 1 else M
+    bias, bias_gate = (rng.standard_normal(blen).astype(np.float32) for _ in range(2))
+    dA, dG, dB, dmask = dev(torch, A), dev(torch, G), dev(torch, B), dev(torch, mask)
+    dC = torch.full((nb, M, N), -7.0, dtype=torch.bfloat16, device="cuda")
+    g = capi.HipGemmArgs()
+    g.m, g.n, g.k, g.batches, g.dtype, g.path = M, N, K, nb, capi.K_BF16, path
+    g.a, g.a_gate, g.a_stride_m, g.a_stride_k, g.a_stride_batch = dA.data_ptr(), dG.data_ptr(), K, 1, M * K
+    g.b, g.b_stride_n, g.b_stride_k, g.b_stride_batch = dB.data_ptr(), K, 1, N * K
+    g.c, g.c_stride_m, g.c_stride_batch = dC.data_ptr(), N, M * N
+    g.mask, g.mask_stride_batch = dmask.data_ptr(), N
+    keep = [dev(torch, bias, torch.float32), dev(torch, bias_gate, torch.float32)]
+    if bias_axis:
+        g.bias, g.bias_gate, g.bias_axis = keep[0].data_ptr(), keep[1].data_ptr(), bias_axis
+    g.relu = 1 if relu else 0
+    rc = capi.lib().kutacc_hip_gemm(ctypes.byref(g), None)
+    torch.cuda.synchronize()
+    assert rc == 0, rc
+    A, G, B = (round_to_bf16(v) for v in (A, G, B))
+    proj = gemm_ref(A, B, bias, bias_axis, relu)
+    gate = gemm_ref(G, B, bias_gate, bias_axis, False)
+    proj, gate = round_to_bf16(proj.astype(np.float32)).astype(np.float64), round_to_bf16(gate.astype(np.float32)).astype(np.float64)
+    ref = proj * mask[:, None, :] / (1.0 + np.exp(-gate))
+    got = helpers.to_numpy(dC)
+    helpers.assert_within(got, ref, 2e-3 + 1.2e-2 * np.abs(ref), f"gated gemm, bias axis {bias_axis}, relu {relu}")
+    assert np.all(got[np.broadcast_to(mask[:, None, :] == 0, got.shape)] == 0), "masked positions must be exactly zero"
+
+
 def _gemm_sweep():
     rng = np.random.Generator(np.random.PCG64(777))
     cases = []
