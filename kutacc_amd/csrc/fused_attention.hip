@@ -1036,7 +1036,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
 // on the next row's loads and projections while the slower waves of its SIMD still attend, so the
 // latency- and MFMA-bound projection phase overlaps the VALU-heavy attention phase.
 // ------------------------------------------------------------------------------------------------
-template <int C, bool HAS_NB>
+template <int C, bool HAS_NB, bool L2MODE>
 __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(FusedParams p)
 {
     constexpr int CK = C / 16;
@@ -1088,9 +1088,8 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 
     TL(8);
     const int j = wave; // this wave's sequence block
-    const float qmul = p.l2mode ? p.qscale * LOG2E : p.qscale;
-    // uniform, and kept in a scalar register
-    const float mask_scale = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(p.l2mode ? LOG2E : 1.0f)));
+    const float qmul = L2MODE ? p.qscale * LOG2E : p.qscale;
+    const float mask_scale = L2MODE ? LOG2E : 1.0f;
     const bf16x8 sumsel = rowsum_selector(lane);
     for (int n = 0; n < nrows; ++n) {
         const int b = b0 + n * bstep;
@@ -1214,7 +1213,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         float l;
         const uint32_t flags = *flag_word;
         const bf16_t *nb_head = HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr;
-        if (p.l2mode) {
+        if constexpr (L2MODE) {
             const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NT * 2) * 64 + lane : nullptr;
             if (flags == 0u) {
                 attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o,
@@ -1861,10 +1860,10 @@ int launch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t stream)
     return kutacc_hip_status(hipGetLastError());
 }
 
-template <int C, bool HAS_NB>
+template <int C, bool HAS_NB, bool L2MODE>
 int launch_persistent_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
 {
-    auto kern = persistent_head_kernel<C, HAS_NB>;
+    auto kern = persistent_head_kernel<C, HAS_NB, L2MODE>;
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
     if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
         return rc;
@@ -1885,7 +1884,10 @@ int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t strea
 {
     const bool nb = p.nb != nullptr;
     if (pl.persistent) {
-        return nb ? launch_persistent_kernel<C, true>(p, pl, stream) : launch_persistent_kernel<C, false>(p, pl, stream);
+        if (p.l2mode) {
+            return nb ? launch_persistent_kernel<C, true, true>(p, pl, stream) : launch_persistent_kernel<C, false, true>(p, pl, stream);
+        }
+        return nb ? launch_persistent_kernel<C, true, false>(p, pl, stream) : launch_persistent_kernel<C, false, false>(p, pl, stream);
     }
     switch (pl.BPW) {
         case 1: return nb ? launch_head_kernel<C, 1, true>(p, pl, stream) : launch_head_kernel<C, 1, false>(p, pl, stream);
