@@ -469,6 +469,10 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
     if (HAS_NB) {
         wa0 = nbf[0], wa1 = nbf[64];
         wb0 = nbf[2 * 64], wb1 = nbf[3 * 64];
+        // Pinned in this order, ahead of the reload of wa below: the loop then finds the loads in flight in the order it
+        // leaves them in itself (odd tile's words older than the even tile's), and its wait at the top lets the two
+        // newest stay in flight instead of draining the queue.
+        __builtin_amdgcn_sched_barrier(0);
     }
     k0 = kp[0], k1 = kp[64];
     f32x16 xa = init(0), xb;
