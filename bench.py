@@ -26,12 +26,20 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (two runs, scaled against a 256 MiB copy: FETCH x2.000, WRITE x1.000; see
-# profiles/gating_attention_cfg3_hbm_traffic.txt).  Not re-measured live; configurations without an entry report null.
-MEASURED_TRAFFIC_BYTES = {
-    (3, "persistent_head_kernel"): int((23782.8 * 2.0 + 41472.0) * 1024),
-}
+# HBM bytes per launch of each kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command, each
+# counter scaled by what it reads for a 256 MiB copy (profiles/gating_attention_hbm_traffic.txt says how): the file maps
+# "config N" -> kernel name -> bytes.  Not re-measured live; a kernel or configuration without an entry reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(config, kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    v = table.get(f"config {config}", {}).get(kernel)
+    return int(v) if v is not None else None
 
 
 def cpu_baseline(w, budget_s=15.0):
@@ -352,8 +360,14 @@ def main():
     ms = wall / a.steps * 1e3
     tflops = w.flops() / (ms * 1e-3) / 1e12
 
-    # per-kernel durations: same K calls again with hipEvents recorded around each kernel on the stream
+    # per-kernel durations: same K calls again with hipEvents recorded around each kernel on the stream (a few
+    # bracketed calls first, not counted: the first event pairs of a process are slow to create and resolve)
     L.kutacc_hip_profile_enable(1)
+    for _ in range(max(3, min(a.warmup, 10))):
+        op.run()
+    torch.cuda.synchronize()
+    L.kutacc_hip_profile_enable(0)
+    L.kutacc_hip_profile_enable(1)  # enabling clears the totals
     for _ in range(a.steps):
         op.run()
     torch.cuda.synchronize()
@@ -372,7 +386,7 @@ def main():
         ach = dom["flops_per_launch"] / (dom["avg_ms"] * 1e-3) / 1e12
         roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((w.config, dom["name"])),
+                    "traffic": measured_traffic(w.config, dom["name"]),
                     "avg_kernel_ms": round(dom["avg_ms"], 5),
                     "flops_per_launch": dom["flops_per_launch"]}
 

@@ -400,13 +400,19 @@ kutacc_export int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t
 /* ---- runtime control (no counterpart in the reference; the CPU library has no device) ---- */
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.
- * Default: the HIP null stream. */
+ * Default: the HIP null stream.  The setting belongs to the calling host thread (like a framework's current
+ * stream): threads that drive the library on different streams each set their own. */
 kutacc_export void kutacc_hip_set_stream(void *stream);
 kutacc_export void *kutacc_hip_get_stream(void);
 
 /* 1 (default): the handle-based API blocks until the device work has finished, as the CPU library
- * does.  0: it returns after enqueueing when all operands are device pointers. */
+ * does.  0: it returns after enqueueing when all operands are device pointers.  Per host thread, like the stream. */
 kutacc_export void kutacc_hip_set_blocking(int blocking);
+
+/* Calls on host pointers run on device copies of their operands; those copies are kept between calls (a repeated
+ * shape allocates once).  This frees them and returns the number of bytes released.  Call it when no such call is
+ * in flight. */
+kutacc_export int64_t kutacc_hip_release_staging(void);
 
 /* Per-kernel timing for benchmarks.  While enabled, each kernel launched by this library is
  * bracketed by hipEvents on its stream.  kutacc_hip_profile_read(i, ...) waits for the recorded
@@ -421,7 +427,10 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *   "plan"      "bpw,gw": force the long-sequence attention kernel with bpw (1-4) query blocks per wave and gw (1, 2, 4)
  *               weight matrices per LDS group where that fits the device; anything else: the planner decides (default)
  *   "fragments" "0": keep the attention kernels off the fragment-major pair bias (general softmax blocks); "1": default
- *   "debug"     "1": one line per fused call on stderr with the plan taken; "0": default */
+ *   "debug"     "1": one line per fused call on stderr with the plan taken; "0": default
+ *   "pointer_checks" "0": the handle-based attention entry points classify only `input` (host or device) and take the
+ *               caller's word that every other operand lives in the same place, which saves about fifteen driver
+ *               queries per call; "1": every operand is checked and mixed calls are rejected (default) */
 kutacc_export int kutacc_hip_set_tuning(const char *name, const char *value);
 
 /* The process-wide sticky error flag behind KUTACC_CHECK (reference src/utils/check.cpp:16 keeps it

@@ -168,7 +168,7 @@ DECLARED_SYMBOLS = [
     "kutacc_hip_pair_bias", "kutacc_hip_set_stream", "kutacc_hip_get_stream", "kutacc_hip_set_blocking",
     "kutacc_hip_error_flag", "kutacc_hip_clear_error", "kutacc_hip_tensor_create", "kutacc_hip_tensor_destroy",
     "kutacc_hip_profile_enable", "kutacc_hip_profile_read", "kutacc_hip_set_tuning",
-    "kutacc_hip_gating_attention_static",
+    "kutacc_hip_gating_attention_static", "kutacc_hip_release_staging",
 ]
 
 _lib = None
@@ -280,6 +280,7 @@ def lib() -> ctypes.CDLL:
     L.kutacc_hip_profile_read.restype = ctypes.c_int
     L.kutacc_hip_gating_attention_static.argtypes = [ctypes.POINTER(HipAttentionArgs), _vp]
     L.kutacc_hip_gating_attention_static.restype = ctypes.c_int
+    L.kutacc_hip_release_staging.restype = _i64
     L.kutacc_hip_set_tuning.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
     L.kutacc_hip_set_tuning.restype = ctypes.c_int
     _lib = L

@@ -5,11 +5,13 @@
 // reference src/linear/mm.cpp:23-35,80-82 (shape / stride / dtype checks of the GEMM operands).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <climits>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <iostream>
+#include <mutex>
 #include <vector>
 
 #include "check.h"
@@ -45,9 +47,13 @@ const kutacc_version_t k_version = {
     "Kunpeng HPCKit", "26.1.RC1", "KuTACC", "26.1.RC1", "1", "hip-gfx950",
 };
 
-hipStream_t g_stream = nullptr;
-bool g_blocking = true;
+// Stream and blocking mode belong to the calling host thread (as a framework's "current stream" does): two threads
+// that drive the library on different streams do not see each other's settings.
+thread_local hipStream_t g_stream = nullptr;
+thread_local bool g_blocking = true;
 thread_local const char *t_last_path = "none";
+// 0: the handle-based entry points take the caller's word that all operands of a call live where `input` lives
+std::atomic<int> g_pointer_checks{1};
 
 inline hipStream_t pick_stream(void *s) { return s ? (hipStream_t)s : g_stream; }
 
@@ -74,8 +80,57 @@ struct Mirror {
     bool copy_back = false;
 };
 
+// Device buffers of the staged path are kept between calls: a call takes what it needs from the pool (smallest buffer
+// that is large enough, else a new allocation) and gives everything back when it is done, so a caller that repeats a
+// shape pays hipMalloc once.  kutacc_hip_release_staging() frees the pool.
+struct StagingPool {
+    struct Block {
+        void *dev;
+        size_t bytes;
+    };
+    std::mutex mu;
+    std::vector<Block> free_blocks;
+    hipError_t take(size_t bytes, void **out, size_t *got)
+    {
+        {
+            std::lock_guard<std::mutex> lk(mu);
+            int best = -1;
+            for (int i = 0; i < (int)free_blocks.size(); ++i) {
+                if (free_blocks[i].bytes >= bytes && (best < 0 || free_blocks[i].bytes < free_blocks[best].bytes)) {
+                    best = i;
+                }
+            }
+            if (best >= 0) {
+                *out = free_blocks[best].dev, *got = free_blocks[best].bytes;
+                free_blocks.erase(free_blocks.begin() + best);
+                return hipSuccess;
+            }
+        }
+        *got = bytes;
+        return hipMalloc(out, bytes);
+    }
+    void give(void *dev, size_t bytes)
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        free_blocks.push_back({dev, bytes});
+    }
+    size_t release()
+    {
+        std::lock_guard<std::mutex> lk(mu);
+        size_t total = 0;
+        for (auto &b : free_blocks) {
+            total += b.bytes;
+            (void)hipFree(b.dev);
+        }
+        free_blocks.clear();
+        return total;
+    }
+};
+StagingPool g_staging;
+
 struct Stager {
     std::vector<Mirror> items;
+    std::vector<size_t> capacity; // what the pool gave for each item
     hipStream_t stream;
     int rc = 0;
     explicit Stager(hipStream_t s) : stream(s) {}
@@ -89,18 +144,20 @@ struct Stager {
         }
         Mirror m;
         m.host = host, m.bytes = bytes, m.copy_back = back;
-        hipError_t e = hipMalloc(&m.dev, bytes);
+        size_t got = 0;
+        hipError_t e = g_staging.take(bytes, &m.dev, &got);
         if (e == hipSuccess && upload && host) {
             e = hipMemcpyAsync(m.dev, host, bytes, hipMemcpyHostToDevice, stream);
         }
         if (e != hipSuccess) {
             rc = (int)e;
             if (m.dev) {
-                (void)hipFree(m.dev);
+                g_staging.give(m.dev, got);
             }
             return nullptr;
         }
         items.push_back(m);
+        capacity.push_back(got);
         return m.dev;
     }
     int finish()
@@ -117,10 +174,11 @@ struct Stager {
         if (rc == 0 && e != hipSuccess) {
             rc = (int)e;
         }
-        for (auto &m : items) {
-            (void)hipFree(m.dev);
+        for (size_t i = 0; i < items.size(); ++i) {
+            g_staging.give(items[i].dev, capacity[i]);
         }
         items.clear();
+        capacity.clear();
         return rc;
     }
 };
@@ -179,6 +237,24 @@ void kutacc_hip_tensor_destroy(void *handle) { delete static_cast<kutacc::Tensor
 // ---------------------------------------------------------------------------------------------
 // runtime control
 // ---------------------------------------------------------------------------------------------
+int64_t kutacc_hip_release_staging(void) { return (int64_t)g_staging.release(); }
+
+// the hooks of the attention launcher live with it; "pointer_checks" belongs to the entry points here
+namespace kutacc_launch {
+int fused_attention_tuning(const char *name, const char *value);
+}
+int kutacc_hip_set_tuning(const char *name, const char *value)
+{
+    if (!name) {
+        return KUTACC_HIP_EINVAL;
+    }
+    if (!std::strcmp(name, "pointer_checks")) {
+        g_pointer_checks.store((value && value[0] == '0') ? 0 : 1);
+        return 0;
+    }
+    return kutacc_launch::fused_attention_tuning(name, value);
+}
+
 void kutacc_hip_set_stream(void *stream) { g_stream = (hipStream_t)stream; }
 void *kutacc_hip_get_stream(void) { return (void *)g_stream; }
 void kutacc_hip_set_blocking(int blocking) { g_blocking = blocking != 0; }
@@ -365,8 +441,10 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
     const Space sp = space_of(in.data);
     const void *all_ptrs[] = {bs.data, ot.data, q.data, k.data, v.data, gt.data, av.data, wq.data,
                               wk.data, wv.data, wg.data, bg.data, wo.data, bo.data, has_nb ? nb.data : in.data};
-    for (const void *p : all_ptrs) {
-        KUTACC_CHECK(space_of(p) == sp, "kutacc_af2_gating_attention: host and device pointers mixed in one call");
+    if (g_pointer_checks.load(std::memory_order_relaxed)) {
+        for (const void *p : all_ptrs) {
+            KUTACC_CHECK(space_of(p) == sp, "kutacc_af2_gating_attention: host and device pointers mixed in one call");
+        }
     }
     if (KUTACC_FAILED()) {
         return;
@@ -492,8 +570,10 @@ void kutacc_af2_global_attention(kutacc_af2_attention_inputs_t *q_based_ptr, kut
     hipStream_t s = g_stream;
     const Space sp = space_of(x.data);
     const void *all_ptrs[] = {mk.data, ot.data, qa.data, wq.data, wk.data, wv.data, wg.data, bg.data, wo.data, bo.data};
-    for (const void *ptr : all_ptrs) {
-        KUTACC_CHECK(space_of(ptr) == sp, "kutacc_af2_global_attention: host and device pointers mixed in one call");
+    if (g_pointer_checks.load(std::memory_order_relaxed)) {
+        for (const void *ptr : all_ptrs) {
+            KUTACC_CHECK(space_of(ptr) == sp, "kutacc_af2_global_attention: host and device pointers mixed in one call");
+        }
     }
     if (KUTACC_FAILED()) {
         return;

@@ -2206,11 +2206,8 @@ extern "C" kutacc_export int kutacc_hip_gating_attention_static(const kutacc_hip
 // Tuning hooks for tests and experiments: "plan" = "bpw,gw" forces the long-sequence kernel with that many query blocks
 // per wave and weight matrices per group where it fits (anything else: the planner decides), "fragments" = "0" keeps the
 // kernels off the fragment-major pair bias (general attention blocks), "debug" = "1" prints the plan of every call.
-extern "C" kutacc_export int kutacc_hip_set_tuning(const char *name, const char *value)
+int kutacc_launch::fused_attention_tuning(const char *name, const char *value)
 {
-    if (!name) {
-        return KUTACC_HIP_EINVAL;
-    }
     const bool on = value && value[0] != '\0' && value[0] != '0';
     if (!strcmp(name, "plan")) {
         int bpw = 0, gw = 0;

@@ -94,6 +94,9 @@ bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &args, in
 int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream,
                            const FusedAttentionOptions &opt = FusedAttentionOptions());
 
+// "plan" / "fragments" / "debug" hooks of the attention launcher (kutacc_hip_set_tuning); KUTACC_HIP_EINVAL for other names
+int fused_attention_tuning(const char *name, const char *value);
+
 bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
                              int64_t m, int64_t n, int64_t k);
 int row_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld, int64_t m,

@@ -338,6 +338,30 @@ def test_host_pointers_are_staged_and_match_device_pointers(torch_cuda):
     np.testing.assert_array_equal(hten["out"], dev_bits)
     avg_bits = scratch["avg"].view(torch_cuda.int16).cpu().numpy().view(np.uint16)
     np.testing.assert_array_equal(hscratch["avg"], avg_bits)
+    # the device copies are kept between calls: a second call (buffers reused, whatever they held) gives the same bits,
+    # and releasing the pool reports what it held
+    hten["out"][:] = 0
+    hop.run()
+    assert not capi.error_flag()
+    np.testing.assert_array_equal(hten["out"], dev_bits)
+    assert capi.lib().kutacc_hip_release_staging() > 0
+    assert capi.lib().kutacc_hip_release_staging() == 0
+
+
+def test_pointer_checks_can_be_switched_off(torch_cuda):
+    """With "pointer_checks" off the entry point classifies `input` only; results on device memory are unchanged."""
+    w = make_workload(3, batch=3, seq_len=96)
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    want = ten["out"].clone()
+    ten["out"].zero_()
+    assert capi.set_tuning("pointer_checks", "0") == 0
+    try:
+        op.run()
+    finally:
+        capi.set_tuning("pointer_checks", "1")
+    assert not capi.error_flag() and helpers.same_bits(ten["out"], want)
+    assert capi.set_tuning("no such hook", "1") == capi.EINVAL
 
 
 def test_mixed_host_and_device_pointers_are_rejected(torch_cuda):
