@@ -428,6 +428,11 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *               weight matrices per LDS group where that fits the device; anything else: the planner decides (default)
  *   "fragments" "0": keep the attention kernels off the fragment-major pair bias (general softmax blocks); "1": default
  *   "debug"     "1": one line per fused call on stderr with the plan taken; "0": default
+ *   "layernorm" "fused": kutacc_hip_triangle_attention and kutacc_hip_msa_attention let the attention kernel normalise its
+ *               input rows itself where it can (sequence lengths of the persistent kernel), which drops the normalised
+ *               copy from the workspace and costs 8-15 % of the block's time; "separate" or "auto" (default): the
+ *               LayerNorm runs as a pass of its own.  The workspace functions answer for the mode in force when they are
+ *               called: query and call under the same setting.
  *   "pointer_checks" "0": the handle-based attention entry points classify only `input` (host or device) and take the
  *               caller's word that every other operand lives in the same place, which saves about fifteen driver
  *               queries per call; "1": every operand is checked and mixed calls are rejected (default) */

@@ -54,6 +54,7 @@ thread_local bool g_blocking = true;
 thread_local const char *t_last_path = "none";
 // 0: the handle-based entry points take the caller's word that all operands of a call live where `input` lives
 std::atomic<int> g_pointer_checks{1};
+std::atomic<int> g_block_layernorm{0};
 
 inline hipStream_t pick_stream(void *s) { return s ? (hipStream_t)s : g_stream; }
 
@@ -252,6 +253,10 @@ int kutacc_hip_set_tuning(const char *name, const char *value)
         g_pointer_checks.store((value && value[0] == '0') ? 0 : 1);
         return 0;
     }
+    if (!std::strcmp(name, "layernorm")) {
+        g_block_layernorm.store(value && !std::strcmp(value, "fused") ? 1 : (value && !std::strcmp(value, "separate") ? 2 : 0));
+        return 0;
+    }
     return kutacc_launch::fused_attention_tuning(name, value);
 }
 
@@ -346,6 +351,7 @@ hipStream_t default_stream() { return g_stream; }
 hipStream_t stream_or_default(void *s) { return pick_stream(s); }
 bool on_device(const void *p) { return space_of(p) == Space::Device; }
 int finish(int rc, hipStream_t s) { return finish_device_call(rc, s); }
+int block_layernorm_mode() { return g_block_layernorm.load(std::memory_order_relaxed); }
 } // namespace kutacc_api
 
 void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inputs_t *q_based_ptr, kutacc_tensor_h bias,

@@ -26,17 +26,74 @@ struct Workspace {
     int64_t z_norm, nb, bias, q, avg, total; // byte offsets
 };
 
-Workspace layout(int64_t n, int64_t heads)
+// fused_ln: the head kernel normalises the rows of the pair tensor itself, so no normalised copy is kept
+Workspace layout(int64_t n, int64_t heads, bool fused_ln)
 {
     const int64_t c = heads * HEAD, act = align256(n * n * c * 2);
     Workspace w;
     w.z_norm = 0;
-    w.nb = w.z_norm + act;
+    w.nb = w.z_norm + (fused_ln ? 0 : act);
     w.bias = w.nb + align256(heads * n * n * 2);
     w.q = w.bias + align256(n * n * 2);
     w.avg = w.q + act;
     w.total = w.avg + act;
     return w;
+}
+// Argument block of the attention call inside the triangle-attention block, on a workspace laid out by layout();
+// `ws` may be a null base when only the plan is of interest (the offsets are then the pointers).
+kutacc_hip_attention_args_t triangle_attention_call(const kutacc_hip_triangle_attention_args_t *a, char *ws, const Workspace &w,
+                                                    bool fused_ln)
+{
+    const int64_t n = a->n_res, heads = a->nheads, c = heads * HEAD;
+    const bool ending = a->ending_node != 0;
+    kutacc_hip_attention_args_t g;
+    std::memset(&g, 0, sizeof(g));
+    g.batch = n, g.seq_len = n, g.nheads = heads, g.head_size = HEAD;
+    g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_FUSED;
+    if (fused_ln) {
+        // the un-normalised pair tensor itself: row (b, s) of the attention's input is row (s, b) of it for the ending node
+        g.input = a->pair_act, g.input_ld = ending ? n * c : c;
+    } else {
+        g.input = ws + w.z_norm, g.input_ld = c;
+    }
+    g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
+    g.gating_b = a->gating_b, g.output_b = a->output_b;
+    g.bias = a->pair_mask, g.bias_stride_b = ending ? 1 : n;
+    g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n * n, g.nb_stride_q = n;
+    g.q = ws + w.q, g.q_stride_b = n * c, g.q_stride_s = c, g.q_stride_h = HEAD;
+    g.avg = ws + w.avg, g.avg_stride_b = n * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
+    g.out = a->pair_act, g.out_ld = c;
+    return g;
+}
+
+// Whether the block at this size lets the head kernel do the LayerNorm: asked with stand-in pointers (only sizes,
+// strides and alignment matter to the plan).
+// The policy both blocks share.  Inside the head kernel the LayerNorm is repeated by every head's workgroup and sits on
+// the kernel's critical path (the projection phase of the wave that finishes its attention last, which is latency bound);
+// against that stands one write and one read of the normalised activation, a pass the memory system does in 6-15 us.
+// Measured on one MI355X the fused form is slower at both block shapes (triangle attention, 384 residues x 128
+// channels: 133-140 against 119 us; MSA row-wise, 512 x 256 x 256 channels: 238 against 221 us), so the separate pass is
+// the default and the fused form is for callers who want the workspace without the normalised copy.
+bool layernorm_policy_allows(int64_t)
+{
+    return kutacc_api::block_layernorm_mode() == 1;
+}
+
+bool triangle_block_fuses_layernorm(int64_t n, int64_t heads)
+{
+    if (!layernorm_policy_allows(heads * HEAD)) {
+        return false;
+    }
+    kutacc_hip_triangle_attention_args_t a;
+    std::memset(&a, 0, sizeof(a));
+    char *fake = reinterpret_cast<char *>(uintptr_t(1) << 20);
+    a.n_res = n, a.nheads = heads, a.dtype = KUTACC_DTYPE_BF16;
+    a.pair_act = fake, a.pair_mask = fake;
+    a.query_w = a.key_w = a.value_w = a.gating_w = a.output_w = fake;
+    a.gating_b = a.output_b = reinterpret_cast<const float *>(fake);
+    const Workspace w = layout(n, heads, true);
+    const kutacc_hip_attention_args_t g = triangle_attention_call(&a, fake, w, true);
+    return kutacc_launch::fused_layernorm_supported(g, kutacc_launch::FusedAttentionOptions());
 }
 } // namespace
 
@@ -71,7 +128,7 @@ int64_t kutacc_hip_triangle_attention_workspace(int64_t n_res, int64_t nheads)
     if (n_res <= 0 || nheads <= 0 || n_res > 65536 || nheads > 64) {
         return -1;
     }
-    return layout(n_res, nheads).total;
+    return layout(n_res, nheads, triangle_block_fuses_layernorm(n_res, nheads)).total;
 }
 
 int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a, void *stream)
@@ -84,7 +141,11 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
         return KUTACC_HIP_EINVAL;
     }
     const int64_t n = a->n_res, heads = a->nheads, c = heads * HEAD;
-    const Workspace w = layout(n, heads);
+    // Where the persistent head kernel takes the call, it normalises the rows of the pair tensor itself (LayerNorm is
+    // then the first link of the fused chain, and the workspace holds no normalised copy); elsewhere the producer below
+    // writes one.
+    const bool fused_ln = triangle_block_fuses_layernorm(n, heads);
+    const Workspace w = layout(n, heads, fused_ln);
     if (a->workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
         return KUTACC_HIP_EINVAL;
     }
@@ -92,28 +153,18 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     hipStream_t s = kutacc_api::stream_or_default(stream);
     const int ending = a->ending_node != 0;
 
-    kutacc_hip_attention_args_t g;
-    std::memset(&g, 0, sizeof(g));
-    g.batch = n, g.seq_len = n, g.nheads = heads, g.head_size = HEAD;
-    g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_FUSED;
-    g.input = ws + w.z_norm, g.input_ld = c;
-    g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
-    g.gating_b = a->gating_b, g.output_b = a->output_b;
-    g.bias = a->pair_mask, g.bias_stride_b = ending ? 1 : n;
-    g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n * n, g.nb_stride_q = n;
-    g.q = ws + w.q, g.q_stride_b = n * c, g.q_stride_s = c, g.q_stride_h = HEAD;
-    g.avg = ws + w.avg, g.avg_stride_b = n * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
-    g.out = a->pair_act, g.out_ld = c;
+    const kutacc_hip_attention_args_t g = triangle_attention_call(a, ws, w, fused_ln);
     if (!kutacc_launch::fused_attention_supports(g)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
     // 1. LayerNorm + pair-bias projection in one pass over the pair tensor; the ending node reads it transposed
     //    -- and, where the grid allows it, writes the fragment-major copy the attention kernels read as well
+    void *z_norm = fused_ln ? nullptr : ws + w.z_norm;
     int frag_nb = 0, frag_nt = 0;
     const bool fragments = kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt) &&
-                           kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, ws + w.z_norm, n, n, c, heads,
+                           kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, z_norm, n, n, c, heads,
                                                                      KUTACC_DTYPE_BF16);
-    int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, ws + w.z_norm, n, n, c, heads,
+    int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, z_norm, n, n, c, heads,
                                       a->ln_eps, KUTACC_DTYPE_BF16, ending, s, fragments ? g.q : nullptr, frag_nb, frag_nt);
     if (rc != 0) {
         return rc;
@@ -125,6 +176,10 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     opt.bias_is_mask = true; // element (b, k) of the mask bias comes from mask[b, k], or mask[k, b] for the ending node
     opt.bias_stride_k = ending ? n : 1;
     opt.nb_fragments_ready = fragments;
+    if (fused_ln) {
+        opt.ln_gamma = a->ln_gamma, opt.ln_beta = a->ln_beta, opt.ln_eps = a->ln_eps;
+        opt.input_stride_b = ending ? c : n * c;
+    }
     return kutacc_launch::gating_attention_fused(g, s, opt);
 }
 
@@ -327,17 +382,65 @@ struct MsaWorkspace {
     int64_t m_norm, nb, bias, q, avg, total;
 };
 
-MsaWorkspace msa_layout(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
+// fused_ln: the head kernel normalises the msa rows itself, so no normalised copy is kept
+MsaWorkspace msa_layout(int64_t n_seq, int64_t n_res, int64_t heads, bool column, bool fused_ln)
 {
     const int64_t act = align256(n_seq * n_res * heads * HEAD * 2);
     MsaWorkspace w;
     w.m_norm = 0;
-    w.nb = w.m_norm + act;
+    w.nb = w.m_norm + (fused_ln ? 0 : act);
     w.bias = w.nb + (column ? 0 : align256(heads * n_res * n_res * 2));
     w.q = w.bias + align256(n_seq * n_res * 2);
     w.avg = w.q + act;
     w.total = w.avg + act;
     return w;
+}
+// Argument block of the attention call inside the MSA attention block (see triangle_attention_call)
+kutacc_hip_attention_args_t msa_attention_call(const kutacc_hip_msa_attention_args_t *a, char *ws, const MsaWorkspace &w,
+                                               bool fused_ln)
+{
+    const bool column = a->column != 0;
+    const int64_t n_seq = a->n_seq, n_res = a->n_res, heads = a->nheads, c = heads * HEAD;
+    // row-wise: every sequence attends over the residues; column-wise: every residue attends over the sequences,
+    // i.e. the same operator on the msa with its two leading axes exchanged
+    const int64_t batch = column ? n_res : n_seq, seq = column ? n_seq : n_res;
+    kutacc_hip_attention_args_t g;
+    std::memset(&g, 0, sizeof(g));
+    g.batch = batch, g.seq_len = seq, g.nheads = heads, g.head_size = HEAD;
+    g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_FUSED;
+    if (fused_ln) {
+        // the un-normalised msa itself; column-wise, row (b, s) of the attention's input is row (s, b) of it
+        g.input = a->msa_act, g.input_ld = column ? n_res * c : c;
+    } else {
+        g.input = ws + w.m_norm, g.input_ld = c;
+    }
+    g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
+    g.gating_b = a->gating_b, g.output_b = a->output_b;
+    g.bias = a->msa_mask, g.bias_stride_b = column ? 1 : n_res;
+    if (!column) {
+        g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n_res * n_res, g.nb_stride_q = n_res;
+    }
+    g.q = ws + w.q, g.q_stride_b = seq * c, g.q_stride_s = c, g.q_stride_h = HEAD;
+    g.avg = ws + w.avg, g.avg_stride_b = seq * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
+    g.out = a->msa_act, g.out_ld = c;
+    return g;
+}
+
+bool msa_block_fuses_layernorm(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
+{
+    if (!layernorm_policy_allows(heads * HEAD)) {
+        return false;
+    }
+    kutacc_hip_msa_attention_args_t a;
+    std::memset(&a, 0, sizeof(a));
+    char *fake = reinterpret_cast<char *>(uintptr_t(1) << 20);
+    a.n_seq = n_seq, a.n_res = n_res, a.nheads = heads, a.dtype = KUTACC_DTYPE_BF16, a.column = column ? 1 : 0;
+    a.msa_act = fake, a.msa_mask = fake;
+    a.query_w = a.key_w = a.value_w = a.gating_w = a.output_w = fake;
+    a.gating_b = a.output_b = reinterpret_cast<const float *>(fake);
+    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column, true);
+    const kutacc_hip_attention_args_t g = msa_attention_call(&a, fake, w, true);
+    return kutacc_launch::fused_layernorm_supported(g, kutacc_launch::FusedAttentionOptions());
 }
 } // namespace
 
@@ -346,7 +449,7 @@ int64_t kutacc_hip_msa_attention_workspace(int64_t n_seq, int64_t n_res, int64_t
     if (n_seq <= 0 || n_res <= 0 || nheads <= 0 || n_seq > 1 << 20 || n_res > 65536 || nheads > 64) {
         return -1;
     }
-    return msa_layout(n_seq, n_res, nheads, column != 0).total;
+    return msa_layout(n_seq, n_res, nheads, column != 0, msa_block_fuses_layernorm(n_seq, n_res, nheads, column != 0)).total;
 }
 
 int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *stream)
@@ -363,36 +466,22 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
         return KUTACC_HIP_EINVAL;
     }
     const int64_t n_seq = a->n_seq, n_res = a->n_res, heads = a->nheads, c = heads * HEAD;
-    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column);
+    // where the persistent head kernel takes the call it normalises the msa rows itself: no normalised copy, no LayerNorm pass
+    const bool fused_ln = msa_block_fuses_layernorm(n_seq, n_res, heads, column);
+    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column, fused_ln);
     if (a->workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
         return KUTACC_HIP_EINVAL;
     }
     char *ws = static_cast<char *>(a->workspace);
     hipStream_t s = kutacc_api::stream_or_default(stream);
-    // row-wise: every sequence attends over the residues; column-wise: every residue attends over the sequences,
-    // i.e. the same operator on the msa with its two leading axes exchanged
-    const int64_t batch = column ? n_res : n_seq, seq = column ? n_seq : n_res;
-
-    kutacc_hip_attention_args_t g;
-    std::memset(&g, 0, sizeof(g));
-    g.batch = batch, g.seq_len = seq, g.nheads = heads, g.head_size = HEAD;
-    g.dtype = KUTACC_DTYPE_BF16, g.path = KUTACC_HIP_PATH_FUSED;
-    g.input = ws + w.m_norm, g.input_ld = c;
-    g.query_w = a->query_w, g.key_w = a->key_w, g.value_w = a->value_w, g.gating_w = a->gating_w, g.output_w = a->output_w;
-    g.gating_b = a->gating_b, g.output_b = a->output_b;
-    g.bias = a->msa_mask, g.bias_stride_b = column ? 1 : n_res;
-    if (!column) {
-        g.nonbatched_bias = ws + w.nb, g.nb_stride_h = n_res * n_res, g.nb_stride_q = n_res;
-    }
-    g.q = ws + w.q, g.q_stride_b = seq * c, g.q_stride_s = c, g.q_stride_h = HEAD;
-    g.avg = ws + w.avg, g.avg_stride_b = seq * c, g.avg_stride_s = c, g.avg_stride_h = HEAD;
-    g.out = a->msa_act, g.out_ld = c;
+    const kutacc_hip_attention_args_t g = msa_attention_call(a, ws, w, fused_ln);
     if (!kutacc_launch::fused_attention_supports(g)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
-    // 1. LayerNorm of the msa rows, read transposed for the column-wise form
-    int rc = kutacc_launch::layernorm_rows(a->msa_act, c, a->ln_gamma, a->ln_beta, ws + w.m_norm, c, n_seq * n_res, c, a->ln_eps,
-                                           KUTACC_DTYPE_BF16, s, column ? n_seq : 0);
+    // 1. LayerNorm of the msa rows, read transposed for the column-wise form (unless the head kernel does it)
+    int rc = fused_ln ? 0
+                      : kutacc_launch::layernorm_rows(a->msa_act, c, a->ln_gamma, a->ln_beta, ws + w.m_norm, c, n_seq * n_res, c,
+                                                      a->ln_eps, KUTACC_DTYPE_BF16, s, column ? n_seq : 0);
     // 2. pair bias from the pair activation (row-wise form only)
     //    -- with the fragment-major copy the attention kernels read, where the grid allows it
     bool fragments = false;
@@ -413,6 +502,10 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
         opt.bias_is_mask = true; // msa_mask[s, r] is element (b = s, k = r) row-wise and (b = r, k = s) column-wise
         opt.bias_stride_k = column ? n_res : 1;
         opt.nb_fragments_ready = fragments;
+        if (fused_ln) {
+            opt.ln_gamma = a->ln_gamma, opt.ln_beta = a->ln_beta, opt.ln_eps = a->ln_eps;
+            opt.input_stride_b = column ? c : n_res * c;
+        }
         rc = kutacc_launch::gating_attention_fused(g, s, opt);
     }
     return rc;

@@ -90,7 +90,9 @@ struct FusedParams {
     const bf16_t *bias;
     const bf16_t *nb;
     bf16_t *avg;
-    int64_t x_ld, bias_sb, bias_sk, nb_sh, nb_sq, avg_sb, avg_ss, avg_sh;
+    int64_t x_ld, x_sb, bias_sb, bias_sk, nb_sh, nb_sq, avg_sb, avg_ss, avg_sh; // x_sb: from one batch row of x to the next
+    const float *ln_gamma, *ln_beta; // fused LayerNorm of the input rows (persistent kernel), else nullptr
+    float ln_eps;
     int bias_is_mask; // bias holds the 0/1 mask; the kernels form 1e9*(mask-1) themselves
     int B, S, H, NB, NW, GW;
     int nb_vec;   // pair-bias rows may be read with 16-byte loads
@@ -862,7 +864,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             asm volatile("" : "+s"(j));
             bf16x8 xf[CK];
             if (staged_input) {
-                const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
+                const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
                 uint4 *kslot = lds_k + j * 128, *vslot = lds_v + j * 128 - 128; // panel slots 0-127 and 128-255
                 if constexpr (V_ALIAS) {
                     kslot = vslot = own_panel;
@@ -887,7 +889,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             } else {
                 int srow = j * 32 + prow;
                 srow = srow < S ? srow : S - 1; // rows past the end repeat the last row; they are never stored
-                const bf16_t *xrow = p.x + ((int64_t)b * S + srow) * p.x_ld + g * 8;
+                const bf16_t *xrow = p.x + (int64_t)b * p.x_sb + (int64_t)srow * p.x_ld + g * 8;
 #pragma unroll
                 for (int ks = 0; ks < CK; ++ks) {
                     xf[ks] = as_bf16x8(*reinterpret_cast<const uint4 *>(xrow + ks * 16));
@@ -1040,7 +1042,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
 // on the next row's loads and projections while the slower waves of its SIMD still attend, so the
 // latency- and MFMA-bound projection phase overlaps the VALU-heavy attention phase.
 // ------------------------------------------------------------------------------------------------
-template <int C, bool HAS_NB, bool L2MODE>
+template <int C, bool HAS_NB, bool L2MODE, bool FUSED_LN>
 __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(FusedParams p)
 {
     constexpr int CK = C / 16;
@@ -1118,9 +1120,89 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 
         // ---- input rows of the block -> fragments, 64 channels per staging panel ----
         const int prow_x = pi_row(lane_x & 31), g_x = lane_x >> 5;
-        const bf16_t *xb = p.x + (int64_t)b * S * p.x_ld;
+        const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
         bf16x8 xf[CK];
-        {
+        if constexpr (FUSED_LN) {
+            // The rows arrive un-normalised and are normalised between their load and their staging (arithmetic of
+            // reference src/normalization/layernorm_kernel.h:21-53, result rounded to bf16 as the tensor it replaces
+            // was).  A lane holds 8 channels per panel of four rows; a row's C channels sit in the 8 lanes that loaded
+            // it, so its two sums cross three DPP steps.
+            PanelRegs t[NP];
+#pragma unroll
+            for (int c = 0; c < NP; ++c) {
+                t[c] = panel_load(xb, p.x_ld, j * 32, S - 1, c * 64, lane_x);
+            }
+            float gm[NP][8], bt[NP][8];
+#pragma unroll
+            for (int c = 0; c < NP; ++c) {
+                const float *gsrc = p.ln_gamma + c * 64 + (lane_x & 7) * 8, *bsrc = p.ln_beta + c * 64 + (lane_x & 7) * 8;
+#pragma unroll
+                for (int e = 0; e < 8; e += 4) {
+                    const f32x4 gv = *reinterpret_cast<const f32x4 *>(gsrc + e), bv = *reinterpret_cast<const f32x4 *>(bsrc + e);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        gm[c][e + k] = gv[k], bt[c][e + k] = bv[k];
+                    }
+                }
+            }
+            auto normalise_row = [&](uint4 (&words)[NP]) {
+                float v[NP][8];
+#pragma unroll
+                for (int c = 0; c < NP; ++c) {
+                    const bf16x8 in = as_bf16x8(words[c]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        v[c][e] = to_f32(in[e]);
+                    }
+                }
+                const float x0 = __shfl(v[0][0], lane_x & ~7, 64); // first element of the row
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int c = 0; c < NP; ++c) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float d = v[c][e] - x0;
+                        s1 += d;
+                        s2 = fmaf(d, d, s2);
+                    }
+                }
+                s1 = group_sum<8>(s1), s2 = group_sum<8>(s2);
+                const float nch = (float)C;
+                const float mean = s1 / nch + x0;
+                const float var = fmaxf((s2 - s1 * s1 / nch) / nch, 0.f);
+                const float rstd = 1.0f / sqrtf(var + p.ln_eps);
+                const float shift = -rstd * mean;
+#pragma unroll
+                for (int c = 0; c < NP; ++c) {
+                    bf16x8 o;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        o[e] = (bf16_t)fmaf(fmaf(v[c][e], rstd, shift), gm[c][e], bt[c][e]);
+                    }
+                    words[c] = as_uint4(o);
+                }
+            };
+            {
+                uint4 w0[NP], w1[NP], w2[NP], w3[NP];
+#pragma unroll
+                for (int c = 0; c < NP; ++c) {
+                    w0[c] = t[c].r0, w1[c] = t[c].r1, w2[c] = t[c].r2, w3[c] = t[c].r3;
+                }
+                normalise_row(w0), normalise_row(w1), normalise_row(w2), normalise_row(w3);
+#pragma unroll
+                for (int c = 0; c < NP; ++c) {
+                    t[c].r0 = w0[c], t[c].r1 = w1[c], t[c].r2 = w2[c], t[c].r3 = w3[c];
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < NP; ++c) {
+                panel_store(panel, lane_x, t[c]);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    xf[4 * c + k] = as_bf16x8(panel[panel_slot(prow_x, 2 * k + g_x)]);
+                }
+            }
+        } else {
             PanelRegs ta, tb;
             ta = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane_x);
 #pragma unroll
@@ -1864,10 +1946,10 @@ int launch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t stream)
     return kutacc_hip_status(hipGetLastError());
 }
 
-template <int C, bool HAS_NB, bool L2MODE>
+template <int C, bool HAS_NB, bool L2MODE, bool FUSED_LN = false>
 int launch_persistent_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
 {
-    auto kern = persistent_head_kernel<C, HAS_NB, L2MODE>;
+    auto kern = persistent_head_kernel<C, HAS_NB, L2MODE, FUSED_LN>;
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
     if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
         return rc;
@@ -1888,6 +1970,10 @@ int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t strea
 {
     const bool nb = p.nb != nullptr;
     if (pl.persistent) {
+        if (p.ln_gamma != nullptr) { // only asked for where fused_layernorm_supported says so: log2 units
+            return nb ? launch_persistent_kernel<C, true, true, true>(p, pl, stream)
+                      : launch_persistent_kernel<C, false, true, true>(p, pl, stream);
+        }
         if (p.l2mode) {
             return nb ? launch_persistent_kernel<C, true, true>(p, pl, stream) : launch_persistent_kernel<C, false, true>(p, pl, stream);
         }
@@ -1944,6 +2030,17 @@ bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &a, int *
     return true;
 }
 
+bool fused_layernorm_supported(const kutacc_hip_attention_args_t &a, const FusedAttentionOptions &opt)
+{
+    Plan pl;
+    if (!fused_attention_supports(a) || !make_plan(a.seq_len, (int)(a.nheads * a.head_size), pl) || !pl.persistent ||
+        fragments_disabled()) {
+        return false;
+    }
+    // log2 units need the fragment-major pair bias (none without a pair bias)
+    return a.nonbatched_bias == nullptr || fragment_home(a, pl.NB, opt) != nullptr;
+}
+
 bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
 {
     if (a.dtype != KUTACC_DTYPE_BF16 || a.head_size != HEAD) {
@@ -1987,6 +2084,8 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     p.nb = (const bf16_t *)a.nonbatched_bias;
     p.avg = (bf16_t *)a.avg;
     p.x_ld = a.input_ld, p.bias_sb = a.bias_stride_b, p.nb_sh = a.nb_stride_h, p.nb_sq = a.nb_stride_q;
+    p.x_sb = opt.input_stride_b != 0 ? opt.input_stride_b : a.seq_len * a.input_ld;
+    p.ln_gamma = nullptr, p.ln_beta = nullptr, p.ln_eps = 0.f;
     p.bias_sk = opt.bias_stride_k, p.bias_is_mask = opt.bias_is_mask ? 1 : 0;
     p.avg_sb = a.avg_stride_b, p.avg_ss = a.avg_stride_s, p.avg_sh = a.avg_stride_h;
     p.B = (int)a.batch, p.S = (int)a.seq_len, p.H = (int)a.nheads, p.NB = pl.NB, p.NW = pl.NW, p.GW = pl.GW;
@@ -2021,6 +2120,12 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
         p.nbf = (const uint4 *)fragments;
     }
     p.l2mode = ((p.nb == nullptr || p.nbf != nullptr) && !fragments_disabled()) ? 1 : 0;
+    if (opt.ln_gamma != nullptr) {
+        if (!pl.persistent || !p.l2mode || opt.ln_beta == nullptr || !aligned(opt.ln_gamma, 16) || !aligned(opt.ln_beta, 16)) {
+            return KUTACC_HIP_EUNSUPPORTED; // the caller asks fused_layernorm_supported first
+        }
+        p.ln_gamma = opt.ln_gamma, p.ln_beta = opt.ln_beta, p.ln_eps = opt.ln_eps;
+    }
     if (g_debug.load(std::memory_order_relaxed)) {
         fprintf(stderr,
                 "[kutacc] fused plan: persistent=%d C=%d NB=%d NT=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d log2_units=%d "

@@ -87,7 +87,16 @@ struct FusedAttentionOptions {
     // neither read nor written; a call whose copy does not fit is rejected with KUTACC_HIP_EINVAL
     void *fragment_workspace = nullptr;
     size_t fragment_workspace_bytes = 0;
+    // LayerNorm of the input rows inside the head kernel (args.input is then the un-normalised tensor): fp32 gamma and
+    // beta of nheads*head_size values, 16-byte aligned.  Only where fused_layernorm_supported says so.
+    const float *ln_gamma = nullptr, *ln_beta = nullptr;
+    float ln_eps = 0.f;
+    // elements from one batch row of args.input to the next; 0 = seq_len * input_ld (dense).  With input_ld as the
+    // stride between sequence positions this lets the kernels read an [S, B, C] tensor as [B, S, C] without a copy.
+    int64_t input_stride_b = 0;
 };
+// Whether gating_attention_fused can normalise the input rows itself for this call (the persistent kernel in log2 units)
+bool fused_layernorm_supported(const kutacc_hip_attention_args_t &args, const FusedAttentionOptions &opt);
 // Whether gating_attention_fused would keep a fragment-major copy of the pair bias in args.q, and the copy's extent:
 // [nheads][*nb query blocks][*nt key tiles][2][64 lanes] x 16 bytes.
 bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &args, int *nb, int *nt);

@@ -101,6 +101,15 @@ def test_pair_bias_transposed_equals_pair_bias_of_the_swapped_tensor(torch_cuda,
 
 
 # ---- the block ---------------------------------------------------------------------------------------------------
+@pytest.fixture(params=["fused", "separate"])
+def layernorm_placement(request):
+    """Both placements of the blocks' LayerNorm: inside the attention kernel's row staging (where that kernel can) and as a
+    pass of its own.  The setting must hold while the block object is built (it sizes its workspace) and run."""
+    assert capi.set_tuning("layernorm", request.param) == 0
+    yield request.param
+    capi.set_tuning("layernorm", "auto")
+
+
 def block_case(seed, n, heads):
     rng = np.random.Generator(np.random.PCG64(seed))
     c = heads * 32
@@ -149,14 +158,14 @@ def run_block(torch, c, ending, z=None, mask=None):
 # 64, 96 and 160: whole key tiles, where the producer of the pair bias also writes the copy the attention kernels read
 # (96 and 160: an odd tile count, padded with a zero tile)
 @pytest.mark.parametrize("n,heads", [(48, 4), (70, 4), (40, 8), (64, 4), (96, 4), (160, 4), (64, 8), (32, 4), (128, 8)])
-def test_triangle_attention_block_against_the_oracle(torch_cuda, n, heads, ending):
+def test_triangle_attention_block_against_the_oracle(torch_cuda, layernorm_placement, n, heads, ending):
     c = block_case(600 + n, n, heads)
     got = run_block(torch_cuda, c, ending)
     helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block n={n} ending={ending}")
 
 
 @pytest.mark.parametrize("index,n", [(i, int(n)) for i, n in enumerate(np.random.Generator(np.random.PCG64(57)).integers(8, 200, size=8))])
-def test_triangle_attention_block_seeded_sweep(torch_cuda, index, n):
+def test_triangle_attention_block_seeded_sweep(torch_cuda, layernorm_placement, index, n):
     """Eight seeded pair sizes between 8 and 199 (ragged key tiles, odd tile counts), four heads, node alternating."""
     ending = bool(index & 1)
     c = block_case(3000 + index, n, 4)
@@ -164,7 +173,7 @@ def test_triangle_attention_block_seeded_sweep(torch_cuda, index, n):
     helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block sweep {index}: n={n} ending={ending}")
 
 
-def test_triangle_attention_block_full_size_orientation_identity(torch_cuda):
+def test_triangle_attention_block_full_size_orientation_identity(torch_cuda, layernorm_placement):
     """384 residues: the ending-node block equals the starting-node block on the transposed pair tensor and mask,
     transposed back -- the two orientations differ only in which element is read or written where."""
     torch = torch_cuda
@@ -175,6 +184,21 @@ def test_triangle_attention_block_full_size_orientation_identity(torch_cuda):
     start_t = run_block(torch, c, False, z.transpose(0, 1).contiguous(), mask.t().contiguous())
     assert helpers.same_bits(end, start_t.transpose(0, 1).contiguous())
     assert not helpers.same_bits(end, z)
+
+
+def test_fused_layernorm_drops_the_normalised_copy_from_the_workspace(torch_cuda):
+    """With the LayerNorm inside the attention kernel the blocks keep no normalised activation: the workspace is one
+    activation smaller wherever the persistent kernel runs (384 residues), and unchanged where it does not (1024)."""
+    L = capi.lib()
+    sizes = {}
+    for mode in ("fused", "separate"):
+        assert capi.set_tuning("layernorm", mode) == 0
+        sizes[mode] = (L.kutacc_hip_triangle_attention_workspace(384, 4), L.kutacc_hip_triangle_attention_workspace(1024, 4),
+                       L.kutacc_hip_msa_attention_workspace(512, 256, 8, 0))
+    capi.set_tuning("layernorm", "auto")
+    assert sizes["separate"][0] - sizes["fused"][0] == 384 * 384 * 128 * 2
+    assert sizes["separate"][1] == sizes["fused"][1]
+    assert sizes["separate"][2] - sizes["fused"][2] == 512 * 256 * 256 * 2
 
 
 def test_triangle_attention_block_rejects_bad_arguments(torch_cuda):
@@ -421,7 +445,7 @@ def msa_oracle(c, column):
 @pytest.mark.parametrize("column", [False, True], ids=["row-wise with pair bias", "column-wise"])
 @pytest.mark.parametrize("n_seq,n_res,heads,c_z", [(24, 40, 8, 128), (50, 20, 8, 128), (33, 33, 4, 64), (24, 64, 8, 128),
                                                    (20, 96, 8, 128)])
-def test_msa_attention_block_against_the_oracle(torch_cuda, n_seq, n_res, heads, c_z, column):
+def test_msa_attention_block_against_the_oracle(torch_cuda, layernorm_placement, n_seq, n_res, heads, c_z, column):
     torch = torch_cuda
     c = msa_case(1000 + n_seq, n_seq, n_res, heads, c_z)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
