@@ -34,6 +34,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <type_traits>
+#include <vector>
 
 #include "api_internal.h"
 #include "device_util.h"
@@ -1321,6 +1322,9 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, nb_head, p.nb_sq, j * 32, p.nb_vec != 0, panel, q0, q1, sel0,
                                  sel1, NB, S, lane, o, l);
         }
+        if (n == 2) {
+            TL(4);
+        }
         int lane_o = lane; // as above: the addresses of the epilogue are not worth a register during the attention loop
         asm volatile("" : "+v"(lane_o));
         const int qpos = j * 32 + pi_row(lane_o & 31);
@@ -1335,9 +1339,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             }
             store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * (lane_o >> 5), o,
                         __builtin_amdgcn_rcpf(l), gv);
-        }
-        if (n == 2) {
-            TL(4);
         }
         if (n == 2) {
             TL(5);
@@ -2333,3 +2334,111 @@ int kutacc_launch::fused_attention_tuning(const char *name, const char *value)
     }
     return KUTACC_HIP_EINVAL;
 }
+
+#ifdef KUTACC_TIMELINE
+// Development build only: the attention tile loop by itself.  One workgroup per CU, K and V fragments of `nt` key tiles in
+// LDS (arbitrary small values), pair-bias fragments streamed from a buffer that stays in L2, `waves` waves per
+// workgroup (4, 8 or 12: one, two or three per SIMD) each running attend_block_l2 `reps` times.  No projections, no
+// barriers, no epilogue: what the loop costs per key tile when nothing else shares the SIMD.
+namespace {
+template <bool HAS_NB>
+__global__ __launch_bounds__(768) void attention_loop_probe(const uint4 *nbf_g, float *out, int NT, int reps,
+                                                            unsigned long long *clk)
+{
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint4 *lds_k = lds, *lds_v = lds + NT * 2 * 64;
+    for (int i = tid; i < NT * 2 * 64 * 2; i += blockDim.x) {
+        bf16x8 v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[e] = (bf16_t)(((i * 8 + e) * 37 % 101 - 50) * 0.01f);
+        }
+        lds[i] = as_uint4(v);
+    }
+    bf16x8 q0, q1, sel0, sel1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        q0[e] = (bf16_t)(((lane * 8 + e) * 13 % 31 - 15) * 0.02f);
+        q1[e] = (bf16_t)(((lane * 8 + e) * 7 % 29 - 14) * 0.02f);
+    }
+    make_selectors(lane, sel0, sel1);
+    const bf16x8 sumsel = rowsum_selector(lane);
+    __syncthreads();
+    const uint4 *nbf = nbf_g + (int64_t)wave * NT * 2 * 64 + lane;
+    float acc = 0.f;
+    const unsigned long long t0 = clock64();
+    for (int r = 0; r < reps; ++r) {
+        f32x16 o;
+        float l;
+        attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, nullptr, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o, l);
+        acc += o[0] + o[5] + l;
+        asm volatile("" : "+v"(q0), "+v"(q1));
+    }
+    const unsigned long long t1 = clock64();
+    out[blockIdx.x * blockDim.x + tid] = acc;
+    if (lane == 0) {
+        clk[blockIdx.x * 12 + wave] = t1 - t0;
+    }
+}
+} // namespace
+
+// result[0] = kernel time in microseconds, result[1] = shader clocks of the slowest wave (mean over workgroups),
+// result[2] = shader clocks of wave 0.  Returns 0 or a HIP status.
+extern "C" __attribute__((visibility("default"))) int kutacc_debug_attention_loop(int nt, int reps, int waves, int pair_bias,
+                                                                                  double *result)
+{
+    if (nt < 2 || nt > 32 || (nt & 1) || (waves != 4 && waves != 8 && waves != 12) || reps < 1 || !result) {
+        return KUTACC_HIP_EINVAL;
+    }
+    const int ncu = num_cus();
+    uint4 *nbf = nullptr;
+    float *out = nullptr;
+    unsigned long long *clk = nullptr;
+    const size_t nbf_bytes = (size_t)12 * nt * 2 * 64 * 16;
+    hipError_t e = hipMalloc(&nbf, nbf_bytes);
+    e = e == hipSuccess ? hipMalloc(&out, (size_t)ncu * 768 * 4) : e;
+    e = e == hipSuccess ? hipMalloc(&clk, (size_t)ncu * 12 * 8) : e;
+    if (e == hipSuccess) {
+        std::vector<uint16_t> h(nbf_bytes / 2);
+        for (size_t i = 0; i < h.size(); ++i) {
+            h[i] = (uint16_t)(0x3c00 + i * 7 % 64); // bf16 values a little above 0.0078
+        }
+        e = hipMemcpy(nbf, h.data(), nbf_bytes, hipMemcpyHostToDevice);
+    }
+    const size_t lds_bytes = 100 * 1024; // more than half a CU's LDS: one workgroup per CU
+    auto kern = pair_bias ? attention_loop_probe<true> : attention_loop_probe<false>;
+    e = e == hipSuccess ? hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) : e;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    e = e == hipSuccess ? hipEventCreate(&e0) : e;
+    e = e == hipSuccess ? hipEventCreate(&e1) : e;
+    float ms = 0.f;
+    for (int pass = 0; pass < 2 && e == hipSuccess; ++pass) { // the first pass warms up
+        e = hipMemset(clk, 0, (size_t)ncu * 12 * 8);
+        e = e == hipSuccess ? hipEventRecord(e0, nullptr) : e;
+        kern<<<ncu, waves * 64, lds_bytes, nullptr>>>(nbf, out, nt, reps, clk);
+        e = e == hipSuccess ? hipGetLastError() : e;
+        e = e == hipSuccess ? hipEventRecord(e1, nullptr) : e;
+        e = e == hipSuccess ? hipEventSynchronize(e1) : e;
+        e = e == hipSuccess ? hipEventElapsedTime(&ms, e0, e1) : e;
+    }
+    if (e == hipSuccess) {
+        std::vector<unsigned long long> c((size_t)ncu * 12);
+        e = hipMemcpy(c.data(), clk, c.size() * 8, hipMemcpyDeviceToHost);
+        double per_wave[12] = {};
+        for (int w = 0; w < ncu; ++w) {
+            for (int k = 0; k < waves; ++k) {
+                per_wave[k] += (double)c[(size_t)w * 12 + k] / ncu;
+            }
+        }
+        double mx = 0;
+        for (int k = 0; k < waves; ++k) {
+            mx = per_wave[k] > mx ? per_wave[k] : mx;
+        }
+        result[0] = ms * 1e3, result[1] = mx, result[2] = per_wave[0];
+    }
+    (void)hipEventDestroy(e0), (void)hipEventDestroy(e1);
+    (void)hipFree(nbf), (void)hipFree(out), (void)hipFree(clk);
+    return kutacc_hip_status(e);
+}
+#endif // KUTACC_TIMELINE
