@@ -55,6 +55,7 @@ thread_local const char *t_last_path = "none";
 // 0: the handle-based entry points take the caller's word that all operands of a call live where `input` lives
 std::atomic<int> g_pointer_checks{1};
 std::atomic<int> g_block_layernorm{0};
+std::atomic<int> g_reference_scratch{0}; // kutacc_af2_gating_attention fills q, k, v, gate as the reference does
 
 inline hipStream_t pick_stream(void *s) { return s ? (hipStream_t)s : g_stream; }
 
@@ -253,6 +254,10 @@ int kutacc_hip_set_tuning(const char *name, const char *value)
         g_pointer_checks.store((value && value[0] == '0') ? 0 : 1);
         return 0;
     }
+    if (!std::strcmp(name, "scratch")) {
+        g_reference_scratch.store(value && !std::strcmp(value, "reference") ? 1 : 0);
+        return 0;
+    }
     if (!std::strcmp(name, "layernorm")) {
         g_block_layernorm.store(value && !std::strcmp(value, "fused") ? 1 : (value && !std::strcmp(value, "separate") ? 2 : 0));
         return 0;
@@ -423,7 +428,9 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
     kutacc_hip_attention_args_t a;
     std::memset(&a, 0, sizeof(a));
     a.batch = batch, a.seq_len = seq_len, a.nheads = nheads, a.head_size = head_size;
-    a.dtype = (int32_t)dt, a.path = KUTACC_HIP_PATH_AUTO;
+    // "scratch" = "reference": the shape-agnostic kernels, which leave q, k, v and gate as the reference's kernel does
+    // (src/attention/gating_attention.cpp:47-66); the MFMA kernels never form them in memory
+    a.dtype = (int32_t)dt, a.path = g_reference_scratch.load(std::memory_order_relaxed) ? KUTACC_HIP_PATH_GENERIC : KUTACC_HIP_PATH_AUTO;
     a.input = in.data, a.input_ld = nchannels;
     a.query_w = wq.data, a.key_w = wk.data, a.value_w = wv.data, a.gating_w = wg.data, a.output_w = wo.data;
     a.gating_b = (const float *)bg.data, a.output_b = (const float *)bo.data;

@@ -364,6 +364,36 @@ def test_pointer_checks_can_be_switched_off(torch_cuda):
     assert capi.set_tuning("no such hook", "1") == capi.EINVAL
 
 
+def test_reference_scratch_mode_fills_q_k_v_gate(torch_cuda):
+    """The reference's kernel leaves its projections in the caller's scratch tensors (reference
+    src/attention/gating_attention.cpp:47-66: q scaled by 1/sqrt(d), k, v transposed to [H, d, B, S], gate after the
+    sigmoid).  The MFMA kernels never form them in memory; with "scratch" = "reference" the operator runs on the
+    shape-agnostic kernels, and the five tensors must match the oracle's bf16 model of the reference."""
+    from oracle import oracle
+    w = make_workload(3, batch=3, seq_len=80)
+    op, ten, scratch = helpers.make_op(w)
+    assert capi.set_tuning("scratch", "reference") == 0
+    try:
+        op.run()
+        path = capi.last_path()
+    finally:
+        capi.set_tuning("scratch", "default")
+    assert not capi.error_flag() and path == "generic"
+    bits = lambda a: oracle.to_bf16_bits(np.asarray(a, dtype=np.float32))  # noqa: E731
+    _, ref = oracle.gating_attention_bf16(bits(w.x), bits(w.wq), bits(w.wk), bits(w.wv), bits(w.wg), w.bg, bits(w.wo), w.bo,
+                                          bits(w.bias), None if w.nb is None else bits(w.nb), w.H, return_scratch=True)
+    for name in ("q", "k", "gate", "avg"):
+        got = helpers.to_numpy(scratch[name]).reshape(w.B, w.S, w.C)
+        helpers.check_close(got, oracle.from_bf16_bits(ref[name]).reshape(w.B, w.S, w.C), w.dtype, name)
+    helpers.check_close(helpers.to_numpy(scratch["v"]), oracle.from_bf16_bits(ref["v"]), w.dtype, "v")
+    # and the default mode leaves k, v and gate alone
+    for t in scratch.values():
+        t.zero_()
+    op.run()
+    assert capi.last_path() == "fused_mfma"
+    assert not scratch["k"].any() and not scratch["v"].any() and not scratch["gate"].any()
+
+
 def test_mixed_host_and_device_pointers_are_rejected(torch_cuda):
     w = make_workload(3, batch=2, seq_len=64)
     ten, scratch = helpers.to_device(w)
