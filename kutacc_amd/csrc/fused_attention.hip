@@ -99,7 +99,7 @@ struct FusedParams {
     int nb_vec;   // pair-bias rows may be read with 16-byte loads
     float qscale; // 1 / sqrt(head_size)
     int ngrp;     // persistent kernel: batch-row groups per XCD
-    const uint4 *nbf; // pair bias * log2(e) in fragment-major order (pair_bias_fragments_kernel), or nullptr
+    const uint4 *nbf; // pair bias * log2(e), fp16, in fragment-major order (pair_bias_fragments_kernel), or nullptr
     int NT;           // key tiles the LDS arrays are laid out for: NB rounded up to an even number (the log2-unit
                       // loop walks tile pairs; a phantom tile is all zeros behind a -inf mask)
     int l2mode;       // logits in log2 units (attend_block_l2); needs nbf when there is a pair bias
@@ -117,6 +117,19 @@ __device__ __forceinline__ void make_selectors(int lane, bf16x8 &sel0, bf16x8 &s
     for (int e = 0; e < 8; ++e) {
         sel0[e] = (bf16_t)((gi == g && w == e) ? 1.0f : 0.0f);
         sel1[e] = (bf16_t)((gi == g && w == e + 8) ? 1.0f : 0.0f);
+    }
+}
+
+// The same selectors with fp16 ones, for the log2-unit loop, whose pair-bias fragments are fp16.
+__device__ __forceinline__ void make_selectors_f16(int lane, f16x8 &sel0, f16x8 &sel1)
+{
+    const int r = lane & 31, g = lane >> 5;
+    const int gi = (r >> 2) & 1;
+    const int w = 4 * (r >> 3) + (r & 3);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        sel0[e] = (_Float16)((gi == g && w == e) ? 1.0f : 0.0f);
+        sel1[e] = (_Float16)((gi == g && w == e + 8) ? 1.0f : 0.0f);
     }
 }
 
@@ -441,7 +454,7 @@ __device__ __forceinline__ float rowsum_fetch(const f32x4 &lacc, int lane)
 
 template <bool HAS_NB, bool WITH_MASK, bool SHIFT>
 __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4,
-                                                const uint4 *nbf, bf16x8 q0, bf16x8 q1, bf16x8 sel0, bf16x8 sel1,
+                                                const uint4 *nbf, bf16x8 q0, bf16x8 q1, f16x8 sel0, f16x8 sel1,
                                                 bf16x8 sumsel, int NB, int lane, float shift, f32x16 &o_out, float &l_out,
                                                 int prio_phase = -1)
 {
@@ -480,8 +493,8 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
     k0 = kp[0], k1 = kp[64];
     f32x16 xa = init(0), xb;
     if (HAS_NB) {
-        xa = mfma(sel0, as_bf16x8(wa0), xa);
-        xa = mfma(sel1, as_bf16x8(wa1), xa);
+        xa = mfma_f16(sel0, as_f16x8(wa0), xa);
+        xa = mfma_f16(sel1, as_f16x8(wa1), xa);
         wa0 = nbf[clampt(2) * 128], wa1 = nbf[clampt(2) * 128 + 64];
     }
     xa = mfma(as_bf16x8(k0), q0, xa);
@@ -506,10 +519,10 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
         bf16x8 p0, p1;
         xn = init(t_next);
         if (HAS_NB) {
-            xn = mfma(sel0, as_bf16x8(w0), xn);
+            xn = mfma_f16(sel0, as_f16x8(w0), xn);
             exp4(xc, 0);
             fence();
-            xn = mfma(sel1, as_bf16x8(w1), xn);
+            xn = mfma_f16(sel1, as_f16x8(w1), xn);
             w0 = nbf[t_w * 128], w1 = nbf[t_w * 128 + 64];
             exp4(xc, 4);
             p0 = pack8(xc, 0);
@@ -563,7 +576,7 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
 // repeat of attend_block_l2 after an overflow or underflow.  Not a hot path: operands are loaded at use.
 template <bool HAS_NB>
 __device__ __forceinline__ float row_max_l2(const uint4 *lds_k, const f32x4 *mask4, const uint4 *nbf, bf16x8 q0, bf16x8 q1,
-                                            bf16x8 sel0, bf16x8 sel1, int NB, int lane)
+                                            f16x8 sel0, f16x8 sel1, int NB, int lane)
 {
     float mx = -INFINITY;
     for (int t = 0; t < NB; ++t) {
@@ -577,8 +590,8 @@ __device__ __forceinline__ float row_max_l2(const uint4 *lds_k, const f32x4 *mas
             }
         }
         if (HAS_NB) {
-            x = mfma(sel0, as_bf16x8(nbf[t * 128]), x);
-            x = mfma(sel1, as_bf16x8(nbf[t * 128 + 64]), x);
+            x = mfma_f16(sel0, as_f16x8(nbf[t * 128]), x);
+            x = mfma_f16(sel1, as_f16x8(nbf[t * 128 + 64]), x);
         }
         x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
         x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
@@ -982,8 +995,17 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         flags |= part_flags[part] << (2 * part);
     }
     const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
-    bf16x8 sel0, sel1;
-    make_selectors(lane, sel0, sel1);
+    // one pair of selector fragments, as bits: fp16 ones for the log2-unit loop (fp16 pair-bias fragments), bf16 ones otherwise
+    uint4 selw0, selw1;
+    if (p.l2mode) {
+        f16x8 a, b;
+        make_selectors_f16(lane, a, b);
+        selw0 = as_uint4(a), selw1 = as_uint4(b);
+    } else {
+        bf16x8 a, b;
+        make_selectors(lane, a, b);
+        selw0 = as_uint4(a), selw1 = as_uint4(b);
+    }
     const bf16x8 sumsel = rowsum_selector(lane);
 
 #pragma unroll
@@ -999,22 +1021,22 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         if (p.l2mode) {
             const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NT * 2) * 64 + lane : nullptr;
             if (flags == 0u) {
-                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
+                attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], as_f16x8(selw0), as_f16x8(selw1), sumsel, NT,
                                                       lane, 0.f, o, l, (wave >> 2) & 1);
             } else {
-                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
+                attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], as_f16x8(selw0), as_f16x8(selw1), sumsel, NT,
                                                      lane, 0.f, o, l, (wave >> 2) & 1);
             }
             __builtin_amdgcn_s_setprio(0);
             if (__any(!(l > 1e-30f && l < 1e30f))) {
                 // some probability overflowed or a whole row underflowed: shift by the true row maxima
-                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, NT, lane);
-                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], sel0, sel1, sumsel, NT,
+                const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, qf[i][0], qf[i][1], as_f16x8(selw0), as_f16x8(selw1), NT, lane);
+                attend_block_l2<HAS_NB, true, true>(lds_k, lds_v, mask4, nbf, qf[i][0], qf[i][1], as_f16x8(selw0), as_f16x8(selw1), sumsel, NT,
                                                     lane, m, o, l);
             }
         } else {
             const bf16_t *nbrow = HAS_NB ? p.nb + (int64_t)h * p.nb_sh + (int64_t)qrow * p.nb_sq + 16 * g : nullptr;
-            attend_block_direct<HAS_NB>(lds_k, lds_v, mask4, flags, nbrow, p.nb_vec != 0, qf[i][0], qf[i][1], sel0, sel1, NB,
+            attend_block_direct<HAS_NB>(lds_k, lds_v, mask4, flags, nbrow, p.nb_vec != 0, qf[i][0], qf[i][1], as_bf16x8(selw0), as_bf16x8(selw1), NB,
                                         S, lane, o, l);
         }
         TL(5);
@@ -1089,8 +1111,12 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             lds_v[NB * 2 * 64 + idx] = z4;
         }
     }
-    bf16x8 sel0, sel1;
-    make_selectors(lane, sel0, sel1);
+    std::conditional_t<L2MODE, f16x8, bf16x8> sel0, sel1; // fp16 ones for the log2-unit loop, whose pair-bias fragments are fp16
+    if constexpr (L2MODE) {
+        make_selectors_f16(lane, sel0, sel1);
+    } else {
+        make_selectors(lane, sel0, sel1);
+    }
     __syncthreads();
 
     TL(8);
@@ -1791,17 +1817,18 @@ __global__ __launch_bounds__(64) void pair_bias_fragments_kernel(const bf16_t *_
         w0.x = wds[0], w0.y = wds[1], w0.z = wds[2], w0.w = wds[3];
         w1.x = wds[4], w1.y = wds[5], w1.z = wds[6], w1.w = wds[7];
     }
-    // into log2 units, rounded to bf16 again (the logits MFMAs of attend_block_l2 accumulate exponents of 2)
+    // into log2 units (the logits MFMAs of attend_block_l2 accumulate exponents of 2), as fp16: the product of a bf16 value
+    // with log2(e) keeps eleven significant bits instead of eight, so the second rounding costs 2^-12 of the bias, not 2^-9
     const bf16x8 s0 = as_bf16x8(w0), s1 = as_bf16x8(w1);
-    bf16x8 d0, d1;
+    uint32_t d[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        d0[e] = (bf16_t)(to_f32(s0[e]) * LOG2E);
-        d1[e] = (bf16_t)(to_f32(s1[e]) * LOG2E);
+    for (int e = 0; e < 4; ++e) {
+        d[e] = (uint32_t)pair_bias_log2_f16(to_f32(s0[2 * e])) | ((uint32_t)pair_bias_log2_f16(to_f32(s0[2 * e + 1])) << 16);
+        d[4 + e] = (uint32_t)pair_bias_log2_f16(to_f32(s1[2 * e])) | ((uint32_t)pair_bias_log2_f16(to_f32(s1[2 * e + 1])) << 16);
     }
     uint4 *dst = out + ((((int64_t)h * NB + j) * NT + t) * 2) * 64 + lane;
-    dst[0] = as_uint4(d0);
-    dst[64] = as_uint4(d1);
+    dst[0] = make_uint4(d[0], d[1], d[2], d[3]);
+    dst[64] = make_uint4(d[4], d[5], d[6], d[7]);
 }
 
 // Tuning hooks (kutacc_hip_set_tuning): a forced plan of the long-sequence kernel, the fragment-major pair bias switched
@@ -2356,13 +2383,14 @@ __global__ __launch_bounds__(768) void attention_loop_probe(const uint4 *nbf_g, 
         }
         lds[i] = as_uint4(v);
     }
-    bf16x8 q0, q1, sel0, sel1;
+    bf16x8 q0, q1;
+    f16x8 sel0, sel1;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         q0[e] = (bf16_t)(((lane * 8 + e) * 13 % 31 - 15) * 0.02f);
         q1[e] = (bf16_t)(((lane * 8 + e) * 7 % 29 - 14) * 0.02f);
     }
-    make_selectors(lane, sel0, sel1);
+    make_selectors_f16(lane, sel0, sel1);
     const bf16x8 sumsel = rowsum_selector(lane);
     __syncthreads();
     const uint4 *nbf = nbf_g + (int64_t)wave * NT * 2 * 64 + lane;

@@ -28,6 +28,48 @@ __device__ __forceinline__ f32x16 mfma(bf16x8 a, bf16x8 b, f32x16 c)
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// The same product with fp16 operands (same operand and accumulator layout, same rate): used where an operand needs the
+// eleven significand bits of fp16 rather than the eight of bf16.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
+__device__ __forceinline__ f32x16 mfma_f16(f16x8 a, f16x8 b, f32x16 c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f16x8 as_f16x8(uint4 u)
+{
+    union {
+        uint4 u;
+        f16x8 h;
+    } c;
+    c.u = u;
+    return c.h;
+}
+
+__device__ __forceinline__ uint4 as_uint4(f16x8 h)
+{
+    union {
+        uint4 u;
+        f16x8 h;
+    } c;
+    c.h = h;
+    return c.u;
+}
+
+// nb * log2(e) as an fp16 bit pattern, for the fragment-major pair bias: finite whatever nb is (magnitudes past fp16's
+// range, |nb| > 45 403, act as that bound -- 2^-65504 is zero all the same)
+__device__ __forceinline__ uint16_t pair_bias_log2_f16(float nb)
+{
+    const float t = fminf(fmaxf(nb * LOG2E, -65504.0f), 65504.0f);
+    union {
+        _Float16 h;
+        uint16_t u;
+    } c;
+    c.h = (_Float16)t;
+    return c.u;
+}
+
 __device__ __forceinline__ f32x16 zero16()
 {
     const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};

@@ -301,14 +301,15 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
         if (nbf != nullptr) {
             // The copy the attention kernels read (rows_j a multiple of 32: the wave's rows are key tile t of one query
             // q): for head h, query block j, key tile t, 16-key half g' and 8-key half e the 16 bytes of lane
-            // (pi^-1(q mod 32), g'), pi being the row order of the attention's accumulators; values in log2 units,
-            // rounded to bf16 a second time.  Through the wave's tile, which nobody reads any more: [head][32 keys].
+            // (pi^-1(q mod 32), g'), pi being the row order of the attention's accumulators; values in log2 units as
+            // fp16 (the bf16 pair bias times log2(e), eleven significant bits kept).  Through the wave's tile, which nobody
+            // reads any more: [head][32 keys].
             static_assert(RB == 1, "the transposing buffer lies on the first row block of the tile");
-            bf16_t *t16 = reinterpret_cast<bf16_t *>(tile);
+            uint16_t *t16 = reinterpret_cast<uint16_t *>(tile);
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 if (4 * g + v < H) {
-                    t16[(4 * g + v) * 32 + col] = (bf16_t)((float)(bf16_t)acc[v] * kutacc_dev::LOG2E);
+                    t16[(4 * g + v) * 32 + col] = kutacc_dev::pair_bias_log2_f16((float)(bf16_t)acc[v]);
                 }
             }
             __builtin_amdgcn_wave_barrier(); // other lanes' stores: keep the loads below behind them

@@ -243,6 +243,31 @@ def test_uniform_pair_bias_offset_changes_nothing(torch_cuda, offset):
     helpers.check_close(b2, helpers.oracle_out(w3), w.dtype, "constant pair bias vs oracle")
 
 
+@pytest.mark.parametrize("seq_len,batch", [(128, 8), (384, 16), (520, 24)])
+def test_large_pair_bias_keeps_its_precision(torch_cuda, seq_len, batch):
+    """A pair bias with entries up to +-30, sigma 10 (what a trained pair representation can reach): the reference adds the
+    bf16 values exactly in fp32 (src/attention/gating_attention.cpp:113-117).  The log2-unit route carries nb * log2(e) as
+    fp16, 2^-12 of the bias at worst (0.007 nat at |nb| = 30, below the 2^-9 rounding of the bf16 probabilities themselves).
+    Carried as bf16 (2^-9 of the bias, 0.06 nat) the same inputs miss the parity bar: 0.13-0.18 off on the gated average,
+    rms 9e-3.  Bar here: 3e-2 + 1e-2 |ref| elementwise and rms error below 4e-3 (measured 2.0e-3; 1.7e-3 with the exact adds of
+    the natural-log route); persistent kernel (128, 384 keys) and long-sequence kernel (520)."""
+    w = make_workload(3, batch=batch, seq_len=seq_len)
+    rng = np.random.default_rng(seq_len)
+    w.nb = round_to_bf16(np.clip(rng.normal(0.0, 10.0, size=w.nb.shape), -30.0, 30.0).astype(np.float32))
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    assert not capi.error_flag() and capi.last_path() == "fused_mfma"
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    got = helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C)
+    # elementwise 3e-2 + 1e-2 |ref| (the usual 2e-2 floor is passed by all but one element in 786 432: with logit gaps of
+    # +-30 a softmax is nearly one-hot and a single bf16 rounding of q or k can move a weight; the exact-add route shows
+    # the same tail)
+    helpers.assert_within(got, ref_avg, 3e-2 + 1e-2 * np.abs(ref_avg), "gated average with a large pair bias")
+    rms = float(np.sqrt(np.mean((got - ref_avg) ** 2)))
+    assert rms < 4e-3, f"rms error of the gated average {rms:.3g}"
+    helpers.assert_within(helpers.to_numpy(ten["out"]), ref_out, 3e-2 + 1e-2 * np.abs(ref_out), "out with a large pair bias")
+
+
 def test_fully_masked_and_leading_masked_rows_short_sequence(torch_cuda):
     """Rows whose every key is masked (uniform average of V) and rows whose first key tile is masked, at a
     sequence length the one-workgroup-per-head kernel handles."""
