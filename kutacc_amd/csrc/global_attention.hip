@@ -54,12 +54,13 @@ __device__ __forceinline__ int gate_channel(int rb, int v, int g)
 
 // CACHED: the row has at most 32 tiles (seq_len <= 1024), so each wave keeps the fragments of its (at most 8) tiles
 // in registers after phase A and the row is read from memory once; otherwise every phase streams the row again.
-template <bool CACHED>
-__global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p)
+template <bool CACHED, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalParams p)
 {
-    constexpr int MAXI = CACHED ? 8 : (1 << 24); // tiles per wave
-    constexpr int UNR = CACHED ? 8 : 1;          // the cached tile array needs compile-time indices
-    bf16x8 xs[CACHED ? 8 : 1][4];
+    constexpr int NTHR = 64 * NW;
+    constexpr int MAXI = CACHED ? 32 / NW : (1 << 24); // tiles per wave
+    constexpr int UNR = CACHED ? 32 / NW : 1;          // the cached tile array needs compile-time indices
+    bf16x8 xs[CACHED ? 32 / NW : 1][4];
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
@@ -71,19 +72,40 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
     uint4 *wv_frag = qk_frag + 256;  // [4][64]
     uint4 *wg_frag = wv_frag + 256;  // [2 row blocks][4][64]
     uint4 *wo_frag = wg_frag + 512;  // [2 row blocks][4][64]
-    uint4 *panel = wo_frag + 512 + wave * 256;
-    float *maskb = reinterpret_cast<float *>(wo_frag + 512 + 4 * 256); // mask bias per token, -inf past S
+    uint4 *wk_rows = wo_frag + 512;  // the key weights as they lie in memory, [d][64 channels] bf16 (d <= 32)
+    uint4 *panel = wk_rows + 256 + wave * 256;
+    float *maskb = reinterpret_cast<float *>(wk_rows + 256 + NW * 256); // mask bias per token, -inf past S
     float *mask01 = maskb + spad;                                       // mask value per token, 0 past S
-    float *part = mask01 + spad;                                        // [4 waves][68]: channel sums, mask sum
-    float *qavg = part + 4 * 68;                                        // [64]
+    float *part = mask01 + spad;                                        // [NW waves][68]: channel sums, mask sum
+    float *qavg = part + NW * 68;                                        // [64]
     float *qv = qavg + GC;                                              // [64] q, bf16-rounded
     float *wavg = qv + GC;                                              // [64]
-    float *merge = wavg + GC;                                           // [4 waves][64 lanes][MERGE_LD]
+    float *merge = wavg + GC;                                           // [NW waves][64 lanes][MERGE_LD]
 
     const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
 
+    // Requested before anything else, so that their latency passes under the staging of the weights: the first tiles of
+    // the row (all of a wave's tiles when they are kept in registers and there are at most four) and this thread's slice
+    // of the query weights (output o = tid / TPR, channels part * 64 / TPR ...).
+    constexpr int PRE = CACHED ? (MAXI < 4 ? MAXI : 4) : 1;
+    PanelRegs ahead[PRE];
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+        const int t = wave + NW * i;
+        ahead[i] = panel_load(xb, p.x_ss, (t < NT ? t : NT - 1) * 32, S - 1, 0, lane);
+    }
+    constexpr int TPR = NTHR / GC, WQV = GC / TPR / 8; // threads per output of q, 16-byte pieces per thread
+    uint4 wq_part[WQV];
+#pragma unroll
+    for (int v = 0; v < WQV; ++v) {
+        wq_part[v] = *reinterpret_cast<const uint4 *>(p.wq + (tid / TPR) * GC + (tid % TPR) * (GC / TPR) + v * 8);
+    }
+
     // ---- weights of phases B and C as MFMA fragments; mask ----
-    for (int idx = tid; idx < 256; idx += 256) {
+    for (int idx = tid; idx < d * 8; idx += NTHR) {
+        wk_rows[idx] = reinterpret_cast<const uint4 *>(p.wk)[idx];
+    }
+    for (int idx = tid; idx < 256; idx += NTHR) {
         const int ks = idx >> 6, l = idx & 63, e = l & 31, gg = l >> 5;
         uint4 v = {0u, 0u, 0u, 0u};
         if (e < d) {
@@ -91,14 +113,14 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
         }
         wv_frag[idx] = v;
     }
-    for (int idx = tid; idx < 512; idx += 256) {
+    for (int idx = tid; idx < 512; idx += NTHR) {
         const int rb = idx >> 8, ks = (idx >> 6) & 3, l = idx & 63, i = l & 31, gg = l >> 5;
         const int ch = gate_channel(rb, 4 * (i >> 3) + (i & 3), (i >> 2) & 1);
         wg_frag[idx] = *reinterpret_cast<const uint4 *>(p.wg + ch * GC + ks * 16 + gg * 8);
         const int o = 32 * rb + pi_row(i);
         wo_frag[idx] = *reinterpret_cast<const uint4 *>(p.wo + o * GC + ks * 16 + gg * 8);
     }
-    for (int s = tid; s < spad; s += 256) {
+    for (int s = tid; s < spad; s += NTHR) {
         float m = 0.f, mb = -INFINITY;
         if (s < S) {
             m = to_f32(p.mask[(int64_t)b * p.mask_sb + s]);
@@ -120,17 +142,19 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
             }
         }
         float msum = 0.f;
-        // the loads of the next tile are in flight while this one is summed
-        PanelRegs nxt = panel_load(xb, p.x_ss, wave * 32, S - 1, 0, lane);
+        // the loads of the next PRE tiles are in flight while this one is summed
 #pragma unroll(UNR)
         for (int i = 0; i < MAXI; ++i) {
-            const int t = wave + 4 * i;
+            const int t = wave + NW * i;
             if (t >= NT) {
                 break;
             }
             bf16x8 xf[4];
-            panel_store(panel, lane, nxt);
-            nxt = panel_load(xb, p.x_ss, (t + 4 < NT ? t + 4 : t) * 32, S - 1, 0, lane);
+            panel_store(panel, lane, ahead[i % PRE]);
+            if (!CACHED || i + PRE < MAXI) {
+                const int tn = t + NW * PRE;
+                ahead[i % PRE] = panel_load(xb, p.x_ss, (tn < NT ? tn : NT - 1) * 32, S - 1, 0, lane);
+            }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
@@ -175,8 +199,12 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
     }
     __syncthreads();
     if (tid < GC) {
-        const float tot = part[tid] + part[68 + tid] + part[2 * 68 + tid] + part[3 * 68 + tid];
-        const float ms = part[64] + part[68 + 64] + part[2 * 68 + 64] + part[3 * 68 + 64];
+        float tot = 0.f, ms = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            tot += part[w * 68 + tid];
+            ms += part[w * 68 + 64];
+        }
         const bf16_t qa = (bf16_t)(tot * (1.0f / (ms + 1e-10f))); // reference :66-74
         qavg[tid] = to_f32(qa);
         if (p.q_avg != nullptr) {
@@ -184,34 +212,44 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
         }
     }
     __syncthreads();
-    if (tid < GC) {
-        const bf16_t *wrow = p.wq + tid * GC;
+    {
+        // q[o] = sum_c q_avg[c] wq[o][c]: TPR neighbouring threads share an output, each with the slice it fetched at the start
         float a = 0.f;
 #pragma unroll
-        for (int c8 = 0; c8 < 8; ++c8) {
-            const bf16x8 w8 = as_bf16x8(*reinterpret_cast<const uint4 *>(wrow + c8 * 8));
+        for (int v = 0; v < WQV; ++v) {
+            const bf16x8 w8 = as_bf16x8(wq_part[v]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                a = fmaf(qavg[c8 * 8 + e], to_f32(w8[e]), a);
+                a = fmaf(qavg[(tid % TPR) * (GC / TPR) + v * 8 + e], to_f32(w8[e]), a);
             }
         }
-        qv[tid] = to_f32((bf16_t)a); // the reference stores q as bf16 (:76-80)
+#pragma unroll
+        for (int off = TPR / 2; off > 0; off >>= 1) {
+            a += __shfl_xor(a, off, 64);
+        }
+        if (tid % TPR == 0) {
+            qv[tid / TPR] = to_f32((bf16_t)a); // the reference stores q as bf16 (:76-80)
+        }
     }
     __syncthreads();
-    {
+    if (tid < 256) {
         // B operand of the logits product: column h (zero for h >= H), 8 channels per lane and k-step
         const int ks = tid >> 6, h = r;
+        float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (h < H) {
+            for (int e = 0; e < d; ++e) {
+                const bf16x8 w8 = as_bf16x8(wk_rows[e * 8 + ks * 2 + g]); // channels ks*16 + g*8 .. +8 of key row e
+                const float qe = qv[h * d + e];
+#pragma unroll
+                for (int e8 = 0; e8 < 8; ++e8) {
+                    a[e8] = fmaf(qe, to_f32(w8[e8]), a[e8]);
+                }
+            }
+        }
         bf16x8 f;
 #pragma unroll
         for (int e8 = 0; e8 < 8; ++e8) {
-            const int c = ks * 16 + g * 8 + e8;
-            float a = 0.f;
-            if (h < H) {
-                for (int e = 0; e < d; ++e) {
-                    a = fmaf(qv[h * d + e], to_f32(p.wk[e * GC + c]), a);
-                }
-            }
-            f[e8] = (bf16_t)(a * p.scale);
+            f[e8] = (bf16_t)(a[e8] * p.scale);
         }
         qk_frag[ks * 64 + lane] = as_uint4(f);
     }
@@ -227,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
         }
 #pragma unroll(UNR)
         for (int i = 0; i < MAXI; ++i) {
-            const int t = wave + 4 * i;
+            const int t = wave + NW * i;
             if (t >= NT) {
                 break;
             }
@@ -239,7 +277,7 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
                 }
             } else {
                 panel_store(panel, lane, nxt);
-                nxt = panel_load(xb, p.x_ss, (t + 4 < NT ? t + 4 : t) * 32, S - 1, 0, lane);
+                nxt = panel_load(xb, p.x_ss, (t + NW < NT ? t + NW : t) * 32, S - 1, 0, lane);
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
@@ -294,17 +332,17 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
     }
     __syncthreads();
     if (wave == 0) {
-        float mw[4], lw[4];
+        float mw[NW], lw[NW];
         float M = -1e30f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < NW; ++w) {
             mw[w] = merge[(w * 64 + lane) * MERGE_LD];
             lw[w] = merge[(w * 64 + lane) * MERGE_LD + 1];
             M = fmaxf(M, mw[w]);
         }
         float L = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < NW; ++w) {
             mw[w] = __builtin_amdgcn_exp2f((mw[w] - M) * LOG2E);
             L = fmaf(lw[w], mw[w], L);
         }
@@ -313,7 +351,7 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
         for (int v = 0; v < 16; ++v) {
             float a = 0.f;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
+            for (int w = 0; w < NW; ++w) {
                 a = fmaf(merge[(w * 64 + lane) * MERGE_LD + 2 + v], mw[w], a);
             }
             const int e = 8 * (v >> 2) + 4 * g + (v & 3);
@@ -341,7 +379,7 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
         }
 #pragma unroll(UNR)
         for (int i = 0; i < MAXI; ++i) {
-            const int t = wave + 4 * i;
+            const int t = wave + NW * i;
             if (t >= NT) {
                 break;
             }
@@ -353,7 +391,7 @@ __global__ __launch_bounds__(256, 2) void global_attention_kernel(GlobalParams p
                 }
             } else {
                 panel_store(panel, lane, nxt);
-                nxt = panel_load(xb, p.x_ss, (t + 4 < NT ? t + 4 : t) * 32, S - 1, 0, lane);
+                nxt = panel_load(xb, p.x_ss, (t + NW < NT ? t + NW : t) * 32, S - 1, 0, lane);
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
@@ -431,24 +469,42 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
     p.B = (int)a.batch, p.S = (int)a.seq_len, p.H = (int)a.nheads, p.d = (int)a.head_size;
     p.NT = (int)((a.seq_len + 31) / 32);
     p.scale = (float)(1.0 / sqrt((double)a.head_size)); // reference :98
-    const size_t lds_bytes = (size_t)(256 + 256 + 512 + 512 + 4 * 256) * 16 +
-                             (size_t)(2 * p.NT * 32 + 4 * 68 + 3 * GC + 4 * 64 * MERGE_LD) * 4;
+    // A batch row is one workgroup and its three phases follow one another (load and mean, logits, gate and output), so what
+    // overlaps them is other rows on the same CU.  With the row kept in registers (up to 1024 positions) four waves hold
+    // 128 + 113 registers and two rows share a CU; eight waves hold half the tiles each (174 registers) and one row has the
+    // CU to itself, which is faster only while there is no second row to put there -- batch <= CUs: 28.1 against 30.7 us at
+    // 256 x 1024, 48.3 against 39.3 us at 384 x 1024.  Rows streamed three times (longer sequences) always take eight
+    // waves: 220 against 282 us at 384 x 5120.
     const bool cached = p.NT <= 32;
-    static size_t configured[2][KUTACC_DEVICE_SLOTS] = {};
+    static int cu_table[KUTACC_DEVICE_SLOTS] = {};
+    const int ncu = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
+    const int nw = (p.NT >= 16 && (!cached || a.batch <= ncu)) ? 8 : 4;
+    const size_t lds_bytes = (size_t)(256 + 256 + 512 + 512 + 256 + nw * 256) * 16 +
+                             (size_t)(2 * p.NT * 32 + nw * 68 + 3 * GC + nw * 64 * MERGE_LD) * 4;
+    static size_t configured[4][KUTACC_DEVICE_SLOTS] = {};
+    const void *fn = nw == 8 ? (cached ? reinterpret_cast<const void *>(global_attention_kernel<true, 8>)
+                                       : reinterpret_cast<const void *>(global_attention_kernel<false, 8>))
+                             : (cached ? reinterpret_cast<const void *>(global_attention_kernel<true, 4>)
+                                       : reinterpret_cast<const void *>(global_attention_kernel<false, 4>));
     {
-        const void *fn = cached ? reinterpret_cast<const void *>(global_attention_kernel<true>)
-                                : reinterpret_cast<const void *>(global_attention_kernel<false>);
-        const hipError_t e = kutacc_opt_in_lds(fn, lds_bytes, configured[cached]);
+        const hipError_t e = kutacc_opt_in_lds(fn, lds_bytes, configured[(nw == 8 ? 2 : 0) + (cached ? 1 : 0)]);
         if (e != hipSuccess) {
             return (int)e;
         }
     }
     const double BS = (double)a.batch * (double)a.seq_len;
     kutacc_prof::KernelTimer t("global_attention_kernel", BS * (4.0 * GC * a.head_size + 4.0 * GC * GC + 4.0 * GC), stream);
-    if (cached) {
-        global_attention_kernel<true><<<dim3((unsigned)a.batch), 256, lds_bytes, stream>>>(p);
+    const dim3 grid((unsigned)a.batch), block((unsigned)(64 * nw));
+    if (nw == 8) {
+        if (cached) {
+            global_attention_kernel<true, 8><<<grid, block, lds_bytes, stream>>>(p);
+        } else {
+            global_attention_kernel<false, 8><<<grid, block, lds_bytes, stream>>>(p);
+        }
+    } else if (cached) {
+        global_attention_kernel<true, 4><<<grid, block, lds_bytes, stream>>>(p);
     } else {
-        global_attention_kernel<false><<<dim3((unsigned)a.batch), 256, lds_bytes, stream>>>(p);
+        global_attention_kernel<false, 4><<<grid, block, lds_bytes, stream>>>(p);
     }
     return kutacc_hip_status(hipGetLastError());
 }
