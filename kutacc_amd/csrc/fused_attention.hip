@@ -120,6 +120,25 @@ __device__ __forceinline__ void make_selectors(int lane, bf16x8 &sel0, bf16x8 &s
     }
 }
 
+// Pair-bias words on their way into a selector MFMA: -inf (and any negative NaN pattern) becomes the most negative finite
+// bf16, since the MFMA multiplies every word by 0 or 1 and 0 x inf is a NaN.  As 16-bit unsigned numbers the negative
+// values sort by magnitude, so this is one packed minimum per word; what the logit then holds is absorbed like a -inf.
+__device__ __forceinline__ uint4 finite_bias_words(uint4 w)
+{
+    typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
+    union {
+        uint4 u;
+        u16x2 h[4];
+    } c;
+    c.u = w;
+    const u16x2 bound = {0xff7f, 0xff7f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        c.h[i] = __builtin_elementwise_min(c.h[i], bound);
+    }
+    return c.u;
+}
+
 // The same selectors with fp16 ones, for the log2-unit loop, whose pair-bias fragments are fp16.
 __device__ __forceinline__ void make_selectors_f16(int lane, f16x8 &sel0, f16x8 &sel1)
 {
@@ -266,8 +285,8 @@ __device__ __forceinline__ void attend_block(const uint4 *lds_k, const uint4 *ld
         if (HAS_NB) {
             uint4 w0, w1;
             nb_words(t, w0, w1);
-            x = mfma(sel0, as_bf16x8(w0), x);
-            x = mfma(sel1, as_bf16x8(w1), x);
+            x = mfma(sel0, as_bf16x8(finite_bias_words(w0)), x);
+            x = mfma(sel1, as_bf16x8(finite_bias_words(w1)), x);
         }
         x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
         x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
@@ -363,8 +382,8 @@ __device__ __forceinline__ void attend_block(const uint4 *lds_k, const uint4 *ld
             x = zero16();
         }
         const int c0 = 4 * (t & 1) + 2 * g;
-        x = mfma(sel0, as_bf16x8(panel[panel_slot(prow, c0)]), x);
-        x = mfma(sel1, as_bf16x8(panel[panel_slot(prow, c0 + 1)]), x);
+        x = mfma(sel0, as_bf16x8(finite_bias_words(panel[panel_slot(prow, c0)])), x);
+        x = mfma(sel1, as_bf16x8(finite_bias_words(panel[panel_slot(prow, c0 + 1)])), x);
         x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
         x = mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
     };
@@ -661,8 +680,8 @@ __device__ __forceinline__ void attend_block_direct(const uint4 *lds_k, const ui
             uint4 w0, w1;
             w0.x = nbw[0], w0.y = nbw[1], w0.z = nbw[2], w0.w = nbw[3];
             w1.x = nbw[4], w1.y = nbw[5], w1.z = nbw[6], w1.w = nbw[7];
-            x = mfma(sel0, as_bf16x8(w0), x);
-            x = mfma(sel1, as_bf16x8(w1), x);
+            x = mfma(sel0, as_bf16x8(finite_bias_words(w0)), x);
+            x = mfma(sel1, as_bf16x8(finite_bias_words(w1)), x);
             if (t + 1 < NB) {
                 fetch_nb(t + 1); // in flight while this tile's MFMAs and the previous tile's softmax run
             }

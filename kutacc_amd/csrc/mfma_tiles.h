@@ -57,11 +57,12 @@ __device__ __forceinline__ uint4 as_uint4(f16x8 h)
     return c.u;
 }
 
-// nb * log2(e) as an fp16 bit pattern, for the fragment-major pair bias: finite whatever nb is (magnitudes past fp16's
-// range, |nb| > 45 403, act as that bound -- 2^-65504 is zero all the same)
+// nb * log2(e) as an fp16 bit pattern, for the fragment-major pair bias: magnitudes past fp16's range (|nb| > 45 403,
+// infinities included) act as that bound -- 2^-65504 is zero all the same, and the selector products stay finite
 __device__ __forceinline__ uint16_t pair_bias_log2_f16(float nb)
 {
-    const float t = fminf(fmaxf(nb * LOG2E, -65504.0f), 65504.0f);
+    float t = nb * LOG2E;
+    t = t > 65504.0f ? 65504.0f : (t < -65504.0f ? -65504.0f : t); // comparisons, not min/max: a NaN stays a NaN
     union {
         _Float16 h;
         uint16_t u;

@@ -268,6 +268,26 @@ def test_large_pair_bias_keeps_its_precision(torch_cuda, seq_len, batch):
     helpers.assert_within(helpers.to_numpy(ten["out"]), ref_out, 3e-2 + 1e-2 * np.abs(ref_out), "out with a large pair bias")
 
 
+@pytest.mark.parametrize("batch,seq_len", [(8, 160), (2, 160), (8, 520), (2, 520)])
+@pytest.mark.parametrize("hole", [-1e9, -np.inf])
+def test_pair_bias_entries_that_mask_single_pairs(torch_cuda, hole, batch, seq_len):
+    """A pair bias used as a per-(query, key) mask: a tenth of its entries at -1e9 or -inf, never a whole row.  The
+    reference's fp32 add (src/attention/gating_attention.cpp:113-117) gives those pairs zero weight.  The fragment-major
+    copy carries them as the largest fp16 magnitude; the routes that read the pair bias in place (batch 2: the copy does
+    not fit the q tensor) turn -inf into the most negative finite bf16 on its way into the selector product."""
+    w = make_workload(3, batch=batch, seq_len=seq_len)
+    rng = np.random.default_rng(5)
+    holes = rng.random(w.nb.shape) < 0.1
+    holes[..., 0] = False  # every query keeps at least one key
+    w.nb = np.where(holes, np.float32(hole), w.nb).astype(np.float32)
+    op, ten, scratch = helpers.make_op(w)
+    op.run()
+    assert not capi.error_flag() and capi.last_path() == "fused_mfma"
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, "gated average")
+    helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
+
+
 def test_fully_masked_and_leading_masked_rows_short_sequence(torch_cuda):
     """Rows whose every key is masked (uniform average of V) and rows whose first key tile is masked, at a
     sequence length the one-workgroup-per-head kernel handles."""
