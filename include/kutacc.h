@@ -100,7 +100,11 @@ typedef struct kutacc_af2_attention_inputs {
  *
  *   input            [batch*seq_len, nchannels], already layer-normalised
  *   bias             [batch, 1, 1, seq_len] mask bias (0 or -1e9), element (b,k) at b*strides[0]+k
- *   nonbatched_bias  [nheads, seq_len, seq_len]; a tensor whose sizes[0]==0 means "absent"
+ *   nonbatched_bias  [nheads, seq_len, seq_len]; a tensor whose sizes[0]==0 means "absent".  Entries of -inf or below
+ *                    -45 000 exclude a (query, key) pair, as in the reference.  One corner differs: for a query that
+ *                    has no key left whose mask bias is 0 and whose pair bias is above that bound, the reference
+ *                    attends uniformly over the keys the mask bias excludes, the MFMA kernels over the keys the pair
+ *                    bias excludes (they carry such entries as the largest fp16 magnitude, which lies above -1e9)
  *   out              [batch, seq_len, nchannels]
  *   block_size       query tiling of the CPU implementation; validated (>0), otherwise advisory
  *
