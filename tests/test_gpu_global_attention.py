@@ -65,6 +65,9 @@ SHAPES = [
     # B, S, H, d, mask
     (4, 128, 8, 8, "random"), (3, 97, 8, 8, "random"), (2, 1024, 8, 8, "random"), (5, 33, 4, 16, "random"),
     (2, 200, 2, 32, "ones"), (3, 1, 8, 8, "ones"), (6, 7, 16, 4, "random"), (2, 1500, 8, 8, "random"),
+    # both workgroup sizes of the kernel: eight waves while a row has a CU to itself (at most 256 rows) or is streamed,
+    # four when two rows share a CU
+    (300, 512, 8, 8, "random"), (257, 1024, 4, 16, "random"), (256, 640, 8, 8, "random"), (3, 2100, 4, 16, "random"),
 ]
 
 
@@ -74,9 +77,10 @@ def test_global_attention_matches_oracle(torch_cuda, B, S, H, d, mask_mode):
     op, ten, scratch = device_op(torch_cuda, c)
     op.run()
     assert not capi.error_flag() and capi.last_path() == "global_mfma"
-    ref, ref_qavg = oracle_out(c)
-    helpers.check_close(helpers.to_numpy(ten["out"]), ref, "bf16", "global attention out")
-    helpers.assert_within(helpers.to_numpy(scratch["avg"]), ref_qavg, 2.0 ** -8 * np.abs(ref_qavg) + 1e-6, "masked mean q_avg")
+    rows = list(range(B)) if B <= 8 else sorted({0, 1, B // 2, B - 2, B - 1})  # large batches: the oracle on a few rows
+    ref, ref_qavg = oracle_out(dict(c, x=c["x"][rows], mask=c["mask"][rows]))
+    helpers.check_close(helpers.to_numpy(ten["out"][rows]), ref, "bf16", "global attention out")
+    helpers.assert_within(helpers.to_numpy(scratch["avg"][rows]), ref_qavg, 2.0 ** -8 * np.abs(ref_qavg) + 1e-6, "masked mean q_avg")
 
 
 def test_global_attention_full_extra_msa_shape(torch_cuda):
