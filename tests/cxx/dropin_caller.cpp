@@ -160,6 +160,68 @@ __attribute__((visibility("default"))) int dropin_gating_attention(void *input, 
     return unset.get_tensor() == nullptr ? 0 : 1;
 }
 
+// kutacc_af2_global_attention on the caller's memory, tensors described as the reference's operator reads them (reference
+// src/attention/global_attention.cpp:30-164, include/kutacc.h:292-307): q_data [batch, seq_len, 64], q_mask
+// [batch, seq_len, 1], query/gating/output weights [64, 64], key/value weights [head_size, 64], scratch q and avg
+// [batch, 64], k [batch*seq_len, head_size], v [head_size, batch*seq_len], gate [batch, seq_len, 64].
+__attribute__((visibility("default"))) int dropin_global_attention(void *q_data, void *q_mask, void *q, void *k, void *v,
+                                                                  void *gate, void *avg, void *query_w, void *key_w,
+                                                                  void *value_w, void *gating_w, void *gating_b, void *output_w,
+                                                                  void *output_b, void *out, int64_t batch, int64_t seq_len,
+                                                                  int64_t nheads, int64_t head_size)
+{
+    const int64_t B = batch, S = seq_len, H = nheads, d = head_size, C = H * d;
+    const kutacc::DType bf16 = kutacc::kBF16;
+    TensorWrapper t_x(q_data, dims({B, S, C}), dims({S * C, C, 1}), 3, bf16);
+    TensorWrapper t_mask(q_mask, dims({B, S, 1}), dims({S, 1, 1}), 3, bf16);
+    TensorWrapper t_q(q, dims({B, C}), dims({C, 1}), 2, bf16), t_avg(avg, dims({B, C}), dims({C, 1}), 2, bf16);
+    TensorWrapper t_k(k, dims({B * S, d}), dims({d, 1}), 2, bf16), t_v(v, dims({d, B * S}), dims({B * S, 1}), 2, bf16);
+    TensorWrapper t_gate(gate, dims({B, S, C}), dims({S * C, C, 1}), 3, bf16);
+    TensorWrapper t_wq(query_w, dims({C, C}), dims({C, 1}), 2, bf16), t_wk(key_w, dims({d, C}), dims({C, 1}), 2, bf16);
+    TensorWrapper t_wv(value_w, dims({d, C}), dims({C, 1}), 2, bf16), t_wg(gating_w, dims({C, C}), dims({C, 1}), 2, bf16);
+    TensorWrapper t_wo(output_w, dims({C, C}), dims({C, 1}), 2, bf16);
+    TensorWrapper t_bg(gating_b, dims({C}), dims({1}), 1, bf16), t_bo(output_b, dims({C}), dims({1}), 1, bf16);
+    TensorWrapper t_out(out, dims({B, S, C}), dims({S * C, C, 1}), 3, bf16);
+    kutacc_af2_attention_weights_t weights = {C,
+                                              H,
+                                              d,
+                                              t_wq.get_tensor(),
+                                              t_wk.get_tensor(),
+                                              t_wv.get_tensor(),
+                                              t_wg.get_tensor(),
+                                              t_bg.get_tensor(),
+                                              t_wo.get_tensor(),
+                                              t_bo.get_tensor()};
+    kutacc_af2_attention_inputs_t inputs = {B,
+                                            S,
+                                            t_q.get_tensor(),
+                                            t_k.get_tensor(),
+                                            t_v.get_tensor(),
+                                            t_gate.get_tensor(),
+                                            t_avg.get_tensor()};
+    kutacc_af2_global_attention(&inputs, t_x.get_tensor(), t_mask.get_tensor(), &weights, t_out.get_tensor());
+    return 0;
+}
+
+// kutacc_af2_transition on the caller's memory (reference src/attention/transition.cpp:21-67, include/kutacc.h:194-214,
+// 321-322): input_act and out [batch, n_res, c_o], linear1_w [c_i, c_o], linear2_w [c_o, c_i], fp32 biases,
+// intermediate_act [batch*n_res, c_i].
+__attribute__((visibility("default"))) int dropin_transition(void *input_act, void *intermediate_act, void *linear1_w,
+                                                            void *linear1_b, void *linear2_w, void *linear2_b, void *out,
+                                                            int64_t batch, int64_t n_res, int64_t c_o, int64_t c_i)
+{
+    const kutacc::DType bf16 = kutacc::kBF16;
+    TensorWrapper t_x(input_act, dims({batch, n_res, c_o}), dims({n_res * c_o, c_o, 1}), 3, bf16);
+    TensorWrapper t_mid(intermediate_act, dims({batch * n_res, c_i}), dims({c_i, 1}), 2, bf16);
+    TensorWrapper t_w1(linear1_w, dims({c_i, c_o}), dims({c_o, 1}), 2, bf16), t_w2(linear2_w, dims({c_o, c_i}), dims({c_i, 1}), 2, bf16);
+    TensorWrapper t_b1(linear1_b, dims({c_i}), dims({1}), 1, bf16), t_b2(linear2_b, dims({c_o}), dims({1}), 1, bf16);
+    TensorWrapper t_out(out, dims({batch, n_res, c_o}), dims({n_res * c_o, c_o, 1}), 3, bf16);
+    kutacc_af2_trans_act_inputs_t inputs = {batch, n_res, t_x.get_tensor(), t_mid.get_tensor()};
+    kutacc_af2_trans_weights_t weights = {c_o, c_i, t_w1.get_tensor(), t_b1.get_tensor(), t_w2.get_tensor(), t_b2.get_tensor()};
+    kutacc_af2_transition(&inputs, &weights, t_out.get_tensor());
+    return 0;
+}
+
 // kutacc_af2_linear_weight_prepack through the header's prototype, default argument included
 __attribute__((visibility("default"))) void dropin_prepack(const void *weight, void *result, int64_t n, int64_t k, int64_t ldb)
 {

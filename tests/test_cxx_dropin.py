@@ -41,6 +41,8 @@ def load(which):
     L.dropin_gating_attention.argtypes = [_vp] * 16 + [_i64] * 5
     L.dropin_prepack.argtypes = [_vp, _vp, _i64, _i64, _i64]
     L.dropin_prepack.restype = None
+    L.dropin_global_attention.argtypes = [_vp] * 15 + [_i64] * 4
+    L.dropin_transition.argtypes = [_vp] * 7 + [_i64] * 4
     return L
 
 
@@ -112,6 +114,44 @@ def test_cxx_caller_matches_ctypes_handle_path(which, config, batch, seq):
     assert helpers.same_bits(ten2["out"], ten["out"]), "out differs from the ctypes-handle path"
     assert helpers.same_bits(scratch2["avg"], scratch["avg"]), "gated average differs from the ctypes-handle path"
     helpers.check_close(helpers.to_numpy(ten2["out"]), helpers.oracle_out(w), w.dtype, "out")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", ["own_header", "reference_header"])
+def test_cxx_caller_global_attention_and_transition(which):
+    """The other two operators with struct arguments, called from C++ through TensorWrapper handles
+    (kutacc_af2_global_attention, reference include/kutacc.h:292-307; kutacc_af2_transition, :194-214, 321-322): results
+    equal the ctypes-handle path bit for bit."""
+    import torch
+    assert torch.cuda.is_available(), "this test needs the GPU"
+    import test_gpu_global_attention as G
+    import test_gpu_pair_stack as P
+    L = load(which)
+    capi.set_stream(None)
+    capi.set_blocking(True)
+    c = G.make_case(31, 5, 300, 8, 8, "random")
+    op, ten, scratch = G.device_op(torch, c)
+    op.run()
+    assert not capi.error_flag()
+    op2, ten2, scratch2 = G.device_op(torch, c)  # a second set of tensors; op2 itself is not run
+    rc = L.dropin_global_attention(_ptr(ten2["x"]), _ptr(ten2["mask"]), _ptr(scratch2["q"]), _ptr(scratch2["k"]),
+                                   _ptr(scratch2["v"]), _ptr(scratch2["gate"]), _ptr(scratch2["avg"]), _ptr(ten2["wq"]),
+                                   _ptr(ten2["wk"]), _ptr(ten2["wv"]), _ptr(ten2["wg"]), _ptr(ten2["bg"]), _ptr(ten2["wo"]),
+                                   _ptr(ten2["bo"]), _ptr(ten2["out"]), 5, 300, 8, 8)
+    torch.cuda.synchronize()
+    assert rc == 0 and not capi.error_flag() and capi.last_path() == "global_mfma"
+    assert helpers.same_bits(ten2["out"], ten["out"]), "global attention: out differs from the ctypes-handle path"
+
+    t = P.transition_case(77, 2, 90, 128, 512)
+    want, _ = P.run_transition(torch, t)
+    x, w1, w2 = (P.dev(torch, t[k]) for k in ("x", "w1", "w2"))
+    b1, b2 = P.dev(torch, t["b1"], torch.float32), P.dev(torch, t["b2"], torch.float32)
+    mid = torch.zeros((2 * 90, 512), dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros((2, 90, 128), dtype=torch.bfloat16, device="cuda")
+    rc = L.dropin_transition(_ptr(x), _ptr(mid), _ptr(w1), _ptr(b1), _ptr(w2), _ptr(b2), _ptr(out), 2, 90, 128, 512)
+    torch.cuda.synchronize()
+    assert rc == 0 and not capi.error_flag()
+    assert helpers.same_bits(out, want), "transition: out differs from the ctypes-handle path"
 
 
 @pytest.mark.gpu
