@@ -423,7 +423,11 @@ def main():
                    "flops_per_call": w.flops(), "algorithmic_bytes_per_call": w.algorithmic_bytes(),
                    "path": capi.last_path()},
         "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        "kernels": [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in kk.items()} for kk in kernels],
+        # avg_ms: net of the event-bracket overhead (see above); avg_ms_bracketed: as the event pair read it
+        "kernels": [{**{k: (round(v, 5) if isinstance(v, float) else v) for k, v in kk.items()},
+                     "avg_ms": round(kk["avg_ms"] - overhead_ms, 5), "avg_ms_bracketed": round(kk["avg_ms"], 5)}
+                    for kk in kernels],
+        "event_bracket_overhead_ms": round(overhead_ms, 5),
         "roofline": roofline,
         "cpu_baseline": None if a.no_cpu else cpu_baseline(w),
     }
