@@ -89,16 +89,25 @@ struct StagingPool {
     struct Block {
         void *dev;
         size_t bytes;
+        int device; // the device the memory lives on: a block is only handed out again there
     };
     std::mutex mu;
     std::vector<Block> free_blocks;
+    static int current_device()
+    {
+        int d = 0;
+        (void)hipGetDevice(&d);
+        return d;
+    }
     hipError_t take(size_t bytes, void **out, size_t *got)
     {
         {
+            const int here = current_device();
             std::lock_guard<std::mutex> lk(mu);
             int best = -1;
             for (int i = 0; i < (int)free_blocks.size(); ++i) {
-                if (free_blocks[i].bytes >= bytes && (best < 0 || free_blocks[i].bytes < free_blocks[best].bytes)) {
+                if (free_blocks[i].device == here && free_blocks[i].bytes >= bytes &&
+                    (best < 0 || free_blocks[i].bytes < free_blocks[best].bytes)) {
                     best = i;
                 }
             }
@@ -113,8 +122,9 @@ struct StagingPool {
     }
     void give(void *dev, size_t bytes)
     {
+        const int here = current_device(); // a call takes and gives on the same current device
         std::lock_guard<std::mutex> lk(mu);
-        free_blocks.push_back({dev, bytes});
+        free_blocks.push_back({dev, bytes, here});
     }
     size_t release()
     {
