@@ -157,6 +157,7 @@ __device__ __forceinline__ void make_selectors_f16(int lane, f16x8 &sel0, f16x8 
 // [64w, 64w+64); *flag_word must have been zeroed before, with a barrier in between.
 // bias_row[k * stride_k] is the mask bias itself, or (from_mask) the 0/1 mask, turned into 1e9*(mask-1) here with the
 // same multiply-add and bf16 rounding as the stand-alone mask-bias pass.
+template <bool NEAR = false> // NEAR: S * stride_k < 2^31 and stride_k < 2^24 (checked on the host), 32-bit offsets
 __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *mask, uint32_t *flag_word, int S, int NB,
                                                 int wave, int lane, float scale = 1.0f, int64_t stride_k = 1,
                                                 bool from_mask = false)
@@ -165,7 +166,7 @@ __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *m
     if (wave * 64 < NB * 32) {
         float mv = -INFINITY;
         if (k < S) {
-            mv = to_f32(bias_row[k * stride_k]);
+            mv = to_f32(bias_row[NEAR ? (int64_t)__umul24((uint32_t)k, (uint32_t)stride_k) : k * stride_k]);
             if (from_mask) {
                 mv = to_f32((bf16_t)fmaf(mv, 1e9f, -1e9f));
             }
@@ -1161,12 +1162,13 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         // loop, where there is no register for them -- spilled, each costs a scratch round trip per batch row.
         int lane_x = lane;
         asm volatile("" : "+v"(lane_x));
-        stage_mask_part(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane_x, mask_scale, p.bias_sk,
-                        p.bias_is_mask != 0);
+        stage_mask_part<true>(p.bias + (int64_t)b * p.bias_sb, mask, flag_word, S, NT, wave, lane_x, mask_scale, p.bias_sk,
+                              p.bias_is_mask != 0);
 
         // ---- input rows of the block -> fragments, 64 channels per staging panel ----
         const int prow_x = pi_row(lane_x & 31), g_x = lane_x >> 5;
         const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
+        const uint32_t x_pitch = (uint32_t)p.x_ld; // the host sends only near-addressable rows here
         bf16x8 xf[CK];
         if constexpr (FUSED_LN) {
             // The rows arrive un-normalised and are normalised between their load and their staging (arithmetic of
@@ -1176,7 +1178,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             PanelRegs t[NP];
 #pragma unroll
             for (int c = 0; c < NP; ++c) {
-                t[c] = panel_load(xb, p.x_ld, j * 32, S - 1, c * 64, lane_x);
+                t[c] = panel_load_near(xb + c * 64, x_pitch, j * 32, S - 1, 0, lane_x);
             }
             float gm[NP][8], bt[NP][8];
 #pragma unroll
@@ -1250,11 +1252,11 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             }
         } else {
             PanelRegs ta, tb;
-            ta = panel_load(xb, p.x_ld, j * 32, S - 1, 0, lane_x);
+            ta = panel_load_near(xb, x_pitch, j * 32, S - 1, 0, lane_x);
 #pragma unroll
             for (int c = 0; c < NP; c += 2) {
                 if (c + 1 < NP) {
-                    tb = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 1) * 64, lane_x);
+                    tb = panel_load_near(xb + (c + 1) * 64, x_pitch, j * 32, S - 1, 0, lane_x);
                 }
                 panel_store(panel, lane_x, ta);
 #pragma unroll
@@ -1263,7 +1265,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                 }
                 if (c + 1 < NP) {
                     if (c + 2 < NP) {
-                        ta = panel_load(xb, p.x_ld, j * 32, S - 1, (c + 2) * 64, lane_x);
+                        ta = panel_load_near(xb + (c + 2) * 64, x_pitch, j * 32, S - 1, 0, lane_x);
                     }
                     panel_store(panel, lane_x, tb);
 #pragma unroll
@@ -1307,19 +1309,23 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             }
             q0 = pack8(acc, 0);
             q1 = pack8(acc, 8);
-            acc = zero16();
-#pragma unroll
-            for (int ks = 0; ks < CK; ++ks) {
-                acc = mfma(as_bf16x8(wsrc[(PROJ_G * CK + ks) * 64]), xf[ks], acc);
-            }
+            // the gate's accumulator starts at its bias (register v of a lane holds feature 8 (v / 4) + 4 g + v % 4)
             const float *bgp = p.bg + h * HEAD + 4 * g_x;
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 const f32x4 bv = *reinterpret_cast<const f32x4 *>(bgp + 8 * a);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    acc[4 * a + c] = sigmoid_fast(acc[4 * a + c] + bv[c]);
+                    acc[4 * a + c] = bv[c];
                 }
+            }
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                acc = mfma(as_bf16x8(wsrc[(PROJ_G * CK + ks) * 64]), xf[ks], acc);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                acc[v] = sigmoid_fast(acc[v]);
             }
             gate_park_x[0] = as_uint4(pack8(acc, 0));
             gate_park_x[64] = as_uint4(pack8(acc, 8));
@@ -2100,6 +2106,10 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
     if (a.batch > (1 << 24) || a.seq_len > 1024) {
         return false;
     }
+    // the kernels address the rows of one batch row with 32-bit byte offsets from its first element
+    if (a.input_ld <= 0 || a.input_ld > (1 << 19)) {
+        return false;
+    }
     // 16-byte row loads of input and weights, 8-byte stores of avg/out rows
     if (a.input_ld % 8 != 0 || !aligned(a.input, 16) || !aligned(a.query_w, 16) || !aligned(a.key_w, 16) ||
         !aligned(a.value_w, 16) || !aligned(a.gating_w, 16) || !aligned(a.output_w, 16) || !aligned(a.gating_b, 16) ||
@@ -2121,6 +2131,9 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     Plan pl;
     if (!make_plan(a.seq_len, C, pl)) {
         return KUTACC_HIP_EUNSUPPORTED;
+    }
+    if (opt.bias_stride_k < 0 || opt.bias_stride_k > (1 << 20) || a.input_ld <= 0 || a.input_ld > (1 << 19)) {
+        return KUTACC_HIP_EUNSUPPORTED; // 32-bit offsets within a batch row (fused_attention_supports checks input_ld too)
     }
     FusedParams p;
     p.x = (const bf16_t *)a.input;

@@ -153,13 +153,34 @@ __device__ __forceinline__ PanelRegs panel_load(const bf16_t *base, int64_t ld, 
     return p;
 }
 
+// The same four loads for a matrix whose last wanted element lies less than 2^31 bytes past `base` and whose row pitch
+// is below 2^23 elements (the host checks both before it picks a kernel that calls this): the lane's part of each
+// address is then a 32-bit byte offset from the wave-uniform base -- one 24-bit multiply, and an add and a min per
+// row -- where 64-bit pointer arithmetic spends three quarter-rate multiplies per row.
+__device__ __forceinline__ PanelRegs panel_load_near(const bf16_t *base, uint32_t ld, int row0, int last_row, int col0, int lane)
+{
+    const char *bytes = reinterpret_cast<const char *>(base);
+    const uint32_t pitch = 2u * ld;
+    const uint32_t col = 2u * (uint32_t)col0 + 16u * (uint32_t)(lane & 7);
+    const uint32_t last = (uint32_t)last_row * pitch + col;
+    const uint32_t first = __umul24((uint32_t)(row0 + (lane >> 3)), pitch) + col;
+    PanelRegs p;
+    p.r0 = *reinterpret_cast<const uint4 *>(bytes + min(first, last));
+    p.r1 = *reinterpret_cast<const uint4 *>(bytes + min(first + 8u * pitch, last));
+    p.r2 = *reinterpret_cast<const uint4 *>(bytes + min(first + 16u * pitch, last));
+    p.r3 = *reinterpret_cast<const uint4 *>(bytes + min(first + 24u * pitch, last));
+    return p;
+}
+
 __device__ __forceinline__ void panel_store(uint4 *panel, int lane, const PanelRegs &p)
 {
-    const int row = lane >> 3, chunk = lane & 7;
-    panel[panel_slot(row, chunk)] = p.r0;
-    panel[panel_slot(row + 8, chunk)] = p.r1;
-    panel[panel_slot(row + 16, chunk)] = p.r2;
-    panel[panel_slot(row + 24, chunk)] = p.r3;
+    // panel_slot(lane / 8 + 8 i, lane % 8) for i = 0..3, written out: rows 0..7 swizzle by the row itself, and rows
+    // 16..31 flip bit 0 on top of that
+    const int s0 = (lane & 0x38) | ((lane ^ (lane >> 3)) & 7);
+    panel[s0] = p.r0;
+    panel[s0 + 64] = p.r1;
+    panel[(s0 ^ 1) + 128] = p.r2;
+    panel[(s0 ^ 1) + 192] = p.r3;
 }
 
 // 8 x 8 transposition of 16-bit elements over the eight lanes that differ in lane bits 3, 4, 5 (same lane & 7).
