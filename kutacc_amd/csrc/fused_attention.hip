@@ -886,6 +886,104 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         if (pi == 0) {
             TL(2);
         }
+        if constexpr (C == 128 && BPW >= 3) {
+            // Two blocks of the wave per walk over the weight fragments: the input fragments of both stay in registers
+            // (64 of them) and every fragment of the weights is read from LDS once for the pair (1 KB per MFMA when the
+            // blocks are projected one after the other); all rows of a pair are asked for at once.  A pair whose second
+            // block does not exist projects the first one twice and stores it once.
+#pragma unroll
+            for (int i0 = 0; i0 < BPW; i0 += 2) {
+                constexpr int PAIR = 2;
+                int j0 = wave + i0 * NW;
+                if (j0 >= NB) {
+                    continue;
+                }
+                asm volatile("" : "+s"(j0)); // opaque, as below: addresses are formed per pair, not kept across the loop
+                const bool second = i0 + 1 < BPW && j0 + NW < NB;
+                const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
+                bf16x8 xf[PAIR][CK];
+                int jn[PAIR];
+                jn[0] = j0, jn[1] = second ? j0 + NW : j0;
+                PanelRegs t[PAIR][CK / 4];
+#pragma unroll
+                for (int n = 0; n < PAIR; ++n) {
+#pragma unroll
+                    for (int c = 0; c < CK / 4; ++c) {
+                        t[n][c] = panel_load_near(xb + c * 64, (uint32_t)p.x_ld, jn[n] * 32, S - 1, 0, lane);
+                    }
+                }
+#pragma unroll
+                for (int n = 0; n < PAIR; ++n) {
+                    const int j = jn[n];
+                    uint4 *kslot = lds_k + j * 128, *vslot = lds_v + j * 128 - 128; // panel slots 0-127 and 128-255
+                    const uint4 *fsrc = prow < 16 ? kslot : vslot;
+                    const int srow8 = lane >> 3, chunk = lane & 7;
+#pragma unroll
+                    for (int c = 0; c < CK / 4; ++c) {
+                        kslot[panel_slot(srow8, chunk)] = t[n][c].r0;
+                        kslot[panel_slot(srow8 + 8, chunk)] = t[n][c].r1;
+                        vslot[panel_slot(srow8 + 16, chunk)] = t[n][c].r2;
+                        vslot[panel_slot(srow8 + 24, chunk)] = t[n][c].r3;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            xf[n][4 * c + k] = as_bf16x8(fsrc[panel_slot(prow, 2 * k + g)]);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const uint4 *wsrc = lds_w + m * CK * 64 + lane;
+                    f32x16 acc[PAIR];
+                    acc[0] = zero16(), acc[1] = zero16();
+#pragma unroll
+                    for (int ks = 0; ks < CK; ++ks) {
+                        const bf16x8 wf = as_bf16x8(wsrc[ks * 64]);
+#pragma unroll
+                        for (int n = 0; n < PAIR; ++n) {
+                            // V[s][d]: rows = sequence positions; the others W_h . x^T: rows = head-dim
+                            acc[n] = m == PROJ_V ? mfma(xf[n][ks], wf, acc[n]) : mfma(wf, xf[n][ks], acc[n]);
+                        }
+                    }
+#pragma unroll
+                    for (int n = 0; n < PAIR; ++n) {
+                        if (n == 1 && i0 + 1 >= BPW) {
+                            continue;
+                        }
+                        const int i = i0 + n;
+                        if (m == PROJ_V) {
+                            if (n == 0 || second) {
+                                lds_v[(jn[n] * 2 + 0) * 64 + lane] = as_uint4(pack8(acc[n], 0));
+                                lds_v[(jn[n] * 2 + 1) * 64 + lane] = as_uint4(pack8(acc[n], 8));
+                            }
+                        } else if (m == PROJ_K) {
+                            if (n == 0 || second) {
+                                lds_k[(jn[n] * 2 + 0) * 64 + lane] = as_uint4(pack8(acc[n], 0));
+                                lds_k[(jn[n] * 2 + 1) * 64 + lane] = as_uint4(pack8(acc[n], 8));
+                            }
+                        } else if (m == PROJ_Q) {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                acc[n][v] *= qmul;
+                            }
+                            qf[i][0] = pack8(acc[n], 0);
+                            qf[i][1] = pack8(acc[n], 8);
+                        } else {
+                            const float *bgp = p.bg + h * HEAD + 4 * g;
+#pragma unroll
+                            for (int a = 0; a < 4; ++a) {
+                                const f32x4 bv = *reinterpret_cast<const f32x4 *>(bgp + 8 * a);
+#pragma unroll
+                                for (int c = 0; c < 4; ++c) {
+                                    acc[n][4 * a + c] = sigmoid_fast(acc[n][4 * a + c] + bv[c]);
+                                }
+                            }
+                            gate[i][0] = pack8(acc[n], 0);
+                            gate[i][1] = pack8(acc[n], 8);
+                        }
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < BPW; ++i) {
             int j = wave + i * NW;
@@ -978,6 +1076,7 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
                 }
             }
         }
+        } // one block at a time
     }
     TL(3);
     __syncthreads(); // K and V of the whole sequence are in LDS; the weight fragments are no longer read
