@@ -38,6 +38,9 @@ extern "C" {
 #define KUTACC_HIP_PATH_AUTO 0    /* fused MFMA kernels when the shape allows, else generic      */
 #define KUTACC_HIP_PATH_GENERIC 1 /* shape-agnostic scalar kernels (any head_size, bf16 or fp32)  */
 #define KUTACC_HIP_PATH_FUSED 2   /* bf16 MFMA kernels only; EUNSUPPORTED if the shape is not covered */
+/* The MFMA kernels cover bf16, head_size 32, nheads * 32 in {128, 256}, seq_len <= 1024, 16-byte aligned operands with
+ * leading dimensions that are multiples of 8, and an input row pitch of at most 2^19 elements (they address the rows of
+ * a batch row with 32-bit byte offsets). */
 
 /*
  * Flat argument block of the gated-attention operator.  Replaces, for the launch layer, the

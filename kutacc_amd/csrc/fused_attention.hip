@@ -1531,7 +1531,9 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
     constexpr int NP = CK / 4;
     constexpr int SLABS = C / 128, WAVES = 4 * SLABS, THREADS = 64 * WAVES;
     extern __shared__ uint4 lds[]; // W slabs [SLABS][4 feature blocks][CK][64 lanes], then one panel of 256 per wave
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr bool NEAR = C == 128; // 32-bit row offsets from a wave-uniform base; measured slower with 256 features
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = NEAR ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;
     const int r = lane & 31, g = lane >> 5;
     const int nbase = blockIdx.y * (128 * SLABS);               // first output feature of this workgroup
     // slabs it has: with two per workgroup the last workgroup of a row of them may have one
@@ -1544,11 +1546,21 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
     // stored; those of the first step while the weight slab is staged.
     const int64_t start = ((int64_t)blockIdx.x * WAVES + wave) * rows_per_wave;
     const int64_t stop = start + rows_per_wave < M ? start + rows_per_wave : M;
-    const int last_row = (int)(stop - 1);
+    // With 128 features rows are addressed relative to the wave's first one: 32-bit byte offsets from a wave-uniform
+    // base (the host keeps a wave's range below 2^31 bytes), no 64-bit multiply per row.
+    const int last_rel = (int)(stop - 1 - start);
+    const bf16_t *avg_w = avg + start * avg_ld;
+    auto load_panel = [&](int rel_row, int c, int ln) { // 32 rows from rel_row (relative to start), channels 64 c .. 64 c + 63
+        if constexpr (NEAR) {
+            return panel_load_near(avg_w + c * 64, (uint32_t)avg_ld, rel_row, last_rel, 0, ln);
+        } else {
+            return panel_load(avg, avg_ld, (int)start + rel_row, (int)(stop - 1), c * 64, ln);
+        }
+    };
     PanelRegs ta, tb;
     if (start < stop) {
-        ta = panel_load(avg, avg_ld, (int)start, last_row, 0, lane);
-        tb = panel_load(avg, avg_ld, (int)start, last_row, 64, lane);
+        ta = load_panel(0, 0, lane);
+        tb = load_panel(0, 1, lane);
     }
     {
         constexpr int PER = SLABS * 4 * CK * 64 / THREADS; // weight fragments per thread, all loads issued before the first store
@@ -1569,7 +1581,7 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
     }
     __syncthreads();
     for (int64_t rbase = start; rbase < stop; rbase += 32) {
-        const int row0 = (int)rbase;
+        const int row0 = (int)rbase, rel0 = (int)(rbase - start);
         // With 256 input features the lane index is opaque to the optimiser, so that addresses and panel offsets are
         // formed per step instead of being kept (and partly spilled) across the loop.  With 128 the kernel fits either
         // way, and the smaller footprint would let a third workgroup onto some CUs of a grid sized for two.
@@ -1591,7 +1603,7 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
         }
 #pragma unroll
         for (int c = 2; c < NP; ++c) {
-            ta = panel_load(avg, avg_ld, row0, last_row, c * 64, lv);
+            ta = load_panel(rel0, c, lv);
             panel_store(panel, lv, ta);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -1600,9 +1612,9 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
         }
         {
             // clamped to the last step instead of a branch: one harmless re-read at the end
-            const int rnext = rbase + 32 < stop ? row0 + 32 : row0;
-            ta = panel_load(avg, avg_ld, rnext, last_row, 0, lv);
-            tb = panel_load(avg, avg_ld, rnext, last_row, 64, lv);
+            const int rnext = rbase + 32 < stop ? rel0 + 32 : rel0;
+            ta = load_panel(rnext, 0, lv);
+            tb = load_panel(rnext, 1, lv);
         }
 #pragma unroll 1
         for (int slab = 0; slab < nslab; ++slab) {
@@ -1673,7 +1685,12 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
                     v = as_uint4(res);
                 }
                 if (row < stop) {
-                    *reinterpret_cast<uint4 *>(out + target_row(row) * out_ld + n0 + half * 64 + (lv & 7) * 8) = v;
+                    if constexpr (EPILOGUE == EPILOGUE_RESIDUAL || !NEAR) {
+                        *reinterpret_cast<uint4 *>(out + target_row(row) * out_ld + n0 + half * 64 + (lv & 7) * 8) = v;
+                    } else {
+                        char *out_w = reinterpret_cast<char *>(out + start * out_ld + n0 + half * 64);
+                        *reinterpret_cast<uint4 *>(out_w + (__umul24((uint32_t)(rel0 + prow_), 2u * (uint32_t)out_ld) + 16u * (lv & 7))) = v;
+                    }
                 }
             }
         }
@@ -2161,6 +2178,10 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
     gx = gx > cap ? cap : gx;
     const int64_t rpw = ((M + gx * WAVES - 1) / (gx * WAVES) + 7) / 8 * 8;
     const int64_t gy = (N / 128 + SLABS - 1) / SLABS;
+    const int64_t pitch = a_ld > out_ld ? a_ld : out_ld;
+    if (a_ld <= 0 || out_ld <= 0 || pitch >= (1 << 23) || (rpw + 32) * pitch * 2 >= ((int64_t)1 << 31)) {
+        return KUTACC_HIP_EUNSUPPORTED; // the kernel addresses a wave's rows with 32-bit byte offsets
+    }
     kern<<<dim3((unsigned)gx, (unsigned)gy), 64 * WAVES, lds_bytes, stream>>>(
         (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)N, (int)rpw, (const bf16_t *)gate,
         gate_ld, swap_n);
