@@ -1317,7 +1317,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                 const float nch = (float)C;
                 const float mean = s1 / nch + x0;
                 const float var = fmaxf((s2 - s1 * s1 / nch) / nch, 0.f);
-                const float rstd = 1.0f / sqrtf(var + p.ln_eps);
+                const float rstd = __builtin_amdgcn_rsqf(var + p.ln_eps); // as the row kernels form it
                 const float shift = -rstd * mean;
 #pragma unroll
                 for (int c = 0; c < NP; ++c) {

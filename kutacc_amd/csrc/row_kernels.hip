@@ -5,6 +5,8 @@
 // and reference src/linear/linear.cpp:21-42 (bf16 operands, result rounded to the storage type).
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "device_util.h"
 #include "launch_internal.h"
 #include "mfma_tiles.h"
@@ -142,11 +144,17 @@ __device__ __forceinline__ void group_stats(const float (&x)[8], float x0, float
     s2 = group_sum<LPR>(s2);
     const float mean = s1 / n + x0;
     const float var = fmaxf((s2 - s1 * s1 / n) / n, 0.f);
-    rstd = 1.0f / sqrtf(var + eps);
+    // The hardware's reciprocal square root (1 ulp) instead of an IEEE square root and division: every lane of a row
+    // forms it, the two correctly rounded operations expand to some 25 instructions per lane and row, and the normalised
+    // value is rounded to bf16 afterwards.
+    rstd = __builtin_amdgcn_rsqf(var + eps);
     shift = -rstd * mean;
 }
 
-template <int LPR>
+// NEAR: fewer than 2^24 rows, row pitches below 2^23 elements and less than 2^31 bytes from the first row to the end of
+// the last (the launcher checks): rows are counted in 32 bits and addressed by 32-bit byte offsets from the tensors'
+// first elements -- a 24-bit multiply per row where 64-bit pointer arithmetic spends three quarter-rate ones.
+template <int LPR, bool NEAR>
 __global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *__restrict__ x, int64_t ld_x,
                                                                   const float *__restrict__ gamma,
                                                                   const float *__restrict__ beta, bf16_t *__restrict__ out,
@@ -156,25 +164,36 @@ __global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *
     constexpr int U = 4;          // steps in flight
     const int lane = threadIdx.x & 63;
     const int sub = lane % LPR, grp = lane / LPR;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wave_in_block = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform
     float gm[8], bt[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         gm[e] = gamma[sub * 8 + e];
         bt[e] = beta[sub * 8 + e];
     }
-    const int64_t r0 = wave * (RPS * U);
+    using index_t = std::conditional_t<NEAR, uint32_t, int64_t>;
+    const index_t nrows = (index_t)rows, swap = (index_t)swap_j;
+    const index_t r0 = ((index_t)blockIdx.x * 4 + wave_in_block) * (RPS * U);
+    auto row_ptr = [&](auto *base, int64_t ld, index_t r) {
+        if constexpr (NEAR) {
+            using byte_t = std::conditional_t<std::is_const_v<std::remove_pointer_t<decltype(base)>>, const char, char>;
+            return reinterpret_cast<decltype(base)>(reinterpret_cast<byte_t *>(base) +
+                                                    (__umul24(r, 2u * (uint32_t)ld) + 16u * (uint32_t)sub));
+        } else {
+            return base + r * ld + sub * 8;
+        }
+    };
     Pack16 in[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        int64_t r = r0 + u * RPS + grp;
-        r = r < rows ? r : rows - 1;
-        r = swap_j ? (r % swap_j) * (rows / swap_j) + r / swap_j : r; // input row (j, i) for output row (i, j)
-        in[u].u = *reinterpret_cast<const uint4 *>(x + r * ld_x + sub * 8);
+        index_t r = r0 + u * RPS + grp;
+        r = r < nrows ? r : nrows - 1;
+        r = swap ? (r % swap) * (nrows / swap) + r / swap : r; // input row (j, i) for output row (i, j)
+        in[u].u = *reinterpret_cast<const uint4 *>(row_ptr(x, ld_x, r));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * RPS + grp;
+        const index_t r = r0 + u * RPS + grp;
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -188,8 +207,8 @@ __global__ __launch_bounds__(256) void layernorm_rows_bf16_kernel(const bf16_t *
         for (int e = 0; e < 8; ++e) {
             o.b[e] = (bf16_t)fmaf(fmaf(v[e], rstd, shift), gm[e], bt[e]);
         }
-        if (r < rows) {
-            *reinterpret_cast<uint4 *>(out + r * ld_out + sub * 8) = o.u;
+        if (r < nrows) {
+            *reinterpret_cast<uint4 *>(row_ptr(out, ld_out, r)) = o.u;
         }
     }
 }
@@ -215,24 +234,29 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
     __shared__ uint4 tiles[4][RB * 2 * 256]; // per wave: its rows x 128 channels as 32 x 64 panels
     const int lane = threadIdx.x & 63;
     const int sub = lane & 15, grp = lane >> 4;
-    const int64_t r0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * PAIR_BIAS_ROWS_PER_WAVE;
-    if (r0 >= rows) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: the wave's first row stays in scalar registers
+    // Rows are counted in 32 bits and addressed by 32-bit byte offsets from the tensors' first elements (the launcher
+    // sends at most 2^23 rows here: 2 GiB of z), not by 64-bit products per lane and row.
+    const uint32_t nrows = (uint32_t)rows, ncol = (uint32_t)rows_j, nrow_i = (uint32_t)rows_i;
+    const uint32_t r0 = ((uint32_t)blockIdx.x * 4 + wave) * PAIR_BIAS_ROWS_PER_WAVE;
+    if (r0 >= nrows) {
         return;
     }
-    uint4 *tile = tiles[threadIdx.x >> 6];
+    const char *zbytes = reinterpret_cast<const char *>(z);
+    uint4 *tile = tiles[wave];
     Pack16 in[STEPS];
     {
         // transposed: output row (i, j) is computed from row (j, i) of z, stored [rows_j, rows_i, c_z]; the walk
         // over consecutive output rows then steps through z with stride rows_i rows
-        int64_t r = r0 + grp * STEPS;
-        int64_t i = transposed ? r / rows_j : 0, j = transposed ? r % rows_j : 0;
+        uint32_t r = r0 + grp * STEPS;
+        uint32_t i = transposed ? r / ncol : 0, j = transposed ? r % ncol : 0;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
-            int64_t src = transposed ? j * rows_i + i : r;
-            src = r < rows ? src : 0;
-            in[s].u = *reinterpret_cast<const uint4 *>(z + src * CZ + sub * 8);
+            uint32_t src = transposed ? j * nrow_i + i : r;
+            src = r < nrows ? src : 0;
+            in[s].u = *reinterpret_cast<const uint4 *>(zbytes + (src * (2u * CZ) + 16u * sub));
             ++r;
-            if (++j == rows_j) {
+            if (++j == ncol) {
                 j = 0, ++i;
             }
         }
@@ -259,7 +283,7 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
         const int row_local = grp * STEPS + s;
-        const int64_t r = r0 + row_local;
+        const uint32_t r = r0 + row_local;
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -273,8 +297,8 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
         for (int e = 0; e < 8; ++e) {
             o.b[e] = (bf16_t)fmaf(fmaf(v[e], rstd, shift), gm[e], bt[e]);
         }
-        if (z_norm != nullptr && r < rows) {
-            *reinterpret_cast<uint4 *>(z_norm + r * CZ + sub * 8) = o.u;
+        if (z_norm != nullptr && r < nrows) {
+            *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(z_norm) + (r * (2u * CZ) + 16u * sub)) = o.u;
         }
         tile[((row_local >> 5) * 2 + (sub >> 3)) * 256 + kutacc_dev::panel_slot(row_local & 31, sub & 7)] = o.u;
     }
@@ -289,12 +313,14 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
             acc = kutacc_dev::mfma(wf[ks], kutacc_dev::as_bf16x8(zf), acc);
         }
         // accumulator v < 4 of lane (col, g) is head 4 g + v of z row r0 + 32 rb + col
-        const int64_t r = r0 + rb * 32 + col;
-        if (r < rows) {
+        const uint32_t r = r0 + rb * 32 + col;
+        if (r < nrows) {
+            char *nbytes = reinterpret_cast<char *>(nb);
+            const uint32_t first = 2u * (__umul24(4u * g, nrows) + r); // head 4 g of row r, in bytes; H * rows * 2 < 2^28
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 if (4 * g + v < H) {
-                    nb[(int64_t)(4 * g + v) * rows + r] = (bf16_t)acc[v];
+                    *reinterpret_cast<bf16_t *>(nbytes + (first + 2u * v * nrows)) = (bf16_t)acc[v];
                 }
             }
         }
@@ -316,8 +342,8 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
             if (lane < 4 * H) {
                 const int h = lane >> 2, c = lane & 3;
                 const uint4 val = *reinterpret_cast<const uint4 *>(t16 + h * 32 + c * 8);
-                const int64_t r0b = r0 + rb * 32;
-                const int q = (int)(r0b / rows_j), t = (int)(r0b % rows_j) >> 5, qr = q & 31;
+                const uint32_t r0b = r0 + rb * 32;
+                const int q = (int)(r0b / ncol), t = (int)(r0b % ncol) >> 5, qr = q & 31;
                 const int qlane = (qr & 3) | (((qr >> 4) & 1) << 2) | (((qr >> 2) & 3) << 3);
                 uint4 *dst = nbf + ((((int64_t)h * frag_nb + (q >> 5)) * frag_nt + t) * 2 + (c & 1)) * 64 + qlane + 32 * (c >> 1);
                 *dst = val;
@@ -343,11 +369,14 @@ int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const floa
         }
         const bf16_t *xi = (const bf16_t *)x;
         bf16_t *oi = (bf16_t *)out;
+        const int64_t pitch = ld_x > ld_out ? ld_x : ld_out;
+        const bool near = rows < (1 << 24) && pitch < (1 << 23) && rows * pitch * 2 < ((int64_t)1 << 31);
+        auto launch = [&](auto kernel) { kernel<<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); };
         switch (lpr) {
-            case 8: layernorm_rows_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
-            case 16: layernorm_rows_bf16_kernel<16><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
-            case 32: layernorm_rows_bf16_kernel<32><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
-            default: layernorm_rows_bf16_kernel<64><<<(unsigned)nblk, 256, 0, stream>>>(xi, ld_x, gamma, beta, oi, ld_out, rows, eps, swap_j); break;
+            case 8: near ? launch(layernorm_rows_bf16_kernel<8, true>) : launch(layernorm_rows_bf16_kernel<8, false>); break;
+            case 16: near ? launch(layernorm_rows_bf16_kernel<16, true>) : launch(layernorm_rows_bf16_kernel<16, false>); break;
+            case 32: near ? launch(layernorm_rows_bf16_kernel<32, true>) : launch(layernorm_rows_bf16_kernel<32, false>); break;
+            default: near ? launch(layernorm_rows_bf16_kernel<64, true>) : launch(layernorm_rows_bf16_kernel<64, false>); break;
         }
         return kutacc_hip_status(hipGetLastError());
     }
@@ -372,7 +401,8 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
          frag_nb != rows_j / 32 || frag_nt != ((frag_nb + 1) & ~1))) {
         return KUTACC_HIP_EINVAL;
     }
-    if (sizeof(T) == 2 && c_z == 128 && (nheads == 4 || nheads == 8) &&
+    // the MFMA kernel counts rows and byte offsets in 32 bits: at most 2^23 rows of 256 bytes
+    if (sizeof(T) == 2 && c_z == 128 && (nheads == 4 || nheads == 8) && rows <= ((int64_t)1 << 23) &&
         (reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(z_norm)) % 16 == 0) {
         const int64_t nblk = (rows + 4 * PAIR_BIAS_ROWS_PER_WAVE - 1) / (4 * PAIR_BIAS_ROWS_PER_WAVE);
         if (nblk > INT32_MAX) {
