@@ -1514,7 +1514,11 @@ constexpr int EPILOGUE_STORE = 0, EPILOGUE_GATED_RESIDUAL = 1, EPILOGUE_RESIDUAL
 // With 256 input features a workgroup has eight waves and keeps two 128-feature slabs of Wo (128 KB, the whole matrix of
 // the attention's output projection), so a row is read once for all 256 output features; with 128 it has four waves,
 // one slab, and two workgroups share a CU.
-template <int C, int EPILOGUE>
+// NEAR_OUT (residual epilogue only): fewer than 2^24 rows, less than 2^31 bytes of `out`, swap_n zero or at least 32 (the
+// launcher checks): the rows of `out` are found with 32-bit arithmetic -- one division of a wave-uniform row index per
+// 32-row step and an add, a compare and two 24-bit multiplies per row -- where 64-bit division and remainder per lane
+// and row are some 300 quarter-rate instructions per step.
+template <int C, int EPILOGUE, bool NEAR_OUT = false>
 __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output_projection_kernel(
     const bf16_t *__restrict__ avg, int64_t avg_ld, const bf16_t *__restrict__ wo, const float *__restrict__ bo,
     bf16_t *__restrict__ out, int64_t out_ld, int64_t M, int N, int rows_per_wave, const bf16_t *__restrict__ gate,
@@ -1610,6 +1614,27 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
                 af[4 * c + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
             }
         }
+        uint32_t out_off[4]; // NEAR_OUT: byte offsets of this lane's four rows of `out` (rows past the end: the last one)
+        if constexpr (EPILOGUE == EPILOGUE_RESIDUAL && NEAR_OUT) {
+            const uint32_t n32 = (uint32_t)swap_n, nb32 = n32 ? (uint32_t)M / n32 : 0u;
+            const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane(row0);
+            const uint32_t b0 = n32 ? first / n32 : 0u, s0 = first - b0 * n32; // row (b0, s0) of the [M / n, n] grid
+            const uint32_t last_rel = (uint32_t)(stop - 1 - rbase);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t pr = 8u * i + ((uint32_t)lv >> 3);
+                pr = pr < last_rel ? pr : last_rel;
+                uint32_t target = first + pr;
+                if (n32) { // (b, s) -> (s, b); the 32 rows of a step wrap at most once (n >= 32)
+                    uint32_t sq = s0 + pr, bq = b0;
+                    if (sq >= n32) {
+                        sq -= n32, bq += 1;
+                    }
+                    target = __umul24(sq, nb32) + bq;
+                }
+                out_off[i] = __umul24(target, 2u * (uint32_t)out_ld) + 16u * ((uint32_t)lv & 7u);
+            }
+        }
         {
             // clamped to the last step instead of a branch: one harmless re-read at the end
             const int rnext = rbase + 32 < stop ? rel0 + 32 : rel0;
@@ -1633,7 +1658,11 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
                     if constexpr (EPILOGUE == EPILOGUE_GATED_RESIDUAL) {
                         gq[i] = *reinterpret_cast<const uint4 *>(gate + row * gate_ld + col);
                     }
-                    zq[i] = *reinterpret_cast<const uint4 *>(out + target_row(row) * out_ld + col);
+                    if constexpr (EPILOGUE == EPILOGUE_RESIDUAL && NEAR_OUT) {
+                        zq[i] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(out + n0 + half * 64) + out_off[i]);
+                    } else {
+                        zq[i] = *reinterpret_cast<const uint4 *>(out + target_row(row) * out_ld + col);
+                    }
                 }
             }
             f32x16 acc[2];
@@ -1685,7 +1714,9 @@ __global__ __launch_bounds__(C == 128 ? 256 : 512, C == 128 ? 2 : 1) void output
                     v = as_uint4(res);
                 }
                 if (row < stop) {
-                    if constexpr (EPILOGUE == EPILOGUE_RESIDUAL || !NEAR) {
+                    if constexpr (EPILOGUE == EPILOGUE_RESIDUAL && NEAR_OUT) {
+                        *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(out + n0 + half * 64) + out_off[i]) = v;
+                    } else if constexpr (EPILOGUE == EPILOGUE_RESIDUAL || !NEAR) {
                         *reinterpret_cast<uint4 *>(out + target_row(row) * out_ld + n0 + half * 64 + (lv & 7) * 8) = v;
                     } else {
                         char *out_w = reinterpret_cast<char *>(out + start * out_ld + n0 + half * 64);
@@ -1722,33 +1753,38 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
 {
     constexpr int C = 128, CK = C / 16;
     extern __shared__ uint4 lds[]; // [Wo, Wg][4 feature blocks][CK][64 lanes], then 4 panels of 256
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform
     uint4 *panel = lds + 2 * 4 * CK * 64 + wave * 256;
     const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
     const int64_t stop = start + rows_per_wave < M ? start + rows_per_wave : M;
-    const int last_row = (int)(stop - 1);
+    // Rows are addressed relative to the wave's first one, by 32-bit byte offsets from wave-uniform bases; positions of
+    // the channel-first tensor by 32-bit offsets from its first element (the launcher checks that both fit).
+    const int last_rel = (int)(stop - 1 - start);
+    const bf16_t *y_w = y + start * y_ld, *x_w = x + start * x_ld;
+    const uint32_t y_pitch = (uint32_t)y_ld, x_pitch = (uint32_t)x_ld, m32 = (uint32_t)M;
     // the first 64 features of the next step's rows of y and x are requested a step ahead; the second 64 at the top of
     // their own step, behind the first (four sets of registers held across a step do not fit)
     // channel-first x: 64 channels (from c0) x 32 positions (from p0), lane -> channel c0 + 16 i + lane / 4, positions
     // p0 + 8 (lane & 3) .. +7; a chunk past the end of the tensor repeats the last one (M is a multiple of 8)
     auto load_cf = [&](int c0, int64_t p0, int ln) {
-        int64_t pos = p0 + 8 * (ln & 3);
-        pos = pos + 8 <= M ? pos : M - 8;
+        uint32_t pos = (uint32_t)p0 + 8u * (ln & 3);
+        pos = pos + 8u <= m32 ? pos : m32 - 8u;
         PanelRegs t;
-        const bf16_t *src = x + (int64_t)(c0 + (ln >> 2)) * x_ld + pos;
-        t.r0 = *reinterpret_cast<const uint4 *>(src);
-        t.r1 = *reinterpret_cast<const uint4 *>(src + 16 * x_ld);
-        t.r2 = *reinterpret_cast<const uint4 *>(src + 32 * x_ld);
-        t.r3 = *reinterpret_cast<const uint4 *>(src + 48 * x_ld);
+        const char *src = reinterpret_cast<const char *>(x + (int64_t)c0 * x_ld);
+        const uint32_t off = 2u * (__umul24((uint32_t)(ln >> 2), x_pitch) + pos), step = 32u * x_pitch; // 16 channels on
+        t.r0 = *reinterpret_cast<const uint4 *>(src + off);
+        t.r1 = *reinterpret_cast<const uint4 *>(src + (off + step));
+        t.r2 = *reinterpret_cast<const uint4 *>(src + (off + 2u * step));
+        t.r3 = *reinterpret_cast<const uint4 *>(src + (off + 3u * step));
         return t;
     };
     PanelRegs ya, xa;
     if (start < stop) {
-        ya = panel_load(y, y_ld, (int)start, last_row, 0, lane);
+        ya = panel_load_near(y_w, y_pitch, 0, last_rel, 0, lane);
         if constexpr (X_CHANNEL_FIRST) {
             xa = load_cf(0, start, lane);
         } else {
-            xa = panel_load(x, x_ld, (int)start, last_row, 0, lane);
+            xa = panel_load_near(x_w, x_pitch, 0, last_rel, 0, lane);
         }
     }
     {
@@ -1769,16 +1805,16 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
     __syncthreads();
     const uint4 *wo_s = lds, *wg_s = lds + 4 * CK * 64;
     for (int64_t rbase = start; rbase < stop; rbase += 32) {
-        const int row0 = (int)rbase;
+        const int rel0 = (int)(rbase - start);
         int lv = lane; // opaque: addresses and panel offsets are formed per step, not kept across the loop
         asm volatile("" : "+v"(lv));
         const int rv = lv & 31, gv = lv >> 5;
-        const int rnext = rbase + 32 < stop ? row0 + 32 : row0; // clamped: one harmless re-read at the end
+        const int rnext = rbase + 32 < stop ? rel0 + 32 : rel0; // clamped: one harmless re-read at the end
         // ---- gate: 128 features of the 32 rows, rounded to bf16, kept in accumulator order ----
         bf16x8 gate[4][2];
         {
             bf16x8 yf[CK];
-            const PanelRegs yb = panel_load(y, y_ld, row0, last_row, 64, lv);
+            const PanelRegs yb = panel_load_near(y_w + 64, y_pitch, rel0, last_rel, 0, lv);
             panel_store(panel, lv, ya);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -1789,7 +1825,7 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
             for (int k = 0; k < 4; ++k) {
                 yf[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
             }
-            ya = panel_load(y, y_ld, rnext, last_row, 0, lv);
+            ya = panel_load_near(y_w, y_pitch, rnext, last_rel, 0, lv);
             const float *gbias = bg + 4 * gv;
 #pragma unroll
             for (int nb_ = 0; nb_ < 4; ++nb_) {
@@ -1859,7 +1895,7 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
                 xf[k] = o;
             }
         } else {
-            const PanelRegs xb = panel_load(x, x_ld, row0, last_row, 64, lv);
+            const PanelRegs xb = panel_load_near(x_w + 64, x_pitch, rel0, last_rel, 0, lv);
             panel_store(panel, lv, xa);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -1870,17 +1906,20 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
             for (int k = 0; k < 4; ++k) {
                 xf[4 + k] = as_bf16x8(panel[panel_slot(rv, 2 * k + gv)]);
             }
-            xa = panel_load(x, x_ld, rnext, last_row, 0, lv);
+            xa = panel_load_near(x_w, x_pitch, rnext, last_rel, 0, lv);
         }
         const float *bias = bo + 4 * gv;
 #pragma unroll
         for (int half = 0; half < 2; ++half) { // 64 output features per panel
             uint4 zq[4]; // the rows of `out` to add to, requested before the MFMAs
+            char *out_w = reinterpret_cast<char *>(out + start * out_ld + half * 64);
+            uint32_t out_off[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                int64_t row = (int64_t)row0 + 8 * i + (lv >> 3);
-                row = row < stop ? row : stop - 1;
-                zq[i] = *reinterpret_cast<const uint4 *>(out + row * out_ld + half * 64 + (lv & 7) * 8);
+                int rel = rel0 + 8 * i + (lv >> 3);
+                rel = rel < last_rel ? rel : last_rel;
+                out_off[i] = __umul24((uint32_t)rel, 2u * (uint32_t)out_ld) + 16u * (lv & 7);
+                zq[i] = *reinterpret_cast<const uint4 *>(out_w + out_off[i]);
             }
             f32x16 acc[2];
             acc[0] = zero16(), acc[1] = zero16();
@@ -1916,9 +1955,8 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
                 for (int e = 0; e < 8; ++e) {
                     res[e] = (bf16_t)(to_f32(z[e]) + to_f32(u[e]));
                 }
-                const int64_t row = (int64_t)row0 + prow_;
-                if (row < stop) {
-                    *reinterpret_cast<uint4 *>(out + row * out_ld + half * 64 + (lv & 7) * 8) = as_uint4(res);
+                if (rel0 + prow_ <= last_rel) {
+                    *reinterpret_cast<uint4 *>(out_w + out_off[i]) = as_uint4(res);
                 }
             }
         }
@@ -2163,11 +2201,14 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
                              int64_t M, int64_t N, hipStream_t stream, const void *gate = nullptr, int64_t gate_ld = 0,
                              int64_t swap_n = 0)
 {
-    auto kern = output_projection_kernel<C, EPILOGUE>;
+    // the residual epilogue finds its rows of `out` with 32-bit arithmetic where the tensor allows
+    const bool near_out = EPILOGUE == EPILOGUE_RESIDUAL && M < (1 << 24) && out_ld > 0 && out_ld < (1 << 22) &&
+                          M * out_ld * 2 < ((int64_t)1 << 31) && (swap_n == 0 || (swap_n >= 32 && M % swap_n == 0));
+    auto kern = near_out ? output_projection_kernel<C, EPILOGUE, EPILOGUE == EPILOGUE_RESIDUAL> : output_projection_kernel<C, EPILOGUE, false>;
     constexpr int SLABS = C / 128, WAVES = 4 * SLABS;
     const size_t lds_bytes = (size_t)SLABS * 4 * (C / 16) * 64 * 16 + WAVES * 4096;
-    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
-    if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
+    static size_t configured[2][KUTACC_DEVICE_SLOTS] = {}; // one table per kernel the pointer may hold
+    if (const int rc = opt_in_lds(kern, lds_bytes, configured[near_out ? 1 : 0])) {
         return rc;
     }
     const int64_t tiles = (M + 31) / 32;
@@ -2376,7 +2417,12 @@ bool row_projection_projected_gate_supports(const void *a, int64_t a_ld, const v
                                             int64_t y_ld, const void *wg, const float *bg, const void *acc, int64_t acc_ld,
                                             int64_t m, int64_t n, int64_t k, int64_t ky)
 {
-    return k == 128 && ky == 128 && n == 128 && m > 0 && m <= INT32_MAX - 64 && bias && bg && y && wg && a_ld % 8 == 0 &&
+    // the kernel addresses rows by 32-bit byte offsets: of a wave's rows from its first one, of a channel-first `a`
+    // (a_ld >= m) from its first element
+    const int64_t lim = (int64_t)1 << 31;
+    const bool near = m < (1 << 23) && a_ld > 0 && a_ld < (1 << 23) && y_ld > 0 && acc_ld > 0 && m * y_ld * 2 < lim &&
+                      m * acc_ld * 2 < lim && (a_ld >= m || m * a_ld * 2 < lim);
+    return k == 128 && ky == 128 && n == 128 && m > 0 && near && bias && bg && y && wg && a_ld % 8 == 0 &&
            y_ld % 8 == 0 && acc_ld % 8 == 0 && aligned(a, 16) && aligned(w, 16) && aligned(bias, 16) && aligned(y, 16) &&
            aligned(wg, 16) && aligned(bg, 16) && aligned(acc, 16);
 }
