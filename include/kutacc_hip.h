@@ -111,7 +111,9 @@ kutacc_export int kutacc_hip_gating_attention_static(const kutacc_hip_attention_
  * :167-205 (entry).  One query per batch row and head (the masked mean of the row), one key/value head
  * shared by all heads.  bf16 storage, nheads*head_size == 64 (the reference hard-wires nchannels == 64,
  * :172), nheads <= 32, head_size <= 32.  The reference's scratch tensors q, k, v, gate are not needed and
- * not touched; q_avg ([B, 64], may be NULL) receives the masked mean as the reference leaves it in `avg`. */
+ * not touched; q_avg ([B, 64], may be NULL) receives the masked mean as the reference leaves it in `avg`.
+ * seq_len <= 16384; the tokens of a batch row must lie within 2 GiB of its first one in q_data and in out (32-bit
+ * offsets in the kernel), else KUTACC_HIP_EUNSUPPORTED. */
 typedef struct kutacc_hip_global_attention_args {
     int64_t batch;     /* B */
     int64_t seq_len;   /* S */

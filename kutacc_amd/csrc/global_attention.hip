@@ -83,6 +83,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
     float *merge = wavg + GC;                                           // [NW waves][64 lanes][MERGE_LD]
 
     const bf16_t *xb = p.x + (int64_t)b * p.x_sb;
+    const uint32_t x_pitch = (uint32_t)p.x_ss; // tokens of a row by 32-bit byte offsets from xb (the launcher checks the range)
 
     // Requested before anything else, so that their latency passes under the staging of the weights: the first tiles of
     // the row (all of a wave's tiles when they are kept in registers and there are at most four) and this thread's slice
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
 #pragma unroll
     for (int i = 0; i < PRE; ++i) {
         const int t = wave + NW * i;
-        ahead[i] = panel_load(xb, p.x_ss, (t < NT ? t : NT - 1) * 32, S - 1, 0, lane);
+        ahead[i] = panel_load_near(xb, x_pitch, (t < NT ? t : NT - 1) * 32, S - 1, 0, lane);
     }
     constexpr int TPR = NTHR / GC, WQV = GC / TPR / 8; // threads per output of q, 16-byte pieces per thread
     uint4 wq_part[WQV];
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
             panel_store(panel, lane, ahead[i % PRE]);
             if (!CACHED || i + PRE < MAXI) {
                 const int tn = t + NW * PRE;
-                ahead[i % PRE] = panel_load(xb, p.x_ss, (tn < NT ? tn : NT - 1) * 32, S - 1, 0, lane);
+                ahead[i % PRE] = panel_load_near(xb, x_pitch, (tn < NT ? tn : NT - 1) * 32, S - 1, 0, lane);
             }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
         float m_run = -1e30f, lsum = 0.f;
         PanelRegs nxt;
         if (!CACHED) {
-            nxt = panel_load(xb, p.x_ss, wave * 32, S - 1, 0, lane);
+            nxt = panel_load_near(xb, x_pitch, wave * 32, S - 1, 0, lane);
         }
 #pragma unroll(UNR)
         for (int i = 0; i < MAXI; ++i) {
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
                 }
             } else {
                 panel_store(panel, lane, nxt);
-                nxt = panel_load(xb, p.x_ss, (t + NW < NT ? t + NW : t) * 32, S - 1, 0, lane);
+                nxt = panel_load_near(xb, x_pitch, (t + NW < NT ? t + NW : t) * 32, S - 1, 0, lane);
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
         const float *bop = p.bo + 16 * g;
         PanelRegs nxt;
         if (!CACHED) {
-            nxt = panel_load(xb, p.x_ss, wave * 32, S - 1, 0, lane);
+            nxt = panel_load_near(xb, x_pitch, wave * 32, S - 1, 0, lane);
         }
 #pragma unroll(UNR)
         for (int i = 0; i < MAXI; ++i) {
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
                 }
             } else {
                 panel_store(panel, lane, nxt);
-                nxt = panel_load(xb, p.x_ss, (t + NW < NT ? t + NW : t) * 32, S - 1, 0, lane);
+                nxt = panel_load_near(xb, x_pitch, (t + NW < NT ? t + NW : t) * 32, S - 1, 0, lane);
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     xf[ks] = as_bf16x8(panel[panel_slot(r, 2 * ks + g)]);
@@ -429,9 +430,10 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
                     }
                 }
                 if (s < S) {
-                    bf16_t *dst = p.out + (int64_t)b * p.out_sb + (int64_t)s * p.out_ss + 32 * ob + 16 * g;
-                    *reinterpret_cast<uint4 *>(dst) = as_uint4(pack8(oa, 0));
-                    *reinterpret_cast<uint4 *>(dst + 8) = as_uint4(pack8(oa, 8));
+                    char *row_out = reinterpret_cast<char *>(p.out + (int64_t)b * p.out_sb + 32 * ob); // uniform
+                    uint4 *dst = reinterpret_cast<uint4 *>(row_out + (__umul24((uint32_t)s, 2u * (uint32_t)p.out_ss) + 32u * g));
+                    dst[0] = as_uint4(pack8(oa, 0));
+                    dst[1] = as_uint4(pack8(oa, 8));
                 }
             }
         }
@@ -450,6 +452,12 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
     }
     if (a.dtype != KUTACC_DTYPE_BF16 || a.nheads * a.head_size != GC || a.nheads > 32 || a.head_size > 32 ||
         a.batch > INT32_MAX || a.seq_len > 16384) {
+        return KUTACC_HIP_EUNSUPPORTED;
+    }
+    // tokens of a batch row are addressed by 32-bit byte offsets from its first one
+    if (a.q_data_stride_s <= 0 || a.out_stride_s <= 0 || a.q_data_stride_s >= (1 << 22) || a.out_stride_s >= (1 << 22) ||
+        a.seq_len >= (1 << 23) || (a.seq_len + 32) * a.q_data_stride_s * 2 >= ((int64_t)1 << 31) ||
+        (a.seq_len + 32) * a.out_stride_s * 2 >= ((int64_t)1 << 31)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
     // 16-byte row loads of x and the weights, 16-byte stores of out rows
