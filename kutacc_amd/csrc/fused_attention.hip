@@ -1755,10 +1755,15 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
     extern __shared__ uint4 lds[]; // [Wo, Wg][4 feature blocks][CK][64 lanes], then 4 panels of 256
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform
     uint4 *panel = lds + 2 * 4 * CK * 64 + wave * 256;
-    const int64_t start = ((int64_t)blockIdx.x * 4 + wave) * rows_per_wave;
-    const int64_t stop = start + rows_per_wave < M ? start + rows_per_wave : M;
-    // Rows are addressed relative to the wave's first one, by 32-bit byte offsets from wave-uniform bases; positions of
+    // The workgroup owns 4 * rows_per_wave consecutive rows and its waves take the 32-row steps of that range in turn
+    // (wave w: steps w, w + 4, ...): neighbouring steps run at the same time, so the two 64-byte halves of a 128-byte
+    // line of the channel-first tensor (32 positions each) are asked for together instead of a whole step apart, by
+    // which time the line has left the L2.
+    // Rows are addressed relative to the workgroup's first one, by 32-bit byte offsets from uniform bases; positions of
     // the channel-first tensor by 32-bit offsets from its first element (the launcher checks that both fit).
+    const int64_t start = (int64_t)blockIdx.x * 4 * rows_per_wave;
+    const int64_t stop = start + 4 * rows_per_wave < M ? start + 4 * rows_per_wave : M;
+    const int64_t first = start + 32 * wave; // this wave's first step
     const int last_rel = (int)(stop - 1 - start);
     const bf16_t *y_w = y + start * y_ld, *x_w = x + start * x_ld;
     const uint32_t y_pitch = (uint32_t)y_ld, x_pitch = (uint32_t)x_ld, m32 = (uint32_t)M;
@@ -1779,12 +1784,12 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
         return t;
     };
     PanelRegs ya, xa;
-    if (start < stop) {
-        ya = panel_load_near(y_w, y_pitch, 0, last_rel, 0, lane);
+    if (first < stop) {
+        ya = panel_load_near(y_w, y_pitch, 32 * wave, last_rel, 0, lane);
         if constexpr (X_CHANNEL_FIRST) {
-            xa = load_cf(0, start, lane);
+            xa = load_cf(0, first, lane);
         } else {
-            xa = panel_load_near(x_w, x_pitch, 0, last_rel, 0, lane);
+            xa = panel_load_near(x_w, x_pitch, 32 * wave, last_rel, 0, lane);
         }
     }
     {
@@ -1804,12 +1809,12 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
     }
     __syncthreads();
     const uint4 *wo_s = lds, *wg_s = lds + 4 * CK * 64;
-    for (int64_t rbase = start; rbase < stop; rbase += 32) {
+    for (int64_t rbase = first; rbase < stop; rbase += 128) {
         const int rel0 = (int)(rbase - start);
         int lv = lane; // opaque: addresses and panel offsets are formed per step, not kept across the loop
         asm volatile("" : "+v"(lv));
         const int rv = lv & 31, gv = lv >> 5;
-        const int rnext = rbase + 32 < stop ? rel0 + 32 : rel0; // clamped: one harmless re-read at the end
+        const int rnext = rbase + 128 < stop ? rel0 + 128 : rel0; // clamped: one harmless re-read at the end
         // ---- gate: 128 features of the 32 rows, rounded to bf16, kept in accumulator order ----
         bf16x8 gate[4][2];
         {
@@ -1861,7 +1866,7 @@ __global__ __launch_bounds__(256, 2) void projected_gate_residual_kernel(
             for (int k = 0; k < 4; ++k) {
                 xf[4 + k] = lds_transposed_fragment(tile + tr_off + k * 1024, tile + tr_off + k * 1024 + 256);
             }
-            xa = load_cf(0, rbase + 32 < stop ? rbase + 32 : rbase, lv);
+            xa = load_cf(0, rbase + 128 < stop ? rbase + 128 : rbase, lv);
             // LayerNorm over the 128 channels of the lane's position: this lane holds channels 16 k + 8 g + 0..7
             float x0 = to_f32(xf[0][0]);
             x0 = __shfl(x0, lv & 31, 64); // channel 0 sits in the lane of the lower half
@@ -2453,7 +2458,7 @@ int row_projection_projected_gate_residual(const void *a, int64_t a_ld, const vo
     int64_t gx = (tiles + 3) / 4;
     const int64_t cap = (int64_t)num_cus() * 2; // two workgroups per CU, each wave with an equal share of the rows
     gx = gx > cap ? cap : gx;
-    const int64_t rpw = ((m + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8;
+    const int64_t rpw = ((m + gx * 4 - 1) / (gx * 4) + 7) / 8 * 8; // a workgroup's range, 4 rpw rows, is whole 32-row steps
     auto kern = cf ? projected_gate_residual_kernel<true> : projected_gate_residual_kernel<false>;
     kern<<<dim3((unsigned)gx), 256, lds_bytes, stream>>>((const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (const bf16_t *)y, y_ld,
                                                          (const bf16_t *)wg, bg, (bf16_t *)acc, acc_ld, m, (int)rpw, ln_gamma,
