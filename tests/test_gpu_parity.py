@@ -505,6 +505,30 @@ def test_non_blocking_mode_on_caller_stream(torch_cuda):
 
 
 # ---- row operators in front of the path ----------------------------------------------------------------------
+
+def test_layernorm_rows_with_a_pitch_beyond_32_bit_offsets(torch_cuda):
+    """The bf16 LayerNorm kernel addresses rows with 32-bit byte offsets where the tensors allow it and keeps a 64-bit form
+    for the rest: a row pitch of 2^23 elements (16 MiB between rows) must take that form and give the same rows as the
+    dense call."""
+    torch = torch_cuda
+    rows, size, ld = 40, 128, 1 << 23
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = (torch.randn(rows, size, device="cuda", generator=g) * 2 + 0.5).bfloat16()
+    gamma, beta = torch.randn(size, device="cuda", generator=g), torch.randn(size, device="cuda", generator=g)
+    wide_in = torch.zeros(rows, ld, device="cuda", dtype=torch.bfloat16)
+    wide_in[:, :size] = x
+    wide_out = torch.full((rows, ld), 3.0, device="cuda", dtype=torch.bfloat16)
+    dense_out = torch.zeros_like(x)
+    L = capi.lib()
+    assert L.kutacc_hip_layernorm_rows(x.data_ptr(), size, gamma.data_ptr(), beta.data_ptr(), dense_out.data_ptr(), size, rows,
+                                       size, 1e-5, capi.K_BF16, None) == 0
+    assert L.kutacc_hip_layernorm_rows(wide_in.data_ptr(), ld, gamma.data_ptr(), beta.data_ptr(), wide_out.data_ptr(), ld, rows,
+                                       size, 1e-5, capi.K_BF16, None) == 0
+    torch.cuda.synchronize()
+    assert helpers.same_bits(wide_out[:, :size].contiguous(), dense_out)
+    assert bool((wide_out[:, size:size + 64] == 3.0).all()), "columns beyond the row were written"
+
+
 @pytest.mark.parametrize("size", [128, 256, 100])
 def test_layernorm_rows_match_oracle(torch_cuda, size):
     from oracle import oracle
