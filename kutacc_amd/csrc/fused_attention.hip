@@ -2273,8 +2273,9 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
     if (a.batch > (1 << 24) || a.seq_len > 1024) {
         return false;
     }
-    // the kernels address the rows of one batch row with 32-bit byte offsets from its first element
-    if (a.input_ld <= 0 || a.input_ld > (1 << 19)) {
+    // the kernels address the rows of one batch row (the output projection: of a wave's range) with 32-bit byte offsets
+    if (a.input_ld <= 0 || a.input_ld > (1 << 19) || a.out_ld <= 0 || a.out_ld > (1 << 19) || a.avg_stride_s <= 0 ||
+        a.avg_stride_s > (1 << 19)) {
         return false;
     }
     // 16-byte row loads of input and weights, 8-byte stores of avg/out rows
@@ -2389,7 +2390,9 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
 bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
                              int64_t m, int64_t n, int64_t k)
 {
-    return (k == 128 || k == 256) && n > 0 && n % 128 == 0 && n / 128 <= 65535 && m > 0 && m <= INT32_MAX - 64 && bias &&
+    // row pitches the kernel's 32-bit offsets within a wave's range of rows can take for any split of the rows
+    const bool pitches = a_ld > 0 && out_ld > 0 && a_ld <= (1 << 19) && out_ld <= (1 << 19);
+    return (k == 128 || k == 256) && n > 0 && n % 128 == 0 && n / 128 <= 65535 && m > 0 && m <= INT32_MAX - 64 && bias && pitches &&
            a_ld % 8 == 0 && out_ld % 8 == 0 && aligned(a, 16) && aligned(w, 16) && aligned(bias, 16) && aligned(out, 16);
 }
 

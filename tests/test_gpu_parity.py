@@ -369,23 +369,28 @@ def test_strided_tensors_through_the_launch_layer(torch_cuda, path, nb_pad):
     assert bool((out_p[:, C:] == -3.0).all()), "columns beyond C of the padded out rows were written"
 
 
-def test_row_pitch_beyond_the_mfma_kernels_addressing_takes_the_generic_kernels(torch_cuda):
-    """The MFMA kernels address the rows of a batch row with 32-bit byte offsets and accept a row pitch of up to 2^19
-    elements; a wider one must not reach them: the automatic choice falls back to the generic kernels (and is right),
-    the forced MFMA path refuses."""
+@pytest.mark.parametrize("wide", ["input", "out"])
+def test_row_pitch_beyond_the_mfma_kernels_addressing_takes_the_generic_kernels(torch_cuda, wide):
+    """The MFMA kernels address rows with 32-bit byte offsets and accept row pitches of up to 2^19 elements; a wider one
+    must not reach them: the automatic choice falls back to the generic kernels (and is right), the forced MFMA path
+    refuses."""
     torch = torch_cuda
     w = make_workload(3, batch=1, seq_len=40)
     B, S, C = w.B, w.S, w.C
     ten, scratch = helpers.to_device(w)
     ld = (1 << 19) + 8
-    x_p = torch.zeros((B * S, ld), dtype=torch.bfloat16, device="cuda")
-    x_p[:, :C] = ten["x"].reshape(B * S, C)
     a = helpers.hip_args(w, ten, scratch, capi.PATH_AUTO)
-    a.input, a.input_ld = x_p.data_ptr(), ld
+    wide_t = torch.zeros((B * S, ld), dtype=torch.bfloat16, device="cuda")
+    if wide == "input":
+        wide_t[:, :C] = ten["x"].reshape(B * S, C)
+        a.input, a.input_ld = wide_t.data_ptr(), ld
+    else:
+        a.out, a.out_ld = wide_t.data_ptr(), ld
     rc = capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None)
     torch.cuda.synchronize()
     assert rc == 0 and capi.last_path() == "generic"
-    helpers.check_close(helpers.to_numpy(ten["out"]), helpers.oracle_out(w), w.dtype, "wide-pitch out")
+    got = ten["out"] if wide == "input" else wide_t[:, :C].reshape(B, S, C)
+    helpers.check_close(helpers.to_numpy(got), helpers.oracle_out(w), w.dtype, "wide-pitch out")
     a.path = capi.PATH_FUSED
     assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None) != 0
     torch.cuda.synchronize()
