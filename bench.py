@@ -1,14 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the fused gated-attention operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--windows 5] [--no-cpu] [--no-all-configs]
 
 A "step" is one kutacc_af2_gating_attention call on device-resident synthetic inputs of the chosen
 configuration (default: config 3, the N_res=384 triangle-attention shape the headline metric is
 quoted on).  Prints ONE JSON line: whole-call TFLOP/s from algorithmic flops
-(10*B*S*C^2 + 4*B*S^2*C), ms per call, the roofline of the dominant kernel (live hipEvent timing on
-the launch stream, read back through kutacc_hip_profile_*) and a CPU baseline (the bf16
-restatement of the reference algorithm in oracle/, timed on this host on a bounded batch sample).
+(10*B*S*C^2 + 4*B*S^2*C), ms per call (median of --windows timed windows of exactly K steps; the minimum is
+reported too), the shader clock the driver reported during those windows, the roofline of the dominant kernel (live
+hipEvent timing on the launch stream, read back through kutacc_hip_profile_*), ms and TFLOP/s of the other four
+configurations ("all_configs") and a CPU baseline (the bf16 restatement of the reference algorithm in oracle/, timed
+on this host on a bounded batch sample).
 """
 from __future__ import annotations
 
@@ -306,13 +308,219 @@ def msa_block_rates(reps=20):
     return res
 
 
+def device_workload(config):
+    """Inputs of configuration `config` drawn on the GPU (torch's generator, seed 1000 + config): the same shapes,
+    distributions and mask rules as kutacc_amd.workloads.make_workload, without its minute of host-side drawing for the
+    large pair tensors.  Used for the timing of the configurations beside the headline one; the parity tests and the
+    headline measurement use the seeded numpy workloads.  Returns (op, tensors, scratch, spec)."""
+    import numpy as np
+    import torch
+    from kutacc_amd import capi
+    from kutacc_amd.workloads import CONFIGS, C_Z, HEAD_SIZE, MASK_BIAS
+
+    spec = CONFIGS[config]
+    B, S, H = spec["B"], spec["S"], spec["H"]
+    C = H * HEAD_SIZE
+    dt = torch.bfloat16 if spec["dtype"] == "bf16" else torch.float32
+    code = capi.K_BF16 if spec["dtype"] == "bf16" else capi.K_FP32
+    g = torch.Generator(device="cuda").manual_seed(1000 + config)
+    L = capi.lib()
+
+    def normal(*shape, scale=1.0):
+        return (torch.randn(*shape, device="cuda", generator=g) * scale).to(dt)
+
+    def layernorm(t):
+        rows, size = t.numel() // t.shape[-1], t.shape[-1]
+        out = torch.empty_like(t)
+        ones, zeros = torch.ones(size, device="cuda"), torch.zeros(size, device="cuda")
+        assert L.kutacc_hip_layernorm_rows(t.data_ptr(), size, ones.data_ptr(), zeros.data_ptr(), out.data_ptr(), size, rows,
+                                           size, 1e-5, code, None) == 0
+        torch.cuda.synchronize()
+        return out
+
+    nb = None
+    if config in (3, 5):  # the pair tensor is the attention input and the source of the pair bias
+        z = normal(S, S, C_Z)
+        w_bias = normal(H, C_Z, scale=C_Z ** -0.5)
+        x = torch.empty_like(z)
+        nb = torch.empty((H, S, S), device="cuda", dtype=dt)
+        ones, zeros = torch.ones(C_Z, device="cuda"), torch.zeros(C_Z, device="cuda")
+        assert L.kutacc_hip_pair_bias(z.data_ptr(), ones.data_ptr(), zeros.data_ptr(), w_bias.data_ptr(), nb.data_ptr(),
+                                      x.data_ptr(), S, S, C_Z, H, 1e-5, code, None) == 0
+        torch.cuda.synchronize()
+        del z
+    else:
+        x = layernorm(normal(B, S, C))
+        if spec["pair_bias"]:
+            zn = layernorm(normal(S, S, C_Z))
+            w_bias = normal(H, C_Z, scale=C_Z ** -0.5)
+            nb = torch.einsum("ijc,hc->hij", zn.float(), w_bias.float()).to(dt).contiguous()
+            del zn
+    wq, wk, wv, wg, wo = (normal(C, C, scale=C ** -0.5) for _ in range(5))
+    bg, bo = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
+    rng = np.random.Generator(np.random.PCG64(1000 + config))
+    bias = np.zeros((B, S), dtype=np.float32)
+    if config in (2, 4):  # residues (2) or sequences (4) padded, the same keys for every batch row
+        keep = rng.random(S) >= (0.05 if config == 2 else 0.10)
+        keep[0] = True
+        bias[:] = (MASK_BIAS * (1.0 - keep.astype(np.float32)))[None, :]
+    elif config == 5:  # last 0-15 % of the residues padded, as a pair mask
+        pad = int(np.floor(rng.random() * 0.15 * S))
+        r = (np.arange(S) < S - pad).astype(np.float32)
+        bias[:] = MASK_BIAS * (1.0 - r[:B, None] * r[None, :])
+    bias = torch.from_numpy(bias).to(device="cuda", dtype=dt)
+    ten = dict(x=x, wq=wq, wk=wk, wv=wv, wg=wg, wo=wo, bg=bg, bo=bo, bias=bias, nb=nb,
+               out=torch.zeros((B, S, C), device="cuda", dtype=dt))
+    scratch = {n: torch.zeros((B, S, H, HEAD_SIZE), device="cuda", dtype=dt) for n in ("q", "k", "gate", "avg")}
+    scratch["v"] = torch.zeros((H, HEAD_SIZE, B, S), device="cuda", dtype=dt)
+    op = capi.GatedAttention(x, wq, wk, wv, wg, bg, wo, bo, bias, nb, H, ten["out"], scratch)
+    return op, ten, scratch, spec
+
+
+def settle(op, seconds=SETTLE_SECONDS):
+    """Untimed calls until the card sits at the clocks it sustains under this load (see main())."""
+    import torch
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            op.run()
+        torch.cuda.synchronize()
+
+
+def timed_window(op, steps):
+    """Wall time of exactly `steps` asynchronous calls between two synchronisations, in ms per call."""
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        op.run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def kernel_times(op, steps, warm):
+    """Per-kernel durations over `steps` calls: hipEvents recorded by the library around each kernel on the launch stream
+    (a few bracketed calls first, not counted: the first event pairs of a process are slow to create and resolve)."""
+    import torch
+    from kutacc_amd import capi
+    L = capi.lib()
+    L.kutacc_hip_profile_enable(1)
+    for _ in range(warm):
+        op.run()
+    torch.cuda.synchronize()
+    L.kutacc_hip_profile_enable(0)
+    L.kutacc_hip_profile_enable(1)  # enabling clears the totals
+    for _ in range(steps):
+        op.run()
+    torch.cuda.synchronize()
+    L.kutacc_hip_profile_enable(0)
+    kernels = []
+    name = ctypes.create_string_buffer(128)
+    tot, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+    i = 0
+    while L.kutacc_hip_profile_read(i, name, 128, ctypes.byref(tot), ctypes.byref(cnt), ctypes.byref(fl)) == 0:
+        kernels.append(dict(name=name.value.decode(), avg_ms=tot.value / max(cnt.value, 1), launches=cnt.value,
+                            flops_per_launch=fl.value))
+        i += 1
+    return kernels
+
+
+def empty_event_pair_ms(stream, n=200):
+    """What a pair of events recorded back to back on the launch stream reads with no kernel between them: the part of a
+    bracketed kernel time that is the command processor handling the two event packets.  Median of n pairs."""
+    import torch
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    with torch.cuda.stream(stream):
+        for e0, e1 in pairs:
+            e0.record()
+            e1.record()
+    torch.cuda.synchronize()
+    reads = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return reads[len(reads) // 2]
+
+
+class ClockSampler:
+    """Samples the shader clock the driver reports (sysfs pp_dpm_sclk of the first AMD card: the level marked '*')
+    from a host thread while a timed window runs.  Reports None where the file is missing or unreadable."""
+
+    def __init__(self, period_s=0.002):
+        import glob
+        self.path = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))), None)
+        self.period = period_s
+        self.samples = []
+        self._stop = False
+        self._thread = None
+
+    def _read(self):
+        try:
+            with open(self.path) as f:
+                for line in f:
+                    if "*" in line:
+                        return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        except (OSError, ValueError, IndexError, TypeError):
+            return None
+        return None
+
+    def __enter__(self):
+        import threading
+        if self.path:
+            def loop():
+                while not self._stop:
+                    v = self._read()
+                    if v:
+                        self.samples.append(v)
+                    time.sleep(self.period)
+            self._thread = threading.Thread(target=loop, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+
+    def mean_mhz(self):
+        return round(sum(self.samples) / len(self.samples), 1) if self.samples else None
+
+
+def config_summary(config, steps, warmup):
+    """One of the configurations beside the headline one: settle, warm up, time `steps` calls, per-kernel brackets.
+    Returns {ms, TFLOP/s, frac, dominant kernel, path} plus the kernel list."""
+    import torch
+    from kutacc_amd import capi
+    op, ten, scratch, spec = device_workload(config)
+    B, S, H = spec["B"], spec["S"], spec["H"]
+    C = H * 32
+    flops = 10 * B * S * C * C + 4 * B * S * S * C
+    settle(op)
+    for _ in range(warmup):
+        op.run()
+    ms = timed_window(op, steps)
+    assert not capi.error_flag()
+    kernels = kernel_times(op, steps, max(3, min(warmup, 10)))
+    dom = max(kernels, key=lambda k: k["avg_ms"] * k["launches"])
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {"workload": f"config {config} {spec['name']}: B={B} S={S} C={C} H={H} d=32", "dtype": spec["dtype"], "steps": steps,
+           "ms": round(ms, 5), "TFLOP/s": round(tf, 2),
+           "frac_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4) if spec["dtype"] == "bf16" else None,
+           "path": capi.last_path(), "dominant_kernel": dom["name"], "dominant_kernel_ms": round(dom["avg_ms"], 5),
+           "kernels": [{"name": k["name"], "avg_ms": round(k["avg_ms"], 5), "launches_per_call": k["launches"] // max(steps, 1)}
+                       for k in kernels],
+           "data": "drawn on the GPU (same shapes, distributions and mask rules as the seeded workload)"}
+    del op, ten, scratch
+    torch.cuda.empty_cache()
+    return rec
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3)
+    ap.add_argument("--windows", type=int, default=5, help="timed windows of --steps calls each; the line reports their median and minimum")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-all-configs", action="store_true", help="skip the timing of the other four configurations")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy: a kernel of known traffic to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run against")
@@ -342,7 +550,6 @@ def main():
     stream = torch.cuda.current_stream()
     capi.set_stream(stream.cuda_stream)
     capi.set_blocking(False)
-    L = capi.lib()
 
     if a.calibrate_copy:
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda:0").fill_(1)
@@ -353,66 +560,37 @@ def main():
     # The card idles at its lowest clocks and takes some hundred calls (about 30 ms of work) to settle at the clocks it
     # sustains under this load; the first calls after any pause run up to 25 % slower.  A fixed stretch of untimed calls
     # puts the W warm-up steps and the K timed steps at the sustained state whatever W is.
-    t_settle = time.perf_counter()
-    while time.perf_counter() - t_settle < SETTLE_SECONDS:
-        for _ in range(50):
-            op.run()
-        torch.cuda.synchronize()
+    settle(op)
     for _ in range(a.warmup):
         op.run()
     assert not capi.error_flag()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        op.run()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    # --windows timed windows of exactly K steps each, back to back; ms_per_step is their median
+    with ClockSampler() as clock:
+        windows = [timed_window(op, a.steps) for _ in range(max(1, a.windows))]
     assert not capi.error_flag()
-    ms = wall / a.steps * 1e3
+    ms = sorted(windows)[len(windows) // 2]
     tflops = w.flops() / (ms * 1e-3) / 1e12
 
-    # per-kernel durations: same K calls again with hipEvents recorded around each kernel on the stream (a few
-    # bracketed calls first, not counted: the first event pairs of a process are slow to create and resolve)
-    L.kutacc_hip_profile_enable(1)
-    for _ in range(max(3, min(a.warmup, 10))):
-        op.run()
-    torch.cuda.synchronize()
-    L.kutacc_hip_profile_enable(0)
-    L.kutacc_hip_profile_enable(1)  # enabling clears the totals
-    for _ in range(a.steps):
-        op.run()
-    torch.cuda.synchronize()
-    L.kutacc_hip_profile_enable(0)
-    kernels = []
-    name = ctypes.create_string_buffer(128)
-    tot, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
-    i = 0
-    while L.kutacc_hip_profile_read(i, name, 128, ctypes.byref(tot), ctypes.byref(cnt), ctypes.byref(fl)) == 0:
-        kernels.append(dict(name=name.value.decode(), avg_ms=tot.value / max(cnt.value, 1), launches=cnt.value,
-                            flops_per_launch=fl.value))
-        i += 1
+    kernels = kernel_times(op, a.steps, max(3, min(a.warmup, 10)))
     # An event pair around a kernel reads the kernel plus the time the command processor takes over the two event
-    # packets (an empty pair reads 4-5 us on this part).  The kernels of a call run back to back (the profiler's trace
-    # shows no gap), so what the bracketed times of one call add up to beyond the unbracketed time per call is that
-    # overhead, spread evenly over the brackets; the roofline uses the kernel's time net of it, which is what
-    # rocprofv3 reports (profiles/gating_attention_kernel_stats.txt).
-    per_call = sum(k["avg_ms"] * k["launches"] for k in kernels) / max(a.steps, 1)
-    brackets_per_call = sum(k["launches"] for k in kernels) / max(a.steps, 1)
-    overhead_ms = max(0.0, (per_call - ms) / brackets_per_call) if kernels else 0.0
+    # packets; an empty pair on the same stream measures that part directly.  avg_ms is what the bracket read;
+    # avg_ms_net subtracts the empty pair and is the figure comparable with a profiler's kernel duration.
+    overhead_ms = empty_event_pair_ms(stream)
     dom = max(kernels, key=lambda k: k["avg_ms"] * k["launches"]) if kernels else None
     roofline = None
     if dom:
-        net_ms = dom["avg_ms"] - overhead_ms
-        ach = dom["flops_per_launch"] / (net_ms * 1e-3) / 1e12
+        ach = dom["flops_per_launch"] / (dom["avg_ms"] * 1e-3) / 1e12
+        net_ms = max(dom["avg_ms"] - overhead_ms, 1e-6)
+        ach_net = dom["flops_per_launch"] / (net_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4),
                     "traffic": measured_traffic(w.config, dom["name"]),
-                    "avg_kernel_ms": round(net_ms, 5), "avg_kernel_ms_bracketed": round(dom["avg_ms"], 5),
-                    "event_bracket_overhead_ms": round(overhead_ms, 5),
+                    "traffic_source": "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
+                                      "not re-measured in this run)",
+                    "avg_kernel_ms": round(dom["avg_ms"], 5), "avg_kernel_ms_net": round(net_ms, 5),
+                    "achieved_net": round(ach_net, 2), "frac_net": round(ach_net / MFMA_BF16_PEAK_TFLOPS, 4),
+                    "empty_event_pair_ms": round(overhead_ms, 5),
                     "flops_per_launch": dom["flops_per_launch"]}
-
-    capi.set_blocking(True)
-    capi.set_stream(None)
 
     rec = {
         "metric": "gated-attention TFLOP/s + % bf16 MFMA peak; ms/call at N_res=384 tri-attn",
@@ -423,14 +601,30 @@ def main():
                    "flops_per_call": w.flops(), "algorithmic_bytes_per_call": w.algorithmic_bytes(),
                    "path": capi.last_path()},
         "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        # avg_ms: net of the event-bracket overhead (see above); avg_ms_bracketed: as the event pair read it
+        # ms_per_step and value are the median window; each window is exactly `steps` calls
+        "timed_windows": {"count": len(windows), "steps_each": a.steps, "median_ms": round(ms, 5),
+                          "min_ms": round(min(windows), 5), "max_ms": round(max(windows), 5),
+                          "all_ms": [round(v, 5) for v in windows]},
+        "shader_clock_mhz": clock.mean_mhz(), "shader_clock_samples": len(clock.samples),
         "kernels": [{**{k: (round(v, 5) if isinstance(v, float) else v) for k, v in kk.items()},
-                     "avg_ms": round(kk["avg_ms"] - overhead_ms, 5), "avg_ms_bracketed": round(kk["avg_ms"], 5)}
-                    for kk in kernels],
-        "event_bracket_overhead_ms": round(overhead_ms, 5),
+                     "avg_ms_net": round(max(kk["avg_ms"] - overhead_ms, 0.0), 5)} for kk in kernels],
+        "empty_event_pair_ms": round(overhead_ms, 5),
         "roofline": roofline,
-        "cpu_baseline": None if a.no_cpu else cpu_baseline(w),
     }
+    del op, ten, scratch
+    torch.cuda.empty_cache()
+    if not a.no_all_configs:
+        # the other configurations, same settle + warm-up, at least 50 steps each (no CPU leg)
+        rec["all_configs"] = {f"config {w.config}": {"ms": round(ms, 5), "TFLOP/s": round(tflops, 2),
+                                                      "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                                                      "path": rec["config"]["path"],
+                                                      "dominant_kernel": dom["name"] if dom else None}}
+        for c in (1, 2, 4, 5):
+            if c != w.config:
+                rec["all_configs"][f"config {c}"] = config_summary(c, max(50, min(a.steps, 100)), a.warmup)
+    capi.set_blocking(True)
+    capi.set_stream(None)
+    rec["cpu_baseline"] = None if a.no_cpu else cpu_baseline(w)
     if a.producers:
         rec["producers"] = producer_rates(a.config)
     if a.pair_stack:

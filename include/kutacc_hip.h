@@ -103,6 +103,9 @@ kutacc_export int kutacc_hip_gating_attention(const kutacc_hip_attention_args_t 
  * whose copy, nheads * ceil(S/32) * 2*ceil(S/64) * 2048 bytes, exceeds the array is rejected with KUTACC_HIP_EINVAL
  * and a line on stderr (16 MiB holds 8 heads at 1024 positions).  All calls on one GPU share the array, which keeps
  * the last call's contents: every call rewrites the part it reads, and calls that overlap in time on one GPU race.
+ * The first call on a device looks up the array's address (hipGetSymbolAddress) and the first call of a kernel
+ * variant raises its dynamic-LDS limit (hipFuncSetAttribute, device-attribute queries); neither may be recorded into
+ * a graph, so make one warm-up call per device and shape outside stream capture before capturing this entry point.
  */
 #define KUTACC_HIP_STATIC_SCRATCH_BYTES (16u << 20)
 kutacc_export int kutacc_hip_gating_attention_static(const kutacc_hip_attention_args_t *args, void *stream);
@@ -112,7 +115,8 @@ kutacc_export int kutacc_hip_gating_attention_static(const kutacc_hip_attention_
  * shared by all heads.  bf16 storage, nheads*head_size == 64 (the reference hard-wires nchannels == 64,
  * :172), nheads <= 32, head_size <= 32.  The reference's scratch tensors q, k, v, gate are not needed and
  * not touched; q_avg ([B, 64], may be NULL) receives the masked mean as the reference leaves it in `avg`.
- * seq_len <= 16384; the tokens of a batch row must lie within 2 GiB of its first one in q_data and in out (32-bit
+ * seq_len <= 12288 (what a workgroup's LDS holds of a row's mask and logits; longer rows return
+ * KUTACC_HIP_EUNSUPPORTED before anything is launched); the tokens of a batch row must lie within 2 GiB of its first one in q_data and in out (32-bit
  * offsets in the kernel), else KUTACC_HIP_EUNSUPPORTED. */
 typedef struct kutacc_hip_global_attention_args {
     int64_t batch;     /* B */
@@ -406,12 +410,13 @@ kutacc_export int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t
 
 /* Stream used when a `stream` argument is NULL and by the handle-based API of kutacc.h.
  * Default: the HIP null stream.  The setting belongs to the calling host thread (like a framework's current
- * stream): threads that drive the library on different streams each set their own. */
+ * stream): threads that drive the library on different streams each set their own.  A thread that has never set one
+ * uses the value set last by any thread, so worker threads of a host that configured the library once inherit it. */
 kutacc_export void kutacc_hip_set_stream(void *stream);
 kutacc_export void *kutacc_hip_get_stream(void);
 
 /* 1 (default): the handle-based API blocks until the device work has finished, as the CPU library
- * does.  0: it returns after enqueueing when all operands are device pointers.  Per host thread, like the stream. */
+ * does.  0: it returns after enqueueing when all operands are device pointers.  Per host thread, inherited like the stream. */
 kutacc_export void kutacc_hip_set_blocking(int blocking);
 
 /* Calls on host pointers run on device copies of their operands; those copies are kept between calls (a repeated

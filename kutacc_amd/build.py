@@ -1,7 +1,6 @@
 """Compile libkutacc.so for gfx950 with hipcc (cross-compiles without a GPU).
 
     python -m kutacc_amd.build          # rebuild kutacc_amd/lib/libkutacc.so
-    python -m kutacc_amd.build --dev    # ... and the development variant with clock probes (kutacc_amd.devtools)
 """
 from __future__ import annotations
 
@@ -35,7 +34,7 @@ def hipcc() -> str:
 
 def build(verbose: bool = False) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
-    extra = os.environ.get("KUTACC_EXTRA_HIPFLAGS", "").split()  # e.g. -DKUTACC_TIMELINE for tuning builds
+    extra = os.environ.get("KUTACC_EXTRA_HIPFLAGS", "").split()  # extra hipcc flags for one-off tuning builds
     objs = []
     procs = []
     for src in SOURCES:
@@ -62,31 +61,6 @@ def build(verbose: bool = False) -> str:
     subprocess.check_call(cmd)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
-
-
-DEV_LIB_PATH = os.path.join(LIB_DIR, "libkutacc_dev.so")
-
-
-def build_dev() -> str:
-    """The development variant of the library (kutacc_amd/lib/libkutacc_dev.so): the attention source compiled with
-    -DKUTACC_TIMELINE, which adds clock probes to the head kernels and exports kutacc_debug_timeline and
-    kutacc_debug_attention_loop (read by kutacc_amd.devtools).  Every other object is the product build's, so build()
-    runs first.  The probes cost a few per cent; nothing ships from this build."""
-    if not os.path.exists(LIB_PATH):
-        build()
-    obj = os.path.join(LIB_DIR, "fused_attention_dev.o")
-    cmd = [hipcc(), *HIP_FLAGS, "-DKUTACC_TIMELINE", "-x", "hip", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-c",
-           os.path.join(CSRC, "fused_attention.hip"), "-o", obj]
-    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    lines = [ln for ln in p.stdout.splitlines() if "packed-fp32-ops" not in ln]
-    if p.returncode != 0:
-        print("\n".join(lines), flush=True)
-        raise RuntimeError("hipcc failed")
-    objs = [os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o") for src in SOURCES if src != "fused_attention.hip"]
-    tmp = DEV_LIB_PATH + ".tmp"
-    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, obj, "-o", tmp])
-    os.replace(tmp, DEV_LIB_PATH)
-    return DEV_LIB_PATH
 
 
 def host_cxx() -> str:
@@ -123,5 +97,3 @@ def build_dropin_callers() -> list:
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
     print("\n".join(build_dropin_callers()))
-    if "--dev" in sys.argv:
-        print(build_dev())

@@ -18,6 +18,7 @@
 #include "kutacc.h"
 #include "kutacc_hip.h"
 #include "api_internal.h"
+#include "staging.h"
 #include "launch_internal.h"
 #include "tensor_view.h"
 
@@ -48,16 +49,22 @@ const kutacc_version_t k_version = {
 };
 
 // Stream and blocking mode belong to the calling host thread (as a framework's "current stream" does): two threads
-// that drive the library on different streams do not see each other's settings.
-thread_local hipStream_t g_stream = nullptr;
-thread_local bool g_blocking = true;
+// that each set theirs do not see each other's settings.  A thread that never set one (a worker of a pool whose owner
+// configured the library) inherits the value set last by any thread.
+std::atomic<hipStream_t> g_shared_stream{nullptr};
+std::atomic<bool> g_shared_blocking{true};
+thread_local bool t_own_stream = false, t_own_blocking = false;
+thread_local hipStream_t t_stream = nullptr;
+thread_local bool t_blocking = true;
+inline hipStream_t current_stream() { return t_own_stream ? t_stream : g_shared_stream.load(std::memory_order_relaxed); }
+inline bool current_blocking() { return t_own_blocking ? t_blocking : g_shared_blocking.load(std::memory_order_relaxed); }
 thread_local const char *t_last_path = "none";
 // 0: the handle-based entry points take the caller's word that all operands of a call live where `input` lives
 std::atomic<int> g_pointer_checks{1};
 std::atomic<int> g_block_layernorm{0};
 std::atomic<int> g_reference_scratch{0}; // kutacc_af2_gating_attention fills q, k, v, gate as the reference does
 
-inline hipStream_t pick_stream(void *s) { return s ? (hipStream_t)s : g_stream; }
+inline hipStream_t pick_stream(void *s) { return s ? (hipStream_t)s : current_stream(); }
 
 // Where does a data pointer live?  Plain malloc memory is unknown to HIP (the query fails and leaves
 // a sticky error behind, which is cleared here); pinned host memory counts as host.
@@ -74,127 +81,11 @@ Space space_of(const void *p)
     return (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged) ? Space::Device : Space::Host;
 }
 
-// Device mirror of a host range, for the staged (host-pointer) path.
-struct Mirror {
-    void *dev = nullptr;
-    void *host = nullptr;
-    size_t bytes = 0;
-    bool copy_back = false;
-};
-
-// Device buffers of the staged path are kept between calls: a call takes what it needs from the pool (smallest buffer
-// that is large enough, else a new allocation) and gives everything back when it is done, so a caller that repeats a
-// shape pays hipMalloc once.  kutacc_hip_release_staging() frees the pool.
-struct StagingPool {
-    struct Block {
-        void *dev;
-        size_t bytes;
-        int device; // the device the memory lives on: a block is only handed out again there
-    };
-    std::mutex mu;
-    std::vector<Block> free_blocks;
-    static int current_device()
-    {
-        int d = 0;
-        (void)hipGetDevice(&d);
-        return d;
-    }
-    hipError_t take(size_t bytes, void **out, size_t *got)
-    {
-        {
-            const int here = current_device();
-            std::lock_guard<std::mutex> lk(mu);
-            int best = -1;
-            for (int i = 0; i < (int)free_blocks.size(); ++i) {
-                if (free_blocks[i].device == here && free_blocks[i].bytes >= bytes &&
-                    (best < 0 || free_blocks[i].bytes < free_blocks[best].bytes)) {
-                    best = i;
-                }
-            }
-            if (best >= 0) {
-                *out = free_blocks[best].dev, *got = free_blocks[best].bytes;
-                free_blocks.erase(free_blocks.begin() + best);
-                return hipSuccess;
-            }
-        }
-        *got = bytes;
-        return hipMalloc(out, bytes);
-    }
-    void give(void *dev, size_t bytes)
-    {
-        const int here = current_device(); // a call takes and gives on the same current device
-        std::lock_guard<std::mutex> lk(mu);
-        free_blocks.push_back({dev, bytes, here});
-    }
-    size_t release()
-    {
-        std::lock_guard<std::mutex> lk(mu);
-        size_t total = 0;
-        for (auto &b : free_blocks) {
-            total += b.bytes;
-            (void)hipFree(b.dev);
-        }
-        free_blocks.clear();
-        return total;
-    }
-};
-StagingPool g_staging;
-
-struct Stager {
-    std::vector<Mirror> items;
-    std::vector<size_t> capacity; // what the pool gave for each item
-    hipStream_t stream;
-    int rc = 0;
-    explicit Stager(hipStream_t s) : stream(s) {}
-    void *in(const void *host, size_t bytes) { return add(const_cast<void *>(host), bytes, true, false); }
-    void *scratch(size_t bytes) { return add(nullptr, bytes, false, false); }
-    void *out(void *host, size_t bytes, bool preload) { return add(host, bytes, preload, true); }
-    void *add(void *host, size_t bytes, bool upload, bool back)
-    {
-        if (rc != 0 || bytes == 0) {
-            return nullptr;
-        }
-        Mirror m;
-        m.host = host, m.bytes = bytes, m.copy_back = back;
-        size_t got = 0;
-        hipError_t e = g_staging.take(bytes, &m.dev, &got);
-        if (e == hipSuccess && upload && host) {
-            e = hipMemcpyAsync(m.dev, host, bytes, hipMemcpyHostToDevice, stream);
-        }
-        if (e != hipSuccess) {
-            rc = (int)e;
-            if (m.dev) {
-                g_staging.give(m.dev, got);
-            }
-            return nullptr;
-        }
-        items.push_back(m);
-        capacity.push_back(got);
-        return m.dev;
-    }
-    int finish()
-    {
-        for (auto &m : items) {
-            if (rc == 0 && m.copy_back) {
-                const hipError_t e = hipMemcpyAsync(m.host, m.dev, m.bytes, hipMemcpyDeviceToHost, stream);
-                if (e != hipSuccess) {
-                    rc = (int)e;
-                }
-            }
-        }
-        const hipError_t e = hipStreamSynchronize(stream);
-        if (rc == 0 && e != hipSuccess) {
-            rc = (int)e;
-        }
-        for (size_t i = 0; i < items.size(); ++i) {
-            g_staging.give(items[i].dev, capacity[i]);
-        }
-        items.clear();
-        capacity.clear();
-        return rc;
-    }
-};
+using kutacc_api::g_staging;
+using kutacc_api::Stager;
 } // namespace
+
+kutacc_api::StagingPool kutacc_api::g_staging;
 
 int kutacc_get_version(kutacc_version_t *version)
 {
@@ -275,9 +166,17 @@ int kutacc_hip_set_tuning(const char *name, const char *value)
     return kutacc_launch::fused_attention_tuning(name, value);
 }
 
-void kutacc_hip_set_stream(void *stream) { g_stream = (hipStream_t)stream; }
-void *kutacc_hip_get_stream(void) { return (void *)g_stream; }
-void kutacc_hip_set_blocking(int blocking) { g_blocking = blocking != 0; }
+void kutacc_hip_set_stream(void *stream)
+{
+    t_stream = (hipStream_t)stream, t_own_stream = true;
+    g_shared_stream.store(t_stream, std::memory_order_relaxed);
+}
+void *kutacc_hip_get_stream(void) { return (void *)current_stream(); }
+void kutacc_hip_set_blocking(int blocking)
+{
+    t_blocking = blocking != 0, t_own_blocking = true;
+    g_shared_blocking.store(t_blocking, std::memory_order_relaxed);
+}
 int kutacc_hip_error_flag(void) { return kutacc::kutacc_check_err_set ? 1 : 0; }
 void kutacc_hip_clear_error(void) { kutacc::kutacc_check_err_set = false; }
 const char *kutacc_hip_last_path(void) { return t_last_path; }
@@ -354,7 +253,7 @@ inline size_t span2(int64_t rows, int64_t row_stride, int64_t cols) { return (si
 
 int finish_device_call(int rc, hipStream_t s)
 {
-    if (rc == 0 && g_blocking) {
+    if (rc == 0 && current_blocking()) {
         rc = kutacc_hip_status(hipStreamSynchronize(s));
     }
     return rc;
@@ -362,7 +261,7 @@ int finish_device_call(int rc, hipStream_t s)
 } // namespace
 
 namespace kutacc_api {
-hipStream_t default_stream() { return g_stream; }
+hipStream_t default_stream() { return current_stream(); }
 hipStream_t stream_or_default(void *s) { return pick_stream(s); }
 bool on_device(const void *p) { return space_of(p) == Space::Device; }
 int finish(int rc, hipStream_t s) { return finish_device_call(rc, s); }
@@ -460,7 +359,7 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
         a.q = nullptr;
     }
 
-    hipStream_t s = g_stream;
+    hipStream_t s = current_stream();
     const Space sp = space_of(in.data);
     const void *all_ptrs[] = {bs.data, ot.data, q.data, k.data, v.data, gt.data, av.data, wq.data,
                               wk.data, wv.data, wg.data, bg.data, wo.data, bo.data, has_nb ? nb.data : in.data};
@@ -590,7 +489,7 @@ void kutacc_af2_global_attention(kutacc_af2_attention_inputs_t *q_based_ptr, kut
     a.q_avg = qa.data, a.q_avg_stride_b = nchannels;
     a.out = ot.data, a.out_stride_s = ot.stride(ot.dim >= 3 ? 1 : 0), a.out_stride_b = seq_len * a.out_stride_s;
 
-    hipStream_t s = g_stream;
+    hipStream_t s = current_stream();
     const Space sp = space_of(x.data);
     const void *all_ptrs[] = {mk.data, ot.data, qa.data, wq.data, wk.data, wv.data, wg.data, bg.data, wo.data, bo.data};
     if (g_pointer_checks.load(std::memory_order_relaxed)) {
@@ -642,7 +541,7 @@ void kutacc_af2_layernorm(__bf16 *data, float *gamma, float *beta, int64_t size,
     if (KUTACC_FAILED()) {
         return;
     }
-    hipStream_t s = g_stream;
+    hipStream_t s = current_stream();
     int rc;
     if (space_of(data) == Space::Device) {
         rc = finish_device_call(
@@ -703,7 +602,7 @@ void kutacc_af2_linear(kutacc_tensor_h act, kutacc_tensor_h weight, float *bias_
     if (KUTACC_FAILED()) {
         return;
     }
-    hipStream_t s = g_stream;
+    hipStream_t s = current_stream();
     int rc;
     if (sp == Space::Device) {
         rc = finish_device_call(
@@ -747,9 +646,9 @@ void kutacc_af2_linear_weight_prepack(const __bf16 *weight, __bf16 *result, int6
         return;
     }
     hipError_t e = hipMemcpy2DAsync(result, (size_t)k * 2, weight, (size_t)ldb * 2, (size_t)k * 2, (size_t)n,
-                                    hipMemcpyDeviceToDevice, g_stream);
-    if (e == hipSuccess && g_blocking) {
-        e = hipStreamSynchronize(g_stream);
+                                    hipMemcpyDeviceToDevice, current_stream());
+    if (e == hipSuccess && current_blocking()) {
+        e = hipStreamSynchronize(current_stream());
     }
     KUTACC_CHECK(e == hipSuccess, "kutacc_af2_linear_weight_prepack: ", hipGetErrorString(e));
 }

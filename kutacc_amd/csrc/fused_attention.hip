@@ -44,32 +44,6 @@
 
 using namespace kutacc_dev;
 
-// Phase timestamps for kernel tuning, compiled in only with -DKUTACC_TIMELINE (never in the shipped
-// library): wave leaders of every 256th workgroup record clock64() at the probes below, and
-// kutacc_debug_timeline() copies the table out.
-#ifdef KUTACC_TIMELINE
-__device__ unsigned long long g_timeline[8 * 16 * 12];
-#define TL(i)                                                                                 \
-    do {                                                                                      \
-        if ((blockIdx.x & 255) == 77 && (threadIdx.x & 63) == 0 && (blockIdx.x >> 8) < 8) {   \
-            g_timeline[((blockIdx.x >> 8) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = clock64(); \
-        }                                                                                     \
-    } while (0)
-extern "C" __attribute__((visibility("default"))) int kutacc_debug_timeline(unsigned long long *out, int n)
-{
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_timeline), (size_t)n * 8);
-}
-#define TLV(i, val)                                                                           \
-    do {                                                                                      \
-        if ((blockIdx.x & 255) == 77 && (threadIdx.x & 63) == 0 && (blockIdx.x >> 8) < 8) {   \
-            g_timeline[((blockIdx.x >> 8) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = (val);     \
-        }                                                                                     \
-    } while (0)
-#else
-#define TL(i) ((void)0)
-#define TLV(i, val) ((void)0)
-#endif
-
 namespace {
 
 constexpr int HEAD = 32;            // head_size the MFMA kernels are written for
@@ -821,7 +795,6 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         return;
     }
     const int tid = threadIdx.x;
-    TL(0);
     const int nthreads = p.NW * 64;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, kept in a scalar register
     const int r = lane & 31, g = lane >> 5;
@@ -879,12 +852,10 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         if (pi > 0) {
             __syncthreads(); // previous group's fragments are no longer being read
         } else {
-            TL(1);
         }
         stage_weight_fragments<C>(lds_w, p, pass * GW, GW, h, wave, NW, lane);
         __syncthreads();
         if (pi == 0) {
-            TL(2);
         }
         if constexpr (C == 128 && BPW >= 3) {
             // Two blocks of the wave per walk over the weight fragments: the input fragments of both stay in registers
@@ -1078,7 +1049,6 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         }
         } // one block at a time
     }
-    TL(3);
     __syncthreads(); // K and V of the whole sequence are in LDS; the weight fragments are no longer read
     if constexpr (V_ALIAS) {
 #pragma unroll
@@ -1106,7 +1076,6 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
         }
     }
     __syncthreads();
-    TL(4);
 
     // ---- attention: each wave walks the key tiles for its own query blocks ----
     uint32_t flags = 0; // bit t: key tile t needs the mask added (non-zero bias or ragged tail)
@@ -1158,7 +1127,6 @@ __global__ __launch_bounds__(64 * max_waves(C, BPW)) void fused_head_kernel(Fuse
             attend_block_direct<HAS_NB>(lds_k, lds_v, mask4, flags, nbrow, p.nb_vec != 0, qf[i][0], qf[i][1], as_bf16x8(selw0), as_bf16x8(selw1), NB,
                                         S, lane, o, l);
         }
-        TL(5);
         if (qpos < S) {
             f32x16 gv;
 #pragma unroll
@@ -1190,7 +1158,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     constexpr int CK = C / 16;
     constexpr int NP = CK / 4; // staging panels (64 channels each) per input row block
     extern __shared__ uint4 lds[];
-    TL(7);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: values derived from it stay in scalar registers
     const int r = lane & 31, g = lane >> 5;
@@ -1238,7 +1205,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     }
     __syncthreads();
 
-    TL(8);
     const int j = wave; // this wave's sequence block
     const float qmul = L2MODE ? p.qscale * LOG2E : p.qscale;
     const float mask_scale = L2MODE ? LOG2E : 1.0f;
@@ -1247,15 +1213,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         const int b = b0 + n * bstep;
         uint32_t *flag_word = flag_words + (n & 1);
         float *mask = mask_base + (n & 1) * NT * 32;
-        if (n == 2) {
-            TL(0);
-        }
-        if (n == 1) {
-            TL(9);
-        }
-        if (n == nrows - 1) {
-            TL(10);
-        }
         // The lane index is opaque to the optimiser here: the row addresses and panel offsets derived from it are then
         // formed anew for every batch row (a few dozen vector instructions) instead of being kept across the attention
         // loop, where there is no register for them -- spilled, each costs a scratch round trip per batch row.
@@ -1374,9 +1331,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                 }
             }
         }
-        if (n == 2) {
-            TL(1);
-        }
         // ---- four projections of the block ----
         bf16x8 q0, q1;
         uint4 kfrag0, kfrag1, vfrag0, vfrag1; // this block's K and V fragments, parked until the LDS arrays are free
@@ -1429,9 +1383,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             gate_park_x[0] = as_uint4(pack8(acc, 0));
             gate_park_x[64] = as_uint4(pack8(acc, 8));
         }
-        if (n == 2) {
-            TL(2);
-        }
         __syncthreads(); // every wave is done with the previous row's attention: the K and V arrays are free
         lds_k[(j * 2 + 0) * 64 + lane] = kfrag0;
         lds_k[(j * 2 + 1) * 64 + lane] = kfrag1;
@@ -1441,9 +1392,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             flag_words[(n + 1) & 1] = 0; // its readers (previous row) are done, its writers (next row) start after the next barrier
         }
         __syncthreads(); // K, V and the mask of this batch row are complete
-        if (n == 2) {
-            TL(3);
-        }
 
         const f32x4 *mask4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
         f32x16 o;
@@ -1460,9 +1408,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
                                                      l);
             }
             const bool ok = !__any(!(l > 1e-30f && l < 1e30f));
-            if (n == 2) {
-                TLV(6, ok ? 1 : 0);
-            }
             if (!ok) {
                 // some probability overflowed or a whole row underflowed: shift by the true row maxima
                 const float m = row_max_l2<HAS_NB>(lds_k, mask4, nbf, q0, q1, sel0, sel1, NT, lane);
@@ -1471,9 +1416,6 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
         } else {
             attend_block<HAS_NB>(lds_k, lds_v, mask4, flags, nb_head, p.nb_sq, j * 32, p.nb_vec != 0, panel, q0, q1, sel0,
                                  sel1, NB, S, lane, o, l);
-        }
-        if (n == 2) {
-            TL(4);
         }
         int lane_o = lane; // as above: the addresses of the epilogue are not worth a register during the attention loop
         asm volatile("" : "+v"(lane_o));
@@ -1490,11 +1432,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * (lane_o >> 5), o,
                         __builtin_amdgcn_rcpf(l), gv);
         }
-        if (n == 2) {
-            TL(5);
-        }
     }
-    TL(11);
 }
 
 // out[t][o] = sum_c avg[t][c] * Wo[o][c] + bo[o]  (reference src/attention/gating_attention.cpp:152-157).
@@ -2200,6 +2138,32 @@ int dispatch_head_kernel(const FusedParams &p, const Plan &pl, hipStream_t strea
     }
 }
 
+// How output_projection_kernel<C, .> splits M rows: workgroups along the rows and rows per wave (a multiple of 8).  Two
+// workgroups of four waves per CU, or one of eight: each wave with an equal share of the rows (a third resident
+// workgroup, where the registers allow one, measured slower: the weight slab is staged per workgroup).
+inline void output_projection_split(int C, int64_t M, int64_t &gx, int64_t &rpw)
+{
+    const int waves = 4 * (C / 128);
+    const int64_t tiles = (M + 31) / 32;
+    gx = (tiles + waves - 1) / waves;
+    const int64_t cap = (int64_t)num_cus() * (C == 128 ? 2 : 1);
+    gx = gx > cap ? cap : gx;
+    rpw = ((M + gx * waves - 1) / (gx * waves) + 7) / 8 * 8;
+}
+
+// The kernel addresses a wave's rows with 32-bit byte offsets from the wave's first row: true when that range fits for
+// these row pitches under the split the launcher will choose.
+inline bool output_projection_rows_fit(int C, int64_t M, int64_t a_ld, int64_t out_ld)
+{
+    if (a_ld <= 0 || out_ld <= 0 || M <= 0) {
+        return false;
+    }
+    int64_t gx, rpw;
+    output_projection_split(C, M, gx, rpw);
+    const int64_t pitch = a_ld > out_ld ? a_ld : out_ld;
+    return pitch < (1 << 23) && (rpw + 32) * pitch * 2 < ((int64_t)1 << 31);
+}
+
 // out[M, N] = a[M, K] . w[N, K]^T + bias with K = C and N a multiple of 128 (one grid row per 128-feature slab)
 template <int C, int EPILOGUE = EPILOGUE_STORE>
 int launch_output_projection(const void *a, int64_t a_ld, const void *w, const float *bias, void *out, int64_t out_ld,
@@ -2217,18 +2181,12 @@ int launch_output_projection(const void *a, int64_t a_ld, const void *w, const f
     if (const int rc = opt_in_lds(kern, lds_bytes, configured[near_out ? 1 : 0])) {
         return rc;
     }
-    const int64_t tiles = (M + 31) / 32;
-    // two workgroups of four waves per CU, or one of eight: each wave with an equal share of the rows (a third resident
-    // workgroup, where the registers allow one, measured slower: the weight slab is staged per workgroup)
-    int64_t gx = (tiles + WAVES - 1) / WAVES;
-    const int64_t cap = (int64_t)num_cus() * (C == 128 ? 2 : 1);
-    gx = gx > cap ? cap : gx;
-    const int64_t rpw = ((M + gx * WAVES - 1) / (gx * WAVES) + 7) / 8 * 8;
-    const int64_t gy = (N / 128 + SLABS - 1) / SLABS;
-    const int64_t pitch = a_ld > out_ld ? a_ld : out_ld;
-    if (a_ld <= 0 || out_ld <= 0 || pitch >= (1 << 23) || (rpw + 32) * pitch * 2 >= ((int64_t)1 << 31)) {
-        return KUTACC_HIP_EUNSUPPORTED; // the kernel addresses a wave's rows with 32-bit byte offsets
+    if (!output_projection_rows_fit(C, M, a_ld, out_ld)) {
+        return KUTACC_HIP_EUNSUPPORTED; // the callers' support checks ask the same question first
     }
+    int64_t gx, rpw;
+    output_projection_split(C, M, gx, rpw);
+    const int64_t gy = (N / 128 + SLABS - 1) / SLABS;
     kern<<<dim3((unsigned)gx, (unsigned)gy), 64 * WAVES, lds_bytes, stream>>>(
         (const bf16_t *)a, a_ld, (const bf16_t *)w, bias, (bf16_t *)out, out_ld, M, (int)N, (int)rpw, (const bf16_t *)gate,
         gate_ld, swap_n);
@@ -2286,6 +2244,10 @@ bool fused_attention_supports(const kutacc_hip_attention_args_t &a)
     }
     if (a.avg_stride_h != HEAD || a.avg_stride_s % 8 != 0 || a.avg_stride_b != a.seq_len * a.avg_stride_s ||
         !aligned(a.avg, 16) || a.out_ld % 8 != 0 || !aligned(a.out, 16)) {
+        return false;
+    }
+    // ... and the output projection a wave's range of the batch * seq_len rows of avg and out
+    if (!output_projection_rows_fit((int)C, a.batch * a.seq_len, a.avg_stride_s, a.out_ld)) {
         return false;
     }
     Plan pl;
@@ -2390,9 +2352,13 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
 bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
                              int64_t m, int64_t n, int64_t k)
 {
-    // row pitches the kernel's 32-bit offsets within a wave's range of rows can take for any split of the rows
-    const bool pitches = a_ld > 0 && out_ld > 0 && a_ld <= (1 << 19) && out_ld <= (1 << 19);
-    return (k == 128 || k == 256) && n > 0 && n % 128 == 0 && n / 128 <= 65535 && m > 0 && m <= INT32_MAX - 64 && bias && pitches &&
+    // row pitches the kernel's 32-bit offsets within a wave's range of rows can take under the launcher's split of m rows
+    if (k != 128 && k != 256) {
+        return false;
+    }
+    const bool pitches = a_ld > 0 && out_ld > 0 && a_ld <= (1 << 19) && out_ld <= (1 << 19) && m > 0 &&
+                         output_projection_rows_fit((int)k, m, a_ld, out_ld);
+    return n > 0 && n % 128 == 0 && n / 128 <= 65535 && m > 0 && m <= INT32_MAX - 64 && bias && pitches &&
            a_ld % 8 == 0 && out_ld % 8 == 0 && aligned(a, 16) && aligned(w, 16) && aligned(bias, 16) && aligned(out, 16);
 }
 
@@ -2568,112 +2534,3 @@ int kutacc_launch::fused_attention_tuning(const char *name, const char *value)
     }
     return KUTACC_HIP_EINVAL;
 }
-
-#ifdef KUTACC_TIMELINE
-// Development build only: the attention tile loop by itself.  One workgroup per CU, K and V fragments of `nt` key tiles in
-// LDS (arbitrary small values), pair-bias fragments streamed from a buffer that stays in L2, `waves` waves per
-// workgroup (4, 8 or 12: one, two or three per SIMD) each running attend_block_l2 `reps` times.  No projections, no
-// barriers, no epilogue: what the loop costs per key tile when nothing else shares the SIMD.
-namespace {
-template <bool HAS_NB>
-__global__ __launch_bounds__(768) void attention_loop_probe(const uint4 *nbf_g, float *out, int NT, int reps,
-                                                            unsigned long long *clk)
-{
-    extern __shared__ uint4 lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint4 *lds_k = lds, *lds_v = lds + NT * 2 * 64;
-    for (int i = tid; i < NT * 2 * 64 * 2; i += blockDim.x) {
-        bf16x8 v;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            v[e] = (bf16_t)(((i * 8 + e) * 37 % 101 - 50) * 0.01f);
-        }
-        lds[i] = as_uint4(v);
-    }
-    bf16x8 q0, q1;
-    f16x8 sel0, sel1;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        q0[e] = (bf16_t)(((lane * 8 + e) * 13 % 31 - 15) * 0.02f);
-        q1[e] = (bf16_t)(((lane * 8 + e) * 7 % 29 - 14) * 0.02f);
-    }
-    make_selectors_f16(lane, sel0, sel1);
-    const bf16x8 sumsel = rowsum_selector(lane);
-    __syncthreads();
-    const uint4 *nbf = nbf_g + (int64_t)wave * NT * 2 * 64 + lane;
-    float acc = 0.f;
-    const unsigned long long t0 = clock64();
-    for (int r = 0; r < reps; ++r) {
-        f32x16 o;
-        float l;
-        attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, nullptr, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o, l);
-        acc += o[0] + o[5] + l;
-        asm volatile("" : "+v"(q0), "+v"(q1));
-    }
-    const unsigned long long t1 = clock64();
-    out[blockIdx.x * blockDim.x + tid] = acc;
-    if (lane == 0) {
-        clk[blockIdx.x * 12 + wave] = t1 - t0;
-    }
-}
-} // namespace
-
-// result[0] = kernel time in microseconds, result[1] = shader clocks of the slowest wave (mean over workgroups),
-// result[2] = shader clocks of wave 0.  Returns 0 or a HIP status.
-extern "C" __attribute__((visibility("default"))) int kutacc_debug_attention_loop(int nt, int reps, int waves, int pair_bias,
-                                                                                  double *result)
-{
-    if (nt < 2 || nt > 32 || (nt & 1) || (waves != 4 && waves != 8 && waves != 12) || reps < 1 || !result) {
-        return KUTACC_HIP_EINVAL;
-    }
-    const int ncu = num_cus();
-    uint4 *nbf = nullptr;
-    float *out = nullptr;
-    unsigned long long *clk = nullptr;
-    const size_t nbf_bytes = (size_t)12 * nt * 2 * 64 * 16;
-    hipError_t e = hipMalloc(&nbf, nbf_bytes);
-    e = e == hipSuccess ? hipMalloc(&out, (size_t)ncu * 768 * 4) : e;
-    e = e == hipSuccess ? hipMalloc(&clk, (size_t)ncu * 12 * 8) : e;
-    if (e == hipSuccess) {
-        std::vector<uint16_t> h(nbf_bytes / 2);
-        for (size_t i = 0; i < h.size(); ++i) {
-            h[i] = (uint16_t)(0x3c00 + i * 7 % 64); // bf16 values a little above 0.0078
-        }
-        e = hipMemcpy(nbf, h.data(), nbf_bytes, hipMemcpyHostToDevice);
-    }
-    const size_t lds_bytes = 100 * 1024; // more than half a CU's LDS: one workgroup per CU
-    auto kern = pair_bias ? attention_loop_probe<true> : attention_loop_probe<false>;
-    e = e == hipSuccess ? hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) : e;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    e = e == hipSuccess ? hipEventCreate(&e0) : e;
-    e = e == hipSuccess ? hipEventCreate(&e1) : e;
-    float ms = 0.f;
-    for (int pass = 0; pass < 2 && e == hipSuccess; ++pass) { // the first pass warms up
-        e = hipMemset(clk, 0, (size_t)ncu * 12 * 8);
-        e = e == hipSuccess ? hipEventRecord(e0, nullptr) : e;
-        kern<<<ncu, waves * 64, lds_bytes, nullptr>>>(nbf, out, nt, reps, clk);
-        e = e == hipSuccess ? hipGetLastError() : e;
-        e = e == hipSuccess ? hipEventRecord(e1, nullptr) : e;
-        e = e == hipSuccess ? hipEventSynchronize(e1) : e;
-        e = e == hipSuccess ? hipEventElapsedTime(&ms, e0, e1) : e;
-    }
-    if (e == hipSuccess) {
-        std::vector<unsigned long long> c((size_t)ncu * 12);
-        e = hipMemcpy(c.data(), clk, c.size() * 8, hipMemcpyDeviceToHost);
-        double per_wave[12] = {};
-        for (int w = 0; w < ncu; ++w) {
-            for (int k = 0; k < waves; ++k) {
-                per_wave[k] += (double)c[(size_t)w * 12 + k] / ncu;
-            }
-        }
-        double mx = 0;
-        for (int k = 0; k < waves; ++k) {
-            mx = per_wave[k] > mx ? per_wave[k] : mx;
-        }
-        result[0] = ms * 1e3, result[1] = mx, result[2] = per_wave[0];
-    }
-    (void)hipEventDestroy(e0), (void)hipEventDestroy(e1);
-    (void)hipFree(nbf), (void)hipFree(out), (void)hipFree(clk);
-    return kutacc_hip_status(e);
-}
-#endif // KUTACC_TIMELINE

@@ -440,6 +440,17 @@ __global__ __launch_bounds__(64 * NW, 2) void global_attention_kernel(GlobalPara
     }
 }
 
+// Dynamic LDS of global_attention_kernel<., NW> for NT key tiles: staged weights and the waves' panels (16-byte units),
+// then mask and logits rows, per-wave states and the merge area (floats).
+constexpr size_t LDS_PER_WORKGROUP = 160 * 1024;
+constexpr size_t lds_bytes_for(int nw, int nt)
+{
+    return (size_t)(256 + 256 + 512 + 512 + 256 + nw * 256) * 16 + (size_t)(2 * nt * 32 + nw * 68 + 3 * GC + nw * 64 * MERGE_LD) * 4;
+}
+constexpr int MAX_SEQ_LEN = 12288; // what the four-wave layout holds
+static_assert(lds_bytes_for(4, MAX_SEQ_LEN / 32) <= LDS_PER_WORKGROUP && lds_bytes_for(4, MAX_SEQ_LEN / 32 + 1) > LDS_PER_WORKGROUP,
+              "MAX_SEQ_LEN must be the longest row whose four-wave layout fits the LDS");
+
 } // namespace
 
 namespace kutacc_launch {
@@ -451,7 +462,7 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
         return KUTACC_HIP_EINVAL;
     }
     if (a.dtype != KUTACC_DTYPE_BF16 || a.nheads * a.head_size != GC || a.nheads > 32 || a.head_size > 32 ||
-        a.batch > INT32_MAX || a.seq_len > 16384) {
+        a.batch > INT32_MAX || a.seq_len > MAX_SEQ_LEN) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
     // tokens of a batch row are addressed by 32-bit byte offsets from its first one
@@ -486,9 +497,16 @@ int global_attention(const kutacc_hip_global_attention_args_t &a, hipStream_t st
     const bool cached = p.NT <= 32;
     static int cu_table[KUTACC_DEVICE_SLOTS] = {};
     const int ncu = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
-    const int nw = (p.NT >= 16 && (!cached || a.batch <= ncu)) ? 8 : 4;
-    const size_t lds_bytes = (size_t)(256 + 256 + 512 + 512 + 256 + nw * 256) * 16 +
-                             (size_t)(2 * p.NT * 32 + nw * 68 + 3 * GC + nw * 64 * MERGE_LD) * 4;
+    // ... as long as the eight-wave layout fits the LDS: its fixed part is 36 KB larger than the four-wave one's, and
+    // both grow by 256 bytes per key tile (7808 positions with eight waves, MAX_SEQ_LEN with four).
+    int nw = (p.NT >= 16 && (!cached || a.batch <= ncu)) ? 8 : 4;
+    if (nw == 8 && lds_bytes_for(8, p.NT) > LDS_PER_WORKGROUP) {
+        nw = 4;
+    }
+    const size_t lds_bytes = lds_bytes_for(nw, p.NT);
+    if (lds_bytes > LDS_PER_WORKGROUP) {
+        return KUTACC_HIP_EUNSUPPORTED; // not reached while MAX_SEQ_LEN is what four waves can hold
+    }
     static size_t configured[4][KUTACC_DEVICE_SLOTS] = {};
     const void *fn = nw == 8 ? (cached ? reinterpret_cast<const void *>(global_attention_kernel<true, 8>)
                                        : reinterpret_cast<const void *>(global_attention_kernel<false, 8>))

@@ -25,8 +25,10 @@
  *     force on tiny shapes, and closed-form invariants.
  *   - Rbf16 rounding points: pinned only relative to R32 (must agree within bf16 tolerances);
  *     the closed GEMM library's accumulation order is unknown -> bit-level parity unpinned.
- *   - exp_mode 1 (emulation of the SVE FEXPA based fast_exp): parity unpinned; the instruction's
- *     table cannot be checked on this machine.
+ *   - exp_mode 1 (emulation of the SVE FEXPA based fast_exp, exported as oracle_ref_exp): the instruction itself cannot
+ *     be run on this machine; the emulation is pinned by what the arithmetic of fast_exp.h:21-27 fixes (results are
+ *     integer powers of 2^(1/64), the nearest one to exp(x) with ties away from zero, exactly 1 at 0, exactly 0 below
+ *     the u32 saturation, constant above the clamp, monotone), tests/test_oracle_pinning.py.
  */
 #include <math.h>
 #include <stdint.h>
@@ -316,6 +318,14 @@ static inline float ref_exp(float x, int exp_mode)
     float outv;
     memcpy(&outv, &bits, 4);
     return outv;
+}
+
+/* ref_exp over an array, for the tests that pin it. */
+void oracle_ref_exp(const float *x, float *y, int64_t n, int exp_mode)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        y[i] = ref_exp(x[i], exp_mode);
+    }
 }
 
 /* y[rows, n] (bf16, row stride ldy, col stride cs) = x[rows, kdim] . w[n, kdim]^T (+ bias[n]),

@@ -50,6 +50,14 @@ def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
 
+def ref_exp(x, exp_mode=1):
+    """The oracle's model of the reference's fast_exp (src/math/fast_exp.h:21-27) on an array of float32."""
+    x = _f32(x).ravel()
+    y = np.empty_like(x)
+    lib().oracle_ref_exp(x.ctypes.data_as(_f32p), y.ctypes.data_as(_f32p), _i64(x.size), ctypes.c_int(exp_mode))
+    return y
+
+
 def _u16(a):
     a = np.ascontiguousarray(a)
     assert a.dtype == np.uint16, a.dtype

@@ -287,3 +287,51 @@ def test_glue_launch_layer_rejects_bad_arguments_without_a_device():
     act = n * n * h * 32 * 2
     assert L.kutacc_hip_triangle_attention_workspace(n, h) == 3 * act + h * n * n * 2 + n * n * 2
     assert L.kutacc_hip_triangle_attention_workspace(-1, h) == -1
+
+
+def test_global_attention_launch_layer_rejects_long_rows_before_any_launch():
+    """A row's mask and logits must fit the workgroup's LDS: 12288 positions.  Longer rows are refused by the argument
+    checks, before any HIP call, so this runs without a GPU (the pointers are never dereferenced)."""
+    a = capi.HipGlobalAttentionArgs()
+    fake = 1 << 20  # 16-byte aligned, non-null
+    a.batch, a.nheads, a.head_size, a.dtype = 2, 8, 8, capi.K_BF16
+    for f in ("q_data", "q_mask", "query_w", "key_w", "value_w", "gating_w", "output_w", "gating_b", "output_b", "out"):
+        setattr(a, f, fake)
+    a.q_data_stride_s = a.out_stride_s = 64
+    for seq_len in (12320, 16384):
+        a.seq_len = seq_len
+        a.q_data_stride_b = a.out_stride_b = 64 * seq_len
+        a.q_mask_stride_b = seq_len
+        assert capi.lib().kutacc_hip_global_attention(ctypes.byref(a), None) == capi.EUNSUPPORTED
+
+
+def test_stream_and_blocking_are_inherited_by_threads_that_never_set_them():
+    """A thread that sets a stream keeps its own; one that never did sees the value set last by anyone (a host that
+    configures the library on one thread and calls it from pool workers).  No GPU needed: the stream is only stored."""
+    import threading
+    lib = capi.lib()
+    lib.kutacc_hip_get_stream.restype = ctypes.c_void_p
+    seen = {}
+    try:
+        lib.kutacc_hip_set_stream(ctypes.c_void_p(0x1000))
+
+        def fresh():
+            seen["fresh"] = lib.kutacc_hip_get_stream()
+
+        def own():
+            lib.kutacc_hip_set_stream(ctypes.c_void_p(0x2000))
+            seen["own"] = lib.kutacc_hip_get_stream()
+
+        for fn in (fresh, own, fresh):
+            t = threading.Thread(target=fn)
+            t.start()
+            t.join()
+            if fn is fresh and "first" not in seen:
+                seen["first"] = seen.pop("fresh")
+        assert seen["first"] == 0x1000        # inherited from the configuring thread
+        assert seen["own"] == 0x2000          # a thread's own setting
+        assert seen["fresh"] == 0x2000        # a later fresh thread inherits the value set last
+        assert lib.kutacc_hip_get_stream() == 0x1000  # and this thread keeps its own
+    finally:
+        lib.kutacc_hip_set_stream(None)
+        assert not lib.kutacc_hip_get_stream()

@@ -68,6 +68,8 @@ SHAPES = [
     # both workgroup sizes of the kernel: eight waves while a row has a CU to itself (at most 256 rows) or is streamed,
     # four when two rows share a CU
     (300, 512, 8, 8, "random"), (257, 1024, 4, 16, "random"), (256, 640, 8, 8, "random"), (3, 2100, 4, 16, "random"),
+    # streamed rows on either side of what the eight-wave layout's LDS holds (7808 positions), and the longest row
+    (2, 7808, 8, 8, "random"), (2, 8192, 8, 8, "random"), (1, 12288, 8, 8, "random"),
 ]
 
 
@@ -121,3 +123,11 @@ def test_global_attention_rejects_other_channel_counts(torch_cuda, capfd):
     op.run()
     assert capi.error_flag()
     assert "invalid int value" in capfd.readouterr().err
+
+
+def test_global_attention_rejects_rows_beyond_the_lds(torch_cuda):
+    c = make_case(5, 1, 12320, 8, 8)
+    op, ten, _ = device_op(torch_cuda, c)
+    op.run()
+    assert capi.error_flag()
+    capi.clear_error()

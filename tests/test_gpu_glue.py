@@ -186,6 +186,39 @@ def test_triangle_attention_block_full_size_orientation_identity(torch_cuda, lay
     assert not helpers.same_bits(end, z)
 
 
+def block_oracle_rows(c, ending, rows):
+    """block_oracle for the batch rows `rows` of the attention only (rows i of the pair tensor for the starting node,
+    columns for the ending node): rows of the attention are independent, so the oracle's LayerNorm and pair bias run on
+    the whole tensor and its attention on the sample.  Returns the updated pair_act entries [len(rows), n, c] in the
+    orientation of the attention (entry [a, k] is pair_act[rows[a], k] or, ending node, pair_act[k, rows[a]])."""
+    from oracle import oracle
+    z, mask = c["z"], c["mask"]
+    if ending:
+        z, mask = z.transpose(1, 0, 2), mask.T
+    n, _, ch = z.shape
+    zn = oracle.layernorm_rows_f32(np.ascontiguousarray(z).reshape(-1, ch), c["gamma"], c["beta"], 1e-5).reshape(n, n, ch)
+    nb = np.ascontiguousarray(oracle.linear_f32(zn.reshape(-1, ch), c["bias_w"]).reshape(n, n, c["heads"]).transpose(2, 0, 1))
+    bias = (np.ascontiguousarray(mask[rows]) * np.float32(1e9) - np.float32(1e9)).astype(np.float32)
+    out = oracle.gating_attention_f32(np.ascontiguousarray(zn[rows]), c["wq"], c["wk"], c["wv"], c["wg"], c["bg"], c["wo"],
+                                      c["bo"], bias, nb, c["heads"])
+    return z[rows] + out
+
+
+@pytest.mark.parametrize("n", [384, 1024])
+def test_triangle_attention_block_full_size_sampled_rows(torch_cuda, n):
+    """The pair sizes the block is benchmarked at, both orientations: the oracle on a sample of attention rows (first,
+    last, the padded residues, rows on either side of 32-row tile edges), every other entry checked for finiteness."""
+    torch = torch_cuda
+    c = block_case(7000 + n, n, 4)
+    rows = sorted({0, 1, 31, 32, 33, n // 2 - 1, n // 2, n - 34, n - 33, n - 32, n - 4, n - 3, n - 2, n - 1})
+    for ending in (False, True):
+        got = run_block(torch, c, ending)
+        assert bool(torch.isfinite(got).all())
+        want = block_oracle_rows(c, ending, rows)
+        sample = got[:, rows].transpose(0, 1) if ending else got[rows]
+        helpers.check_close(helpers.to_numpy(sample.contiguous()), want, "bf16", f"block n={n} ending={ending}, sampled rows")
+
+
 def test_fused_layernorm_drops_the_normalised_copy_from_the_workspace(torch_cuda):
     """With the LayerNorm inside the attention kernel the blocks keep no normalised activation: the workspace is one
     activation smaller wherever the persistent kernel runs (384 residues), and unchanged where it does not (1024)."""
@@ -525,3 +558,41 @@ def test_pair_stack_blocks_replay_from_a_hip_graph(torch_cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert helpers.same_bits(z, want)
+
+
+def test_msa_attention_blocks_full_size_sampled_rows(torch_cuda):
+    """The MSA shapes the blocks are benchmarked at -- row-wise with pair bias at 512 sequences x 256 residues, column-wise
+    at 1024 sequences x 384 residues -- against the oracle on a sample of attention rows (sequences for the row-wise
+    form, residues for the column-wise one), every other entry checked for finiteness."""
+    from oracle import oracle
+    torch = torch_cuda
+    for column, n_seq, n_res in ((False, 512, 256), (True, 1024, 384)):
+        c = msa_case(8000 + n_seq, n_seq, n_res, 8, 128)
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+            device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+        msa = dev(c["m"])
+        w = {k: dev(c[k]) for k in ("ln_gamma", "ln_beta", "wq", "wk", "wv", "wg", "bg", "wo", "bo")}
+        pair = None if column else {"pair_act": dev(c["z"]), "pair_ln_gamma": dev(c["pair_ln_gamma"]),
+                                    "pair_ln_beta": dev(c["pair_ln_beta"]), "bias_w": dev(c["bias_w"])}
+        blk = capi.MsaAttentionBlock(msa, dev(c["mask"]), w, 8, pair)
+        rc = blk.run()
+        torch.cuda.synchronize()
+        assert rc == 0, rc
+        assert bool(torch.isfinite(msa).all())
+        m, mask = (c["m"].transpose(1, 0, 2), c["mask"].T) if column else (c["m"], c["mask"])
+        B = m.shape[0]
+        rows = sorted({0, 1, 7, 8, 9, B // 2, B - 10, B - 9, B - 8, B - 3, B - 2, B - 1})
+        ch = m.shape[-1]
+        mn = oracle.layernorm_rows_f32(np.ascontiguousarray(m[rows]).reshape(-1, ch), c["ln_gamma"], c["ln_beta"], 1e-5)
+        mn = mn.reshape(len(rows), -1, ch)
+        nb = None
+        if not column:
+            cz = c["z"].shape[-1]
+            zn = oracle.layernorm_rows_f32(c["z"].reshape(-1, cz), c["pair_ln_gamma"], c["pair_ln_beta"], 1e-5)
+            nb = np.ascontiguousarray(oracle.linear_f32(zn, c["bias_w"]).reshape(n_res, n_res, 8).transpose(2, 0, 1))
+        bias = (np.ascontiguousarray(mask[rows]) * np.float32(1e9) - np.float32(1e9)).astype(np.float32)
+        out = oracle.gating_attention_f32(mn, c["wq"], c["wk"], c["wv"], c["wg"], c["bg"], c["wo"], c["bo"], bias, nb, 8)
+        want = m[rows] + out
+        sample = msa[:, rows].transpose(0, 1) if column else msa[rows]
+        helpers.check_close(helpers.to_numpy(sample.contiguous()), want, "bf16",
+                            f"msa block {n_seq}x{n_res} column={column}, sampled rows")

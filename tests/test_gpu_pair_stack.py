@@ -487,3 +487,93 @@ def test_pair_stack_against_the_golden_fixture(torch_cuda):
     assert not capi.error_flag()
     helpers.check_close(helpers.to_numpy(gate), g["tm.gate"], "bf16", "fixture gate")
     helpers.check_close(helpers.to_numpy(res), g["tm.last"], "bf16", "fixture gated output")
+
+
+# ---- host pointers: staged through the device, bit-identical to the device-pointer call -----------------------
+def _bits(t):
+    """bf16 torch tensor (device) -> its bit patterns as a numpy uint16 array."""
+    import torch
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _host_bits(a):
+    """float32 numpy array that holds bf16-representable values -> bf16 bit patterns (what a host caller passes)."""
+    from oracle import oracle
+    return oracle.to_bf16_bits(np.ascontiguousarray(a, dtype=np.float32))
+
+
+def test_transition_host_pointers_match_device_pointers(torch_cuda):
+    """The reference's callers hand kutacc_af2_transition host tensors (reference src/attention/transition.cpp:42-67)."""
+    torch = torch_cuda
+    for shape in [(2, 37, 128, 512), (1, 9, 24, 40)]:  # one-kernel form, two GEMM launches
+        c = transition_case(77, *shape)
+        out, _ = run_transition(torch, c)
+        batch, n_res, c_o, c_i = shape
+        h_out = np.zeros((batch, n_res, c_o), np.uint16)
+        h_mid = np.zeros((batch * n_res, c_i), np.uint16)
+        op = capi.Transition(_host_bits(c["x"]), _host_bits(c["w1"]), c["b1"], _host_bits(c["w2"]), c["b2"], h_mid, h_out)
+        op.run()
+        assert not capi.error_flag()
+        np.testing.assert_array_equal(h_out, _bits(out))
+    # mixed memory spaces are rejected
+    x = dev(torch, c["x"])
+    op = capi.Transition(x, _host_bits(c["w1"]), c["b1"], _host_bits(c["w2"]), c["b2"], h_mid, h_out)
+    op.run()
+    assert capi.error_flag()
+    capi.clear_error()
+
+
+@pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
+def test_triangle_multiplication_host_pointers_match_device_pointers(torch_cuda, incoming):
+    """All four steps on host arrays (reference src/attention/triangle_multiplication.cpp:153-240 takes host tensors)
+    against the same steps on device tensors, bit for bit, each step fed the device result of the step before."""
+    torch = torch_cuda
+    n, c_o, c_i = 40, 128, 128
+    c = tm_case(901, n, c_o, c_i)
+    dx, dmask = dev(torch, c["x"]), dev(torch, c["mask"])
+    hx, hmask = _host_bits(c["x"]), _host_bits(c["mask"])
+    sides = {}
+    for side in "lr":
+        d_proj = calc_proj(torch, c, side, n, c_o, c_i, dx, dmask)
+        h_proj = np.zeros((c_i, n, n), np.uint16)
+        h_gate = np.zeros_like(h_proj)
+        keep = [_host_bits(c[side + "pw"]), c[side + "pb"], _host_bits(c[side + "gw"]), c[side + "gb"]]
+        h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]
+        hp, hxx, hg, hm = capi.tensor(h_proj), capi.tensor(hx), capi.tensor(h_gate), capi.tensor(hmask)
+        acts = capi.TmActInputs(n, n, hp.handle, hxx.handle, hg.handle)
+        weights = capi.TmProjWeights(c_o, c_i, h[0].handle, h[1].handle, h[2].handle, h[3].handle)
+        capi.kutacc_af2_triangle_multiplication_calc_proj(acts, hm, weights, False)
+        assert not capi.error_flag()
+        np.testing.assert_array_equal(h_proj, _bits(d_proj))
+        sides[side] = (d_proj, h_proj)
+    d_center = equation(torch, sides["l"][0], sides["r"][0], n, incoming)
+    h_center = np.zeros((c_i, n, n), np.uint16)
+    hc, hl, hr = capi.tensor(h_center), capi.tensor(sides["l"][1]), capi.tensor(sides["r"][1])
+    capi.kutacc_af2_triangle_multiplication_equation(hc, hl, hr, n, incoming)
+    assert not capi.error_flag()
+    np.testing.assert_array_equal(h_center, _bits(d_center))
+    # gate and output projection on a channel-last centre
+    d_ctr = (d_center.permute(1, 2, 0).float() / math.sqrt(n)).to(torch.bfloat16).contiguous()
+    h_ctr = _bits(d_ctr)
+    d_gate = torch.zeros((n, n, c_o), dtype=torch.bfloat16, device="cuda")
+    d_out = torch.zeros_like(d_gate)
+    dkeep = [dev(torch, c["gating_w"]), dev(torch, c["gating_b"], torch.float32), dev(torch, c["out_w"]),
+             dev(torch, c["out_b"], torch.float32)]
+    hkeep = [_host_bits(c["gating_w"]), c["gating_b"], _host_bits(c["out_w"]), c["out_b"]]
+    h_gate, h_out = np.zeros((n, n, c_o), np.uint16), np.zeros((n, n, c_o), np.uint16)
+    results = []
+    for keep, x_, gate_, out_, ctr_ in [(dkeep, dx, d_gate, d_out, d_ctr), (hkeep, hx, h_gate, h_out, h_ctr)]:
+        h = [capi.tensor(keep[0]), capi.tensor(keep[1], capi.K_FP32), capi.tensor(keep[2]), capi.tensor(keep[3], capi.K_FP32)]
+        hxx, hg, ho, hcc = capi.tensor(x_), capi.tensor(gate_), capi.tensor(out_), capi.tensor(ctr_)
+        acts = capi.TmActInputs(n, n, None, hxx.handle, None)
+        weights = capi.TmLinearWeights(c_o, c_i, h[0].handle, h[1].handle, h[2].handle, h[3].handle)
+        capi.kutacc_af2_triangle_multiplication_gate_and_out_linear(hg, ho, acts, hcc, weights, False)
+        assert not capi.error_flag()
+        results.append((hg, ho))
+    np.testing.assert_array_equal(h_gate, _bits(d_gate))
+    np.testing.assert_array_equal(h_out, _bits(d_out))
+    for hg, ho in results:
+        capi.kutacc_af2_triangle_multiplication_last(ho, hg, n, n, c_o)
+        assert not capi.error_flag()
+    np.testing.assert_array_equal(h_out, _bits(d_out))
+    assert np.any(h_out != 0)

@@ -224,6 +224,81 @@ def test_absent_pair_bias_equals_zero_pair_bias():
     np.testing.assert_array_equal(run_f32(c2), out)
 
 
+# ---- fast_exp emulation (reference src/math/fast_exp.h:21-27) -----------------------------------------
+# The FEXPA instruction cannot be run here.  What the arithmetic around it fixes: the result is 2^(n/64) for the integer
+# n nearest to x * 64 / ln 2 (ties away from zero), assembled from n's low six bits (table index) and the bits above
+# (exponent); a negative n + 8128 saturates to 0 in the unsigned conversion and gives +0.0; x is clamped at ln(FLT_MAX).
+def _fexpa_grid():
+    rng = np.random.default_rng(7)
+    xs = [np.linspace(-100.0, 95.0, 200001), rng.uniform(-20.0, 20.0, 200000), rng.normal(0.0, 1.0, 100000),
+          np.array([0.0, -0.0, 1.0, -1.0, 88.0, 88.72283, 88.72284, 88.8, 100.0, 1e30, -87.9, -88.0, -88.1, -1e30])]
+    return np.concatenate(xs).astype(np.float32)
+
+
+def test_fast_exp_emulation_returns_the_nearest_64th_octave():
+    x = _fexpa_grid()
+    y = oracle.ref_exp(x, 1).astype(np.float64)
+    inside = (x > -87.3) & (x < 88.7)  # below -87.34 the exponent field is 0 and the table bits read as a subnormal
+    xi, yi = x[inside].astype(np.float64), y[inside]
+    steps = 64.0 * np.log2(yi)  # must be integers: the result is a power of 2^(1/64) (mantissa from a 64-entry table)
+    n = np.rint(steps)
+    assert np.abs(steps - n).max() < 2e-5  # 1 ulp of fp32 in the mantissa is 64 * 1.7e-7 of a step
+    # ... and the nearest one to exp(x): the exact position is x * 64 / ln 2; fp32 rounding of the constant 92.33248
+    # and of the multiply-add moves it by < 1e-3 of a step at |x| < 88, which only matters next to a tie
+    pos = xi * (64.0 / np.log(2.0))
+    dist = np.abs(pos - n)
+    assert dist.max() <= 0.5 + 2e-3
+    # relative error against exp: at most half a step, 2^(1/128) - 1 = 0.543 %
+    rel = np.abs(yi / np.exp(xi) - 1.0)
+    assert rel.max() <= 2.0 ** (1.0 / 128.0) - 1.0 + 3e-5
+    assert rel.max() > 4e-3  # and it is that coarse: a libm exp would pass everything above but this
+
+
+def test_fast_exp_emulation_ties_round_away_from_zero():
+    # x = (k + 0.5) * ln 2 / 64 cannot be hit exactly in fp32, but the integer-valued products can: with x = m / 92.33248
+    # rounded to fp32 the fma lands within an ulp of m + 8128, so walk fp32 neighbours until the product is the exact
+    # half-integer and check the direction of rounding on the bit level instead
+    k = np.arange(-200, 200, dtype=np.float64)
+    c = np.float32(92.33248)
+    hits = 0
+    for kk in k:
+        target = kk + 0.5 + 8128.0
+        x0 = np.float32((kk + 0.5) / float(c))
+        for _ in range(8):  # search the neighbourhood for an x whose single-rounded fma equals the tie exactly
+            t = np.float32(np.float64(x0) * np.float64(c) + 8128.0)  # double product is exact enough: one rounding
+            if float(t) == target:
+                y = float(oracle.ref_exp(np.array([x0], np.float32), 1)[0])
+                want = 2.0 ** ((kk + 1.0) / 64.0)  # half away from zero in the biased (positive) domain
+                assert abs(y / want - 1.0) < 2e-7, (kk, y, want)
+                hits += 1
+                break
+            x0 = np.nextafter(x0, np.float32(np.inf if float(t) < target else -np.inf), dtype=np.float32)
+    assert hits > 50
+
+
+def test_fast_exp_emulation_special_values():
+    e = lambda v: oracle.ref_exp(np.array(v, np.float32), 1)
+    assert e([0.0])[0] == 1.0 and e([-0.0])[0] == 1.0
+    ln2 = np.float32(np.log(2.0))
+    got = e([ln2, -ln2, 2 * ln2])  # n = +-64, 128 exactly (the products are within 1e-5 of the integers)
+    np.testing.assert_array_equal(got, np.array([2.0, 0.5, 4.0], np.float32))
+    # below -8128 / 92.33248 = -88.03 the biased integer is <= 0, the unsigned conversion saturates and FEXPA(0) is +0.0
+    z = e([-88.04, -88.5, -100.0, -1e9, -3e38, -np.inf])
+    assert np.all(z == 0.0) and not np.any(np.signbit(z))
+    assert e([-88.02])[0] > 0.0
+    # the clamp at ln(FLT_MAX): everything at or above it gives the same result (exponent field 255, fraction 0)
+    top = e([88.72284, 88.8, 100.0, 1e30, np.inf])
+    assert np.all(top == top[0]) and np.isinf(top[0])
+    assert np.isfinite(e([88.7])[0])
+    # monotone non-decreasing over the whole grid
+    x = np.sort(_fexpa_grid())
+    y = oracle.ref_exp(x, 1).astype(np.float64)
+    assert np.all(np.diff(y[np.isfinite(y)]) >= 0.0) and np.all(np.isinf(y[x >= 88.72284]))
+    # exp_mode 0 is libm
+    xm = np.linspace(-30, 30, 1001).astype(np.float32)
+    np.testing.assert_allclose(oracle.ref_exp(xm, 0), np.exp(xm.astype(np.float64)), rtol=3e-7)
+
+
 # ---- Rbf16 (reference rounding points) ---------------------------------------------------------------
 def to_bits_case(c):
     b = oracle.to_bf16_bits

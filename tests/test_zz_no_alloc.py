@@ -68,3 +68,41 @@ def test_static_scratch_entry_rejects_what_it_cannot_run():
     assert capi.lib().kutacc_hip_gating_attention_static(ctypes.byref(a), None) == capi.EUNSUPPORTED
     assert capi.lib().kutacc_hip_gating_attention_static(None, None) == capi.EINVAL
     assert not bool(ten["out"].any())
+
+
+def test_static_scratch_entry_allocates_nothing_and_records_no_events():
+    """After one warm-up call per shape, a run of calls with per-kernel profiling switched on leaves the device's free
+    memory where it was (hipMemGetInfo) and adds no entry to the profile (no events are created for this entry)."""
+    import torch
+    assert torch.cuda.is_available(), "this test needs the GPU"
+    capi.set_stream(None)
+    lib = capi.lib()
+    w = make_workload(3, batch=12, seq_len=384)
+    ten, scratch = helpers.to_device(w)
+    a = helpers.hip_args(w, ten, scratch, capi.PATH_FUSED)
+    a.q = a.k = a.v = a.gate = None
+    assert lib.kutacc_hip_gating_attention_static(ctypes.byref(a), None) == 0  # warm-up: symbol address, LDS opt-in
+    torch.cuda.synchronize()
+    want = ten["out"].clone()
+
+    def profile_entries():
+        name = ctypes.create_string_buffer(128)
+        ms, launches, flops = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+        n = 0
+        while lib.kutacc_hip_profile_read(n, name, 128, ctypes.byref(ms), ctypes.byref(launches), ctypes.byref(flops)) == 0:
+            n += 1
+        return n
+
+    lib.kutacc_hip_profile_enable(1)
+    try:
+        entries_before = profile_entries()
+        free_before, _ = torch.cuda.mem_get_info()
+        for _ in range(20):
+            assert lib.kutacc_hip_gating_attention_static(ctypes.byref(a), None) == 0
+        torch.cuda.synchronize()
+        free_after, _ = torch.cuda.mem_get_info()
+        assert free_after == free_before, (free_before, free_after)
+        assert profile_entries() == entries_before
+    finally:
+        lib.kutacc_hip_profile_enable(0)
+    assert helpers.same_bits(ten["out"], want)
