@@ -49,6 +49,7 @@ namespace {
 constexpr int HEAD = 32;            // head_size the MFMA kernels are written for
 constexpr int WEIGHT_LOADS_IN_FLIGHT = 8; // per wave, while the weight fragments of a head are copied into LDS
 constexpr int MAX_WAVES = 12;       // fused_head_kernel: 768 threads, 3 waves per SIMD, 168 VGPRs each
+constexpr int FAIR_SLICE_SHIFT = 11;  // log2 of the clocks a wave keeps one issue priority (timeslice_priority); 2^8 to 2^13 measured alike
 constexpr float RESCALE_GAP = 5.5f; // running max may lag the true max by this much (natural log units, ~8 octaves)
 
 // Waves per workgroup a given fused_head_kernel instantiation may be launched with.  One query block
@@ -420,6 +421,34 @@ __device__ __forceinline__ void attend_block(const uint4 *lds_k, const uint4 *ld
 //   nbf : this wave's fragment-major pair bias, already offset by the lane: tile t at nbf[(2t+m)*64]
 //   returns the row sum of every lane's query in l_out
 
+// Issue priority of a wave among the (up to three) waves of its workgroup on one SIMD, by time slices of the clock they
+// all see: in slice s the wave with turn (s + d) mod 3 gets priority 2 - d, so over three slices every wave is first,
+// second and third once, however far it has come.  Left to the arbiter's oldest-first rule the oldest wave runs its
+// attention almost alone and the youngest is left to finish by itself while the others wait at the barrier.  The
+// branches sit inside one asm statement: as branches of a loop body they split the body into blocks, and the register
+// allocator spills across them.  Call once per tile pair; reset with s_setprio 0 after the loop.
+__device__ __forceinline__ void timeslice_priority(uint32_t turn, int shift)
+{
+    const uint32_t tick = ((uint32_t)__builtin_amdgcn_s_memtime() >> shift) & 0x3fffu;
+    const uint32_t slice = tick - 3u * ((tick * 0x5556u) >> 16); // tick mod 3
+    const uint32_t d = turn >= slice ? turn - slice : turn + 3u - slice;
+    asm volatile("s_cmp_eq_u32 %0, 0\n\t"
+                 "s_cbranch_scc1 .Lfirst_%=\n\t"
+                 "s_cmp_eq_u32 %0, 1\n\t"
+                 "s_cbranch_scc1 .Lsecond_%=\n\t"
+                 "s_setprio 0\n\t"
+                 "s_branch .Ldone_%=\n"
+                 ".Lfirst_%=:\n\t"
+                 "s_setprio 2\n\t"
+                 "s_branch .Ldone_%=\n"
+                 ".Lsecond_%=:\n\t"
+                 "s_setprio 1\n"
+                 ".Ldone_%=:"
+                 :
+                 : "s"(d)
+                 : "scc");
+}
+
 // A operand of the row-sum MFMA (16x16x32: lane -> row lane&15, k-chunk lane>>4).  The B operand is a
 // probability fragment of the 32x32x16 layout (lane -> query lane&31, 8 keys of half lane>>5), which the
 // 16x16x32 shape reads as column lane&15, k-chunk lane>>4: chunks 0 and 2 belong to query n, chunks 1 and
@@ -450,7 +479,7 @@ template <bool HAS_NB, bool WITH_MASK, bool SHIFT>
 __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4,
                                                 const uint4 *nbf, bf16x8 q0, bf16x8 q1, f16x8 sel0, f16x8 sel1,
                                                 bf16x8 sumsel, int NB, int lane, float shift, f32x16 &o_out, float &l_out,
-                                                int prio_phase = -1)
+                                                int prio_phase = -1, int fair_turn = -1)
 {
     const int npairs = NB >> 1;
     const uint4 *kp = lds_k + lane;
@@ -542,6 +571,9 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
     };
 
     for (int pair = 0; pair < npairs; ++pair) {
+        if (fair_turn >= 0) {
+            timeslice_priority((uint32_t)fair_turn, FAIR_SLICE_SHIFT);
+        }
         if (prio_phase >= 0) {
             // two waves of one workgroup share a SIMD in lock step; the arbiter prefers the older one, which then runs
             // ahead and leaves the other to finish alone.  Alternating the issue priority per tile pair keeps them level.
@@ -561,6 +593,9 @@ __device__ __forceinline__ void attend_block_l2(const uint4 *lds_k, const uint4 
         half_step(xb, xa, tn, wa0, wa1, clampt(tn + 2), tn + 1);
         v0 = vp[(tn * 2 + 0) * 64], v1 = vp[(tn * 2 + 1) * 64];
         fence();
+    }
+    if (fair_turn >= 0) {
+        __builtin_amdgcn_s_setprio(0);
     }
     o_out = o;
     l_out = rowsum_fetch(lacc, lane);
@@ -1206,6 +1241,9 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
     __syncthreads();
 
     const int j = wave; // this wave's sequence block
+    // With three waves per SIMD (128 channels) the waves take turns at the issue priorities during the attention; with two
+    // (256 channels) the arbiter's own order measured 2 % faster.
+    const int fair_turn = C == 128 ? wave >> 2 : -1;
     const float qmul = L2MODE ? p.qscale * LOG2E : p.qscale;
     const float mask_scale = L2MODE ? LOG2E : 1.0f;
     const bf16x8 sumsel = rowsum_selector(lane);
@@ -1402,10 +1440,10 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             const uint4 *nbf = HAS_NB ? p.nbf + ((int64_t)(h * NB + j) * NT * 2) * 64 + lane : nullptr;
             if (flags == 0u) {
                 attend_block_l2<HAS_NB, false, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o,
-                                                      l);
+                                                      l, -1, fair_turn);
             } else {
                 attend_block_l2<HAS_NB, true, false>(lds_k, lds_v, mask4, nbf, q0, q1, sel0, sel1, sumsel, NT, lane, 0.f, o,
-                                                     l);
+                                                     l, -1, fair_turn);
             }
             const bool ok = !__any(!(l > 1e-30f && l < 1e30f));
             if (!ok) {
@@ -1431,6 +1469,518 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
             }
             store_gated(p.avg + (int64_t)b * p.avg_sb + (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * (lane_o >> 5), o,
                         __builtin_amdgcn_rcpf(l), gv);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// persistent_pair_kernel: persistent_head_kernel walking its batch rows two at a time (128 channels, log2 units).
+// The pair bias of a (head, query block, key tile) is the same for every batch row, so a wave that attends the same query
+// block of two rows at once fetches it once -- as fp32, in accumulator order, straight into the C operand of the logits
+// MFMAs of both rows (pair_bias_tiles_kernel writes that copy).  Per row and key tile this moves the same bytes as the
+// fp16 fragments of persistent_head_kernel and takes the two selector MFMAs out of the loop (matrix pipe 224 -> 160 clocks
+// per tile); the two rows' instruction streams are independent, which gives the scheduler what a fourth wave per SIMD
+// would; and every weight fragment read from LDS in the projection phase serves two rows.
+// LDS, 16-byte units: W[4][CK][64]  K[2 rows][NT][2][64]  V[2 rows][NT][2][64]  panel[NB waves][128];
+// then floats mask[2 pairs in flight][2 rows][NT*32] and four uint32 of tile flags.  At 384 positions that is
+// 32 + 96 + 24 + 6 KB: the panels are half the size of persistent_head_kernel's (32 rows x 32 channels); during the
+// attention a wave's panel holds the sigmoid of the first row's gate, the second row's waits in eight registers.
+// ------------------------------------------------------------------------------------------------
+
+// Wave-private 2 KB staging panel: 32 rows x 64 bytes in 16-byte slots, filled with two coalesced loads (lane l -> row
+// l / 4 + 16 i, chunk l % 4) and read back in MFMA fragment order; the chunk index is XOR-swizzled by row so that both
+// access patterns are free of LDS bank conflicts.
+__device__ __forceinline__ int panel32_slot(int row, int chunk) { return row * 4 + (chunk ^ (((row >> 2) & 1) | (((row >> 4) & 1) << 1))); }
+
+struct Panel32Regs {
+    uint4 r0, r1;
+};
+
+// rows row0 .. row0 + 31 (clamped to last_row) of a row-major bf16 matrix, 32 columns from col0; 32-bit byte offsets from
+// a wave-uniform base as in panel_load_near
+__device__ __forceinline__ Panel32Regs panel32_load_near(const bf16_t *base, uint32_t ld, int row0, int last_row, int col0, int lane)
+{
+    const char *bytes = reinterpret_cast<const char *>(base);
+    const uint32_t pitch = 2u * ld;
+    const uint32_t col = 2u * (uint32_t)col0 + 16u * (uint32_t)(lane & 3);
+    const uint32_t last = (uint32_t)last_row * pitch + col;
+    const uint32_t first = __umul24((uint32_t)(row0 + (lane >> 2)), pitch) + col;
+    Panel32Regs p;
+    p.r0 = *reinterpret_cast<const uint4 *>(bytes + min(first, last));
+    p.r1 = *reinterpret_cast<const uint4 *>(bytes + min(first + 16u * pitch, last));
+    return p;
+}
+
+__device__ __forceinline__ void panel32_store(uint4 *panel, int lane, const Panel32Regs &p)
+{
+    const int row = lane >> 2, chunk = lane & 3;
+    panel[panel32_slot(row, chunk)] = p.r0;
+    panel[panel32_slot(row + 16, chunk)] = p.r1;
+}
+
+// Pair bias [H, S, S] -> fp32 tiles in accumulator order, in log2 units: for head h, query block j and key tile t,
+// [h][j][t][4][64 lanes] x 16 bytes; lane (r, g) holds keys 32 t + 16 g .. + 15 of query 32 j + pi(r), four per 16-byte
+// piece -- registers 4 a .. 4 a + 3 of the logits accumulator.  Queries past S repeat row S - 1, keys past S read as zero
+// (their mask bias is -inf); -inf entries become the most negative finite value so that a row of them still has a
+// finite maximum.
+__global__ __launch_bounds__(64) void pair_bias_tiles_kernel(const bf16_t *__restrict__ nb, int64_t nb_sh, int64_t nb_sq, int S,
+                                                             int NB, int NT, int vec, f32x4 *__restrict__ out)
+{
+    const int lane = threadIdx.x;
+    const int r = lane & 31, g = lane >> 5;
+    const int t = blockIdx.x % NT, j = blockIdx.x / NT, h = blockIdx.y;
+    int q = 32 * j + pi_row(r);
+    q = q < S ? q : S - 1;
+    const int key0 = 32 * t + 16 * g;
+    const bf16_t *src = nb + (int64_t)h * nb_sh + (int64_t)q * nb_sq + key0;
+    float v[16];
+    if (vec && key0 + 16 <= S) {
+        const bf16x8 s0 = as_bf16x8(*reinterpret_cast<const uint4 *>(src)), s1 = as_bf16x8(*reinterpret_cast<const uint4 *>(src + 8));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[e] = to_f32(s0[e]), v[8 + e] = to_f32(s1[e]);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            v[e] = key0 + e < S ? to_f32(src[e]) : 0.f;
+        }
+    }
+    f32x4 *dst = out + ((((int64_t)h * NB + j) * NT + t) * 4) * 64 + lane;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        f32x4 o;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const float x = v[4 * a + c] * LOG2E;
+            o[c] = x < -3.0e38f ? -3.0e38f : x; // a comparison, not a max: a NaN stays a NaN
+        }
+        dst[a * 64] = o;
+    }
+}
+
+// Attention of one 32-query block of two batch rows A and B (same head) in log2 units; see attend_block_l2 for the
+// formulation.  Tiles are walked A(0) B(0) A(1) B(1) ...: while the softmax and P.V of one (row, tile) run on the vector
+// ALU, the logits MFMAs of the next one are in the matrix pipe.
+//   lds_kA/vA/kB/vB : K and V fragments of the two rows, [tile][kstep][lane]
+//   maskA4 / maskB4 : fp32 mask bias of the rows (log2 units), offset by 16 g floats; added to every tile (WITH_MASK only)
+//   nbc             : fp32 pair-bias tiles of this head and query block, offset by the lane: tile t, piece a at
+//                     nbc[(4 t + a) * 64]; nullptr without a pair bias
+template <bool HAS_NB, bool WITH_MASK>
+__device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 *lds_vA, const uint4 *lds_kB, const uint4 *lds_vB,
+                                               const f32x4 *maskA4, const f32x4 *maskB4, const f32x4 *nbc, bf16x8 qA0, bf16x8 qA1,
+                                               bf16x8 qB0, bf16x8 qB1, int NB, int lane, f32x16 &oA_out,
+                                               float &lA_out, f32x16 &oB_out, float &lB_out, uint32_t turn)
+{
+    const int npairs = NB >> 1;
+    const uint4 *kA = lds_kA + lane, *vA = lds_vA + lane, *kB = lds_kB + lane, *vB = lds_vB + lane;
+    auto clampt = [&](int t) { return t < NB ? t : NB - 1; };
+    auto loadC = [&](int t) {
+        f32x16 c;
+        if constexpr (HAS_NB) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 v = nbc[(t * 4 + a) * 64];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    c[4 * a + e] = v[e];
+                }
+            }
+        } else {
+            c = zero16();
+        }
+        return c;
+    };
+    f32x16 C0 = loadC(0), C1 = loadC(1);
+    uint4 k0 = kA[0], k1 = kA[64], v0, v1;
+    f32x16 xa, xb;
+    xa = mfma(as_bf16x8(k0), qA0, C0);
+    xa = mfma(as_bf16x8(k1), qA1, xa);
+    k0 = kB[0], k1 = kB[64];
+    v0 = vA[0], v1 = vA[64];
+    f32x16 oA = zero16(), oB = zero16();
+    float lsumA = 0.f, lsumB = 0.f; // this lane's share of the row sums; the two halves of the wave are added at the end
+    bf16x2 one2;
+    one2[0] = (bf16_t)1.0f, one2[1] = (bf16_t)1.0f;
+    // Probabilities -> bf16 by truncation: one byte permute per pair of values where the rounding conversion is a slower
+    // instruction.  The row sums are taken over the same truncated values, so the bias (2^-9 on average) cancels in the
+    // normalisation and what is left is a rounding error of up to 2^-8 per probability instead of 2^-9.
+    auto pack_trunc = [&](const f32x16 &x, int base) {
+        uint4 u;
+        u.x = __builtin_amdgcn_perm(__float_as_uint(x[base + 1]), __float_as_uint(x[base + 0]), 0x07060302u);
+        u.y = __builtin_amdgcn_perm(__float_as_uint(x[base + 3]), __float_as_uint(x[base + 2]), 0x07060302u);
+        u.z = __builtin_amdgcn_perm(__float_as_uint(x[base + 5]), __float_as_uint(x[base + 4]), 0x07060302u);
+        u.w = __builtin_amdgcn_perm(__float_as_uint(x[base + 7]), __float_as_uint(x[base + 6]), 0x07060302u);
+        return as_bf16x8(u);
+    };
+    // row sums on the vector ALU, two probabilities per dot2: with two rows in flight the row-sum MFMAs of
+    // attend_block_l2 (a selector fragment and an accumulator per row) cost more registers than the loop has
+    auto rowsum = [&](float &lsum, bf16x8 pv) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            bf16x2 a;
+            a[0] = pv[2 * v], a[1] = pv[2 * v + 1];
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(a, one2, lsum, false);
+        }
+    };
+    // what is left to add to the logits of a finished tile before the exponential: the row's mask bias (the pair-bias
+    // seed is shared by the two rows, their masks are not).  Added to every tile, flagged or not: a branch per tile
+    // splits the loop into pieces that the register allocator handles worse than sixteen adds.
+    auto finish_logits = [&](f32x16 &x, const f32x4 *mask4, int t) {
+        if constexpr (WITH_MASK) {
+            __builtin_amdgcn_sched_barrier(0); // the four reads and sixteen adds stay together: spread out, their
+                                               // temporaries push the loop past its registers
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 mv = mask4[t * 8 + a];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    x[4 * a + c] += mv[c];
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+    auto exp4 = [&](f32x16 &x, int base) {
+#pragma unroll
+        for (int v = base; v < base + 4; ++v) {
+            x[v] = __builtin_amdgcn_exp2f(x[v]);
+        }
+    };
+    // softmax and P.V of the finished tile xc (into o, lacc); logits of the next tile into xn from seed C with query
+    // fragments q0, q1; then k0, k1 <- knext[0], knext[64].  No scheduling fences inside: with two independent rows in
+    // flight the compiler's own interleaving measured faster than a fixed one.  The empty asm keeps C live past the MFMA
+    // that reads it: the compiler then writes xn to registers of its own (D != C) instead of computing it in place in
+    // C's registers, which rotated the roles of the register blocks from one iteration to the next and cost 40 copies
+    // per iteration, behind a wait for every load in flight.
+    auto half_step = [&](f32x16 &xc, f32x16 &xn, const f32x16 &C, bf16x8 q0, bf16x8 q1, f32x16 &o, float &lsum, const uint4 *knext) {
+        bf16x8 p0, p1;
+        exp4(xc, 0);
+        exp4(xc, 4);
+        p0 = pack_trunc(xc, 0);
+        xn = mfma(as_bf16x8(k0), q0, C);
+        asm volatile("" ::"v"(C));
+        o = mfma(as_bf16x8(v0), p0, o);
+        exp4(xc, 8);
+        xn = mfma(as_bf16x8(k1), q1, xn);
+        rowsum(lsum, p0);
+        k0 = knext[0], k1 = knext[64];
+        exp4(xc, 12);
+        p1 = pack_trunc(xc, 8);
+        o = mfma(as_bf16x8(v1), p1, o);
+        rowsum(lsum, p1);
+    };
+    for (int pair = 0; pair < npairs; ++pair) {
+        timeslice_priority(turn, FAIR_SLICE_SHIFT);
+        const int t0 = 2 * pair, t1 = t0 + 1;
+        const int tn = pair + 1 < npairs ? t0 + 2 : t0; // next pair's first tile, clamped
+        // (A, t0) finished; logits of (B, t0) from C0
+        finish_logits(xa, maskA4, t0);
+        half_step(xa, xb, C0, qB0, qB1, oA, lsumA, kA + t1 * 128);
+        v0 = vB[t0 * 128], v1 = vB[t0 * 128 + 64];
+        fence(); // the loads stay behind the last reader of the registers they fill
+        C0 = loadC(clampt(t0 + 2));
+        fence();
+        // (B, t0) finished; logits of (A, t1) from C1
+        finish_logits(xb, maskB4, t0);
+        half_step(xb, xa, C1, qA0, qA1, oB, lsumB, kB + t1 * 128);
+        v0 = vA[t1 * 128], v1 = vA[t1 * 128 + 64];
+        // (A, t1) finished; logits of (B, t1) from C1
+        finish_logits(xa, maskA4, t1);
+        half_step(xa, xb, C1, qB0, qB1, oA, lsumA, kA + tn * 128);
+        v0 = vB[t1 * 128], v1 = vB[t1 * 128 + 64];
+        fence();
+        C1 = loadC(clampt(t1 + 2));
+        fence();
+        // (B, t1) finished; logits of (A, tn) from C0
+        finish_logits(xb, maskB4, t1);
+        half_step(xb, xa, C0, qA0, qA1, oB, lsumB, kB + tn * 128);
+        v0 = vA[tn * 128], v1 = vA[tn * 128 + 64];
+    }
+    __builtin_amdgcn_s_setprio(0);
+    oA_out = oA, oB_out = oB;
+    lA_out = half_swap_sum(lsumA), lB_out = half_swap_sum(lsumB);
+}
+
+// The repeat of one row's block after an overflow or underflow of the unshifted exponentials, with the pair bias as fp32
+// tiles: a first pass over the key tiles for the true row maxima, a second one with them subtracted.  Not a hot path:
+// one row, nothing prefetched, few registers.
+template <bool HAS_NB>
+__device__ __forceinline__ void attend_row_shifted(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4, const f32x4 *nbc, bf16x8 q0,
+                                                bf16x8 q1, int NB, int lane, f32x16 &o_out, float &l_out)
+{
+    auto logits = [&](int t) {
+        f32x16 x;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            f32x4 mv = mask4[t * 8 + a];
+            if constexpr (HAS_NB) {
+                const f32x4 cv = nbc[(t * 4 + a) * 64];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    mv[c] += cv[c];
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                x[4 * a + c] = mv[c];
+            }
+        }
+        x = mfma(as_bf16x8(lds_k[(t * 2 + 0) * 64 + lane]), q0, x);
+        return mfma(as_bf16x8(lds_k[(t * 2 + 1) * 64 + lane]), q1, x);
+    };
+    float mx = -INFINITY;
+    for (int t = 0; t < NB; ++t) {
+        const f32x16 x = logits(t);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            mx = fmaxf(mx, x[v]);
+        }
+    }
+    mx = half_swap_max(mx); // finite: a fully masked row has -1e9*log2(e) everywhere
+    f32x16 o = zero16();
+    float lsum = 0.f;
+    bf16x2 one2;
+    one2[0] = (bf16_t)1.0f, one2[1] = (bf16_t)1.0f;
+    for (int t = 0; t < NB; ++t) {
+        f32x16 x = logits(t);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            x[v] = __builtin_amdgcn_exp2f(x[v] - mx);
+        }
+        const bf16x8 p0 = pack8(x, 0), p1 = pack8(x, 8);
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 0) * 64 + lane]), p0, o);
+        o = mfma(as_bf16x8(lds_v[(t * 2 + 1) * 64 + lane]), p1, o);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            bf16x2 a, c;
+            a[0] = p0[2 * v], a[1] = p0[2 * v + 1];
+            c[0] = p1[2 * v], c[1] = p1[2 * v + 1];
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(a, one2, lsum, false);
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(c, one2, lsum, false);
+        }
+    }
+    o_out = o;
+    l_out = half_swap_sum(lsum);
+}
+
+template <bool HAS_NB>
+__global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedParams p)
+{
+    constexpr int C = 128, CK = C / 16;
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int S = p.S, NB = p.NB, NT = p.NT;
+    const int nthreads = NB * 64;
+
+    // workgroup -> (XCD, head, batch-row group) as in persistent_head_kernel
+    const int w = blockIdx.x;
+    const int xcd = w & 7;
+    const int slot = w >> 3;
+    const int h = slot % p.H;
+    const int grp = slot / p.H;
+    const int b0 = xcd + 8 * grp;
+    const int bstep = 8 * p.ngrp;
+    const int nrows = b0 < p.B ? (p.B - b0 + bstep - 1) / bstep : 0;
+
+    uint4 *lds_w = lds;
+    uint4 *lds_k = lds_w + 4 * CK * 64;     // [row of the pair][NT][2][64]
+    uint4 *lds_v = lds_k + 2 * NT * 2 * 64; // likewise
+    uint4 *panel = lds_v + 2 * NT * 2 * 64 + wave * 128;
+    float *mask_base = reinterpret_cast<float *>(lds_v + 2 * NT * 2 * 64 + NB * 128); // [pair parity][row of the pair][NT*32]
+    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 4 * NT * 32);     // [pair parity][row of the pair]
+
+    stage_weight_fragments<C>(lds_w, p, 0, 4, h, wave, nthreads >> 6, lane);
+    if (tid < 4) {
+        flag_words[tid] = 0;
+    }
+    if (NT > NB) { // phantom key tile of both rows: zero K and V fragments, never written again
+        const uint4 z4 = {0u, 0u, 0u, 0u};
+        for (int idx = tid; idx < 256; idx += nthreads) {
+            const int row = idx >> 7, i = idx & 127;
+            lds_k[(row * NT + NB) * 128 + i] = z4;
+            lds_v[(row * NT + NB) * 128 + i] = z4;
+        }
+    }
+    __syncthreads();
+
+    const int j = wave; // this wave's sequence block
+    const float qmul = p.qscale * LOG2E;
+    const uint32_t x_pitch = (uint32_t)p.x_ld; // the host sends only near-addressable rows here
+    for (int n = 0; n < nrows; n += 2) {
+        const int par = (n >> 1) & 1;
+        const bool have_b = n + 1 < nrows; // an odd row count: the last pair attends its one row twice and stores it once
+        const int bA = b0 + n * bstep, bB = have_b ? bA + bstep : bA;
+        uint32_t *flag_word = flag_words + 2 * par;
+        float *mask = mask_base + par * 2 * NT * 32;
+        // opaque lane index: addresses derived from it are formed anew per pair instead of living across the attention loop
+        int lane_x = lane;
+        asm volatile("" : "+v"(lane_x));
+        stage_mask_part<true>(p.bias + (int64_t)bA * p.bias_sb, mask, flag_word, S, NT, wave, lane_x, LOG2E, p.bias_sk,
+                              p.bias_is_mask != 0);
+        stage_mask_part<true>(p.bias + (int64_t)bB * p.bias_sb, mask + NT * 32, flag_word + 1, S, NT, wave, lane_x, LOG2E, p.bias_sk,
+                              p.bias_is_mask != 0);
+
+        // ---- input rows of the block, both batch rows -> fragments, 32 channels per staging panel ----
+        const int prow_x = pi_row(lane_x & 31), g_x = lane_x >> 5;
+        const bf16_t *xA = p.x + (int64_t)bA * p.x_sb, *xB = p.x + (int64_t)bB * p.x_sb;
+        bf16x8 xfA[CK], xfB[CK];
+        {
+            Panel32Regs ta[4], tb[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                ta[c] = panel32_load_near(xA, x_pitch, j * 32, S - 1, 32 * c, lane_x);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                tb[c] = panel32_load_near(xB, x_pitch, j * 32, S - 1, 32 * c, lane_x);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                panel32_store(panel, lane_x, ta[c]);
+                xfA[2 * c] = as_bf16x8(panel[panel32_slot(prow_x, g_x)]);
+                xfA[2 * c + 1] = as_bf16x8(panel[panel32_slot(prow_x, 2 + g_x)]);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                panel32_store(panel, lane_x, tb[c]);
+                xfB[2 * c] = as_bf16x8(panel[panel32_slot(prow_x, g_x)]);
+                xfB[2 * c + 1] = as_bf16x8(panel[panel32_slot(prow_x, 2 + g_x)]);
+            }
+        }
+        // ---- four projections of the block, both rows per weight fragment ----
+        // Gate first, then Q, K, V, each packed to bf16 as soon as it is complete;
+        // the scheduling barriers keep the compiler from running the four loops into one another, which needs four
+        // pairs of accumulators at once and spilled the input fragments.
+        bf16x8 qA0, qA1, qB0, qB1;
+        bf16x8 gateB0, gateB1;                                  // sigmoid(gate) of the second row, until the epilogue
+        bf16x8 kfA0, kfA1, vfA0, vfA1, kfB0, kfB1, vfB0, vfB1; // parked until the LDS arrays are free
+        {
+            const uint4 *wsrc = lds_w + lane_x;
+            auto project = [&](int proj, f32x16 &accA, f32x16 &accB, bool weights_left) {
+#pragma unroll
+                for (int ks = 0; ks < CK; ++ks) {
+                    const bf16x8 wf = as_bf16x8(wsrc[(proj * CK + ks) * 64]);
+                    if (weights_left) {
+                        accA = mfma(wf, xfA[ks], accA);
+                        accB = mfma(wf, xfB[ks], accB);
+                    } else {
+                        accA = mfma(xfA[ks], wf, accA);
+                        accB = mfma(xfB[ks], wf, accB);
+                    }
+                }
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                // the gate's accumulator starts at its bias (register v of a lane holds feature 8 (v / 4) + 4 g + v % 4)
+                f32x16 accA, accB;
+                const float *bgp = p.bg + h * HEAD + 4 * g_x;
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4 bv = *reinterpret_cast<const f32x4 *>(bgp + 8 * a);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        accA[4 * a + c] = bv[c], accB[4 * a + c] = bv[c];
+                    }
+                }
+                project(PROJ_G, accA, accB, true);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    accA[v] = sigmoid_fast(accA[v]), accB[v] = sigmoid_fast(accB[v]);
+                }
+                // the first row's into the wave's panel (its input rows are all staged), the second row's stay in registers
+                panel[lane_x] = as_uint4(pack8(accA, 0));
+                panel[64 + lane_x] = as_uint4(pack8(accA, 8));
+                gateB0 = pack8(accB, 0), gateB1 = pack8(accB, 8);
+                asm volatile("" : "+v"(gateB0), "+v"(gateB1));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                f32x16 accA = zero16(), accB = zero16();
+                project(PROJ_Q, accA, accB, true);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    accA[v] *= qmul, accB[v] *= qmul;
+                }
+                qA0 = pack8(accA, 0), qA1 = pack8(accA, 8);
+                qB0 = pack8(accB, 0), qB1 = pack8(accB, 8);
+                asm volatile("" : "+v"(qA0), "+v"(qA1), "+v"(qB0), "+v"(qB1)); // packed here, not after the barrier
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                f32x16 accA = zero16(), accB = zero16();
+                project(PROJ_K, accA, accB, true);
+                kfA0 = pack8(accA, 0), kfA1 = pack8(accA, 8);
+                kfB0 = pack8(accB, 0), kfB1 = pack8(accB, 8);
+                asm volatile("" : "+v"(kfA0), "+v"(kfA1), "+v"(kfB0), "+v"(kfB1));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                f32x16 accA = zero16(), accB = zero16();
+                project(PROJ_V, accA, accB, false);
+                vfA0 = pack8(accA, 0), vfA1 = pack8(accA, 8);
+                vfB0 = pack8(accB, 0), vfB1 = pack8(accB, 8);
+                asm volatile("" : "+v"(vfA0), "+v"(vfA1), "+v"(vfB0), "+v"(vfB1));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads(); // every wave is done with the previous pair's attention: the K and V arrays are free
+        {
+            uint4 *ka = lds_k + (j * 2) * 64 + lane, *va = lds_v + (j * 2) * 64 + lane;
+            ka[0] = as_uint4(kfA0), ka[64] = as_uint4(kfA1), va[0] = as_uint4(vfA0), va[64] = as_uint4(vfA1);
+            ka[NT * 128] = as_uint4(kfB0), ka[NT * 128 + 64] = as_uint4(kfB1);
+            va[NT * 128] = as_uint4(vfB0), va[NT * 128 + 64] = as_uint4(vfB1);
+        }
+        if (tid < 2) {
+            flag_words[2 * (par ^ 1) + tid] = 0; // its readers (previous pair) are done, its writers (next pair) start after the next barrier
+        }
+        __syncthreads(); // K, V and the masks of this pair are complete
+
+        // opaque once more: the loops' LDS and pair-bias addresses are formed here, per pair,
+        // rather than hoisted out of the pair loop and spilled
+        int lane_a = lane;
+        asm volatile("" : "+v"(lane_a));
+        const int g = lane_a >> 5;
+        const f32x4 *maskA4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
+        const f32x4 *maskB4 = reinterpret_cast<const f32x4 *>(mask + NT * 32 + 16 * g);
+        const uint32_t flagsA = flag_word[0], flagsB = flag_word[1];
+        const f32x4 *nbc = HAS_NB ? reinterpret_cast<const f32x4 *>(p.nbf) + ((int64_t)(h * NB + j) * NT * 4) * 64 + lane_a : nullptr;
+        const uint4 *kA = lds_k, *vA = lds_v, *kB = lds_k + NT * 128, *vB = lds_v + NT * 128;
+        f32x16 oA, oB;
+        float lA, lB;
+        if ((flagsA | flagsB) == 0u) {
+            attend_pair_l2<HAS_NB, false>(kA, vA, kB, vB, maskA4, maskB4, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
+        } else {
+            attend_pair_l2<HAS_NB, true>(kA, vA, kB, vB, maskA4, maskB4, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
+        }
+        // some probability overflowed or a whole row underflowed: repeat that row shifted by its true row maxima
+        if (__any(!(lA > 1e-30f && lA < 1e30f))) {
+            attend_row_shifted<HAS_NB>(kA, vA, maskA4, nbc, qA0, qA1, NT, lane_a, oA, lA);
+        }
+        if (__any(!(lB > 1e-30f && lB < 1e30f))) {
+            attend_row_shifted<HAS_NB>(kB, vB, maskB4, nbc, qB0, qB1, NT, lane_a, oB, lB);
+        }
+        int lane_o = lane; // as above: the addresses of the epilogue are not worth a register during the attention loop
+        asm volatile("" : "+v"(lane_o));
+        const int qpos = j * 32 + pi_row(lane_o & 31);
+        if (qpos < S) {
+            const int64_t off = (int64_t)qpos * p.avg_ss + (int64_t)h * p.avg_sh + 4 * (lane_o >> 5);
+            const bf16x8 gateA0 = as_bf16x8(panel[lane_o]), gateA1 = as_bf16x8(panel[64 + lane_o]);
+            f32x16 gv;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                gv[v] = to_f32(gateA0[v]), gv[8 + v] = to_f32(gateA1[v]);
+            }
+            store_gated(p.avg + (int64_t)bA * p.avg_sb + off, oA, __builtin_amdgcn_rcpf(lA), gv);
+            if (have_b) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) {
+                    gv[v] = to_f32(gateB0[v]), gv[8 + v] = to_f32(gateB1[v]);
+                }
+                store_gated(p.avg + (int64_t)bB * p.avg_sb + off, oB, __builtin_amdgcn_rcpf(lB), gv);
+            }
         }
     }
 }
@@ -1956,6 +2506,7 @@ __global__ __launch_bounds__(64) void pair_bias_fragments_kernel(const bf16_t *_
 // Tuning hooks (kutacc_hip_set_tuning): a forced plan of the long-sequence kernel, the fragment-major pair bias switched
 // off, one line per call on stderr.  Plain atomics: set from a test or an experiment, read on every launch.
 std::atomic<int> g_forced_bpw{0}, g_forced_gw{0}, g_no_fragments{0}, g_debug{0};
+std::atomic<int> g_pair_mode{0}; // persistent_pair_kernel: 0 = where every workgroup has two batch rows or more, 1 = wherever it can run, 2 = never
 
 bool fragments_disabled() { return g_no_fragments.load(std::memory_order_relaxed) != 0; }
 
@@ -1975,6 +2526,17 @@ int num_cus()
 {
     static int table[KUTACC_DEVICE_SLOTS] = {};
     return kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, table);
+}
+
+// batch-row groups per XCD of the persistent kernels: one workgroup per CU at most; groups of 8*H workgroups share
+// batch-row sequences across the XCDs
+int persistent_groups(int B, int H)
+{
+    const int per_ring = 8 * H;
+    int ngrp = num_cus() / per_ring;
+    const int need = (B + 7) / 8;
+    ngrp = ngrp < 1 ? 1 : ngrp;
+    return ngrp > need ? need : ngrp;
 }
 
 size_t head_kernel_lds(int C, int NB, int GW, int NW, int BPW)
@@ -1997,6 +2559,14 @@ size_t persistent_kernel_lds(int C, int NB)
     const int NT = (NB + 1) & ~1; // key tiles, padded to a pair
     return (size_t)4 * (C / 16) * 64 * 16 + (size_t)NT * 2 * 64 * 16 * 2 + (size_t)NB * (4096 + 2048) +
            (size_t)2 * NT * 32 * 4 + 16;
+}
+
+size_t pair_kernel_lds(int NB)
+{
+    // persistent_pair_kernel (128 channels): the head's four weight matrices, K and V of two batch rows, per wave one
+    // 2 KB panel, two pairs' masks of two rows each, flags
+    const int NT = (NB + 1) & ~1;
+    return (size_t)4 * 8 * 64 * 16 + (size_t)2 * NT * 2 * 64 * 16 * 2 + (size_t)NB * 2048 + (size_t)4 * NT * 32 * 4 + 16;
 }
 
 bool make_plan(int64_t S, int C, Plan &pl)
@@ -2060,12 +2630,13 @@ int64_t fragment_bytes(int64_t nheads, int NB) { return nheads * NB * ((NB + 1) 
 
 // Where the fast attention loop keeps its fragment-major copy of the pair bias, or nullptr when the call gets none: the
 // workspace the options bring, else the caller's q scratch tensor when that is dense, aligned and large enough.
-void *fragment_home(const kutacc_hip_attention_args_t &a, int NB, const kutacc_launch::FusedAttentionOptions &opt)
+// `scale`: 1 for the fp16 fragments, 2 for the fp32 tiles of persistent_pair_kernel
+void *fragment_home(const kutacc_hip_attention_args_t &a, int NB, const kutacc_launch::FusedAttentionOptions &opt, int scale = 1)
 {
     if (a.nonbatched_bias == nullptr || fragments_disabled()) {
         return nullptr;
     }
-    const int64_t nbf_bytes = fragment_bytes(a.nheads, NB);
+    const int64_t nbf_bytes = fragment_bytes(a.nheads, NB) * scale;
     if (opt.fragment_workspace != nullptr) {
         return (aligned(opt.fragment_workspace, 16) && (uint64_t)nbf_bytes <= opt.fragment_workspace_bytes)
                    ? opt.fragment_workspace
@@ -2104,14 +2675,22 @@ int launch_persistent_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
     if (const int rc = opt_in_lds(kern, pl.lds_bytes, configured)) {
         return rc;
     }
-    // one workgroup per CU at most; groups of 8*H workgroups share batch-row sequences across the XCDs
-    const int per_ring = 8 * p.H;
-    int ngrp = num_cus() / per_ring;
-    const int need = (p.B + 7) / 8;
-    ngrp = ngrp < 1 ? 1 : ngrp;
-    ngrp = ngrp > need ? need : ngrp;
-    p.ngrp = ngrp;
-    kern<<<dim3((unsigned)(per_ring * ngrp)), dim3((unsigned)(pl.NW * 64)), pl.lds_bytes, stream>>>(p);
+    p.ngrp = persistent_groups(p.B, p.H);
+    kern<<<dim3((unsigned)(8 * p.H * p.ngrp)), dim3((unsigned)(pl.NW * 64)), pl.lds_bytes, stream>>>(p);
+    return kutacc_hip_status(hipGetLastError());
+}
+
+template <bool HAS_NB>
+int launch_pair_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
+{
+    auto kern = persistent_pair_kernel<HAS_NB>;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    const size_t lds_bytes = pair_kernel_lds(pl.NB);
+    if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
+        return rc;
+    }
+    p.ngrp = persistent_groups(p.B, p.H);
+    kern<<<dim3((unsigned)(8 * p.H * p.ngrp)), dim3((unsigned)(pl.NW * 64)), lds_bytes, stream>>>(p);
     return kutacc_hip_status(hipGetLastError());
 }
 
@@ -2294,10 +2873,30 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     if (opt.fragment_workspace != nullptr && p.nb != nullptr && fragments == nullptr && !fragments_disabled()) {
         return KUTACC_HIP_EINVAL; // the caller's workspace cannot hold the copy
     }
+    // Two batch rows per step (persistent_pair_kernel): 128 channels, log2 units, a home for the fp32 tiles of the pair
+    // bias (twice the fragments' bytes), no LayerNorm inside the kernel and no ready-made fp16 fragments; by default
+    // only where every workgroup walks at least two rows.
+    const int pair_mode = g_pair_mode.load(std::memory_order_relaxed);
+    void *const tiles = fragment_home(a, pl.NB, opt, 2);
+    const bool pair_kernel = pl.persistent && C == 128 && pair_mode != 2 && !fragments_disabled() && opt.ln_gamma == nullptr &&
+                             !opt.nb_fragments_ready && pair_kernel_lds(pl.NB) <= (size_t)max_lds_bytes() &&
+                             (p.nb == nullptr || tiles != nullptr) &&
+                             (pair_mode == 1 || a.batch >= 16 * (int64_t)persistent_groups(p.B, p.H));
 
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
-    if (fragments != nullptr && opt.nb_fragments_ready) {
+    if (pair_kernel) {
+        if (p.nb != nullptr) {
+            kutacc_prof::KernelTimer t("pair_bias_tiles_kernel", 0.0, stream);
+            pair_bias_tiles_kernel<<<dim3((unsigned)(pl.NB * p.NT), (unsigned)a.nheads), 64, 0, stream>>>(
+                p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.NT, p.nb_vec, (f32x4 *)tiles);
+            rc = kutacc_hip_status(hipGetLastError());
+            if (rc != 0) {
+                return rc;
+            }
+            p.nbf = (const uint4 *)tiles;
+        }
+    } else if (fragments != nullptr && opt.nb_fragments_ready) {
         p.nbf = (const uint4 *)fragments; // the producer of the pair bias wrote the copy
     } else if (fragments != nullptr) {
         kutacc_prof::KernelTimer t("pair_bias_fragments_kernel", 0.0, stream);
@@ -2319,14 +2918,16 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     if (g_debug.load(std::memory_order_relaxed)) {
         fprintf(stderr,
                 "[kutacc] fused plan: persistent=%d C=%d NB=%d NT=%d NW=%d BPW=%d GW=%d lds=%zu max_lds=%d cus=%d log2_units=%d "
-                "fragments=%d\n",
+                "fragments=%d row_pairs=%d\n",
                 (int)pl.persistent, C, pl.NB, p.NT, pl.NW, pl.BPW, pl.GW, pl.lds_bytes, max_lds_bytes(), num_cus(), p.l2mode,
-                p.nbf != nullptr ? 1 : 0);
+                p.nbf != nullptr ? 1 : 0, (int)pair_kernel);
     }
     {
-        kutacc_prof::KernelTimer t(pl.persistent ? "persistent_head_kernel" : "fused_head_kernel",
+        kutacc_prof::KernelTimer t(pair_kernel ? "persistent_pair_kernel" : pl.persistent ? "persistent_head_kernel" : "fused_head_kernel",
                                    8.0 * BS * C * C + 4.0 * BS * (double)a.seq_len * C, stream);
-        rc = (C == 128) ? dispatch_head_kernel<128>(p, pl, stream) : dispatch_head_kernel<256>(p, pl, stream);
+        rc = pair_kernel ? (p.nb != nullptr ? launch_pair_kernel<true>(p, pl, stream) : launch_pair_kernel<false>(p, pl, stream))
+             : (C == 128) ? dispatch_head_kernel<128>(p, pl, stream)
+                          : dispatch_head_kernel<256>(p, pl, stream);
         if (rc != 0) {
             return rc;
         }
@@ -2522,6 +3123,10 @@ int kutacc_launch::fused_attention_tuning(const char *name, const char *value)
         } else {
             g_forced_bpw.store(0), g_forced_gw.store(0);
         }
+        return 0;
+    }
+    if (!strcmp(name, "row_pairs")) { // "1": wherever the two-row kernel can run, "0": never, anything else: the default rule
+        g_pair_mode.store(value && value[0] == '1' ? 1 : (value && value[0] == '0' ? 2 : 0));
         return 0;
     }
     if (!strcmp(name, "fragments")) {

@@ -189,6 +189,76 @@ def test_seeded_shape_sweep_matches_oracle(torch_cuda, index, config, batch, seq
     helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, f"sweep {index} out")
 
 
+# ---- the two-row persistent kernel (128 channels, up to 384 keys), forced wherever it can run --------------------------
+@pytest.fixture
+def row_pairs_forced():
+    assert capi.set_tuning("row_pairs", "1") == 0
+    yield
+    capi.set_tuning("row_pairs", None)
+
+
+PAIR_CASES = [
+    # config, batch, seq_len, mask kind: None as drawn, "holes", "tails" (+ one fully masked row), "none"
+    (3, 16, 384, None), (3, 17, 384, "holes"), (3, 9, 200, None), (3, 24, 321, "tails"), (3, 3, 33, "holes"),
+    (3, 1, 64, None), (3, 40, 96, "tails"), (5, 18, 352, None), (5, 7, 70, "holes"), (3, 1, 1, None), (3, 26, 383, "none"),
+]
+
+
+@pytest.mark.parametrize("config,batch,seq,mask", PAIR_CASES)
+@pytest.mark.parametrize("pair_bias", [True, False], ids=["pair bias", "no pair bias"])
+def test_two_row_kernel_matches_the_oracle(torch_cuda, row_pairs_forced, config, batch, seq, mask, pair_bias):
+    """Batches that leave workgroups with one, an odd and an even number of rows (a workgroup walks rows 8 * groups
+    apart), ragged and odd tile counts, every mask kind, with and without pair bias; each row against the oracle."""
+    w = make_workload(config, batch=batch, seq_len=seq)
+    rng = np.random.Generator(np.random.PCG64(900 + batch + seq))
+    if mask == "holes":
+        w.bias[:] = round_to_bf16(np.where(rng.random((batch, seq)) < 0.2, -1e9, 0.0).astype(np.float32))
+    elif mask == "tails":
+        for b in range(batch):
+            w.bias[b, seq - int(rng.integers(0, seq)):] = -1e9
+        w.bias[batch - 1, :] = -1e9
+    elif mask == "none":
+        w.bias[:] = 0.0
+    if not pair_bias:
+        w.nb = None
+    ten, scratch = helpers.to_device(w)
+    capi.set_tuning("debug", "1")
+    try:
+        rc = helpers.run_hip(w, ten, scratch, capi.PATH_FUSED)
+    finally:
+        capi.set_tuning("debug", "0")
+    assert rc == 0, rc
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, "gated average")
+    helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
+
+
+def test_two_row_kernel_is_what_the_headline_shape_runs(torch_cuda, capfd):
+    """Configuration 3 at a batch that gives every workgroup two rows takes the two-row kernel by itself, and a large
+    pair-bias offset (overflow / underflow repeat with shifted rows) leaves its result where the oracle has it."""
+    w = make_workload(3, batch=128)
+    ten, scratch = helpers.to_device(w)
+    capi.set_tuning("debug", "1")
+    try:
+        assert helpers.run_hip(w, ten, scratch, capi.PATH_FUSED) == 0
+    finally:
+        capi.set_tuning("debug", "0")
+    assert "row_pairs=1" in capfd.readouterr().err
+    rows = [0, 1, 63, 64, 127]
+    ref_out, _ = oracle_rows(w, rows)
+    helpers.check_close(helpers.to_numpy(ten["out"][rows]), ref_out, w.dtype, "two-row kernel, config 3")
+    # a constant pair bias of +-150 (exact in bf16; far outside what 2^logit holds unshifted): equals no pair bias at all
+    w0 = make_workload(3, batch=128)
+    w0.nb = np.zeros_like(w0.nb)
+    ref0, _ = oracle_rows(w0, rows)
+    for offset in (150.0, -150.0):
+        w2 = make_workload(3, batch=128)
+        w2.nb = np.full_like(w2.nb, offset)
+        ten2, scratch2 = helpers.to_device(w2)
+        assert helpers.run_hip(w2, ten2, scratch2, capi.PATH_FUSED) == 0
+        helpers.check_close(helpers.to_numpy(ten2["out"][rows]), ref0, w.dtype, f"two-row kernel, constant pair bias {offset:+}")
+
+
 def test_fp32_storage_meets_fp32_tolerance(torch_cuda):
     w = make_workload(1)
     op, ten, scratch = helpers.make_op(w)
