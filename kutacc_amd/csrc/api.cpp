@@ -200,11 +200,17 @@ int kutacc_hip_gating_attention(const kutacc_hip_attention_args_t *a, void *stre
     }
     hipStream_t s = pick_stream(stream);
     const bool fused_ok = kutacc_launch::fused_attention_supports(*a);
-    if (a->path == KUTACC_HIP_PATH_FUSED && !fused_ok) {
+    const bool fp32_ok = !fused_ok && kutacc_launch::fp32_attention_supports(*a);
+    if (a->path == KUTACC_HIP_PATH_FUSED && !fused_ok && !fp32_ok) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
     int rc;
-    if (fused_ok && a->path != KUTACC_HIP_PATH_GENERIC) {
+    if (fp32_ok && a->path != KUTACC_HIP_PATH_GENERIC) {
+        rc = kutacc_launch::gating_attention_fp32(*a, s);
+        if (rc == 0) {
+            t_last_path = "fp32_mfma";
+        }
+    } else if (fused_ok && a->path != KUTACC_HIP_PATH_GENERIC) {
         rc = kutacc_launch::gating_attention_fused(*a, s);
         if (rc == 0) {
             t_last_path = "fused_mfma";

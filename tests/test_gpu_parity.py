@@ -114,8 +114,6 @@ SMALL = [
 @pytest.mark.parametrize("config,batch,seq", SMALL)
 @pytest.mark.parametrize("path", [capi.PATH_GENERIC, capi.PATH_FUSED])
 def test_reduced_shapes_both_kernel_families(torch_cuda, config, batch, seq, path):
-    if path == capi.PATH_FUSED and CONFIGS[config]["dtype"] != "bf16":
-        pytest.skip("the MFMA kernels take bf16 storage only; fp32 runs on the generic kernels")
     w = make_workload(config, batch=batch, seq_len=seq)
     if config == 5:
         w.bias[-1, :] = round_to_bf16(np.full(seq, -1e9, dtype=np.float32))  # a fully masked row
@@ -123,9 +121,38 @@ def test_reduced_shapes_both_kernel_families(torch_cuda, config, batch, seq, pat
     ten, scratch = helpers.to_device(w)
     rc = helpers.run_hip(w, ten, scratch, path)
     assert rc == 0, rc
+    if path == capi.PATH_FUSED:
+        assert capi.last_path() == ("fused_mfma" if w.dtype == "bf16" else "fp32_mfma")
     ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
     helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, w.dtype, "gated average")
     helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, w.dtype, "out")
+
+
+@pytest.mark.parametrize("config,batch,seq", [c for c in SMALL if c[2] <= 224] + [(2, 5, 224), (3, 4, 129), (4, 3, 160)])
+def test_fp32_storage_on_the_fp32_matrix_core(torch_cuda, config, batch, seq):
+    """Every reduced shape of up to 224 positions with its tensors stored as fp32 (the values are those of the bf16
+    workload, which fp32 holds exactly): the fp32 MFMA path, held to the fp32 bar -- 1e-4 relative (+ 1e-5) of the fp32
+    oracle -- with masks, ragged lengths, fully masked rows, with and without pair bias, 128 and 256 channels."""
+    w = make_workload(config, batch=batch, seq_len=seq)
+    w.dtype = "fp32"
+    if config == 5:
+        w.bias[-1, :] = -1e9  # a fully masked row
+    ten, scratch = helpers.to_device(w)
+    rc = helpers.run_hip(w, ten, scratch, capi.PATH_FUSED)
+    assert rc == 0 and capi.last_path() == "fp32_mfma", (rc, capi.last_path())
+    ref_out, ref_avg = helpers.oracle_out(w, return_avg=True)
+    helpers.check_close(helpers.to_numpy(scratch["avg"]).reshape(w.B, w.S, w.C), ref_avg, "fp32", "gated average")
+    helpers.check_close(helpers.to_numpy(ten["out"]), ref_out, "fp32", "out")
+    for name in ("q", "k", "v", "gate"):
+        assert not bool(scratch[name].any()), f"{name} was written"
+
+
+def test_fp32_storage_beyond_the_matrix_core_path_takes_the_generic_kernels(torch_cuda):
+    w = make_workload(1, batch=2, seq_len=225)
+    ten, scratch = helpers.to_device(w)
+    assert helpers.run_hip(w, ten, scratch, capi.PATH_FUSED) == capi.EUNSUPPORTED
+    assert helpers.run_hip(w, ten, scratch, capi.PATH_AUTO) == 0 and capi.last_path() == "generic"
+    helpers.check_close(helpers.to_numpy(ten["out"]), helpers.oracle_out(w), "fp32", "out")
 
 
 @pytest.mark.parametrize("config,batch,seq,plan", [
@@ -263,7 +290,7 @@ def test_fp32_storage_meets_fp32_tolerance(torch_cuda):
     w = make_workload(1)
     op, ten, scratch = helpers.make_op(w)
     op.run()
-    assert not capi.error_flag() and capi.last_path() == "generic"
+    assert not capi.error_flag() and capi.last_path() == "fp32_mfma"  # the fp32 matrix core, not the scalar kernels
     ref = helpers.oracle_out(w)
     got = helpers.to_numpy(ten["out"])
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
