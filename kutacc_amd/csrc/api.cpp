@@ -145,6 +145,7 @@ int64_t kutacc_hip_release_staging(void) { return (int64_t)g_staging.release(); 
 // the hooks of the attention launcher live with it; "pointer_checks" belongs to the entry points here
 namespace kutacc_launch {
 int fused_attention_tuning(const char *name, const char *value);
+int pair_gemm_tuning(const char *name, const char *value);
 }
 int kutacc_hip_set_tuning(const char *name, const char *value)
 {
@@ -161,6 +162,9 @@ int kutacc_hip_set_tuning(const char *name, const char *value)
     }
     if (!std::strcmp(name, "layernorm")) {
         g_block_layernorm.store(value && !std::strcmp(value, "fused") ? 1 : (value && !std::strcmp(value, "separate") ? 2 : 0));
+        return 0;
+    }
+    if (kutacc_launch::pair_gemm_tuning(name, value) == 0) {
         return 0;
     }
     return kutacc_launch::fused_attention_tuning(name, value);

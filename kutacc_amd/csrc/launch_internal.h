@@ -109,6 +109,8 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t 
 
 // "plan" / "fragments" / "debug" hooks of the attention launcher (kutacc_hip_set_tuning); KUTACC_HIP_EINVAL for other names
 int fused_attention_tuning(const char *name, const char *value);
+// "gemm_tile" hook of the matrix products of the pair stack; KUTACC_HIP_EINVAL for other names
+int pair_gemm_tuning(const char *name, const char *value);
 
 bool row_projection_supports(const void *a, int64_t a_ld, const void *w, const float *bias, const void *out, int64_t out_ld,
                              int64_t m, int64_t n, int64_t k);

@@ -24,6 +24,10 @@
 // 16-byte aligned) run on a scalar kernel with the same epilogues.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <cstring>
+#include <type_traits>
+
 #include "launch_internal.h"
 #include "mfma_tiles.h"
 #include "profiler.h"
@@ -326,6 +330,269 @@ __global__ __launch_bounds__(256, (A_MMAJOR && B_MMAJOR) ? 4 : 3) void pair_gemm
                     *reinterpret_cast<const uint4 *>(ct + row * CT_LD + chunk * 8);
             }
         }
+    }
+}
+
+// ---- square products with many tiles: 256 x 256 of C per workgroup, 128 x 128 per wave ----
+//
+// At 64 x 64 per wave the four MFMAs of a k-step need four operand fragments from the LDS, and with the stores that
+// stage the tiles the LDS moves 1.5 KB per MFMA: more than it can deliver at the matrix cores' rate.  Here a wave
+// multiplies 4 x 4 blocks (eight fragments for sixteen MFMAs) and a workgroup stages 512 rows of operands for 256
+// MFMAs, 0.75 KB per MFMA.  The 256 accumulator registers leave room for one wave per SIMD, so nothing but the
+// wave's own instruction order hides a latency: operands are requested two k-steps ahead, fragments one quarter step
+// ahead, and the order is pinned with scheduling barriers (one workgroup barrier per step).  An operand stage holds
+// four sub-tiles of 128 rows x 64 k (16 KB each: A rows 0-127, A rows 128-255, B likewise) in the layout the
+// 128 x 128 kernel uses for that orientation; wave w stages sub-tile w.  Both operands in the same orientation, no
+// epilogue but the rounding: the triangle-multiplication equation.
+constexpr int BIG_TILE = 256;
+constexpr int SUB_SLOTS = 1024;
+constexpr int BIG_STAGE_SLOTS = 4 * SUB_SLOTS;
+constexpr size_t BIG_GEMM_LDS = 2 * BIG_STAGE_SLOTS * 16;
+
+struct SubTileRegs {
+    PanelRegs q0, q1, q2, q3;
+};
+
+// The registers, or zeros, by a mask: a conditional assignment becomes a branch, and a branch inside the k-loop splits
+// the basic block whose instruction order the loop depends on.
+__device__ __forceinline__ PanelRegs keep_if(const PanelRegs &p, bool ok)
+{
+    const uint32_t keep = ok ? 0xffffffffu : 0u;
+    auto m = [&](uint4 v) { return make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep); };
+    return PanelRegs{m(p.r0), m(p.r1), m(p.r2), m(p.r3)};
+}
+
+struct TilePlace {
+    int batch, m0, n0;
+};
+
+// Persistent: one workgroup per CU walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... and its operand pipeline runs
+// on across the tile boundary -- the last two k-steps of a tile request the first two of the next, and the store of
+// the finished tile goes out under the next tile's MFMAs.  With one workgroup per CU nothing else would cover a
+// tile's first loads (about 8000 clocks of a 70000-clock tile at k = 1024) or the acknowledgement of its stores.
+template <bool MMAJOR>
+__global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams p, const int64_t total_tiles)
+{
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, g = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // Workgroup ids are dealt round robin over the 8 XCDs, and id + gridDim.x lands on the same XCD when the grid is a
+    // multiple of 8: each XCD gets a contiguous run of tiles, so that neighbours in the walk (which share an operand
+    // tile) share an L2.
+    const int64_t tiles_per_batch = (int64_t)p.MT * p.NT;
+    auto place = [&](int64_t index) -> TilePlace {
+        // (the launcher keeps the number of tiles within 32 bits: 64-bit divisions cost a few thousand clocks per tile)
+        uint32_t v = (uint32_t)(index < total_tiles ? index : total_tiles - 1); // past the last tile: a valid address, never used
+        const uint32_t per = (uint32_t)total_tiles / 8;
+        if (v < per * 8) {
+            v = (v % 8) * per + v / 8;
+        }
+        const int batch = (int)(v / (uint32_t)tiles_per_batch), t = (int)(v % (uint32_t)tiles_per_batch);
+        int mt, nt;
+        if (p.MT <= p.NT) {
+            mt = t % p.MT, nt = t / p.MT;
+        } else {
+            nt = t % p.NT, mt = t / p.NT;
+        }
+        return TilePlace{batch, mt * BIG_TILE, nt * BIG_TILE};
+    };
+
+    // The sub-tile this wave stages: rows row0.. of A (waves 0, 1) or of B (waves 2, 3).  M, N and K are whole tiles
+    // and steps here, so an address is a wave-uniform pointer (tile, k-step, row block: scalar arithmetic) plus one
+    // 32-bit byte offset per lane that never changes; the loads cost no vector instructions beyond themselves, which
+    // matters with one wave per SIMD, where every vector instruction between two MFMAs comes out of the matrix pipe's time.
+    const bool mine_a = wave < 2;
+    const int64_t ld = mine_a ? (MMAJOR ? p.a_sk : p.a_sm) : (MMAJOR ? p.b_sk : p.b_sn);
+    const uint32_t lane_bytes = (uint32_t)(((MMAJOR ? mm_row(lane >> 3) : (lane >> 3)) * ld + (lane & 7) * 8) * 2);
+    using Source = const char *; // first element of the sub-tile's rows at k = 0
+    auto source = [&](const TilePlace &tp) -> Source {
+        const bf16_t *base = mine_a ? p.a + (int64_t)tp.batch * p.a_sb : p.b + (int64_t)tp.batch * p.b_sb;
+        const int row0 = (mine_a ? tp.m0 : tp.n0) + 128 * (wave & 1);
+        return reinterpret_cast<const char *>(MMAJOR ? base + row0 : base + (int64_t)row0 * ld);
+    };
+    // quarter i of the wave's sub-tile of the k-step at k0; a step past K (an odd number of steps is rounded up) reads
+    // step 0 instead and is cleared on its way to the LDS
+    auto fetch_quarter = [&](Source src, int i, int k0) -> PanelRegs {
+        const int k0c = k0 < p.K ? k0 : 0;
+        // k-major: rows 32 i + 8 e + (lane >> 3), 64 k from k0c; m-major: 64 m from 64 (i & 1), k = k0c + 32 (i >> 1) + 8 e + ...
+        const char *q = MMAJOR ? src + ((int64_t)(k0c + 32 * (i >> 1)) * ld + 64 * (i & 1)) * 2 : src + ((int64_t)32 * i * ld + k0c) * 2;
+        PanelRegs f;
+        f.r0 = *reinterpret_cast<const uint4 *>(q + lane_bytes);
+        f.r1 = *reinterpret_cast<const uint4 *>(q + 16 * ld + lane_bytes);
+        f.r2 = *reinterpret_cast<const uint4 *>(q + 32 * ld + lane_bytes);
+        f.r3 = *reinterpret_cast<const uint4 *>(q + 48 * ld + lane_bytes);
+        return f;
+    };
+    auto fetch = [&](Source src, int k0) -> SubTileRegs {
+        return SubTileRegs{fetch_quarter(src, 0, k0), fetch_quarter(src, 1, k0), fetch_quarter(src, 2, k0), fetch_quarter(src, 3, k0)};
+    };
+    // what fetch(.., k0) brought, zeros for a step past K, into the wave's sub-tile of a stage
+    auto park = [&](uint4 *stage, const SubTileRegs &f, int k0) {
+        uint4 *sub = stage + wave * SUB_SLOTS;
+        const bool ok = k0 < p.K;
+        const PanelRegs q0 = keep_if(f.q0, ok), q1 = keep_if(f.q1, ok), q2 = keep_if(f.q2, ok), q3 = keep_if(f.q3, ok);
+        if constexpr (MMAJOR) {
+            store_mmajor(sub, 0, 0, lane, q0);
+            store_mmajor(sub, 64, 0, lane, q1);
+            store_mmajor(sub, 0, 32, lane, q2);
+            store_mmajor(sub, 64, 32, lane, q3);
+        } else {
+            panel_store(sub, lane, q0);
+            panel_store(sub + 256, lane, q1);
+            panel_store(sub + 512, lane, q2);
+            panel_store(sub + 768, lane, q3);
+        }
+    };
+
+    f32x16 acc[4][4];
+    int mm_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mm_off[i] = mm_fragment_offset(i, lane);
+    }
+
+    // Fragments of k-step s + 1 are requested while the MFMAs of step s issue (two register sets), the next stage's
+    // stores go behind the MFMAs of the last step, and the scheduler is told the interleaving: left to itself it
+    // puts every LDS read directly in front of the four MFMAs that need it, and with one wave per SIMD nothing else
+    // covers that latency.
+    bf16x8 af[2][4], bq[2][4];
+    auto fragments = [&](int set, const uint4 *stage, int s) {
+        const uint4 *sa = stage + wm * SUB_SLOTS;
+        const uint4 *sb = stage + (2 + wn) * SUB_SLOTS;
+        const int slot = panel_slot(r, 2 * s + g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (MMAJOR) {
+                af[set][i] = mm_fragment((const lds_char *)sa, mm_off[i], s);
+                bq[set][i] = mm_fragment((const lds_char *)sb, mm_off[i], s);
+            } else {
+                af[set][i] = as_bf16x8(sa[i * 256 + slot]);
+                bq[set][i] = as_bf16x8(sb[i * 256 + slot]);
+            }
+        }
+    };
+    // The fragments arrive in the order a0 b0 a1 b1 a2 b2 a3 b3, the last ones shortly before the quarter that uses
+    // them begins: the MFMAs go in the order in which their operands arrive, the four that need b3 last.
+    auto multiply = [&](int set) {
+        constexpr int order[16][2] = {{0, 0}, {1, 0}, {0, 1}, {1, 1}, {2, 0}, {2, 1}, {0, 2}, {1, 2},
+                                      {2, 2}, {3, 0}, {3, 1}, {3, 2}, {0, 3}, {1, 3}, {2, 3}, {3, 3}};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int i = order[e][0], j = order[e][1];
+            acc[i][j] = mfma(bq[set][j], af[set][i], acc[i][j]);
+        }
+    };
+    constexpr int READS = MMAJOR ? 16 : 8; // LDS read instructions per k-step of 16
+    // One k-step of 64 from `stage`.  Operands travel two steps ahead of the MFMAs: the step requests the tiles of the
+    // step after next (of `src`, at k_fetch) into `fill` and stores `ahead`, requested a step earlier for k_park, into
+    // the other stage.  The sixteen loads are spread over the MFMAs of the first three quarters: issued together they
+    // hold the wave, and with it the matrix pipe, for as long as the CU's memory path takes to accept 64 KB (1500 to
+    // 2400 clocks of a step of 2048 MFMA clocks, measured).
+    auto k_step = [&](const uint4 *stage, uint4 *other, Source src, int k_fetch, int k_park, const SubTileRegs &ahead,
+                      SubTileRegs &fill) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            if (s < 3) {
+                fragments((s + 1) & 1, stage, s + 1);
+            }
+            if (s == 0) {
+                fill.q0 = fetch_quarter(src, 0, k_fetch);
+                fill.q1 = fetch_quarter(src, 1, k_fetch);
+            } else if (s == 1) {
+                fill.q2 = fetch_quarter(src, 2, k_fetch);
+            } else if (s == 2) {
+                fill.q3 = fetch_quarter(src, 3, k_fetch);
+            }
+            multiply(s & 1);
+            if (s == 3) {
+                park(other, ahead, k_park); // every wave left that stage before the barrier that ended the previous step
+            }
+            if (s < 3) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, READS / 8, 0); // LDS reads
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);         // MFMA
+                    if (s == 0 || (e & 1)) {
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // a global load: eight, four and four per quarter
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // LDS write
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+        fragments(0, other, 0);
+    };
+
+    // Steps go in pairs with one body, so that the 256 accumulators and the two register sets keep their places; an odd
+    // number of steps ends with a step whose operands, past K, were cleared on their way to the LDS.
+    const int KT2 = ((p.K + KSTEP - 1) / KSTEP + 1) & ~1;
+    uint4 *stage0 = lds, *stage1 = lds + BIG_STAGE_SLOTS;
+    int64_t v = blockIdx.x;
+    TilePlace cur = place(v);
+    Source cur_src = source(cur);
+    SubTileRegs even, odd; // tiles of an even / odd k-step on their way to the LDS
+    even = fetch(cur_src, 0);
+    odd = fetch(cur_src, KSTEP);
+    park(stage0, even, 0);
+    __syncthreads();
+    fragments(0, stage0, 0);
+    for (; v < total_tiles; v += gridDim.x) {
+        const Source next_src = source(place(v + gridDim.x));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[i][j] = zero16();
+            }
+        }
+        for (int kt = 0; kt < KT2; kt += 2) {
+            const bool last = kt + 2 == KT2; // the requests go on to the next tile
+            const Source src = last ? next_src : cur_src;
+            k_step(stage0, stage1, src, last ? 0 : (kt + 2) * KSTEP, (kt + 1) * KSTEP, odd, even);
+            k_step(stage1, stage0, src, last ? KSTEP : (kt + 3) * KSTEP, last ? 0 : (kt + 2) * KSTEP, even, odd);
+        }
+
+        // Each wave rounds its 128 x 128 block to bf16 through a 32-row strip in its own sub-tile of the stage the last
+        // step read (the other one already holds the next tile's first step; a wave's LDS accesses complete in order, so
+        // the strip needs no barrier, and the wave itself is the next to store into that sub-tile) and writes whole
+        // 256-byte pieces of rows.
+        bf16_t *ct = reinterpret_cast<bf16_t *>(stage1 + wave * SUB_SLOTS);
+        bf16_t *c = p.c + (int64_t)cur.batch * p.c_sb;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    bf16x4 ov;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        ov[e] = (bf16_t)acc[i][j][4 * q + e];
+                    }
+                    *reinterpret_cast<bf16x4 *>(ct + r * CT_LD + 32 * j + 8 * q + 4 * g) = ov;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int piece = lane + 64 * e;
+                const int row = piece >> 4, chunk = piece & 15;
+                const int64_t gm = cur.m0 + 128 * wm + 32 * i + row, gn = cur.n0 + 128 * wn + chunk * 8;
+                *reinterpret_cast<uint4 *>(c + gm * p.c_sm + gn) = *reinterpret_cast<const uint4 *>(ct + row * CT_LD + chunk * 8);
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        cur = place(v + gridDim.x);
+        cur_src = next_src;
     }
 }
 
@@ -900,6 +1167,32 @@ hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
 }
 constexpr int64_t GATED_STREAMING_MIN_POSITIONS = 512 * 512;
 
+template <bool MM>
+hipError_t launch_big_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
+{
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&pair_gemm_big_kernel<MM>), BIG_GEMM_LDS, configured)) {
+        return e;
+    }
+    int device = 0, cus = 0;
+    if (hipError_t e = hipGetDevice(&device)) {
+        return e;
+    }
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device)) {
+        return e;
+    }
+    // one workgroup per CU; a multiple of 8, so that a workgroup's tiles stay on its XCD's share of the walk
+    const int64_t grid = blocks < cus ? blocks : (cus >= 8 ? cus / 8 * 8 : cus);
+    pair_gemm_big_kernel<MM><<<dim3((unsigned)grid), 256, BIG_GEMM_LDS, stream>>>(p, blocks);
+    return hipGetLastError();
+}
+
+// 0: the 256 x 256 tiles where every CU gets at least four of them (measured at 128 channels: 0.36 of the MFMA peak
+// against 0.31 at 1024 x 1024, 0.31 against 0.29 at 768 x 768, no gain at 512 x 512), 1: wherever the shape allows
+// them, 2: never
+std::atomic<int> g_big_tile_mode{0};
+constexpr int64_t BIG_TILE_MIN_WORKGROUPS = 1024;
+
 // the dedicated kernel of the gated projection: 128 -> 128 channels, dense operands, positions in whole 16-byte runs
 bool gated_projection_fits(const kutacc_hip_gemm_args_t &g)
 {
@@ -1008,6 +1301,15 @@ int transition_block_fused(void *act, const float *ln_gamma, const float *ln_bet
     return kutacc_hip_status(e);
 }
 
+int pair_gemm_tuning(const char *name, const char *value)
+{
+    if (!std::strcmp(name, "gemm_tile")) { // "256": wherever the shape allows the large tiles, "128": never, anything else: the default rule
+        g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : 0));
+        return 0;
+    }
+    return KUTACC_HIP_EINVAL;
+}
+
 int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_hip_gemm_args_t *second)
 {
     if (g.m <= 0 || g.n <= 0 || g.k <= 0 || g.batches <= 0 || !g.a || !g.b || !g.c || g.dtype != KUTACC_DTYPE_BF16) {
@@ -1097,6 +1399,16 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
         kutacc_prof::KernelTimer t("pair_gemm_scalar_kernel", flops, stream);
         pair_gemm_scalar_kernel<<<dim3((unsigned)blocks), 256, 0, stream>>>(p);
         return kutacc_hip_status(hipGetLastError());
+    }
+    // (whole tiles and k-steps, and lane offsets within 32 bits: the kernel's addresses are a uniform pointer plus a lane constant)
+    if (!gated && am == bm && g.bias_axis == 0 && !g.relu && g.m % BIG_TILE == 0 && g.n % BIG_TILE == 0 && g.k % KSTEP == 0 &&
+        (am ? g.a_stride_k : g.a_stride_m) < (1 << 26) && (bm ? g.b_stride_k : g.b_stride_n) < (1 << 26) && g_big_tile_mode.load() != 2) {
+        p.MT = (int)(g.m / BIG_TILE), p.NT = (int)(g.n / BIG_TILE);
+        const int64_t big_blocks = (int64_t)p.MT * p.NT * p.batches;
+        if (big_blocks <= INT32_MAX && (big_blocks >= BIG_TILE_MIN_WORKGROUPS || g_big_tile_mode.load() == 1)) {
+            kutacc_prof::KernelTimer t(am ? "pair_gemm_big_kernel<m-major>" : "pair_gemm_big_kernel", flops, stream);
+            return kutacc_hip_status(am ? launch_big_tiles<true>(p, big_blocks, stream) : launch_big_tiles<false>(p, big_blocks, stream));
+        }
     }
     p.MT = (int)((g.m + (gated ? 64 : 128) - 1) / (gated ? 64 : 128));
     p.NT = (int)((g.n + 127) / 128);

@@ -120,6 +120,74 @@ def test_gemm_m_major_operands(torch_cuda, shape, a_mmajor, b_mmajor):
     helpers.assert_within(got, same, 1e-3 + 8e-3 * np.abs(same), "mfma vs scalar kernel")
 
 
+@pytest.fixture
+def gemm_tile():
+    """Forces the tile size of the matrix products ("256": the large tiles wherever the shape allows, "128": never)."""
+    def choose(value):
+        assert capi.set_tuning("gemm_tile", value) == 0
+    yield choose
+    capi.set_tuning("gemm_tile", None)
+
+
+def first_profiled_kernel(torch, fn):
+    capi.lib().kutacc_hip_profile_enable(1)
+    try:
+        fn()
+        torch.cuda.synchronize()
+        name = ctypes.create_string_buffer(96)
+        ms, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+        assert capi.lib().kutacc_hip_profile_read(0, name, 96, ctypes.byref(ms), ctypes.byref(cnt), ctypes.byref(fl)) == 0
+        return name.value.decode()
+    finally:
+        capi.lib().kutacc_hip_profile_enable(0)
+
+
+@pytest.mark.parametrize("mmajor", [False, True], ids=["k-major", "m-major"])
+@pytest.mark.parametrize("shape", [(2, 256, 256, 64), (1, 512, 256, 192), (3, 256, 768, 320), (9, 256, 256, 128), (300, 256, 256, 64)])
+def test_gemm_large_tiles(torch_cuda, gemm_tile, shape, mmajor):
+    """The 256 x 256 tiles (128 x 128 per wave) against the float64 product and, bit for bit, against the 128 x 128
+    tiles, which add the same products in the same order: one and several k-steps, an odd number of them (the kernel
+    takes them in pairs), several tiles per batch, and more tiles than the chip has CUs (a workgroup then walks several,
+    its operand pipeline running across the tile boundary)."""
+    nb, M, N, K = shape
+    rng = np.random.Generator(np.random.PCG64(300 + M + N + K))
+    A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
+    gemm_tile("256")
+    name = first_profiled_kernel(torch_cuda, lambda: run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED))
+    assert name.startswith("pair_gemm_big_kernel"), name
+    got = run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED, c_pad=8)
+    ref = gemm_ref(A, B)
+    helpers.assert_within(got, ref, GEMM_TOL(ref), f"large tiles {shape}")
+    gemm_tile("128")
+    small = run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED, c_pad=8)
+    assert np.array_equal(got, small)
+
+
+def test_equation_at_768_residues_takes_the_large_tiles(torch_cuda):
+    """128 channels of 768 x 768: nine large tiles per channel, more than four per CU, which is where the default rule
+    switches to them.  Sampled channels against the oracle; the incoming form equals the outgoing one on transposed
+    operands bit for bit."""
+    from oracle import oracle
+    torch = torch_cuda
+    n, c_i = 768, 128
+    g = torch.Generator(device="cuda").manual_seed(77)
+    left = (torch.randn(c_i, n, n, device="cuda", generator=g)).to(torch.bfloat16)
+    right = (torch.randn(c_i, n, n, device="cuda", generator=g) * n ** -0.5).to(torch.bfloat16)
+    for incoming in (False, True):
+        name = first_profiled_kernel(torch, lambda: equation(torch, left, right, n, incoming))
+        assert name == ("pair_gemm_big_kernel<m-major>" if incoming else "pair_gemm_big_kernel"), name
+    out_c = equation(torch, left, right, n, False)
+    in_c = equation(torch, left, right, n, True)
+    chans = [0, 63, 127]
+    l_np, r_np = helpers.to_numpy(left[chans]), helpers.to_numpy(right[chans])
+    for incoming, got in ((False, out_c), (True, in_c)):
+        ref = oracle.tm_equation_f32(l_np, r_np, incoming)
+        helpers.assert_within(helpers.to_numpy(got[chans]), ref, 2e-2 + 6e-3 * np.abs(ref), f"equation incoming={incoming}")
+    lt, rt = left.transpose(1, 2).contiguous(), right.transpose(1, 2).contiguous()
+    swapped = equation(torch, rt, lt, n, False)
+    assert helpers.same_bits(swapped, in_c)
+
+
 @pytest.mark.parametrize("bias_axis,relu", [(1, False), (1, True), (2, False), (2, True), (0, False)])
 @pytest.mark.parametrize("path", [capi.PATH_FUSED, capi.PATH_GENERIC], ids=["mfma", "scalar"])
 def test_gemm_gated_form_bias_axes(torch_cuda, path, bias_axis, relu):
