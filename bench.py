@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 MFMA_BF16_PEAK_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU, dense
+MFMA_FP32_PEAK_TFLOPS = 157.3   # fp32 matrix (32x32x2 f32 MFMA): 256 flop/clk/CU
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of each kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command, each
@@ -502,7 +503,7 @@ def config_summary(config, steps, warmup):
     tf = flops / (ms * 1e-3) / 1e12
     rec = {"workload": f"config {config} {spec['name']}: B={B} S={S} C={C} H={H} d=32", "dtype": spec["dtype"], "steps": steps,
            "ms": round(ms, 5), "TFLOP/s": round(tf, 2),
-           "frac_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4) if spec["dtype"] == "bf16" else None,
+           "frac_mfma_peak": round(tf / (MFMA_BF16_PEAK_TFLOPS if spec["dtype"] == "bf16" else MFMA_FP32_PEAK_TFLOPS), 4),
            "path": capi.last_path(), "dominant_kernel": dom["name"], "dominant_kernel_ms": round(dom["avg_ms"], 5),
            "kernels": [{"name": k["name"], "avg_ms": round(k["avg_ms"], 5), "launches_per_call": k["launches"] // max(steps, 1)}
                        for k in kernels],
@@ -577,18 +578,19 @@ def main():
     # avg_ms_net subtracts the empty pair and is the figure comparable with a profiler's kernel duration.
     overhead_ms = empty_event_pair_ms(stream)
     dom = max(kernels, key=lambda k: k["avg_ms"] * k["launches"]) if kernels else None
+    peak = MFMA_BF16_PEAK_TFLOPS if w.dtype == "bf16" else MFMA_FP32_PEAK_TFLOPS  # fp32 storage runs on the fp32 matrix core
     roofline = None
     if dom:
         ach = dom["flops_per_launch"] / (dom["avg_ms"] * 1e-3) / 1e12
         net_ms = max(dom["avg_ms"] - overhead_ms, 1e-6)
         ach_net = dom["flops_per_launch"] / (net_ms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4),
+        roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": round(ach, 2), "peak": peak,
+                    "unit": "TFLOP/s", "frac": round(ach / peak, 4),
                     "traffic": measured_traffic(w.config, dom["name"]),
                     "traffic_source": "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
                                       "not re-measured in this run)",
                     "avg_kernel_ms": round(dom["avg_ms"], 5), "avg_kernel_ms_net": round(net_ms, 5),
-                    "achieved_net": round(ach_net, 2), "frac_net": round(ach_net / MFMA_BF16_PEAK_TFLOPS, 4),
+                    "achieved_net": round(ach_net, 2), "frac_net": round(ach_net / peak, 4),
                     "empty_event_pair_ms": round(overhead_ms, 5),
                     "flops_per_launch": dom["flops_per_launch"]}
 
@@ -600,7 +602,7 @@ def main():
         "config": {"workload": f"config {w.config} {w.name}: B={w.B} S={w.S} C={w.C} H={w.H} d={w.d}",
                    "flops_per_call": w.flops(), "algorithmic_bytes_per_call": w.algorithmic_bytes(),
                    "path": capi.last_path()},
-        "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        "frac_mfma_peak": round(tflops / peak, 4),
         # ms_per_step and value are the median window; each window is exactly `steps` calls
         "timed_windows": {"count": len(windows), "steps_each": a.steps, "median_ms": round(ms, 5),
                           "min_ms": round(min(windows), 5), "max_ms": round(max(windows), 5),
@@ -616,7 +618,7 @@ def main():
     if not a.no_all_configs:
         # the other configurations, same settle + warm-up, at least 50 steps each (no CPU leg)
         rec["all_configs"] = {f"config {w.config}": {"ms": round(ms, 5), "TFLOP/s": round(tflops, 2),
-                                                      "frac_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                                                      "frac_mfma_peak": round(tflops / peak, 4),
                                                       "path": rec["config"]["path"],
                                                       "dominant_kernel": dom["name"] if dom else None}}
         for c in (1, 2, 4, 5):
