@@ -438,6 +438,11 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *               weight matrices per LDS group where that fits the device; anything else: the planner decides (default)
  *   "fragments" "0": keep the attention kernels off the fragment-major pair bias (general softmax blocks); "1": default
  *   "debug"     "1": one line per fused call on stderr with the plan taken; "0": default
+ *   "row_pairs" "0": never the attention kernel that walks two batch rows per step (128 channels, up to 384 positions);
+ *               "1": wherever it can run; anything else (default): where every workgroup has at least two batch rows
+ *   "gemm_tile" "128" / "256": the batched products of kutacc_af2_triangle_multiplication_equation always on 128 x 128
+ *               tiles / on 256 x 256 tiles wherever the shape has whole ones; anything else (default): 256 x 256 where
+ *               every CU gets at least four tiles
  *   "layernorm" "fused": kutacc_hip_triangle_attention and kutacc_hip_msa_attention let the attention kernel normalise its
  *               input rows itself where it can (sequence lengths of the persistent kernel), which drops the normalised
  *               copy from the workspace and costs 8-15 % of the block's time; "separate" or "auto" (default): the

@@ -315,7 +315,8 @@ def set_blocking(blocking: bool) -> None:
 
 
 def set_tuning(name: str, value: str | None) -> int:
-    """kutacc_hip_set_tuning: "plan" / "fragments" / "debug" hooks of the attention launcher (None = default)."""
+    """kutacc_hip_set_tuning: the hooks include/kutacc_hip.h lists ("plan", "fragments", "debug", "row_pairs",
+    "gemm_tile", "layernorm", "scratch", "pointer_checks"); None = the default of that hook."""
     return lib().kutacc_hip_set_tuning(name.encode(), None if value is None else value.encode())
 
 

@@ -157,29 +157,33 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     if (!kutacc_launch::fused_attention_supports(g)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
-    // 1. LayerNorm + pair-bias projection in one pass over the pair tensor; the ending node reads it transposed
-    //    -- and, where the grid allows it, writes the fragment-major copy the attention kernels read as well
-    void *z_norm = fused_ln ? nullptr : ws + w.z_norm;
-    int frag_nb = 0, frag_nt = 0;
-    const bool fragments = kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt) &&
-                           kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, z_norm, n, n, c, heads,
-                                                                     KUTACC_DTYPE_BF16);
-    int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, z_norm, n, n, c, heads,
-                                      a->ln_eps, KUTACC_DTYPE_BF16, ending, s, fragments ? g.q : nullptr, frag_nb, frag_nt);
-    if (rc != 0) {
-        return rc;
-    }
-    // 2. the operator: it forms the mask bias from the pair mask itself, and its output projection adds straight into
-    //    the pair activation (transposed back for the ending node), so neither costs a pass of its own
+    // The operator forms the mask bias from the pair mask itself, and its output projection adds straight into the pair
+    // activation (transposed back for the ending node), so neither costs a pass of its own.
     kutacc_launch::FusedAttentionOptions opt;
     opt.out_mode = ending ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
     opt.bias_is_mask = true; // element (b, k) of the mask bias comes from mask[b, k], or mask[k, b] for the ending node
     opt.bias_stride_k = ending ? n : 1;
-    opt.nb_fragments_ready = fragments;
     if (fused_ln) {
         opt.ln_gamma = a->ln_gamma, opt.ln_beta = a->ln_beta, opt.ln_eps = a->ln_eps;
         opt.input_stride_b = ending ? c : n * c;
     }
+    // 1. LayerNorm + pair-bias projection in one pass over the pair tensor; the ending node reads it transposed
+    //    -- and, where the grid allows it, writes the copy the attention kernel will read as well: fp32 tiles where
+    //    the operator takes the two-row kernel, fp16 fragments otherwise
+    void *z_norm = fused_ln ? nullptr : ws + w.z_norm;
+    int frag_nb = 0, frag_nt = 0;
+    const bool writes = kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, z_norm, n, n, c, heads, KUTACC_DTYPE_BF16);
+    const bool tiles = writes && heads <= 8 && kutacc_launch::fused_attention_tile_layout(g, opt, &frag_nb, &frag_nt);
+    const bool fragments = !tiles && writes && kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt);
+    int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, z_norm, n, n, c, heads,
+                                      a->ln_eps, KUTACC_DTYPE_BF16, ending, s, (tiles || fragments) ? g.q : nullptr, frag_nb,
+                                      frag_nt, tiles ? 1 : 0);
+    if (rc != 0) {
+        return rc;
+    }
+    // 2. the operator
+    opt.nb_tiles_ready = tiles;
+    opt.nb_fragments_ready = fragments;
     return kutacc_launch::gating_attention_fused(g, s, opt);
 }
 

@@ -158,6 +158,46 @@ __device__ __forceinline__ void stage_mask_part(const bf16_t *bias_row, float *m
     }
 }
 
+// stage_mask_part for the two-row kernel, which adds a row's mask bias to its logits with one more MFMA (a rank-one
+// product of the per-key values with ones) instead of sixteen vector additions per tile: the value of key k is stored
+// as two bf16, v = hi + lo to 2^-17 of |v|, the k-slots 0 and 1 of that MFMA's A operand.  -inf (keys past S): hi = -inf,
+// lo = 0.
+template <bool NEAR = false>
+__device__ __forceinline__ void stage_mask_words(const bf16_t *bias_row, uint32_t *words, uint32_t *flag_word, int S, int NB,
+                                                 int wave, int lane, float scale, int64_t stride_k, bool from_mask)
+{
+    const int k = wave * 64 + lane;
+    if (wave * 64 < NB * 32) {
+        float mv = -INFINITY;
+        if (k < S) {
+            mv = to_f32(bias_row[NEAR ? (int64_t)__umul24((uint32_t)k, (uint32_t)stride_k) : k * stride_k]);
+            if (from_mask) {
+                mv = to_f32((bf16_t)fmaf(mv, 1e9f, -1e9f));
+            }
+            mv *= scale;
+        }
+        if (k < NB * 32) {
+            const bf16_t hi = (bf16_t)mv;
+            const float hf = to_f32(hi);
+            const float rest = (hf == mv || !(fabsf(hf) < INFINITY)) ? 0.f : mv - hf; // a NaN stays one through hi
+            const bf16_t lo = (bf16_t)rest;
+            bf16x2 pair;
+            pair[0] = hi, pair[1] = lo;
+            words[k] = __builtin_bit_cast(uint32_t, pair);
+        }
+        const unsigned long long nz = __ballot(k < NB * 32 && mv != 0.f);
+        const uint32_t bits = (((uint32_t)nz != 0u ? 1u : 0u) | ((uint32_t)(nz >> 32) != 0u ? 2u : 0u)) << (2 * wave);
+        if (lane == 0 && bits != 0u) {
+            atomicOr(flag_word, bits);
+        }
+    }
+}
+
+__device__ __forceinline__ float mask_word_value(uint32_t w)
+{
+    return __uint_as_float(w << 16) + __uint_as_float(w & 0xffff0000u);
+}
+
 // The value stage_mask_part would store for key k, in two steps for kernels that fetch the mask early and store it
 // later, so that nothing waits for the load where it is issued: the raw element of key min(k, S - 1) ...
 __device__ __forceinline__ bf16_t mask_bias_fetch(const bf16_t *bias_row, int S, int k, int64_t stride_k)
@@ -1563,16 +1603,30 @@ __global__ __launch_bounds__(64) void pair_bias_tiles_kernel(const bf16_t *__res
 // formulation.  Tiles are walked A(0) B(0) A(1) B(1) ...: while the softmax and P.V of one (row, tile) run on the vector
 // ALU, the logits MFMAs of the next one are in the matrix pipe.
 //   lds_kA/vA/kB/vB : K and V fragments of the two rows, [tile][kstep][lane]
-//   maskA4 / maskB4 : fp32 mask bias of the rows (log2 units), offset by 16 g floats; added to every tile (WITH_MASK only)
+//   mwA / mwB       : mask bias of the rows (log2 units) as hi/lo bf16 words (stage_mask_words), offset by the key the
+//                     lane's accumulator row stands for; one more MFMA per tile adds them (WITH_MASK only)
 //   nbc             : fp32 pair-bias tiles of this head and query block, offset by the lane: tile t, piece a at
 //                     nbc[(4 t + a) * 64]; nullptr without a pair bias
 template <bool HAS_NB, bool WITH_MASK>
 __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 *lds_vA, const uint4 *lds_kB, const uint4 *lds_vB,
-                                               const f32x4 *maskA4, const f32x4 *maskB4, const f32x4 *nbc, bf16x8 qA0, bf16x8 qA1,
+                                               const uint32_t *mwA, const uint32_t *mwB, const f32x4 *nbc, bf16x8 qA0, bf16x8 qA1,
                                                bf16x8 qB0, bf16x8 qB1, int NB, int lane, f32x16 &oA_out,
                                                float &lA_out, f32x16 &oB_out, float &lB_out, uint32_t turn)
 {
     const int npairs = NB >> 1;
+    // The mask of a row as a rank-one MFMA: A holds (hi, lo) of the key of accumulator row i in k-slots 0 and 1, B holds
+    // ones there, everything else is zero -- in the lanes of the upper half (k-slots 8..15) both operands are all zero,
+    // so that an infinite mask value never meets a zero.
+    const uint32_t lower = lane < 32 ? 0xffffffffu : 0u;
+    uint4 ones4 = {0x3f803f80u & lower, 0u, 0u, 0u};
+    const bf16x8 onesf = as_bf16x8(ones4);
+    auto mask_fragment = [&](const uint32_t *mw, int t) {
+        uint4 u = {0u, 0u, 0u, 0u};
+        if constexpr (WITH_MASK) {
+            u.x = mw[32 * t] & lower;
+        }
+        return as_bf16x8(u);
+    };
     const uint4 *kA = lds_kA + lane, *vA = lds_vA + lane, *kB = lds_kB + lane, *vB = lds_vB + lane;
     auto clampt = [&](int t) { return t < NB ? t : NB - 1; };
     auto loadC = [&](int t) {
@@ -1596,6 +1650,9 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     f32x16 xa, xb;
     xa = mfma(as_bf16x8(k0), qA0, C0);
     xa = mfma(as_bf16x8(k1), qA1, xa);
+    if constexpr (WITH_MASK) {
+        xa = mfma(mask_fragment(mwA, 0), onesf, xa);
+    }
     k0 = kB[0], k1 = kB[64];
     v0 = vA[0], v1 = vA[64];
     f32x16 oA = zero16(), oB = zero16();
@@ -1623,24 +1680,6 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
             lsum = __builtin_amdgcn_fdot2_f32_bf16(a, one2, lsum, false);
         }
     };
-    // what is left to add to the logits of a finished tile before the exponential: the row's mask bias (the pair-bias
-    // seed is shared by the two rows, their masks are not).  Added to every tile, flagged or not: a branch per tile
-    // splits the loop into pieces that the register allocator handles worse than sixteen adds.
-    auto finish_logits = [&](f32x16 &x, const f32x4 *mask4, int t) {
-        if constexpr (WITH_MASK) {
-            __builtin_amdgcn_sched_barrier(0); // the four reads and sixteen adds stay together: spread out, their
-                                               // temporaries push the loop past its registers
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                const f32x4 mv = mask4[t * 8 + a];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    x[4 * a + c] += mv[c];
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
     auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
     auto exp4 = [&](f32x16 &x, int base) {
 #pragma unroll
@@ -1654,8 +1693,10 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     // that reads it: the compiler then writes xn to registers of its own (D != C) instead of computing it in place in
     // C's registers, which rotated the roles of the register blocks from one iteration to the next and cost 40 copies
     // per iteration, behind a wait for every load in flight.
-    auto half_step = [&](f32x16 &xc, f32x16 &xn, const f32x16 &C, bf16x8 q0, bf16x8 q1, f32x16 &o, float &lsum, const uint4 *knext) {
+    auto half_step = [&](f32x16 &xc, f32x16 &xn, const f32x16 &C, bf16x8 q0, bf16x8 q1, f32x16 &o, float &lsum, const uint4 *knext,
+                         const uint32_t *mw_next, int t_next) {
         bf16x8 p0, p1;
+        const bf16x8 mnext = mask_fragment(mw_next, t_next); // requested first, used by the last MFMA of the step
         exp4(xc, 0);
         exp4(xc, 4);
         p0 = pack_trunc(xc, 0);
@@ -1664,6 +1705,9 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
         o = mfma(as_bf16x8(v0), p0, o);
         exp4(xc, 8);
         xn = mfma(as_bf16x8(k1), q1, xn);
+        if constexpr (WITH_MASK) {
+            xn = mfma(mnext, onesf, xn);
+        }
         rowsum(lsum, p0);
         k0 = knext[0], k1 = knext[64];
         exp4(xc, 12);
@@ -1676,26 +1720,22 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
         const int t0 = 2 * pair, t1 = t0 + 1;
         const int tn = pair + 1 < npairs ? t0 + 2 : t0; // next pair's first tile, clamped
         // (A, t0) finished; logits of (B, t0) from C0
-        finish_logits(xa, maskA4, t0);
-        half_step(xa, xb, C0, qB0, qB1, oA, lsumA, kA + t1 * 128);
+        half_step(xa, xb, C0, qB0, qB1, oA, lsumA, kA + t1 * 128, mwB, t0);
         v0 = vB[t0 * 128], v1 = vB[t0 * 128 + 64];
         fence(); // the loads stay behind the last reader of the registers they fill
         C0 = loadC(clampt(t0 + 2));
         fence();
         // (B, t0) finished; logits of (A, t1) from C1
-        finish_logits(xb, maskB4, t0);
-        half_step(xb, xa, C1, qA0, qA1, oB, lsumB, kB + t1 * 128);
+        half_step(xb, xa, C1, qA0, qA1, oB, lsumB, kB + t1 * 128, mwA, t1);
         v0 = vA[t1 * 128], v1 = vA[t1 * 128 + 64];
         // (A, t1) finished; logits of (B, t1) from C1
-        finish_logits(xa, maskA4, t1);
-        half_step(xa, xb, C1, qB0, qB1, oA, lsumA, kA + tn * 128);
+        half_step(xa, xb, C1, qB0, qB1, oA, lsumA, kA + tn * 128, mwB, t1);
         v0 = vB[t1 * 128], v1 = vB[t1 * 128 + 64];
         fence();
         C1 = loadC(clampt(t1 + 2));
         fence();
         // (B, t1) finished; logits of (A, tn) from C0
-        finish_logits(xb, maskB4, t1);
-        half_step(xb, xa, C0, qA0, qA1, oB, lsumB, kB + tn * 128);
+        half_step(xb, xa, C0, qA0, qA1, oB, lsumB, kB + tn * 128, mwA, tn);
         v0 = vA[tn * 128], v1 = vA[tn * 128 + 64];
     }
     __builtin_amdgcn_s_setprio(0);
@@ -1707,14 +1747,16 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
 // tiles: a first pass over the key tiles for the true row maxima, a second one with them subtracted.  Not a hot path:
 // one row, nothing prefetched, few registers.
 template <bool HAS_NB>
-__device__ __forceinline__ void attend_row_shifted(const uint4 *lds_k, const uint4 *lds_v, const f32x4 *mask4, const f32x4 *nbc, bf16x8 q0,
+__device__ __forceinline__ void attend_row_shifted(const uint4 *lds_k, const uint4 *lds_v, const uint32_t *words, const f32x4 *nbc, bf16x8 q0,
                                                 bf16x8 q1, int NB, int lane, f32x16 &o_out, float &l_out)
 {
+    // words: the row's mask words (stage_mask_words), offset by 16 (lane >> 5): register 4 a + c stands for key 4 a + c of them
     auto logits = [&](int t) {
         f32x16 x;
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            f32x4 mv = mask4[t * 8 + a];
+            const uint4 w4 = *reinterpret_cast<const uint4 *>(words + 32 * t + 4 * a);
+            f32x4 mv = {mask_word_value(w4.x), mask_word_value(w4.y), mask_word_value(w4.z), mask_word_value(w4.w)};
             if constexpr (HAS_NB) {
                 const f32x4 cv = nbc[(t * 4 + a) * 64];
 #pragma unroll
@@ -1789,8 +1831,8 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedPa
     uint4 *lds_k = lds_w + 4 * CK * 64;     // [row of the pair][NT][2][64]
     uint4 *lds_v = lds_k + 2 * NT * 2 * 64; // likewise
     uint4 *panel = lds_v + 2 * NT * 2 * 64 + wave * 128;
-    float *mask_base = reinterpret_cast<float *>(lds_v + 2 * NT * 2 * 64 + NB * 128); // [pair parity][row of the pair][NT*32]
-    uint32_t *flag_words = reinterpret_cast<uint32_t *>(mask_base + 4 * NT * 32);     // [pair parity][row of the pair]
+    uint32_t *mask_base = reinterpret_cast<uint32_t *>(lds_v + 2 * NT * 2 * 64 + NB * 128); // [pair parity][row of the pair][NT*32] mask words
+    uint32_t *flag_words = mask_base + 4 * NT * 32;                                         // [pair parity][row of the pair]
 
     stage_weight_fragments<C>(lds_w, p, 0, 4, h, wave, nthreads >> 6, lane);
     if (tid < 4) {
@@ -1814,14 +1856,14 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedPa
         const bool have_b = n + 1 < nrows; // an odd row count: the last pair attends its one row twice and stores it once
         const int bA = b0 + n * bstep, bB = have_b ? bA + bstep : bA;
         uint32_t *flag_word = flag_words + 2 * par;
-        float *mask = mask_base + par * 2 * NT * 32;
+        uint32_t *mask = mask_base + par * 2 * NT * 32;
         // opaque lane index: addresses derived from it are formed anew per pair instead of living across the attention loop
         int lane_x = lane;
         asm volatile("" : "+v"(lane_x));
-        stage_mask_part<true>(p.bias + (int64_t)bA * p.bias_sb, mask, flag_word, S, NT, wave, lane_x, LOG2E, p.bias_sk,
-                              p.bias_is_mask != 0);
-        stage_mask_part<true>(p.bias + (int64_t)bB * p.bias_sb, mask + NT * 32, flag_word + 1, S, NT, wave, lane_x, LOG2E, p.bias_sk,
-                              p.bias_is_mask != 0);
+        stage_mask_words<true>(p.bias + (int64_t)bA * p.bias_sb, mask, flag_word, S, NT, wave, lane_x, LOG2E, p.bias_sk,
+                               p.bias_is_mask != 0);
+        stage_mask_words<true>(p.bias + (int64_t)bB * p.bias_sb, mask + NT * 32, flag_word + 1, S, NT, wave, lane_x, LOG2E, p.bias_sk,
+                               p.bias_is_mask != 0);
 
         // ---- input rows of the block, both batch rows -> fragments, 32 channels per staging panel ----
         const int prow_x = pi_row(lane_x & 31), g_x = lane_x >> 5;
@@ -1943,24 +1985,23 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedPa
         int lane_a = lane;
         asm volatile("" : "+v"(lane_a));
         const int g = lane_a >> 5;
-        const f32x4 *maskA4 = reinterpret_cast<const f32x4 *>(mask + 16 * g);
-        const f32x4 *maskB4 = reinterpret_cast<const f32x4 *>(mask + NT * 32 + 16 * g);
+        const uint32_t *mwA = mask + pi_row(lane_a & 31), *mwB = mwA + NT * 32; // accumulator row i of a tile is its key pi(i)
         const uint32_t flagsA = flag_word[0], flagsB = flag_word[1];
         const f32x4 *nbc = HAS_NB ? reinterpret_cast<const f32x4 *>(p.nbf) + ((int64_t)(h * NB + j) * NT * 4) * 64 + lane_a : nullptr;
         const uint4 *kA = lds_k, *vA = lds_v, *kB = lds_k + NT * 128, *vB = lds_v + NT * 128;
         f32x16 oA, oB;
         float lA, lB;
         if ((flagsA | flagsB) == 0u) {
-            attend_pair_l2<HAS_NB, false>(kA, vA, kB, vB, maskA4, maskB4, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
+            attend_pair_l2<HAS_NB, false>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
         } else {
-            attend_pair_l2<HAS_NB, true>(kA, vA, kB, vB, maskA4, maskB4, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
+            attend_pair_l2<HAS_NB, true>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
         }
         // some probability overflowed or a whole row underflowed: repeat that row shifted by its true row maxima
         if (__any(!(lA > 1e-30f && lA < 1e30f))) {
-            attend_row_shifted<HAS_NB>(kA, vA, maskA4, nbc, qA0, qA1, NT, lane_a, oA, lA);
+            attend_row_shifted<HAS_NB>(kA, vA, mask + 16 * g, nbc, qA0, qA1, NT, lane_a, oA, lA);
         }
         if (__any(!(lB > 1e-30f && lB < 1e30f))) {
-            attend_row_shifted<HAS_NB>(kB, vB, maskB4, nbc, qB0, qB1, NT, lane_a, oB, lB);
+            attend_row_shifted<HAS_NB>(kB, vB, mask + NT * 32 + 16 * g, nbc, qB0, qB1, NT, lane_a, oB, lB);
         }
         int lane_o = lane; // as above: the addresses of the epilogue are not worth a register during the attention loop
         asm volatile("" : "+v"(lane_o));
@@ -2648,6 +2689,19 @@ void *fragment_home(const kutacc_hip_attention_args_t &a, int NB, const kutacc_l
     return (q_dense && nbf_bytes <= a.batch * a.seq_len * C * 2) ? a.q : nullptr;
 }
 
+// Two batch rows per step (persistent_pair_kernel): 128 channels, log2 units, a home for the fp32 tiles of the pair bias
+// (twice the fragments' bytes), no LayerNorm inside the kernel and no ready-made fp16 fragments; by default only where
+// every workgroup walks at least two rows.
+bool pair_kernel_applies(const kutacc_hip_attention_args_t &a, const Plan &pl, const kutacc_launch::FusedAttentionOptions &opt)
+{
+    const int pair_mode = g_pair_mode.load(std::memory_order_relaxed);
+    const int64_t C = a.nheads * a.head_size;
+    return pl.persistent && C == 128 && pair_mode != 2 && !fragments_disabled() && opt.ln_gamma == nullptr &&
+           !opt.nb_fragments_ready && pair_kernel_lds(pl.NB) <= (size_t)max_lds_bytes() &&
+           (a.nonbatched_bias == nullptr || fragment_home(a, pl.NB, opt, 2) != nullptr) &&
+           (pair_mode == 1 || a.batch >= 16 * (int64_t)persistent_groups((int)a.batch, (int)a.nheads));
+}
+
 template <typename K>
 int opt_in_lds(K kern, size_t bytes, size_t *table)
 {
@@ -2787,6 +2841,17 @@ bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &a, int *
     return true;
 }
 
+bool fused_attention_tile_layout(const kutacc_hip_attention_args_t &a, const FusedAttentionOptions &opt, int *nb, int *nt)
+{
+    Plan pl;
+    if (a.nonbatched_bias == nullptr || opt.nb_fragments_ready || !fused_attention_supports(a) ||
+        !make_plan(a.seq_len, (int)(a.nheads * a.head_size), pl) || !pair_kernel_applies(a, pl, opt)) {
+        return false;
+    }
+    *nb = pl.NB, *nt = (pl.NB + 1) & ~1;
+    return true;
+}
+
 bool fused_layernorm_supported(const kutacc_hip_attention_args_t &a, const FusedAttentionOptions &opt)
 {
     Plan pl;
@@ -2873,20 +2938,18 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     if (opt.fragment_workspace != nullptr && p.nb != nullptr && fragments == nullptr && !fragments_disabled()) {
         return KUTACC_HIP_EINVAL; // the caller's workspace cannot hold the copy
     }
-    // Two batch rows per step (persistent_pair_kernel): 128 channels, log2 units, a home for the fp32 tiles of the pair
-    // bias (twice the fragments' bytes), no LayerNorm inside the kernel and no ready-made fp16 fragments; by default
-    // only where every workgroup walks at least two rows.
-    const int pair_mode = g_pair_mode.load(std::memory_order_relaxed);
     void *const tiles = fragment_home(a, pl.NB, opt, 2);
-    const bool pair_kernel = pl.persistent && C == 128 && pair_mode != 2 && !fragments_disabled() && opt.ln_gamma == nullptr &&
-                             !opt.nb_fragments_ready && pair_kernel_lds(pl.NB) <= (size_t)max_lds_bytes() &&
-                             (p.nb == nullptr || tiles != nullptr) &&
-                             (pair_mode == 1 || a.batch >= 16 * (int64_t)persistent_groups(p.B, p.H));
+    const bool pair_kernel = pair_kernel_applies(a, pl, opt);
+    if (opt.nb_tiles_ready && (!pair_kernel || p.nb == nullptr)) {
+        return KUTACC_HIP_EINVAL; // the caller asks fused_attention_tile_layout under the same options and tuning first
+    }
 
     const double BS = (double)a.batch * (double)a.seq_len;
     int rc;
     if (pair_kernel) {
-        if (p.nb != nullptr) {
+        if (p.nb != nullptr && opt.nb_tiles_ready) {
+            p.nbf = (const uint4 *)tiles; // the producer of the pair bias wrote the tiles
+        } else if (p.nb != nullptr) {
             kutacc_prof::KernelTimer t("pair_bias_tiles_kernel", 0.0, stream);
             pair_bias_tiles_kernel<<<dim3((unsigned)(pl.NB * p.NT), (unsigned)a.nheads), 64, 0, stream>>>(
                 p.nb, p.nb_sh, p.nb_sq, p.S, pl.NB, p.NT, p.nb_vec, (f32x4 *)tiles);

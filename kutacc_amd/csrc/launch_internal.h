@@ -87,6 +87,9 @@ struct FusedAttentionOptions {
     // the fragment-major copy of the pair bias already lies in args.q (written by pair_bias with the layout
     // fused_attention_fragment_layout reports): the pass that makes it is skipped
     bool nb_fragments_ready = false;
+    // the fp32 tiles of the pair bias that the two-row kernel reads already lie there (written by pair_bias with the
+    // layout fused_attention_tile_layout reports for the same options): the pass that makes them is skipped
+    bool nb_tiles_ready = false;
     // device memory (16-byte aligned) that takes the fragment-major copy of the pair bias instead of args.q, which is then
     // neither read nor written; a call whose copy does not fit is rejected with KUTACC_HIP_EINVAL
     void *fragment_workspace = nullptr;
@@ -104,6 +107,10 @@ bool fused_layernorm_supported(const kutacc_hip_attention_args_t &args, const Fu
 // Whether gating_attention_fused would keep a fragment-major copy of the pair bias in args.q, and the copy's extent:
 // [nheads][*nb query blocks][*nt key tiles][2][64 lanes] x 16 bytes.
 bool fused_attention_fragment_layout(const kutacc_hip_attention_args_t &args, int *nb, int *nt);
+// Whether gating_attention_fused would run the two-row kernel on this call under these options (and the tuning in force)
+// and keep the fp32 tiles of the pair bias in args.q or the options' workspace, and their extent:
+// [nheads][*nb query blocks][*nt key tiles][4][64 lanes] x 16 bytes.
+bool fused_attention_tile_layout(const kutacc_hip_attention_args_t &args, const FusedAttentionOptions &opt, int *nb, int *nt);
 int gating_attention_fused(const kutacc_hip_attention_args_t &args, hipStream_t stream,
                            const FusedAttentionOptions &opt = FusedAttentionOptions());
 
@@ -160,11 +167,12 @@ int layernorm_channel_first(const void *x, int64_t ld_x, const float *gamma, con
 // row (j, i) of the transposed grid
 int layernorm_rows(const void *x, int64_t ld_x, const float *gamma, const float *beta, void *out, int64_t ld_out,
                    int64_t rows, int64_t size, float eps, int32_t dtype, hipStream_t stream, int64_t swap_j = 0);
-// fragments != nullptr: the fragment-major copy the attention kernels read ([nheads][frag_nb][frag_nt][2][64] x 16 bytes,
-// values times log2(e)) is written as well; only where pair_bias_writes_fragments says so, else KUTACC_HIP_EINVAL
+// fragments != nullptr: the copy the attention kernels read is written as well, values times log2(e): fp16 fragments
+// [nheads][frag_nb][frag_nt][2][64] x 16 bytes, or with frag_tiles != 0 the fp32 tiles of the two-row kernel,
+// [nheads][frag_nb][frag_nt][4][64] x 16 bytes; only where pair_bias_writes_fragments says so, else KUTACC_HIP_EINVAL
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
               int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
-              hipStream_t stream, void *fragments = nullptr, int frag_nb = 0, int frag_nt = 0);
+              hipStream_t stream, void *fragments = nullptr, int frag_nb = 0, int frag_nt = 0, int frag_tiles = 0);
 bool pair_bias_writes_fragments(const void *z, const void *w, const void *z_norm, int64_t rows_i, int64_t rows_j, int64_t c_z,
                                 int64_t nheads, int32_t dtype);
 

@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
                                                              bf16_t *__restrict__ nb, bf16_t *__restrict__ z_norm,
                                                              int64_t rows, float eps, int64_t rows_i, int64_t rows_j,
                                                              int transposed, uint4 *__restrict__ nbf, int frag_nb,
-                                                             int frag_nt)
+                                                             int frag_nt, int frag_tiles)
 {
     constexpr int LPR = 16, CZ = 128, STEPS = PAIR_BIAS_ROWS_PER_WAVE / 4, RB = PAIR_BIAS_ROWS_PER_WAVE / 32;
     __shared__ uint4 tiles[4][RB * 2 * 256]; // per wave: its rows x 128 channels as 32 x 64 panels
@@ -324,7 +324,34 @@ __global__ __launch_bounds__(256) void pair_bias_bf16_kernel(const bf16_t *__res
                 }
             }
         }
-        if (nbf != nullptr) {
+        if (nbf != nullptr && frag_tiles) {
+            // The copy the two-row attention kernel reads: fp32 tiles in the order of its logits accumulators, in log2 units,
+            // [head][query block][key tile][4][64 lanes] x 16 bytes -- lane (pi^-1(q mod 32), g') holds keys 16 g' .. + 15 of
+            // the tile for query q, four per piece.  Through the wave's tile: [head][32 keys] fp32, of which a lane takes
+            // the four keys of one piece.
+            static_assert(RB == 1 && H <= 8, "one lane per piece: 8 pieces per head");
+            float *t32 = reinterpret_cast<float *>(tile);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if (4 * g + v < H) {
+                    const float x = (float)(bf16_t)acc[v] * kutacc_dev::LOG2E;
+                    t32[(4 * g + v) * 32 + col] = x < -3.0e38f ? -3.0e38f : x; // -inf: the most negative finite value
+                }
+            }
+            __builtin_amdgcn_wave_barrier(); // other lanes' stores: keep the loads below behind them
+            if (lane < 8 * H) {
+                const int h = lane >> 3, c = lane & 7; // piece c: keys 4 c .. 4 c + 3 = half g' = c >> 2, piece a = c & 3
+                const uint4 val = *reinterpret_cast<const uint4 *>(t32 + h * 32 + c * 4);
+                const uint32_t r0b = r0 + rb * 32;
+                const int q = (int)(r0b / ncol), t = (int)(r0b % ncol) >> 5, qr = q & 31;
+                const int qlane = (qr & 3) | (((qr >> 4) & 1) << 2) | (((qr >> 2) & 3) << 3);
+                uint4 *dst = nbf + ((((int64_t)h * frag_nb + (q >> 5)) * frag_nt + t) * 4 + (c & 3)) * 64 + qlane + 32 * (c >> 2);
+                *dst = val;
+                if (t + 1 == frag_nb && frag_nt > frag_nb) { // the phantom tile that pads the key tiles to a pair
+                    dst[256] = make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+        } else if (nbf != nullptr) {
             // The copy the attention kernels read (rows_j a multiple of 32: the wave's rows are key tile t of one query
             // q): for head h, query block j, key tile t, 16-key half g' and 8-key half e the 16 bytes of lane
             // (pi^-1(q mod 32), g'), pi being the row order of the attention's accumulators; values in log2 units as
@@ -392,7 +419,7 @@ int launch_layernorm(const void *x, int64_t ld_x, const float *gamma, const floa
 template <typename T>
 int launch_pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
                      int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int transposed,
-                     hipStream_t stream, void *fragments, int frag_nb, int frag_nt)
+                     hipStream_t stream, void *fragments, int frag_nb, int frag_nt, int frag_tiles)
 {
     const int64_t rows = rows_i * rows_j;
     if (fragments != nullptr &&
@@ -411,11 +438,11 @@ int launch_pair_bias(const void *z, const float *gamma, const float *beta, const
         if (nheads == 4) {
             pair_bias_bf16_kernel<4><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
                                                                         (bf16_t *)nb, (bf16_t *)z_norm, rows, eps, rows_i, rows_j,
-                                                                        transposed, (uint4 *)fragments, frag_nb, frag_nt);
+                                                                        transposed, (uint4 *)fragments, frag_nb, frag_nt, frag_tiles);
         } else {
             pair_bias_bf16_kernel<8><<<(unsigned)nblk, 256, 0, stream>>>((const bf16_t *)z, gamma, beta, (const bf16_t *)w,
                                                                         (bf16_t *)nb, (bf16_t *)z_norm, rows, eps, rows_i, rows_j,
-                                                                        transposed, (uint4 *)fragments, frag_nb, frag_nt);
+                                                                        transposed, (uint4 *)fragments, frag_nb, frag_nt, frag_tiles);
         }
         return kutacc_hip_status(hipGetLastError());
     }
@@ -459,18 +486,18 @@ bool pair_bias_writes_fragments(const void *z, const void *w, const void *z_norm
 
 int pair_bias(const void *z, const float *gamma, const float *beta, const void *w, void *nb, void *z_norm,
               int64_t rows_i, int64_t rows_j, int64_t c_z, int64_t nheads, float eps, int32_t dtype, int transposed,
-              hipStream_t stream, void *fragments, int frag_nb, int frag_nt)
+              hipStream_t stream, void *fragments, int frag_nb, int frag_nt, int frag_tiles)
 {
     if (!z || !gamma || !beta || !w || !nb || rows_i <= 0 || rows_j <= 0 || c_z <= 0 || nheads <= 0) {
         return KUTACC_HIP_EINVAL;
     }
     if (dtype == KUTACC_DTYPE_BF16) {
         return launch_pair_bias<bf16_t>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream,
-                                        fragments, frag_nb, frag_nt);
+                                        fragments, frag_nb, frag_nt, frag_tiles);
     }
     if (dtype == KUTACC_DTYPE_FP32) {
         return launch_pair_bias<float>(z, gamma, beta, w, nb, z_norm, rows_i, rows_j, c_z, nheads, eps, transposed, stream,
-                                       fragments, frag_nb, frag_nt);
+                                       fragments, frag_nb, frag_nt, frag_tiles);
     }
     return KUTACC_HIP_EINVAL;
 }

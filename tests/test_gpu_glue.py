@@ -164,6 +164,42 @@ def test_triangle_attention_block_against_the_oracle(torch_cuda, layernorm_place
     helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block n={n} ending={ending}")
 
 
+def profiled_kernels(torch, fn):
+    """Names of the kernels the library timed while fn ran."""
+    import ctypes
+    lib = capi.lib()
+    lib.kutacc_hip_profile_enable(1)
+    try:
+        fn()
+        torch.cuda.synchronize()
+        names, i = [], 0
+        name = ctypes.create_string_buffer(128)
+        ms, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+        while lib.kutacc_hip_profile_read(i, name, 128, ctypes.byref(ms), ctypes.byref(cnt), ctypes.byref(fl)) == 0:
+            names.append(name.value.decode())
+            i += 1
+        return names
+    finally:
+        lib.kutacc_hip_profile_enable(0)
+
+
+@pytest.mark.parametrize("ending", [False, True], ids=["starting node", "ending node"])
+@pytest.mark.parametrize("n", [32, 64, 96, 160, 352])
+def test_triangle_attention_block_on_the_two_row_kernel(torch_cuda, n, ending):
+    """Whole key tiles and the two-row kernel forced wherever it can run: the producer of the pair bias writes the fp32
+    tiles that kernel reads (no pre-pass of the operator), one to eleven key tiles, odd counts padded with a zero tile,
+    one or several rows per workgroup."""
+    c = block_case(900 + n, n, 4)
+    assert capi.set_tuning("row_pairs", "1") == 0
+    try:
+        got = {}
+        names = profiled_kernels(torch_cuda, lambda: got.setdefault("z", run_block(torch_cuda, c, ending)))
+    finally:
+        capi.set_tuning("row_pairs", None)
+    assert "persistent_pair_kernel" in names and "pair_bias_tiles_kernel" not in names and "pair_bias_fragments_kernel" not in names, names
+    helpers.check_close(helpers.to_numpy(got["z"]), block_oracle(c, ending), "bf16", f"block n={n} ending={ending}, two-row kernel")
+
+
 @pytest.mark.parametrize("index,n", [(i, int(n)) for i, n in enumerate(np.random.Generator(np.random.PCG64(57)).integers(8, 200, size=8))])
 def test_triangle_attention_block_seeded_sweep(torch_cuda, layernorm_placement, index, n):
     """Eight seeded pair sizes between 8 and 199 (ragged key tiles, odd tile counts), four heads, node alternating."""
@@ -212,7 +248,12 @@ def test_triangle_attention_block_full_size_sampled_rows(torch_cuda, n):
     c = block_case(7000 + n, n, 4)
     rows = sorted({0, 1, 31, 32, 33, n // 2 - 1, n // 2, n - 34, n - 33, n - 32, n - 4, n - 3, n - 2, n - 1})
     for ending in (False, True):
-        got = run_block(torch, c, ending)
+        res = {}
+        names = profiled_kernels(torch, lambda: res.setdefault("z", run_block(torch, c, ending)))
+        got = res["z"]
+        # 384 residues: the two-row kernel on tiles the producer wrote; 1024: the long-sequence kernel on its fragments
+        assert ("persistent_pair_kernel" if n == 384 else "fused_head_kernel") in names, names
+        assert "pair_bias_tiles_kernel" not in names and "pair_bias_fragments_kernel" not in names, names
         assert bool(torch.isfinite(got).all())
         want = block_oracle_rows(c, ending, rows)
         sample = got[:, rows].transpose(0, 1) if ending else got[rows]
