@@ -486,30 +486,33 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
     int rc = fused_ln ? 0
                       : kutacc_launch::layernorm_rows(a->msa_act, c, a->ln_gamma, a->ln_beta, ws + w.m_norm, c, n_seq * n_res, c,
                                                       a->ln_eps, KUTACC_DTYPE_BF16, s, column ? n_seq : 0);
+    // The operator forms the mask bias from the msa mask on the fly, and its output projection adds into the msa
+    // (transposed back for the column-wise form).
+    kutacc_launch::FusedAttentionOptions opt;
+    opt.out_mode = column ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
+    opt.bias_is_mask = true; // msa_mask[s, r] is element (b = s, k = r) row-wise and (b = r, k = s) column-wise
+    opt.bias_stride_k = column ? n_res : 1;
+    if (fused_ln) {
+        opt.ln_gamma = a->ln_gamma, opt.ln_beta = a->ln_beta, opt.ln_eps = a->ln_eps;
+        opt.input_stride_b = column ? c : n_res * c;
+    }
     // 2. pair bias from the pair activation (row-wise form only)
-    //    -- with the fragment-major copy the attention kernels read, where the grid allows it
-    bool fragments = false;
+    //    -- with the copy the attention kernel will read, where the grid allows it: fp32 tiles for the two-row kernel,
+    //    fp16 fragments otherwise
     if (rc == 0 && !column) {
         int frag_nb = 0, frag_nt = 0;
-        fragments = kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt) &&
-                    kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, nullptr, n_res, n_res, a->c_z, heads,
-                                                              KUTACC_DTYPE_BF16);
+        const bool writes = kutacc_launch::pair_bias_writes_fragments(a->pair_act, a->bias_w, nullptr, n_res, n_res, a->c_z, heads,
+                                                                      KUTACC_DTYPE_BF16);
+        const bool tiles = writes && heads <= 8 && kutacc_launch::fused_attention_tile_layout(g, opt, &frag_nb, &frag_nt);
+        const bool fragments = !tiles && writes && kutacc_launch::fused_attention_fragment_layout(g, &frag_nb, &frag_nt);
         rc = kutacc_launch::pair_bias(a->pair_act, a->pair_ln_gamma, a->pair_ln_beta, a->bias_w, ws + w.nb, nullptr, n_res, n_res,
-                                      a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s, fragments ? g.q : nullptr, frag_nb,
-                                      frag_nt);
-    }
-    // 3. the operator: mask bias formed from the msa mask on the fly, output projection adding into the msa (transposed
-    //    back for the column-wise form)
-    if (rc == 0) {
-        kutacc_launch::FusedAttentionOptions opt;
-        opt.out_mode = column ? kutacc_launch::FUSED_OUT_ADD_TRANSPOSED : kutacc_launch::FUSED_OUT_ADD;
-        opt.bias_is_mask = true; // msa_mask[s, r] is element (b = s, k = r) row-wise and (b = r, k = s) column-wise
-        opt.bias_stride_k = column ? n_res : 1;
+                                      a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s, (tiles || fragments) ? g.q : nullptr,
+                                      frag_nb, frag_nt, tiles ? 1 : 0);
+        opt.nb_tiles_ready = tiles;
         opt.nb_fragments_ready = fragments;
-        if (fused_ln) {
-            opt.ln_gamma = a->ln_gamma, opt.ln_beta = a->ln_beta, opt.ln_eps = a->ln_eps;
-            opt.input_stride_b = column ? c : n_res * c;
-        }
+    }
+    // 3. the operator
+    if (rc == 0) {
         rc = kutacc_launch::gating_attention_fused(g, s, opt);
     }
     return rc;

@@ -1611,7 +1611,7 @@ template <bool HAS_NB, bool WITH_MASK>
 __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 *lds_vA, const uint4 *lds_kB, const uint4 *lds_vB,
                                                const uint32_t *mwA, const uint32_t *mwB, const f32x4 *nbc, bf16x8 qA0, bf16x8 qA1,
                                                bf16x8 qB0, bf16x8 qB1, int NB, int lane, f32x16 &oA_out,
-                                               float &lA_out, f32x16 &oB_out, float &lB_out, uint32_t turn)
+                                               float &lA_out, f32x16 &oB_out, float &lB_out, int turn)
 {
     const int npairs = NB >> 1;
     // The mask of a row as a rank-one MFMA: A holds (hi, lo) of the key of accumulator row i in k-slots 0 and 1, B holds
@@ -1716,7 +1716,9 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
         rowsum(lsum, p1);
     };
     for (int pair = 0; pair < npairs; ++pair) {
-        timeslice_priority(turn, FAIR_SLICE_SHIFT);
+        if (turn >= 0) {
+            timeslice_priority((uint32_t)turn, FAIR_SLICE_SHIFT);
+        }
         const int t0 = 2 * pair, t1 = t0 + 1;
         const int tn = pair + 1 < npairs ? t0 + 2 : t0; // next pair's first tile, clamped
         // (A, t0) finished; logits of (B, t0) from C0
@@ -1807,10 +1809,10 @@ __device__ __forceinline__ void attend_row_shifted(const uint4 *lds_k, const uin
     l_out = half_swap_sum(lsum);
 }
 
-template <bool HAS_NB>
-__global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedParams p)
+template <int C, bool HAS_NB>
+__global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_pair_kernel(FusedParams p)
 {
-    constexpr int C = 128, CK = C / 16;
+    constexpr int CK = C / 16;
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1849,6 +1851,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedPa
     __syncthreads();
 
     const int j = wave; // this wave's sequence block
+    const int fair_turn = C == 128 ? wave >> 2 : -1; // time-sliced priorities pay with three waves per SIMD only
     const float qmul = p.qscale * LOG2E;
     const uint32_t x_pitch = (uint32_t)p.x_ld; // the host sends only near-addressable rows here
     for (int n = 0; n < nrows; n += 2) {
@@ -1869,27 +1872,28 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedPa
         const int prow_x = pi_row(lane_x & 31), g_x = lane_x >> 5;
         const bf16_t *xA = p.x + (int64_t)bA * p.x_sb, *xB = p.x + (int64_t)bB * p.x_sb;
         bf16x8 xfA[CK], xfB[CK];
-        {
+#pragma unroll
+        for (int q = 0; q < C / 128; ++q) { // 128 channels of both rows at a time
             Panel32Regs ta[4], tb[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                ta[c] = panel32_load_near(xA, x_pitch, j * 32, S - 1, 32 * c, lane_x);
+                ta[c] = panel32_load_near(xA, x_pitch, j * 32, S - 1, 128 * q + 32 * c, lane_x);
             }
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                tb[c] = panel32_load_near(xB, x_pitch, j * 32, S - 1, 32 * c, lane_x);
+                tb[c] = panel32_load_near(xB, x_pitch, j * 32, S - 1, 128 * q + 32 * c, lane_x);
             }
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 panel32_store(panel, lane_x, ta[c]);
-                xfA[2 * c] = as_bf16x8(panel[panel32_slot(prow_x, g_x)]);
-                xfA[2 * c + 1] = as_bf16x8(panel[panel32_slot(prow_x, 2 + g_x)]);
+                xfA[8 * q + 2 * c] = as_bf16x8(panel[panel32_slot(prow_x, g_x)]);
+                xfA[8 * q + 2 * c + 1] = as_bf16x8(panel[panel32_slot(prow_x, 2 + g_x)]);
             }
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 panel32_store(panel, lane_x, tb[c]);
-                xfB[2 * c] = as_bf16x8(panel[panel32_slot(prow_x, g_x)]);
-                xfB[2 * c + 1] = as_bf16x8(panel[panel32_slot(prow_x, 2 + g_x)]);
+                xfB[8 * q + 2 * c] = as_bf16x8(panel[panel32_slot(prow_x, g_x)]);
+                xfB[8 * q + 2 * c + 1] = as_bf16x8(panel[panel32_slot(prow_x, 2 + g_x)]);
             }
         }
         // ---- four projections of the block, both rows per weight fragment ----
@@ -1992,9 +1996,9 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void persistent_pair_kernel(FusedPa
         f32x16 oA, oB;
         float lA, lB;
         if ((flagsA | flagsB) == 0u) {
-            attend_pair_l2<HAS_NB, false>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
+            attend_pair_l2<HAS_NB, false>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, fair_turn);
         } else {
-            attend_pair_l2<HAS_NB, true>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, wave >> 2);
+            attend_pair_l2<HAS_NB, true>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, fair_turn);
         }
         // some probability overflowed or a whole row underflowed: repeat that row shifted by its true row maxima
         if (__any(!(lA > 1e-30f && lA < 1e30f))) {
@@ -2602,12 +2606,12 @@ size_t persistent_kernel_lds(int C, int NB)
            (size_t)2 * NT * 32 * 4 + 16;
 }
 
-size_t pair_kernel_lds(int NB)
+size_t pair_kernel_lds(int C, int NB)
 {
-    // persistent_pair_kernel (128 channels): the head's four weight matrices, K and V of two batch rows, per wave one
-    // 2 KB panel, two pairs' masks of two rows each, flags
+    // persistent_pair_kernel: the head's four weight matrices, K and V of two batch rows, per wave one 2 KB panel, two
+    // pairs' masks of two rows each, flags
     const int NT = (NB + 1) & ~1;
-    return (size_t)4 * 8 * 64 * 16 + (size_t)2 * NT * 2 * 64 * 16 * 2 + (size_t)NB * 2048 + (size_t)4 * NT * 32 * 4 + 16;
+    return (size_t)4 * (C / 16) * 64 * 16 + (size_t)2 * NT * 2 * 64 * 16 * 2 + (size_t)NB * 2048 + (size_t)4 * NT * 32 * 4 + 16;
 }
 
 bool make_plan(int64_t S, int C, Plan &pl)
@@ -2696,8 +2700,8 @@ bool pair_kernel_applies(const kutacc_hip_attention_args_t &a, const Plan &pl, c
 {
     const int pair_mode = g_pair_mode.load(std::memory_order_relaxed);
     const int64_t C = a.nheads * a.head_size;
-    return pl.persistent && C == 128 && pair_mode != 2 && !fragments_disabled() && opt.ln_gamma == nullptr &&
-           !opt.nb_fragments_ready && pair_kernel_lds(pl.NB) <= (size_t)max_lds_bytes() &&
+    return pl.persistent && (C == 128 || C == 256) && pair_mode != 2 && !fragments_disabled() && opt.ln_gamma == nullptr &&
+           !opt.nb_fragments_ready && pair_kernel_lds((int)C, pl.NB) <= (size_t)max_lds_bytes() &&
            (a.nonbatched_bias == nullptr || fragment_home(a, pl.NB, opt, 2) != nullptr) &&
            (pair_mode == 1 || a.batch >= 16 * (int64_t)persistent_groups((int)a.batch, (int)a.nheads));
 }
@@ -2734,12 +2738,12 @@ int launch_persistent_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
     return kutacc_hip_status(hipGetLastError());
 }
 
-template <bool HAS_NB>
+template <int C, bool HAS_NB>
 int launch_pair_kernel(FusedParams p, const Plan &pl, hipStream_t stream)
 {
-    auto kern = persistent_pair_kernel<HAS_NB>;
+    auto kern = persistent_pair_kernel<C, HAS_NB>;
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
-    const size_t lds_bytes = pair_kernel_lds(pl.NB);
+    const size_t lds_bytes = pair_kernel_lds(C, pl.NB);
     if (const int rc = opt_in_lds(kern, lds_bytes, configured)) {
         return rc;
     }
@@ -2988,7 +2992,8 @@ int gating_attention_fused(const kutacc_hip_attention_args_t &a, hipStream_t str
     {
         kutacc_prof::KernelTimer t(pair_kernel ? "persistent_pair_kernel" : pl.persistent ? "persistent_head_kernel" : "fused_head_kernel",
                                    8.0 * BS * C * C + 4.0 * BS * (double)a.seq_len * C, stream);
-        rc = pair_kernel ? (p.nb != nullptr ? launch_pair_kernel<true>(p, pl, stream) : launch_pair_kernel<false>(p, pl, stream))
+        rc = pair_kernel ? (C == 128 ? (p.nb != nullptr ? launch_pair_kernel<128, true>(p, pl, stream) : launch_pair_kernel<128, false>(p, pl, stream))
+                                     : (p.nb != nullptr ? launch_pair_kernel<256, true>(p, pl, stream) : launch_pair_kernel<256, false>(p, pl, stream)))
              : (C == 128) ? dispatch_head_kernel<128>(p, pl, stream)
                           : dispatch_head_kernel<256>(p, pl, stream);
         if (rc != 0) {

@@ -535,6 +535,29 @@ def test_msa_attention_block_against_the_oracle(torch_cuda, layernorm_placement,
     helpers.check_close(helpers.to_numpy(msa), msa_oracle(c, column), "bf16", f"msa block {n_seq}x{n_res} column={column}")
 
 
+@pytest.mark.parametrize("n_seq,n_res", [(24, 64), (20, 96), (70, 128), (9, 32)])
+def test_msa_row_attention_block_on_the_two_row_kernel(torch_cuda, n_seq, n_res):
+    """Row-wise MSA attention (256 channels, eight heads) with whole key tiles and the two-row kernel forced: the
+    producer of the pair bias writes that kernel's fp32 tiles, and the operator runs no pre-pass."""
+    torch = torch_cuda
+    heads, c_z = 8, 128
+    c = msa_case(1200 + n_seq, n_seq, n_res, heads, c_z)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    msa = dev(c["m"])
+    w = {k: dev(c[k]) for k in ("ln_gamma", "ln_beta", "wq", "wk", "wv", "wg", "bg", "wo", "bo")}
+    pair = {"pair_act": dev(c["z"]), "pair_ln_gamma": dev(c["pair_ln_gamma"]), "pair_ln_beta": dev(c["pair_ln_beta"]),
+            "bias_w": dev(c["bias_w"])}
+    assert capi.set_tuning("row_pairs", "1") == 0
+    try:
+        blk = capi.MsaAttentionBlock(msa, dev(c["mask"]), w, heads, pair)
+        names = profiled_kernels(torch, lambda: blk.run())
+    finally:
+        capi.set_tuning("row_pairs", None)
+    assert "persistent_pair_kernel" in names and "pair_bias_tiles_kernel" not in names and "pair_bias_fragments_kernel" not in names, names
+    helpers.check_close(helpers.to_numpy(msa), msa_oracle(c, False), "bf16", f"msa row block {n_seq}x{n_res}, two-row kernel")
+
+
 def test_layernorm_rows_transposed(torch_cuda):
     torch = torch_cuda
     g = torch.Generator(device="cuda").manual_seed(4)

@@ -228,6 +228,8 @@ PAIR_CASES = [
     # config, batch, seq_len, mask kind: None as drawn, "holes", "tails" (+ one fully masked row), "none"
     (3, 16, 384, None), (3, 17, 384, "holes"), (3, 9, 200, None), (3, 24, 321, "tails"), (3, 3, 33, "holes"),
     (3, 1, 64, None), (3, 40, 96, "tails"), (5, 18, 352, None), (5, 7, 70, "holes"), (3, 1, 1, None), (3, 26, 383, "none"),
+    # 256 channels, eight heads (up to 256 positions)
+    (2, 16, 256, None), (2, 70, 200, "holes"), (2, 33, 129, "tails"), (2, 3, 33, None), (2, 64, 256, "none"), (4, 40, 224, "holes"),
 ]
 
 
