@@ -438,7 +438,8 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *               weight matrices per LDS group where that fits the device; anything else: the planner decides (default)
  *   "fragments" "0": keep the attention kernels off the fragment-major pair bias (general softmax blocks); "1": default
  *   "debug"     "1": one line per fused call on stderr with the plan taken; "0": default
- *   "row_pairs" "0": never the attention kernel that walks two batch rows per step (128 channels, up to 384 positions);
+ *   "row_pairs" "0": never the attention kernel that walks two batch rows per step (128 channels up to 384 positions,
+ *               256 channels up to 256);
  *               "1": wherever it can run; anything else (default): where every workgroup has at least two batch rows
  *   "gemm_tile" "128" / "256": the batched products of kutacc_af2_triangle_multiplication_equation always on 128 x 128
  *               tiles / on 256 x 256 tiles wherever the shape has whole ones; anything else (default): 256 x 256 where
