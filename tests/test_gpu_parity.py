@@ -225,11 +225,13 @@ def row_pairs_forced():
 
 
 PAIR_CASES = [
-    # config, batch, seq_len, mask kind: None as drawn, "holes", "tails" (+ one fully masked row), "none"
+    # config, batch, seq_len, mask kind: None as drawn, "holes", "tails" (+ one fully masked row), "none", "soft" (a finite
+    # additive bias on every key: the kernel adds it as two bf16 terms)
     (3, 16, 384, None), (3, 17, 384, "holes"), (3, 9, 200, None), (3, 24, 321, "tails"), (3, 3, 33, "holes"),
     (3, 1, 64, None), (3, 40, 96, "tails"), (5, 18, 352, None), (5, 7, 70, "holes"), (3, 1, 1, None), (3, 26, 383, "none"),
     # 256 channels, eight heads (up to 256 positions)
     (2, 16, 256, None), (2, 70, 200, "holes"), (2, 33, 129, "tails"), (2, 3, 33, None), (2, 64, 256, "none"), (4, 40, 224, "holes"),
+    (3, 20, 160, "soft"), (2, 18, 96, "soft"),
 ]
 
 
@@ -248,6 +250,9 @@ def test_two_row_kernel_matches_the_oracle(torch_cuda, row_pairs_forced, config,
         w.bias[batch - 1, :] = -1e9
     elif mask == "none":
         w.bias[:] = 0.0
+    elif mask == "soft":
+        w.bias[:] = round_to_bf16((rng.standard_normal((batch, seq)) * 3.0).astype(np.float32))
+        w.bias[0, : seq // 2] = -np.inf
     if not pair_bias:
         w.nb = None
     ten, scratch = helpers.to_device(w)
