@@ -1514,7 +1514,7 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 }
 
 // ------------------------------------------------------------------------------------------------
-// persistent_pair_kernel: persistent_head_kernel walking its batch rows two at a time (128 channels, log2 units).
+// persistent_pair_kernel: persistent_head_kernel walking its batch rows two at a time (128 or 256 channels, log2 units).
 // The pair bias of a (head, query block, key tile) is the same for every batch row, so a wave that attends the same query
 // block of two rows at once fetches it once -- as fp32, in accumulator order, straight into the C operand of the logits
 // MFMAs of both rows (pair_bias_tiles_kernel writes that copy).  Per row and key tile this moves the same bytes as the
@@ -1522,9 +1522,11 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_head_kernel(F
 // per tile); the two rows' instruction streams are independent, which gives the scheduler what a fourth wave per SIMD
 // would; and every weight fragment read from LDS in the projection phase serves two rows.
 // LDS, 16-byte units: W[4][CK][64]  K[2 rows][NT][2][64]  V[2 rows][NT][2][64]  panel[NB waves][128];
-// then floats mask[2 pairs in flight][2 rows][NT*32] and four uint32 of tile flags.  At 384 positions that is
-// 32 + 96 + 24 + 6 KB: the panels are half the size of persistent_head_kernel's (32 rows x 32 channels); during the
-// attention a wave's panel holds the sigmoid of the first row's gate, the second row's waits in eight registers.
+// then mask words mask[2 pairs in flight][2 rows][NT*32] (a key's mask bias as two bf16: the rows' masks enter the logits
+// by one more MFMA per tile, see stage_mask_words) and four uint32 of tile flags.  At 128 channels and 384 positions that
+// is 32 + 96 + 24 + 6 KB, at 256 channels and 256 positions 64 + 64 + 16 + 4 KB: the panels are half the size of
+// persistent_head_kernel's (32 rows x 32 channels); during the attention a wave's panel holds the sigmoid of the first
+// row's gate, the second row's waits in eight registers.
 // ------------------------------------------------------------------------------------------------
 
 // Wave-private 2 KB staging panel: 32 rows x 64 bytes in 16-byte slots, filled with two coalesced loads (lane l -> row
