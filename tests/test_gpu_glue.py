@@ -383,7 +383,7 @@ def test_triangle_multiplication_block_seeded_sweep(torch_cuda, index, n):
 
 
 @pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
-@pytest.mark.parametrize("n", [384, 512])
+@pytest.mark.parametrize("n", [384, 512, 768])  # 768: the equation on the 256 x 256 tiles
 def test_triangle_multiplication_block_full_size(torch_cuda, incoming, n):
     """384 residues, 128 channels, the real shape, and 512, from where on the gated projections run on the streaming
     kernel (both sides in one pass).  The oracle follows a sample of output positions (i, j) through the

@@ -163,13 +163,14 @@ def test_gemm_large_tiles(torch_cuda, gemm_tile, shape, mmajor):
     assert np.array_equal(got, small)
 
 
-def test_equation_at_768_residues_takes_the_large_tiles(torch_cuda):
-    """128 channels of 768 x 768: nine large tiles per channel, more than four per CU, which is where the default rule
-    switches to them.  Sampled channels against the oracle; the incoming form equals the outgoing one on transposed
-    operands bit for bit."""
+@pytest.mark.parametrize("n", [768, 1024])
+def test_equation_at_768_residues_and_more_takes_the_large_tiles(torch_cuda, n):
+    """128 channels of 768 x 768 (nine large tiles per channel, more than four per CU, which is where the default rule
+    switches to them) and of 1024 x 1024 (eight tiles per workgroup).  Sampled channels against the oracle; the incoming
+    form equals the outgoing one on transposed operands bit for bit."""
     from oracle import oracle
     torch = torch_cuda
-    n, c_i = 768, 128
+    c_i = 128
     g = torch.Generator(device="cuda").manual_seed(77)
     left = (torch.randn(c_i, n, n, device="cuda", generator=g)).to(torch.bfloat16)
     right = (torch.randn(c_i, n, n, device="cuda", generator=g) * n ** -0.5).to(torch.bfloat16)
