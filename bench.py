@@ -218,7 +218,9 @@ def pair_stack_rates(config, reps=20):
     at this configuration's pair tensor: n = S residues, 128 pair channels, 128 projected channels, hidden layer 512.
     Called through the handle-based entry points, asynchronously on torch's stream, hipEvent-bracketed.  Per step:
     microseconds, algorithmic TFLOP/s (2 flops per multiply-add of the products) and algorithmic GB/s (every operand
-    and result of the step once)."""
+    and result of the step once), which of the two rooflines bounds the step (the one whose time at peak is the longer:
+    the equation at 384 residues has 128 flop per byte against the card's 312 and is HBM-bound; from 1024 on it is not)
+    and the fraction of that roofline reached."""
     import torch
     from kutacc_amd import capi
     from kutacc_amd.workloads import CONFIGS
@@ -250,7 +252,10 @@ def pair_stack_rates(config, reps=20):
     res = {"shape": f"pair activation [{n},{n},{c_o}] bf16, c_i={c_i}, transition hidden {hid}"}
 
     def report(name, t, flops, nbytes):
-        res[name] = {"us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1), "GB/s": round(nbytes / t / 1e9, 1)}
+        # the roofline that bounds the step is the one whose time at peak is the longer; frac = that time / measured
+        t_mfma, t_hbm = flops / (MFMA_BF16_PEAK_TFLOPS * 1e12), nbytes / (HBM_PEAK_GBS * 1e9)
+        res[name] = {"us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1), "GB/s": round(nbytes / t / 1e9, 1),
+                     "bound": "mfma" if t_mfma > t_hbm else "hbm", "frac": round(max(t_mfma, t_hbm) / t, 3)}
 
     # transition
     mid = torch.empty(rows, hid, device="cuda", dtype=torch.bfloat16)

@@ -27,6 +27,7 @@
 #include <atomic>
 #include <cstring>
 #include <type_traits>
+#include <utility>
 
 #include "launch_internal.h"
 #include "mfma_tiles.h"
@@ -349,10 +350,6 @@ constexpr int SUB_SLOTS = 1024;
 constexpr int BIG_STAGE_SLOTS = 4 * SUB_SLOTS;
 constexpr size_t BIG_GEMM_LDS = 2 * BIG_STAGE_SLOTS * 16;
 
-struct SubTileRegs {
-    PanelRegs q0, q1, q2, q3;
-};
-
 // The registers, or zeros, by a mask: a conditional assignment becomes a branch, and a branch inside the k-loop splits
 // the basic block whose instruction order the loop depends on.
 __device__ __forceinline__ PanelRegs keep_if(const PanelRegs &p, bool ok)
@@ -366,13 +363,58 @@ struct TilePlace {
     int batch, m0, n0;
 };
 
+// The order of one quarter (k-step of 16) of pair_gemm_big_kernel's k-loop, as scheduling-group barriers, whose sizes
+// must be integer constants: NMFMA MFMAs in pairs, with this quarter's LDS reads, global loads or LDS stores dealt
+// evenly between them.
+template <int COUNT, int SLOT, int SLOTS>
+constexpr int slot_share() { return (COUNT * (SLOT + 1)) / SLOTS - (COUNT * SLOT) / SLOTS; }
+
+template <int NMFMA, int READS, int LOADS, int STORES, int SLOT>
+__device__ __forceinline__ void quarter_slot()
+{
+    constexpr int SLOTS = (NMFMA + 1) / 2;
+    if constexpr (slot_share<READS, SLOT, SLOTS>() > 0) {
+        __builtin_amdgcn_sched_group_barrier(0x100, slot_share<READS, SLOT, SLOTS>(), 0); // LDS reads
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+    if constexpr (slot_share<LOADS, SLOT, SLOTS>() > 0) {
+        __builtin_amdgcn_sched_group_barrier(0x020, slot_share<LOADS, SLOT, SLOTS>(), 0); // global loads
+    }
+    if constexpr (slot_share<STORES, SLOT, SLOTS>() > 0) {
+        __builtin_amdgcn_sched_group_barrier(0x200, slot_share<STORES, SLOT, SLOTS>(), 0); // LDS stores
+    }
+    if constexpr (2 * SLOT + 1 < NMFMA) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+}
+
+template <int NMFMA, int READS, int LOADS, int STORES, int... SLOT>
+__device__ __forceinline__ void quarter_order(std::integer_sequence<int, SLOT...>)
+{
+    (quarter_slot<NMFMA, READS, LOADS, STORES, SLOT>(), ...);
+}
+
+template <int NMFMA, int READS, int LOADS, int STORES>
+__device__ __forceinline__ void quarter_order()
+{
+    quarter_order<NMFMA, READS, LOADS, STORES>(std::make_integer_sequence<int, (NMFMA + 1) / 2>{});
+}
+
 // Persistent: one workgroup per CU walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... and its operand pipeline runs
 // on across the tile boundary -- the last two k-steps of a tile request the first two of the next, and the store of
-// the finished tile goes out under the next tile's MFMAs.  With one workgroup per CU nothing else would cover a
-// tile's first loads (about 8000 clocks of a 70000-clock tile at k = 1024) or the acknowledgement of its stores.
-template <bool MMAJOR>
+// the finished tile goes out under the next tile's MFMAs.
+//
+// BW = 4: 256 x 256 per workgroup (128 x 128 per wave).  BW = 3: 192 x 192 (96 x 96 per wave), for sides that are
+// multiples of 192 but not of 256 (384 residues: four tiles per channel, two per CU, where the 128 x 128 tiles leave
+// the chip one eighth of a round short).  A stage keeps its layout of four 16 KB sub-tiles; with BW = 3 the second
+// sub-tile of each operand is half used.  The operand loads of a step come in pieces of a quarter sub-tile (k-major: 32
+// rows x 64 k; m-major: 64 m x 32 k), 4 BW per step, BW per wave.
+template <bool MMAJOR, int BW>
 __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams p, const int64_t total_tiles)
 {
+    constexpr int TILE_SIDE = 64 * BW; // rows of C per workgroup, and columns
+    constexpr int WAVE_SIDE = 32 * BW;
+    constexpr int NMFMA = BW * BW;     // per wave and k-step of 16
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, g = lane >> 5;
@@ -396,57 +438,80 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams 
         } else {
             nt = t % p.NT, mt = t / p.NT;
         }
-        return TilePlace{batch, mt * BIG_TILE, nt * BIG_TILE};
+        return TilePlace{batch, mt * TILE_SIDE, nt * TILE_SIDE};
     };
 
-    // The sub-tile this wave stages: rows row0.. of A (waves 0, 1) or of B (waves 2, 3).  M, N and K are whole tiles
-    // and steps here, so an address is a wave-uniform pointer (tile, k-step, row block: scalar arithmetic) plus one
-    // 32-bit byte offset per lane that never changes; the loads cost no vector instructions beyond themselves, which
-    // matters with one wave per SIMD, where every vector instruction between two MFMAs comes out of the matrix pipe's time.
-    const bool mine_a = wave < 2;
-    const int64_t ld = mine_a ? (MMAJOR ? p.a_sk : p.a_sm) : (MMAJOR ? p.b_sk : p.b_sn);
-    const uint32_t lane_bytes = (uint32_t)(((MMAJOR ? mm_row(lane >> 3) : (lane >> 3)) * ld + (lane & 7) * 8) * 2);
-    using Source = const char *; // first element of the sub-tile's rows at k = 0
-    auto source = [&](const TilePlace &tp) -> Source {
-        const bf16_t *base = mine_a ? p.a + (int64_t)tp.batch * p.a_sb : p.b + (int64_t)tp.batch * p.b_sb;
-        const int row0 = (mine_a ? tp.m0 : tp.n0) + 128 * (wave & 1);
-        return reinterpret_cast<const char *>(MMAJOR ? base + row0 : base + (int64_t)row0 * ld);
+    // The pieces this wave stages: piece e = wave * BW + i of the step's 4 BW; pieces 0 .. 2 BW - 1 belong to A, the rest
+    // to B.  M, N and K are whole tiles and steps here, so an address is a wave-uniform pointer (tile, k-step, piece:
+    // scalar arithmetic) plus one 32-bit byte offset per lane that never changes; the loads cost no vector instructions
+    // beyond themselves, which matters with one wave per SIMD, where every vector instruction between two MFMAs comes out
+    // of the matrix pipe's time.
+    const int64_t lda = MMAJOR ? p.a_sk : p.a_sm, ldb = MMAJOR ? p.b_sk : p.b_sn;
+    auto piece_is_a = [&](int i) { return wave * BW + i < 2 * BW; };
+    auto piece_index = [&](int i) { const int e = wave * BW + i; return e < 2 * BW ? e : e - 2 * BW; }; // within its operand
+    uint32_t lane_bytes[BW];
+#pragma unroll
+    for (int i = 0; i < BW; ++i) {
+        const int64_t ld = piece_is_a(i) ? lda : ldb;
+        lane_bytes[i] = (uint32_t)(((MMAJOR ? mm_row(lane >> 3) : (lane >> 3)) * ld + (lane & 7) * 8) * 2);
+    }
+    struct Sources {
+        const char *a, *b; // element (row 0 of the tile, k = 0) of each operand
     };
-    // quarter i of the wave's sub-tile of the k-step at k0; a step past K (an odd number of steps is rounded up) reads
-    // step 0 instead and is cleared on its way to the LDS
-    auto fetch_quarter = [&](Source src, int i, int k0) -> PanelRegs {
+    auto sources = [&](const TilePlace &tp) -> Sources {
+        const bf16_t *a = p.a + (int64_t)tp.batch * p.a_sb, *b = p.b + (int64_t)tp.batch * p.b_sb;
+        return Sources{reinterpret_cast<const char *>(MMAJOR ? a + tp.m0 : a + (int64_t)tp.m0 * lda),
+                       reinterpret_cast<const char *>(MMAJOR ? b + tp.n0 : b + (int64_t)tp.n0 * ldb)};
+    };
+    // piece i of this wave for the k-step at k0; a step past K (an odd number of steps is rounded up) reads step 0
+    // instead and is cleared on its way to the LDS
+    auto fetch_piece = [&](const Sources &src, int i, int k0) -> PanelRegs {
         const int k0c = k0 < p.K ? k0 : 0;
-        // k-major: rows 32 i + 8 e + (lane >> 3), 64 k from k0c; m-major: 64 m from 64 (i & 1), k = k0c + 32 (i >> 1) + 8 e + ...
-        const char *q = MMAJOR ? src + ((int64_t)(k0c + 32 * (i >> 1)) * ld + 64 * (i & 1)) * 2 : src + ((int64_t)32 * i * ld + k0c) * 2;
+        const bool is_a = piece_is_a(i);
+        const int64_t ld = is_a ? lda : ldb;
+        const int e = piece_index(i);
+        // k-major: rows 32 e .. + 31, 64 k from k0c; m-major: 64 m from 64 (e / 2), k = k0c + 32 (e % 2) .. + 31
+        const char *base = is_a ? src.a : src.b;
+        const char *q = MMAJOR ? base + ((int64_t)(k0c + 32 * (e & 1)) * ld + 64 * (e >> 1)) * 2 : base + ((int64_t)32 * e * ld + k0c) * 2;
         PanelRegs f;
-        f.r0 = *reinterpret_cast<const uint4 *>(q + lane_bytes);
-        f.r1 = *reinterpret_cast<const uint4 *>(q + 16 * ld + lane_bytes);
-        f.r2 = *reinterpret_cast<const uint4 *>(q + 32 * ld + lane_bytes);
-        f.r3 = *reinterpret_cast<const uint4 *>(q + 48 * ld + lane_bytes);
+        f.r0 = *reinterpret_cast<const uint4 *>(q + lane_bytes[i]);
+        f.r1 = *reinterpret_cast<const uint4 *>(q + 16 * ld + lane_bytes[i]);
+        f.r2 = *reinterpret_cast<const uint4 *>(q + 32 * ld + lane_bytes[i]);
+        f.r3 = *reinterpret_cast<const uint4 *>(q + 48 * ld + lane_bytes[i]);
         return f;
     };
-    auto fetch = [&](Source src, int k0) -> SubTileRegs {
-        return SubTileRegs{fetch_quarter(src, 0, k0), fetch_quarter(src, 1, k0), fetch_quarter(src, 2, k0), fetch_quarter(src, 3, k0)};
-    };
-    // what fetch(.., k0) brought, zeros for a step past K, into the wave's sub-tile of a stage
-    auto park = [&](uint4 *stage, const SubTileRegs &f, int k0) {
-        uint4 *sub = stage + wave * SUB_SLOTS;
-        const bool ok = k0 < p.K;
-        const PanelRegs q0 = keep_if(f.q0, ok), q1 = keep_if(f.q1, ok), q2 = keep_if(f.q2, ok), q3 = keep_if(f.q3, ok);
+    // what fetch_piece(.., i, k0) brought, zeros for a step past K, into its place in a stage: operand o's rows live in
+    // sub-tiles 2 o and 2 o + 1, 128 rows each
+    auto park_piece = [&](uint4 *stage, const PanelRegs &f, int i, int k0) {
+        const PanelRegs q = keep_if(f, k0 < p.K);
+        const int e = piece_index(i);
+        uint4 *operand = stage + (piece_is_a(i) ? 0 : 2 * SUB_SLOTS);
         if constexpr (MMAJOR) {
-            store_mmajor(sub, 0, 0, lane, q0);
-            store_mmajor(sub, 64, 0, lane, q1);
-            store_mmajor(sub, 0, 32, lane, q2);
-            store_mmajor(sub, 64, 32, lane, q3);
+            const int mchunk = e >> 1; // 64 m each
+            store_mmajor(operand + (mchunk >> 1) * SUB_SLOTS, 64 * (mchunk & 1), 32 * (e & 1), lane, q);
         } else {
-            panel_store(sub, lane, q0);
-            panel_store(sub + 256, lane, q1);
-            panel_store(sub + 512, lane, q2);
-            panel_store(sub + 768, lane, q3);
+            panel_store(operand + (e >> 2) * SUB_SLOTS + (e & 3) * 256, lane, q);
+        }
+    };
+    struct Pieces {
+        PanelRegs q[BW];
+    };
+    auto fetch = [&](const Sources &src, int k0) -> Pieces {
+        Pieces f;
+#pragma unroll
+        for (int i = 0; i < BW; ++i) {
+            f.q[i] = fetch_piece(src, i, k0);
+        }
+        return f;
+    };
+    auto park = [&](uint4 *stage, const Pieces &f, int k0) {
+#pragma unroll
+        for (int i = 0; i < BW; ++i) {
+            park_piece(stage, f.q[i], i, k0);
         }
     };
 
-    f32x16 acc[4][4];
+    f32x16 acc[BW][BW];
     int mm_off[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -455,76 +520,70 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams 
 
     // Fragments of k-step s + 1 are requested while the MFMAs of step s issue (two register sets), the next stage's
     // stores go behind the MFMAs of the last step, and the scheduler is told the interleaving: left to itself it
-    // puts every LDS read directly in front of the four MFMAs that need it, and with one wave per SIMD nothing else
+    // puts every LDS read directly in front of the MFMAs that need it, and with one wave per SIMD nothing else
     // covers that latency.
-    bf16x8 af[2][4], bq[2][4];
+    bf16x8 af[2][BW], bq[2][BW];
     auto fragments = [&](int set, const uint4 *stage, int s) {
-        const uint4 *sa = stage + wm * SUB_SLOTS;
-        const uint4 *sb = stage + (2 + wn) * SUB_SLOTS;
         const int slot = panel_slot(r, 2 * s + g);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < BW; ++i) {
+            const int ba = wm * BW + i, bb = wn * BW + i; // 32-row blocks of the operands' 192 or 256 rows
+            const uint4 *sa = stage + (ba >> 2) * SUB_SLOTS, *sb = stage + (2 + (bb >> 2)) * SUB_SLOTS;
             if constexpr (MMAJOR) {
-                af[set][i] = mm_fragment((const lds_char *)sa, mm_off[i], s);
-                bq[set][i] = mm_fragment((const lds_char *)sb, mm_off[i], s);
+                af[set][i] = mm_fragment((const lds_char *)sa, mm_off[ba & 3], s);
+                bq[set][i] = mm_fragment((const lds_char *)sb, mm_off[bb & 3], s);
             } else {
-                af[set][i] = as_bf16x8(sa[i * 256 + slot]);
-                bq[set][i] = as_bf16x8(sb[i * 256 + slot]);
+                af[set][i] = as_bf16x8(sa[(ba & 3) * 256 + slot]);
+                bq[set][i] = as_bf16x8(sb[(bb & 3) * 256 + slot]);
             }
         }
     };
-    // The fragments arrive in the order a0 b0 a1 b1 a2 b2 a3 b3, the last ones shortly before the quarter that uses
-    // them begins: the MFMAs go in the order in which their operands arrive, the four that need b3 last.
+    // The fragments arrive in the order a0 b0 a1 b1 ..., the last ones shortly before the quarter that uses them
+    // begins: the MFMAs go in the order in which their operands arrive, those that need the last fragment last.
     auto multiply = [&](int set) {
-        constexpr int order[16][2] = {{0, 0}, {1, 0}, {0, 1}, {1, 1}, {2, 0}, {2, 1}, {0, 2}, {1, 2},
-                                      {2, 2}, {3, 0}, {3, 1}, {3, 2}, {0, 3}, {1, 3}, {2, 3}, {3, 3}};
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int i = order[e][0], j = order[e][1];
-            acc[i][j] = mfma(bq[set][j], af[set][i], acc[i][j]);
+        for (int m = 0; m < BW; ++m) { // all pairs (i, j) with max(i, j) = m
+#pragma unroll
+            for (int j = 0; j < m; ++j) {
+                acc[m][j] = mfma(bq[set][j], af[set][m], acc[m][j]);
+            }
+#pragma unroll
+            for (int i = 0; i <= m; ++i) {
+                acc[i][m] = mfma(bq[set][m], af[set][i], acc[i][m]);
+            }
         }
     };
-    constexpr int READS = MMAJOR ? 16 : 8; // LDS read instructions per k-step of 16
+    constexpr int READS = (MMAJOR ? 4 : 2) * BW; // LDS read instructions per k-step of 16
     // One k-step of 64 from `stage`.  Operands travel two steps ahead of the MFMAs: the step requests the tiles of the
     // step after next (of `src`, at k_fetch) into `fill` and stores `ahead`, requested a step earlier for k_park, into
-    // the other stage.  The sixteen loads are spread over the MFMAs of the first three quarters: issued together they
-    // hold the wave, and with it the matrix pipe, for as long as the CU's memory path takes to accept 64 KB (1500 to
-    // 2400 clocks of a step of 2048 MFMA clocks, measured).
-    auto k_step = [&](const uint4 *stage, uint4 *other, Source src, int k_fetch, int k_park, const SubTileRegs &ahead,
-                      SubTileRegs &fill) {
+    // the other stage.  The loads are spread over the MFMAs of the first three quarters: issued together they hold the
+    // wave, and with it the matrix pipe, for as long as the CU's memory path takes to accept 64 KB (1500 to 2400 clocks of
+    // a step of 2048 MFMA clocks, measured).
+    auto k_step = [&](const uint4 *stage, uint4 *other, const Sources &src, int k_fetch, int k_park, const Pieces &ahead, Pieces &fill) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             if (s < 3) {
                 fragments((s + 1) & 1, stage, s + 1);
             }
+            // BW = 4: pieces 0 and 1, then 2, then 3; BW = 3: one piece per quarter
             if (s == 0) {
-                fill.q0 = fetch_quarter(src, 0, k_fetch);
-                fill.q1 = fetch_quarter(src, 1, k_fetch);
-            } else if (s == 1) {
-                fill.q2 = fetch_quarter(src, 2, k_fetch);
-            } else if (s == 2) {
-                fill.q3 = fetch_quarter(src, 3, k_fetch);
+                fill.q[0] = fetch_piece(src, 0, k_fetch);
+                if constexpr (BW == 4) {
+                    fill.q[1] = fetch_piece(src, 1, k_fetch);
+                }
+            } else if (s < 3) {
+                fill.q[BW - 3 + s] = fetch_piece(src, BW - 3 + s, k_fetch);
             }
             multiply(s & 1);
             if (s == 3) {
                 park(other, ahead, k_park); // every wave left that stage before the barrier that ended the previous step
             }
-            if (s < 3) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, READS / 8, 0); // LDS reads
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);         // MFMA
-                    if (s == 0 || (e & 1)) {
-                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // a global load: eight, four and four per quarter
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                }
+            if (s == 0) {
+                quarter_order<NMFMA, READS, 4 * (BW - 2), 0>();
+            } else if (s < 3) {
+                quarter_order<NMFMA, READS, 4, 0>();
             } else {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // LDS write
-                }
+                quarter_order<NMFMA, 0, 0, 4 * BW>();
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -532,45 +591,48 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams 
         fragments(0, other, 0);
     };
 
-    // Steps go in pairs with one body, so that the 256 accumulators and the two register sets keep their places; an odd
+    // Steps go in pairs with one body, so that the accumulators and the two register sets keep their places; an odd
     // number of steps ends with a step whose operands, past K, were cleared on their way to the LDS.
     const int KT2 = ((p.K + KSTEP - 1) / KSTEP + 1) & ~1;
     uint4 *stage0 = lds, *stage1 = lds + BIG_STAGE_SLOTS;
     int64_t v = blockIdx.x;
     TilePlace cur = place(v);
-    Source cur_src = source(cur);
-    SubTileRegs even, odd; // tiles of an even / odd k-step on their way to the LDS
+    Sources cur_src = sources(cur);
+    Pieces even, odd; // tiles of an even / odd k-step on their way to the LDS
     even = fetch(cur_src, 0);
     odd = fetch(cur_src, KSTEP);
     park(stage0, even, 0);
     __syncthreads();
     fragments(0, stage0, 0);
     for (; v < total_tiles; v += gridDim.x) {
-        const Source next_src = source(place(v + gridDim.x));
+        const Sources next_src = sources(place(v + gridDim.x));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < BW; ++i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < BW; ++j) {
                 acc[i][j] = zero16();
             }
         }
         for (int kt = 0; kt < KT2; kt += 2) {
             const bool last = kt + 2 == KT2; // the requests go on to the next tile
-            const Source src = last ? next_src : cur_src;
+            const Sources src = last ? next_src : cur_src;
             k_step(stage0, stage1, src, last ? 0 : (kt + 2) * KSTEP, (kt + 1) * KSTEP, odd, even);
             k_step(stage1, stage0, src, last ? KSTEP : (kt + 3) * KSTEP, last ? 0 : (kt + 2) * KSTEP, even, odd);
         }
 
-        // Each wave rounds its 128 x 128 block to bf16 through a 32-row strip in its own sub-tile of the stage the last
-        // step read (the other one already holds the next tile's first step; a wave's LDS accesses complete in order, so
-        // the strip needs no barrier, and the wave itself is the next to store into that sub-tile) and writes whole
-        // 256-byte pieces of rows.
+        // Each wave rounds its block to bf16 through a 32-row strip in the stage the last step read (the other one
+        // already holds the next tile's first step; a wave's LDS accesses complete in order, so the strip needs no
+        // barrier) and writes whole pieces of rows.  The strips lie in sub-tile `wave` of that stage.  With BW = 4 that
+        // sub-tile is also the only place this wave's next stores go, so a wave that is ahead cannot reach a slower one's
+        // strip; with BW = 3 the pieces of a wave spread over sub-tiles, and a barrier keeps the next step's stores behind
+        // every wave's strip.
         bf16_t *ct = reinterpret_cast<bf16_t *>(stage1 + wave * SUB_SLOTS);
         bf16_t *c = p.c + (int64_t)cur.batch * p.c_sb;
+        constexpr int CHUNKS = WAVE_SIDE / 8; // 16-byte pieces per row of the wave's block
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < BW; ++i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < BW; ++j) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     bf16x4 ov;
@@ -583,13 +645,16 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams 
             }
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
+            for (int e = 0; e < (32 * CHUNKS) / 64; ++e) {
                 const int piece = lane + 64 * e;
-                const int row = piece >> 4, chunk = piece & 15;
-                const int64_t gm = cur.m0 + 128 * wm + 32 * i + row, gn = cur.n0 + 128 * wn + chunk * 8;
+                const int row = piece / CHUNKS, chunk = piece % CHUNKS;
+                const int64_t gm = cur.m0 + WAVE_SIDE * wm + 32 * i + row, gn = cur.n0 + WAVE_SIDE * wn + chunk * 8;
                 *reinterpret_cast<uint4 *>(c + gm * p.c_sm + gn) = *reinterpret_cast<const uint4 *>(ct + row * CT_LD + chunk * 8);
             }
             __builtin_amdgcn_wave_barrier();
+        }
+        if constexpr (BW != 4) {
+            __syncthreads();
         }
         cur = place(v + gridDim.x);
         cur_src = next_src;
@@ -1167,11 +1232,11 @@ hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
 }
 constexpr int64_t GATED_STREAMING_MIN_POSITIONS = 512 * 512;
 
-template <bool MM>
+template <bool MM, int BW>
 hipError_t launch_big_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
 {
     static size_t configured[KUTACC_DEVICE_SLOTS] = {};
-    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&pair_gemm_big_kernel<MM>), BIG_GEMM_LDS, configured)) {
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&pair_gemm_big_kernel<MM, BW>), BIG_GEMM_LDS, configured)) {
         return e;
     }
     int device = 0, cus = 0;
@@ -1183,13 +1248,14 @@ hipError_t launch_big_tiles(const GemmParams &p, int64_t blocks, hipStream_t str
     }
     // one workgroup per CU; a multiple of 8, so that a workgroup's tiles stay on its XCD's share of the walk
     const int64_t grid = blocks < cus ? blocks : (cus >= 8 ? cus / 8 * 8 : cus);
-    pair_gemm_big_kernel<MM><<<dim3((unsigned)grid), 256, BIG_GEMM_LDS, stream>>>(p, blocks);
+    pair_gemm_big_kernel<MM, BW><<<dim3((unsigned)grid), 256, BIG_GEMM_LDS, stream>>>(p, blocks);
     return hipGetLastError();
 }
 
 // 0: the 256 x 256 tiles where every CU gets at least four of them (measured at 128 channels: 0.36 of the MFMA peak
-// against 0.31 at 1024 x 1024, 0.31 against 0.29 at 768 x 768, no gain at 512 x 512), 1: wherever the shape allows
-// them, 2: never
+// against 0.31 at 1024 x 1024, 0.31 against 0.29 at 768 x 768, no gain at 512 x 512), else the 192 x 192 tiles where
+// every CU gets at least two (384 x 384: 24.6 us against 25.8-26.6; 576 x 576: 74-78 against 79-86; 192 x 192 loses),
+// else the 128 x 128 tiles; 1: 256 x 256 wherever the shape has whole ones; 3: 192 x 192 wherever it has; 2: neither
 std::atomic<int> g_big_tile_mode{0};
 constexpr int64_t BIG_TILE_MIN_WORKGROUPS = 1024;
 
@@ -1304,7 +1370,7 @@ int transition_block_fused(void *act, const float *ln_gamma, const float *ln_bet
 int pair_gemm_tuning(const char *name, const char *value)
 {
     if (!std::strcmp(name, "gemm_tile")) { // "256": wherever the shape allows the large tiles, "128": never, anything else: the default rule
-        g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : 0));
+        g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : (value && !std::strcmp(value, "192") ? 3 : 0)));
         return 0;
     }
     return KUTACC_HIP_EINVAL;
@@ -1401,13 +1467,26 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
         return kutacc_hip_status(hipGetLastError());
     }
     // (whole tiles and k-steps, and lane offsets within 32 bits: the kernel's addresses are a uniform pointer plus a lane constant)
-    if (!gated && am == bm && g.bias_axis == 0 && !g.relu && g.m % BIG_TILE == 0 && g.n % BIG_TILE == 0 && g.k % KSTEP == 0 &&
-        (am ? g.a_stride_k : g.a_stride_m) < (1 << 26) && (bm ? g.b_stride_k : g.b_stride_n) < (1 << 26) && g_big_tile_mode.load() != 2) {
-        p.MT = (int)(g.m / BIG_TILE), p.NT = (int)(g.n / BIG_TILE);
-        const int64_t big_blocks = (int64_t)p.MT * p.NT * p.batches;
-        if (big_blocks <= INT32_MAX && (big_blocks >= BIG_TILE_MIN_WORKGROUPS || g_big_tile_mode.load() == 1)) {
-            kutacc_prof::KernelTimer t(am ? "pair_gemm_big_kernel<m-major>" : "pair_gemm_big_kernel", flops, stream);
-            return kutacc_hip_status(am ? launch_big_tiles<true>(p, big_blocks, stream) : launch_big_tiles<false>(p, big_blocks, stream));
+    const int tile_mode = g_big_tile_mode.load();
+    if (!gated && am == bm && g.bias_axis == 0 && !g.relu && g.k % KSTEP == 0 && (am ? g.a_stride_k : g.a_stride_m) < (1 << 26) &&
+        (bm ? g.b_stride_k : g.b_stride_n) < (1 << 26) && tile_mode != 2) {
+        // 256 x 256 tiles where every CU gets at least four; else 192 x 192 where every CU gets at least two
+        for (const int side : {BIG_TILE, 192}) {
+            const bool forced = tile_mode == (side == BIG_TILE ? 1 : 3);
+            if (g.m % side != 0 || g.n % side != 0 || (!forced && tile_mode != 0)) {
+                continue;
+            }
+            p.MT = (int)(g.m / side), p.NT = (int)(g.n / side);
+            const int64_t big_blocks = (int64_t)p.MT * p.NT * p.batches;
+            const int64_t enough = side == BIG_TILE ? BIG_TILE_MIN_WORKGROUPS : BIG_TILE_MIN_WORKGROUPS / 2;
+            if (big_blocks <= INT32_MAX && (big_blocks >= enough || forced)) {
+                kutacc_prof::KernelTimer t(side == BIG_TILE ? (am ? "pair_gemm_big_kernel<m-major>" : "pair_gemm_big_kernel")
+                                                            : (am ? "pair_gemm_big_kernel<m-major, 192>" : "pair_gemm_big_kernel<192>"),
+                                           flops, stream);
+                const hipError_t e = side == BIG_TILE ? (am ? launch_big_tiles<true, 4>(p, big_blocks, stream) : launch_big_tiles<false, 4>(p, big_blocks, stream))
+                                                      : (am ? launch_big_tiles<true, 3>(p, big_blocks, stream) : launch_big_tiles<false, 3>(p, big_blocks, stream));
+                return kutacc_hip_status(e);
+            }
         }
     }
     p.MT = (int)((g.m + (gated ? 64 : 128) - 1) / (gated ? 64 : 128));

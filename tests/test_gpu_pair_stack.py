@@ -143,16 +143,19 @@ def first_profiled_kernel(torch, fn):
 
 
 @pytest.mark.parametrize("mmajor", [False, True], ids=["k-major", "m-major"])
-@pytest.mark.parametrize("shape", [(2, 256, 256, 64), (1, 512, 256, 192), (3, 256, 768, 320), (9, 256, 256, 128), (300, 256, 256, 64)])
-def test_gemm_large_tiles(torch_cuda, gemm_tile, shape, mmajor):
-    """The 256 x 256 tiles (128 x 128 per wave) against the float64 product and, bit for bit, against the 128 x 128
-    tiles, which add the same products in the same order: one and several k-steps, an odd number of them (the kernel
-    takes them in pairs), several tiles per batch, and more tiles than the chip has CUs (a workgroup then walks several,
-    its operand pipeline running across the tile boundary)."""
-    nb, M, N, K = shape
+@pytest.mark.parametrize("side", [256, 192])
+@pytest.mark.parametrize("units", [(2, 1, 1, 64), (1, 2, 1, 192), (3, 1, 3, 320), (9, 1, 1, 128), (300, 1, 1, 64)])
+def test_gemm_large_tiles(torch_cuda, gemm_tile, units, side, mmajor):
+    """The 256 x 256 tiles (128 x 128 per wave) and the 192 x 192 ones (96 x 96 per wave) against the float64 product
+    and, bit for bit, against the 128 x 128 tiles, which add the same products in the same order: one and several
+    k-steps, an odd number of them (the kernel takes them in pairs), several tiles per batch, and more tiles than the
+    chip has CUs (a workgroup then walks several, its operand pipeline running across the tile boundary)."""
+    nb, mt, nt, K = units
+    M, N = mt * side, nt * side
+    shape = (nb, M, N, K)
     rng = np.random.Generator(np.random.PCG64(300 + M + N + K))
     A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
-    gemm_tile("256")
+    gemm_tile(str(side))
     name = first_profiled_kernel(torch_cuda, lambda: run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED))
     assert name.startswith("pair_gemm_big_kernel"), name
     got = run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED, c_pad=8)
@@ -163,11 +166,12 @@ def test_gemm_large_tiles(torch_cuda, gemm_tile, shape, mmajor):
     assert np.array_equal(got, small)
 
 
-@pytest.mark.parametrize("n", [768, 1024])
-def test_equation_at_768_residues_and_more_takes_the_large_tiles(torch_cuda, n):
-    """128 channels of 768 x 768 (nine large tiles per channel, more than four per CU, which is where the default rule
-    switches to them) and of 1024 x 1024 (eight tiles per workgroup).  Sampled channels against the oracle; the incoming
-    form equals the outgoing one on transposed operands bit for bit."""
+@pytest.mark.parametrize("n", [384, 576, 768, 1024])
+def test_equation_at_384_residues_and_more_takes_the_large_tiles(torch_cuda, n):
+    """128 channels of 768 x 768 (nine 256 x 256 tiles per channel, more than four per CU, which is where the default
+    rule switches to them) and of 1024 x 1024 (eight tiles per workgroup); of 384 x 384 and 576 x 576, whose sides are
+    whole 192 x 192 tiles (two and four and a half per CU).  Sampled channels against the oracle; the incoming form
+    equals the outgoing one on transposed operands bit for bit."""
     from oracle import oracle
     torch = torch_cuda
     c_i = 128
@@ -176,7 +180,8 @@ def test_equation_at_768_residues_and_more_takes_the_large_tiles(torch_cuda, n):
     right = (torch.randn(c_i, n, n, device="cuda", generator=g) * n ** -0.5).to(torch.bfloat16)
     for incoming in (False, True):
         name = first_profiled_kernel(torch, lambda: equation(torch, left, right, n, incoming))
-        assert name == ("pair_gemm_big_kernel<m-major>" if incoming else "pair_gemm_big_kernel"), name
+        form = ("m-major" if incoming else "") + (", " if incoming and n < 768 else "") + ("192" if n < 768 else "")
+        assert name == "pair_gemm_big_kernel" + (f"<{form}>" if form else ""), name
     out_c = equation(torch, left, right, n, False)
     in_c = equation(torch, left, right, n, True)
     chans = [0, 63, 127]
