@@ -35,12 +35,18 @@ extern "C" {
 #define KUTACC_DTYPE_FP32 2
 
 /* Kernel family selection for kutacc_hip_gating_attention. */
-#define KUTACC_HIP_PATH_AUTO 0    /* fused MFMA kernels when the shape allows, else generic      */
+#define KUTACC_HIP_PATH_AUTO 0    /* fused MFMA kernels when the shape allows, else tiled, else generic */
 #define KUTACC_HIP_PATH_GENERIC 1 /* shape-agnostic scalar kernels (any head_size, bf16 or fp32)  */
-#define KUTACC_HIP_PATH_FUSED 2   /* bf16 MFMA kernels only; EUNSUPPORTED if the shape is not covered */
-/* The MFMA kernels cover bf16, head_size 32, nheads * 32 in {128, 256}, seq_len <= 1024, 16-byte aligned operands with
- * leading dimensions that are multiples of 8, and an input row pitch of at most 2^19 elements (they address the rows of
- * a batch row with 32-bit byte offsets). */
+#define KUTACC_HIP_PATH_FUSED 2   /* MFMA kernels only (fused, fp32, tiled); EUNSUPPORTED if none takes the shape */
+#define KUTACC_HIP_PATH_TILED 3   /* the tiled MFMA route; EUNSUPPORTED if it does not take the shape */
+/* The fused MFMA kernels cover bf16, head_size 32, nheads * 32 in {128, 256}, seq_len <= 1024, 16-byte aligned operands
+ * with leading dimensions that are multiples of 8, and an input row pitch of at most 2^19 elements (they address the
+ * rows of a batch row with 32-bit byte offsets).
+ * The tiled MFMA route covers the other bf16 shapes: any seq_len, head sizes that are multiples of 8 up to 64, any number
+ * of heads; q, k, v, gate and avg laid out as the reference's kernel views them (dense [batch * seq_len, channels]
+ * matrices with row pitches that are multiples of 8, v as [channels, batch * seq_len]).  It follows the reference's data
+ * flow -- projections into q, k, v, gate on the MFMA GEMM, attention on MFMA tiles with an online softmax, output
+ * projection -- and so leaves those tensors as the reference does. */
 
 /*
  * Flat argument block of the gated-attention operator.  Replaces, for the launch layer, the
@@ -71,8 +77,8 @@ typedef struct kutacc_hip_attention_args {
     int64_t nb_stride_h;
     int64_t nb_stride_q;
 
-    /* Caller scratch.  k/v/gate are written only by the generic path; q is written by the generic
-     * path and may be used as workspace by the fused path (a fragment-major copy of the pair bias), so
+    /* Caller scratch.  k/v/gate are written only by the generic and the tiled path; q is written by those
+     * and may be used as workspace by the fused path (a fragment-major copy of the pair bias), so
      * its contents are unspecified after any call; avg (gated weighted average, [B,S,H,d]) is
      * written by every path.  Element (b,s,h,e) of q,k,gate,avg lives at
      * b*stride_b + s*stride_s + h*stride_h + e; v is [H,d,B,S]: (h,e,b,s) at
@@ -149,7 +155,7 @@ typedef struct kutacc_hip_global_attention_args {
 kutacc_export int kutacc_hip_global_attention(const kutacc_hip_global_attention_args_t *args, void *stream);
 
 /* Name of the kernel family the last successful kutacc_hip_gating_attention call used on this
- * thread: "fused_mfma" or "generic".  Static storage. */
+ * thread: "fused_mfma", "fp32_mfma", "tiled_mfma" or "generic".  Static storage. */
 kutacc_export const char *kutacc_hip_last_path(void);
 
 /*

@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libkutacc.so")
 
-SOURCES = ["api.cpp", "api_pair_stack.cpp", "api_glue.cpp", "unsupported.cpp", "profiler.cpp", "generic_kernels.hip", "row_kernels.hip", "fused_attention.hip", "fp32_attention.hip", "global_attention.hip", "pair_stack.hip", "glue_kernels.hip"]
+SOURCES = ["api.cpp", "api_pair_stack.cpp", "api_glue.cpp", "unsupported.cpp", "profiler.cpp", "generic_kernels.hip", "row_kernels.hip", "fused_attention.hip", "fp32_attention.hip", "tiled_attention.hip", "global_attention.hip", "pair_stack.hip", "glue_kernels.hip"]
 
 # -packed-fp32-ops off: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar float code.
 HIP_FLAGS = [

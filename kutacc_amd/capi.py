@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libkutacc.so")
 KUTACC_OK = 0
 KUTACC_ERROR = -1
 K_INT64, K_BF16, K_FP32 = 0, 1, 2
-PATH_AUTO, PATH_GENERIC, PATH_FUSED = 0, 1, 2
+PATH_AUTO, PATH_GENERIC, PATH_FUSED, PATH_TILED = 0, 1, 2, 3
 EINVAL, EUNSUPPORTED = -2, -3
 
 _vp = ctypes.c_void_p

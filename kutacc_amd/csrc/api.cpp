@@ -205,11 +205,17 @@ int kutacc_hip_gating_attention(const kutacc_hip_attention_args_t *a, void *stre
     hipStream_t s = pick_stream(stream);
     const bool fused_ok = kutacc_launch::fused_attention_supports(*a);
     const bool fp32_ok = !fused_ok && kutacc_launch::fp32_attention_supports(*a);
-    if (a->path == KUTACC_HIP_PATH_FUSED && !fused_ok && !fp32_ok) {
+    const bool tiled_ok = kutacc_launch::tiled_attention_supports(*a);
+    if ((a->path == KUTACC_HIP_PATH_FUSED && !fused_ok && !fp32_ok && !tiled_ok) || (a->path == KUTACC_HIP_PATH_TILED && !tiled_ok)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
     int rc;
-    if (fp32_ok && a->path != KUTACC_HIP_PATH_GENERIC) {
+    if (tiled_ok && (a->path == KUTACC_HIP_PATH_TILED || (!fused_ok && a->path != KUTACC_HIP_PATH_GENERIC))) {
+        rc = kutacc_launch::gating_attention_tiled(*a, s);
+        if (rc == 0) {
+            t_last_path = "tiled_mfma";
+        }
+    } else if (fp32_ok && a->path != KUTACC_HIP_PATH_GENERIC) {
         rc = kutacc_launch::gating_attention_fp32(*a, s);
         if (rc == 0) {
             t_last_path = "fp32_mfma";
@@ -347,9 +353,11 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
     kutacc_hip_attention_args_t a;
     std::memset(&a, 0, sizeof(a));
     a.batch = batch, a.seq_len = seq_len, a.nheads = nheads, a.head_size = head_size;
-    // "scratch" = "reference": the shape-agnostic kernels, which leave q, k, v and gate as the reference's kernel does
-    // (src/attention/gating_attention.cpp:47-66); the MFMA kernels never form them in memory
-    a.dtype = (int32_t)dt, a.path = g_reference_scratch.load(std::memory_order_relaxed) ? KUTACC_HIP_PATH_GENERIC : KUTACC_HIP_PATH_AUTO;
+    // "scratch" = "reference": a route that leaves q, k, v and gate as the reference's kernel does
+    // (src/attention/gating_attention.cpp:47-66) -- the tiled MFMA route where it takes the call (decided below, once the
+    // strides are known), else the shape-agnostic kernels; the fused MFMA kernels never form them in memory
+    const bool reference_scratch = g_reference_scratch.load(std::memory_order_relaxed) != 0;
+    a.dtype = (int32_t)dt, a.path = KUTACC_HIP_PATH_AUTO;
     a.input = in.data, a.input_ld = nchannels;
     a.query_w = wq.data, a.key_w = wk.data, a.value_w = wv.data, a.gating_w = wg.data, a.output_w = wo.data;
     a.gating_b = (const float *)bg.data, a.output_b = (const float *)bo.data;
@@ -368,6 +376,12 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
     if (q.numel() < batch * seq_len * nchannels && kutacc_launch::fused_attention_supports(a)) {
         a.q = nullptr;
     }
+    auto pick_path = [&]() {
+        if (reference_scratch) {
+            a.path = kutacc_launch::tiled_attention_supports(a) ? KUTACC_HIP_PATH_TILED : KUTACC_HIP_PATH_GENERIC;
+        }
+    };
+    pick_path();
 
     hipStream_t s = current_stream();
     const Space sp = space_of(in.data);
@@ -414,6 +428,7 @@ void kutacc_af2_gating_attention(kutacc_tensor_h input, kutacc_af2_attention_inp
         KUTACC_CHECK(avg_dense_rows, "avg must be viewable as a [batch*seq_len, nchannels] matrix");
         a.avg = avg_dense_rows ? st.out(av.data, span2(M, a.avg_stride_s, C) * e, false) : nullptr;
         a.out = st.out(ot.data, span2(M, a.out_ld, C) * e, a.out_ld != C);
+        pick_path();
         rc = st.rc;
         if (rc == 0 && !KUTACC_FAILED()) {
             rc = kutacc_hip_gating_attention(&a, s);

@@ -69,6 +69,11 @@ int gating_attention_generic(const kutacc_hip_attention_args_t &args, hipStream_
 int gemm_nt(int32_t dtype, const void *a, int64_t lda, const void *w, int64_t ldw, const float *bias, void *c,
             int64_t c_rs, int64_t c_cs, int64_t m, int64_t n, int64_t k, float beta, hipStream_t stream);
 
+// tiled_attention.hip: bf16, any seq_len, head sizes 8 .. 64; projections into the caller's q, k, v, gate as the reference
+// leaves them, attention on MFMA tiles with an online softmax
+bool tiled_attention_supports(const kutacc_hip_attention_args_t &args);
+int gating_attention_tiled(const kutacc_hip_attention_args_t &args, hipStream_t stream);
+
 // fp32_attention.hip: fp32 storage on the fp32 matrix core (head_size 32, up to 256 channels, up to 224 positions)
 bool fp32_attention_supports(const kutacc_hip_attention_args_t &args);
 int gating_attention_fp32(const kutacc_hip_attention_args_t &args, hipStream_t stream);

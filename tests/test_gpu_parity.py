@@ -496,10 +496,10 @@ def test_strided_tensors_through_the_launch_layer(torch_cuda, path, nb_pad):
 
 
 @pytest.mark.parametrize("wide", ["input", "out"])
-def test_row_pitch_beyond_the_mfma_kernels_addressing_takes_the_generic_kernels(torch_cuda, wide):
-    """The MFMA kernels address rows with 32-bit byte offsets and accept row pitches of up to 2^19 elements; a wider one
-    must not reach them: the automatic choice falls back to the generic kernels (and is right), the forced MFMA path
-    refuses."""
+def test_row_pitch_beyond_the_fused_kernels_addressing_takes_the_tiled_route(torch_cuda, wide):
+    """The fused MFMA kernels address rows with 32-bit byte offsets and accept row pitches of up to 2^19 elements; a wider
+    one must not reach them: the automatic choice, and the choice among MFMA kernels only, go to the tiled route, whose
+    products run on the strided GEMM (and are right)."""
     torch = torch_cuda
     w = make_workload(3, batch=1, seq_len=40)
     B, S, C = w.B, w.S, w.C
@@ -514,12 +514,13 @@ def test_row_pitch_beyond_the_mfma_kernels_addressing_takes_the_generic_kernels(
         a.out, a.out_ld = wide_t.data_ptr(), ld
     rc = capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None)
     torch.cuda.synchronize()
-    assert rc == 0 and capi.last_path() == "generic"
+    assert rc == 0 and capi.last_path() == "tiled_mfma"
     got = ten["out"] if wide == "input" else wide_t[:, :C].reshape(B, S, C)
     helpers.check_close(helpers.to_numpy(got), helpers.oracle_out(w), w.dtype, "wide-pitch out")
     a.path = capi.PATH_FUSED
-    assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None) != 0
+    assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None) == 0 and capi.last_path() == "tiled_mfma"
     torch.cuda.synchronize()
+    helpers.check_close(helpers.to_numpy(got), helpers.oracle_out(w), w.dtype, "wide-pitch out, MFMA kernels only")
 
 
 # ---- boundary behaviour ------------------------------------------------------------------------------------
@@ -564,9 +565,10 @@ def test_pointer_checks_can_be_switched_off(torch_cuda):
 
 def test_reference_scratch_mode_fills_q_k_v_gate(torch_cuda):
     """The reference's kernel leaves its projections in the caller's scratch tensors (reference
-    src/attention/gating_attention.cpp:47-66: q scaled by 1/sqrt(d), k, v transposed to [H, d, B, S], gate after the
-    sigmoid).  The MFMA kernels never form them in memory; with "scratch" = "reference" the operator runs on the
-    shape-agnostic kernels, and the five tensors must match the oracle's bf16 model of the reference."""
+    src/attention/gating_attention.cpp:47-66: q and k as projected, v transposed to [H, d, B, S], gate with its bias,
+    before the sigmoid).  The fused MFMA kernels never form them in memory; with "scratch" = "reference" the operator runs on the
+    tiled MFMA route, which follows the reference's data flow, and the five tensors must match the oracle's bf16 model of
+    the reference."""
     from oracle import oracle
     w = make_workload(3, batch=3, seq_len=80)
     op, ten, scratch = helpers.make_op(w)
@@ -576,7 +578,7 @@ def test_reference_scratch_mode_fills_q_k_v_gate(torch_cuda):
         path = capi.last_path()
     finally:
         capi.set_tuning("scratch", "default")
-    assert not capi.error_flag() and path == "generic"
+    assert not capi.error_flag() and path == "tiled_mfma"
     bits = lambda a: oracle.to_bf16_bits(np.asarray(a, dtype=np.float32))  # noqa: E731
     _, ref = oracle.gating_attention_bf16(bits(w.x), bits(w.wq), bits(w.wk), bits(w.wv), bits(w.wg), w.bg, bits(w.wo), w.bo,
                                           bits(w.bias), None if w.nb is None else bits(w.nb), w.H, return_scratch=True)
