@@ -15,6 +15,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "device_util.h"
 #include "launch_internal.h"
 #include "mfma_tiles.h"
@@ -67,6 +69,19 @@ __device__ __forceinline__ uint4 load8_checked(const bf16_t *src, int valid)
     return c.u;
 }
 
+// acc + the sum of eight bf16: four dot products of a pair with (1, 1)
+__device__ __forceinline__ float pair_sums(bf16x8 v, float acc)
+{
+    typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
+    const pair_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const pair_t pr = {v[2 * i], v[2 * i + 1]};
+        acc = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, acc, false);
+    }
+    return acc;
+}
+
 // KS: k-steps of 16 of the q.k product (head_size <= 16 KS, zero padded); the head's values span DB = ceil(KS / 2)
 // blocks of 32 MFMA rows.
 //
@@ -80,8 +95,8 @@ __device__ __forceinline__ uint4 load8_checked(const bf16_t *src, int valid)
 // Placement: workgroup ids are dealt round robin over the 8 XCDs; the id is decoded so that each XCD works on groups of
 // 8 batch rows x 8 query blocks of one head at a time.  The 64 workgroups of a group sweep the keys roughly together,
 // so the group's K/V (8 rows) and pair bias (8 query blocks) come from HBM once and from the XCD's L2 seven times.
-template <int KS>
-__global__ __launch_bounds__(256) void attention_tiles_kernel(const TileParams p)
+template <int KS, bool HAS_NB>
+__global__ __launch_bounds__(256, 2) void attention_tiles_kernel(const TileParams p)
 {
     constexpr int DB = (KS + 1) / 2;
     constexpr int K_SLOTS = 2 * KS * 64, V_SLOTS = DB * 4 * 64, STAGE_SLOTS = K_SLOTS + V_SLOTS + CHUNK / 4;
@@ -118,162 +133,245 @@ __global__ __launch_bounds__(256) void attention_tiles_kernel(const TileParams p
     const bf16_t *kbase = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
     const bf16_t *vbase = p.v + (int64_t)h * hd * p.v_se + (int64_t)b * p.v_sb;
     const bf16_t *bias_row = p.bias + (int64_t)b * p.bias_sb;
-    const bf16_t *nb_row = p.nb ? p.nb + (int64_t)h * p.nb_sh + (int64_t)query * p.nb_sq : nullptr;
+    const bf16_t *nb_row = HAS_NB ? p.nb + (int64_t)h * p.nb_sh + (int64_t)query * p.nb_sq : nullptr;
 
+    // What a thread stages of every chunk: PK 16-byte pieces of K (key kap, values 8 o .. 8 o + 7 of the head) and DB of
+    // V^T (value d, keys 8 ko .. 8 ko + 7 of the chunk); pieces that lie in the padding are stored as zeros.
+    int k_kap[PK], k_slot[PK], v_slot[DB];
+    int64_t k_off[PK], v_off[DB];
+    bool k_real[PK], v_real[DB];
+#pragma unroll
+    for (int i = 0; i < PK; ++i) {
+        const int idx = tid + 256 * i;
+        const int o = idx % (2 * KS), kap = (idx / (2 * KS)) % CHUNK;
+        k_kap[i] = kap;
+        k_real[i] = 8 * o < hd; // (an index past the last piece repeats piece idx - K_PIECES: same data, same slot)
+        k_off[i] = k_real[i] ? 8 * o : 0;
+        k_slot[i] = ((kap >> 5) * KS + (o >> 1)) * 64 + swap23(kap & 31) + 32 * (o & 1);
+    }
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+        const int idx = tid + 256 * i;
+        const int d = idx >> 3, ko = idx & 7;
+        v_real[i] = d < hd;
+        v_off[i] = (int64_t)(v_real[i] ? d : 0) * p.v_se + 8 * ko;
+        v_slot[i] = K_SLOTS + ((d >> 5) * 4 + (ko >> 1)) * 64 + (d & 31) + 32 * (ko & 1);
+    }
+    auto keep = [](uint4 v, bool ok) { // a select, not a branch around the load
+        const uint32_t m = ok ? 0xffffffffu : 0u;
+        return make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+    };
+    // Two forms of the loads of a chunk.  PLAIN: every key of the chunk exists and every row can be read 16 bytes at a
+    // time -- no condition anywhere (a thread without a piece of its own repeats another thread's, to the same slot), so
+    // that the loop made of such chunks is one basic block per phase and the loads stay in flight across the compute
+    // phase.  Otherwise: the checked form (clamped rows, element-wise reads past alignment or the end).  Nothing touches
+    // what a load returns before park(): a use right behind the load makes the wave wait out the memory latency.
     uint4 kreg[PK], vreg[DB];
-    float bias_reg = 0.f;
-    auto fetch = [&](int c) {
+    bool k_keep[PK];
+    bf16_t bias_raw = (bf16_t)0.f;
+    bool bias_keep = false;
+    auto fetch = [&](int c, auto plain_tag) {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
         const int kc0 = c * CHUNK;
 #pragma unroll
         for (int i = 0; i < PK; ++i) {
-            const int idx = tid + 256 * i;
-            const int o = idx % (2 * KS), key = kc0 + idx / (2 * KS);
-            kreg[i] = zero_u4();
-            if (idx < K_PIECES && key < S && 8 * o < hd) {
-                kreg[i] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)key * p.k_ss + 8 * o);
-            }
+            const int key = kc0 + k_kap[i], key_c = PLAIN || key < S ? key : S - 1;
+            kreg[i] = *reinterpret_cast<const uint4 *>(kbase + (int64_t)key_c * p.k_ss + k_off[i]);
+            k_keep[i] = k_real[i] && (PLAIN || key < S);
         }
+        if constexpr (PLAIN) {
 #pragma unroll
-        for (int i = 0; i < DB; ++i) {
-            const int idx = tid + 256 * i;
-            const int d = idx >> 3, key = kc0 + 8 * (idx & 7);
-            vreg[i] = zero_u4();
-            if (d < hd && key < S) {
-                const bf16_t *src = vbase + (int64_t)d * p.v_se + key;
-                vreg[i] = (p.v_vec && key + 8 <= S) ? *reinterpret_cast<const uint4 *>(src) : load8_checked(src, S - key);
+            for (int i = 0; i < DB; ++i) {
+                vreg[i] = *reinterpret_cast<const uint4 *>(vbase + v_off[i] + kc0);
             }
-        }
-        if (tid < CHUNK) {
-            bias_reg = kc0 + tid < S ? to_f32(bias_row[kc0 + tid]) : -INFINITY;
+            bias_raw = bias_row[kc0 + (tid & (CHUNK - 1))];
+            bias_keep = true;
+        } else {
+#pragma unroll
+            for (int i = 0; i < DB; ++i) {
+                const int key = kc0 + 8 * ((tid + 256 * i) & 7);
+                vreg[i] = zero_u4();
+                if (v_real[i] && key < S) {
+                    const bf16_t *src = vbase + v_off[i] + kc0;
+                    vreg[i] = (p.v_vec && key + 8 <= S) ? *reinterpret_cast<const uint4 *>(src) : load8_checked(src, S - key);
+                }
+            }
+            const int key = kc0 + (tid & (CHUNK - 1));
+            bias_raw = bias_row[key < S ? key : S - 1];
+            bias_keep = key < S;
         }
     };
     auto park = [&](uint4 *stage) {
 #pragma unroll
         for (int i = 0; i < PK; ++i) {
-            const int idx = tid + 256 * i;
-            const int o = idx % (2 * KS), kap = idx / (2 * KS);
-            if (idx < K_PIECES) {
-                stage[((kap >> 5) * KS + (o >> 1)) * 64 + swap23(kap & 31) + 32 * (o & 1)] = kreg[i];
-            }
+            stage[k_slot[i]] = keep(kreg[i], k_keep[i]);
         }
 #pragma unroll
         for (int i = 0; i < DB; ++i) {
-            const int idx = tid + 256 * i;
-            const int d = idx >> 3, ko = idx & 7;
-            stage[K_SLOTS + ((d >> 5) * 4 + (ko >> 1)) * 64 + (d & 31) + 32 * (ko & 1)] = vreg[i];
+            stage[v_slot[i]] = keep(vreg[i], v_real[i]); // (the element-wise form has zeroed what it must already)
         }
-        if (tid < CHUNK) {
-            reinterpret_cast<float *>(stage + K_SLOTS + V_SLOTS)[tid] = bias_reg;
-        }
+        reinterpret_cast<float *>(stage + K_SLOTS + V_SLOTS)[tid & (CHUNK - 1)] = bias_keep ? to_f32(bias_raw) * LOG2E : -INFINITY;
     };
-    // pair bias of this lane's query for the keys of chunk c: [key block][j] holds keys 32 kb + 16 j + 8 g .. + 7
-    auto fetch_nb = [&](int c, uint4 (&dst)[2][2]) {
+    // Pair bias of the wave's 32 queries for the 64 keys of chunk c: 32 rows x 128 bytes.  Read as whole rows (a load
+    // instruction covers 8 rows x 128 contiguous bytes: 8 cache lines; a lane fetching the 16 bytes of its own query for
+    // its own keys would touch 32 lines per instruction, a quarter of each) and passed through a wave-private LDS panel,
+    // from which each lane takes its query's keys in accumulator order.  Rows past the last query repeat it.
+    uint4 *nb_panel = lds + 2 * STAGE_SLOTS + wave * 256;
+    const bf16_t *nb_head = HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr;
+    auto fetch_nb = [&](int c, auto plain_tag) -> PanelRegs {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
+        PanelRegs f = {zero_u4(), zero_u4(), zero_u4(), zero_u4()};
+        if constexpr (HAS_NB) {
+            const int kc0 = c * CHUNK;
+            if constexpr (PLAIN) {
+                return panel_load(nb_head, p.nb_sq, q0 < S ? q0 : S - 1, S - 1, kc0, lane);
+            }
+            const int key = kc0 + 8 * (lane & 7);
+            if (key < S) {
+                uint4 *dst[4] = {&f.r0, &f.r1, &f.r2, &f.r3};
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int key = c * CHUNK + 32 * kb + 16 * j + 8 * g;
-                dst[kb][j] = zero_u4();
-                if (nb_row != nullptr && key < S) {
-                    dst[kb][j] = (p.nb_vec && key + 8 <= S) ? *reinterpret_cast<const uint4 *>(nb_row + key)
-                                                            : load8_checked(nb_row + key, S - key);
+                for (int i = 0; i < 4; ++i) {
+                    const int row = q0 + 8 * i + (lane >> 3);
+                    const bf16_t *src = nb_head + (int64_t)(row < S ? row : S - 1) * p.nb_sq + key;
+                    *dst[i] = (p.nb_vec && key + 8 <= S) ? *reinterpret_cast<const uint4 *>(src) : load8_checked(src, S - key);
                 }
             }
         }
+        return f;
     };
 
     f32x16 oacc[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-        oacc[db] = zero16();
-    }
-    float m_run = -INFINITY, l_run = 0.f; // the sum is this lane's share (its half of the keys)
+    float m_run, l_run; // running maximum (log2 units; SAFE only) and this lane's share of the sum (its half of the keys)
     const int chunks = (S + CHUNK - 1) / CHUNK;
-    uint4 nb_cur[2][2], nb_next[2][2];
-    fetch(0);
-    fetch_nb(0, nb_cur);
-    park(lds);
-    __syncthreads();
-    for (int c = 0; c < chunks; ++c) {
-        const uint4 *stage = lds + (c & 1) * STAGE_SLOTS;
-        const bool more = c + 1 < chunks;
-        if (more) {
-            fetch(c + 1);
-            if (active) {
-                fetch_nb(c + 1, nb_next);
-            }
+    const float scale2 = p.scale * LOG2E;
+    // One pass over all keys.  Everything is in log2 units: x = q.k * (scale * log2 e) + bias * log2 e + nb * log2 e,
+    // p = 2^x.  The fast pass takes 2^x as it stands -- a softmax does not depend on a common shift, and fp32 and bf16
+    // hold 2^-126 .. 2^127 -- and the caller checks the sums afterwards; the SAFE pass keeps a running maximum and
+    // serves the rows the fast one could not (logits beyond that range, rows with every key masked).
+    auto sweep = [&](auto safe_tag) {
+        constexpr bool SAFE = decltype(safe_tag)::value;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            oacc[db] = zero16();
         }
-        if (active) {
-            const float *mask_bias = reinterpret_cast<const float *>(stage + K_SLOTS + V_SLOTS);
+        m_run = -INFINITY, l_run = 0.f;
+        PanelRegs nb_next;
+        // chunks [0, plain) take the PLAIN loads
+        const int plain = (p.v_vec && (!HAS_NB || p.nb_vec)) ? S / CHUNK : 0;
+        if (plain > 0) {
+            fetch(0, std::true_type{});
+            nb_next = fetch_nb(0, std::true_type{});
+        } else {
+            fetch(0, std::false_type{});
+            nb_next = fetch_nb(0, std::false_type{});
+        }
+        if constexpr (HAS_NB) {
+            panel_store(nb_panel, lane, nb_next);
+        }
+        park(lds);
+        __syncthreads();
+        // chunk c from its stage, with the loads of chunk c + 1 (if `more`) in flight meanwhile
+        auto step = [&](int c, bool more, auto plain_tag) {
+            const uint4 *stage = lds + (c & 1) * STAGE_SLOTS;
+            if (more) {
+                fetch(c + 1, plain_tag);
+                nb_next = fetch_nb(c + 1, plain_tag);
+            }
+            if (active) {
+                const float *mask_bias = reinterpret_cast<const float *>(stage + K_SLOTS + V_SLOTS);
+                f32x16 x[2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                f32x16 x = zero16();
+                for (int kb = 0; kb < 2; ++kb) {
+                    x[kb] = zero16();
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    x = mfma(as_bf16x8(stage[(kb * KS + ks) * 64 + lane]), qf[ks], x);
+                    for (int ks = 0; ks < KS; ++ks) {
+                        x[kb] = mfma(as_bf16x8(stage[(kb * KS + ks) * 64 + lane]), qf[ks], x[kb]);
+                    }
                 }
                 float mx = -INFINITY;
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const f32x4 b0 = *reinterpret_cast<const f32x4 *>(mask_bias + 32 * kb + 16 * j + 8 * g);
-                    const f32x4 b1 = *reinterpret_cast<const f32x4 *>(mask_bias + 32 * kb + 16 * j + 8 * g + 4);
-                    const bf16x8 nbv = as_bf16x8(nb_cur[kb][j]);
+                for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        float v = fmaf(x[8 * j + e], p.scale, e < 4 ? b0[e & 3] : b1[e & 3]);
-                        if (nb_row != nullptr) {
-                            v += to_f32(nbv[e]);
+                    for (int j = 0; j < 2; ++j) {
+                        const f32x4 b0 = *reinterpret_cast<const f32x4 *>(mask_bias + 32 * kb + 16 * j + 8 * g);
+                        const f32x4 b1 = *reinterpret_cast<const f32x4 *>(mask_bias + 32 * kb + 16 * j + 8 * g + 4);
+                        const bf16x8 nbv = as_bf16x8(HAS_NB ? nb_panel[panel_slot(r, 4 * kb + 2 * j + g)] : zero_u4());
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            float v = fmaf(x[kb][8 * j + e], scale2, e < 4 ? b0[e & 3] : b1[e & 3]);
+                            if constexpr (HAS_NB) {
+                                v = fmaf(to_f32(nbv[e]), LOG2E, v);
+                            }
+                            x[kb][8 * j + e] = v;
+                            if constexpr (SAFE) {
+                                mx = fmaxf(mx, v);
+                            }
                         }
-                        x[8 * j + e] = v;
-                        mx = fmaxf(mx, v);
                     }
                 }
-                const float m_new = fmaxf(m_run, half_swap_max(mx));
-                // every key so far at -inf: any finite reference point keeps the arithmetic below free of inf - inf
-                const float m_ref = m_new == -INFINITY ? 0.f : m_new;
-                if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-                    const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * LOG2E);
-                    l_run *= alpha;
+                float m_ref = 0.f;
+                if constexpr (SAFE) {
+                    const float m_new = fmaxf(m_run, half_swap_max(mx));
+                    // every key so far at -inf: any finite reference point keeps the arithmetic free of inf - inf
+                    m_ref = m_new == -INFINITY ? 0.f : m_new;
+                    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+                        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+                        l_run *= alpha;
+#pragma unroll
+                        for (int db = 0; db < DB; ++db) {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                oacc[db][v] *= alpha;
+                            }
+                        }
+                        m_run = m_new;
+                    }
+                }
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        // SAFE: (x - m) is exact where x = m, whatever their size (a masked row sits at -1.4e9)
+                        x[kb][v] = __builtin_amdgcn_exp2f(SAFE ? x[kb][v] - m_ref : x[kb][v]);
+                    }
+                    const bf16x8 p0 = pack8(x[kb], 0), p1 = pack8(x[kb], 8);
+                    l_run = pair_sums(p0, pair_sums(p1, l_run)); // of the rounded values, the ones p.v multiplies
 #pragma unroll
                     for (int db = 0; db < DB; ++db) {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            oacc[db][v] *= alpha;
-                        }
+                        oacc[db] = mfma(as_bf16x8(stage[K_SLOTS + (db * 4 + 2 * kb) * 64 + lane]), p0, oacc[db]);
+                        oacc[db] = mfma(as_bf16x8(stage[K_SLOTS + (db * 4 + 2 * kb + 1) * 64 + lane]), p1, oacc[db]);
                     }
-                    m_run = m_new;
-                }
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    // (x - m) first: exact where x = m, whatever their size (a masked row sits at -1e9)
-                    x[v] = __builtin_amdgcn_exp2f((x[v] - m_ref) * LOG2E);
-                    l_run += x[v];
-                }
-                const bf16x8 p0 = pack8(x, 0), p1 = pack8(x, 8);
-#pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    oacc[db] = mfma(as_bf16x8(stage[K_SLOTS + (db * 4 + 2 * kb) * 64 + lane]), p0, oacc[db]);
-                    oacc[db] = mfma(as_bf16x8(stage[K_SLOTS + (db * 4 + 2 * kb + 1) * 64 + lane]), p1, oacc[db]);
                 }
             }
-        }
-        if (more) {
-            park(lds + ((c + 1) & 1) * STAGE_SLOTS); // its last readers passed the barrier that ended the previous chunk
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    nb_cur[kb][j] = nb_next[kb][j];
+            if (more) {
+                park(lds + ((c + 1) & 1) * STAGE_SLOTS); // its last readers passed the barrier that ended the previous chunk
+                if constexpr (HAS_NB) {
+                    panel_store(nb_panel, lane, nb_next); // wave-private, and behind this wave's reads of the chunk just done
                 }
             }
+            __syncthreads();
+        };
+        int c = 0;
+        for (; c + 1 < plain; ++c) {
+            step(c, true, std::true_type{});
         }
-        __syncthreads();
+        for (; c < chunks; ++c) {
+            step(c, c + 1 < chunks, std::false_type{});
+        }
+        l_run = half_swap_sum(l_run);
+    };
+    sweep(std::false_type{});
+    // a sum outside [1e-30, 1e30] (or not a number): the row's logits left the range in which 2^x and the products with
+    // v are safe in fp32, or every key is masked.  The keys are staged by the whole workgroup, so it repeats as one.
+    const bool fast_failed = active && q0 + r < S && !(l_run >= 1e-30f && l_run <= 1e30f);
+    if (__syncthreads_or(fast_failed ? 1 : 0)) {
+        sweep(std::true_type{});
     }
     if (!active || q0 + r >= S) {
         return;
     }
     // weighted average -> bf16, x sigmoid(gate) -> bf16; register 4 a + c of lane half g is value 32 db + 8 a + 4 g + c
-    const float inv = 1.0f / half_swap_sum(l_run);
+    const float inv = 1.0f / l_run;
     const int64_t row = (int64_t)(q0 + r);
     const bf16_t *gp = p.gate + (int64_t)b * p.g_sb + row * p.g_ss + (int64_t)h * p.g_sh;
     bf16_t *ap = p.avg + (int64_t)b * p.a_sb + row * p.a_ss + (int64_t)h * p.a_sh;
@@ -298,13 +396,13 @@ __global__ __launch_bounds__(256) void attention_tiles_kernel(const TileParams p
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <int KS>
+template <int KS, bool HAS_NB>
 hipError_t launch_tiles(const TileParams &p, int64_t blocks, hipStream_t stream)
 {
     constexpr int DB = (KS + 1) / 2;
-    constexpr size_t lds_bytes = 2 * (2 * KS * 64 + DB * 4 * 64 + CHUNK / 4) * 16;
+    constexpr size_t lds_bytes = (2 * (2 * KS * 64 + DB * 4 * 64 + CHUNK / 4) + (HAS_NB ? 4 * 256 : 0)) * 16;
     static_assert(lds_bytes <= 64 * 1024, "two stages fit the LDS a kernel may use without opting in");
-    attention_tiles_kernel<KS><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(p);
+    attention_tiles_kernel<KS, HAS_NB><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(p);
     return hipGetLastError();
 }
 
@@ -385,10 +483,14 @@ int gating_attention_tiled(const kutacc_hip_attention_args_t &a, hipStream_t str
     {
         kutacc_prof::KernelTimer t("attention_tiles_kernel", 4.0 * (double)B * (double)S * (double)S * (double)C, stream);
         const int ks = (int)(hd + 15) / 16;
-        const hipError_t e = ks == 1   ? launch_tiles<1>(p, blocks, stream)
-                             : ks == 2 ? launch_tiles<2>(p, blocks, stream)
-                             : ks == 3 ? launch_tiles<3>(p, blocks, stream)
-                                       : launch_tiles<4>(p, blocks, stream);
+        hipError_t e;
+        if (p.nb != nullptr) {
+            e = ks == 1 ? launch_tiles<1, true>(p, blocks, stream) : ks == 2 ? launch_tiles<2, true>(p, blocks, stream)
+                : ks == 3 ? launch_tiles<3, true>(p, blocks, stream) : launch_tiles<4, true>(p, blocks, stream);
+        } else {
+            e = ks == 1 ? launch_tiles<1, false>(p, blocks, stream) : ks == 2 ? launch_tiles<2, false>(p, blocks, stream)
+                : ks == 3 ? launch_tiles<3, false>(p, blocks, stream) : launch_tiles<4, false>(p, blocks, stream);
+        }
         if ((rc = kutacc_hip_status(e))) {
             return rc;
         }
