@@ -376,6 +376,64 @@ def msa_block_rates(reps=20):
     return res
 
 
+def tiled_route_rates(reps=3):
+    """Times of the operator on the tiled MFMA route (the bf16 shapes beyond the fused head kernels), hipEvent-bracketed
+    calls of kutacc_hip_gating_attention on device tensors drawn with torch's generator: triangle attention at 2048
+    residues (2048 rows of 2048 positions, 4 heads of 32), the row-wise attention of the extra-MSA stack (5120 sequences
+    x 384 residues, 8 heads of 8, pair bias) and, for scale, the headline configuration forced onto this route.  Per
+    shape: milliseconds and TFLOP/s on the operator's algorithmic flops (10 B S C^2 + 4 B S^2 C)."""
+    import ctypes
+
+    import torch
+    from kutacc_amd import capi
+
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {}
+    for name, B, S, H, d, path in (("triangle_attention 2048 residues (B=2048 S=2048 H=4 d=32)", 2048, 2048, 4, 32, capi.PATH_AUTO),
+                                   ("extra_msa_row_attention (B=5120 S=384 H=8 d=8)", 5120, 384, 8, 8, capi.PATH_AUTO),
+                                   ("config 3 forced onto the tiled route (B=384 S=384 H=4 d=32)", 384, 384, 4, 32, capi.PATH_TILED)):
+        C = H * d
+        g = torch.Generator(device="cuda").manual_seed(17)
+        bf = lambda *sh, scale=1.0: (torch.randn(*sh, device="cuda", generator=g) * scale).to(torch.bfloat16)  # noqa: E731
+        x, ws = bf(B, S, C), [bf(C, C, scale=C ** -0.5) for _ in range(5)]
+        bg, bo = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
+        bias, nb = torch.zeros(B, S, device="cuda", dtype=torch.bfloat16), bf(H, S, S)
+        out = torch.empty(B, S, C, device="cuda", dtype=torch.bfloat16)
+        q, k, gate, avg = (torch.empty(B, S, C, device="cuda", dtype=torch.bfloat16) for _ in range(4))
+        v = torch.empty(C, B * S, device="cuda", dtype=torch.bfloat16)
+        a = capi.HipAttentionArgs()
+        a.batch, a.seq_len, a.nheads, a.head_size, a.dtype, a.path = B, S, H, d, capi.K_BF16, path
+        a.input, a.input_ld = x.data_ptr(), C
+        a.query_w, a.key_w, a.value_w, a.gating_w, a.output_w = (w.data_ptr() for w in ws)
+        a.gating_b, a.output_b = bg.data_ptr(), bo.data_ptr()
+        a.bias, a.bias_stride_b = bias.data_ptr(), S
+        a.nonbatched_bias, a.nb_stride_h, a.nb_stride_q = nb.data_ptr(), S * S, S
+        a.q, a.k, a.v, a.gate, a.avg = q.data_ptr(), k.data_ptr(), v.data_ptr(), gate.data_ptr(), avg.data_ptr()
+        for n in ("q", "k", "gate", "avg"):
+            setattr(a, f"{n}_stride_b", S * C), setattr(a, f"{n}_stride_s", C), setattr(a, f"{n}_stride_h", d)
+        a.v_stride_h, a.v_stride_e, a.v_stride_b = d * B * S, B * S, S
+        a.out, a.out_ld = out.data_ptr(), C
+
+        def call():
+            assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), stream) == 0
+        for _ in range(3):
+            call()
+        assert capi.last_path() == "tiled_mfma", capi.last_path()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) / reps * 1e-3
+        flops = 10.0 * B * S * C * C + 4.0 * B * S * S * C
+        res[name] = {"ms": round(t * 1e3, 3), "TFLOP/s": round(flops / t / 1e12, 1),
+                     "frac_of_bf16_mfma_peak": round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 3)}
+        del x, ws, nb, out, q, k, gate, avg, v
+        torch.cuda.empty_cache()
+    return res
+
+
 def device_workload(config):
     """Inputs of configuration `config` drawn on the GPU (torch's generator, seed 1000 + config): the same shapes,
     distributions and mask rules as kutacc_amd.workloads.make_workload, without its minute of host-side drawing for the
@@ -595,6 +653,9 @@ def main():
     ap.add_argument("--msa-blocks", action="store_true",
                     help="also time the row-wise (with pair bias) and column-wise MSA attention blocks at the shapes of "
                          "configurations 2 and 4 and report them in an \"msa_blocks\" object")
+    ap.add_argument("--tiled-route", action="store_true",
+                    help="also time the operator on the tiled MFMA route (rows of 2048 positions, head size 8) and report it "
+                         "in a \"tiled_route\" object")
     ap.add_argument("--pair-stack", action="store_true",
                     help="also time the transition and the triangle-multiplication steps at this configuration's pair "
                          "tensor and report them in a \"pair_stack\" object")
@@ -703,6 +764,8 @@ def main():
         rec["pair_stack"] = pair_stack_rates(a.config)
     if a.msa_blocks:
         rec["msa_blocks"] = msa_block_rates()
+    if a.tiled_route:
+        rec["tiled_route"] = tiled_route_rates()
     print(json.dumps(rec))
 
 

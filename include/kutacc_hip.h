@@ -456,10 +456,11 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *               copy from the workspace and costs 8-15 % of the block's time; "separate" or "auto" (default): the
  *               LayerNorm runs as a pass of its own.  The workspace functions answer for the mode in force when they are
  *               called: query and call under the same setting.
- *   "scratch"   "reference": kutacc_af2_gating_attention runs on the shape-agnostic kernels, which fill the caller's q, k, v
- *               and gate tensors as the reference's kernel does (src/attention/gating_attention.cpp:47-66) -- for callers
- *               or tests that read them; several times slower.  Anything else (default): the MFMA kernels where they
- *               apply, which leave k, v and gate untouched and use q as workspace.
+ *   "scratch"   "reference": kutacc_af2_gating_attention runs on the tiled MFMA route (KUTACC_HIP_PATH_TILED; the
+ *               shape-agnostic kernels where that route does not take the call), which fills the caller's q, k, v and
+ *               gate tensors as the reference's kernel does (src/attention/gating_attention.cpp:47-66) -- for callers or
+ *               tests that read them; about twice the time of the fused kernels.  Anything else (default): the fused MFMA
+ *               kernels where they apply, which leave k, v and gate untouched and use q as workspace.
  *   "pointer_checks" "0": the handle-based attention entry points classify only `input` (host or device) and take the
  *               caller's word that every other operand lives in the same place, which saves about fifteen driver
  *               queries per call; "1": every operand is checked and mixed calls are rejected (default) */

@@ -2,8 +2,10 @@
 // fp32 storage, fp32 arithmetic throughout.  They follow the reference's data flow one to one --
 // four projections into the caller's scratch, per-(batch, head, query) softmax attention with the
 // sigmoid gate applied to the weighted average, output projection (reference
-// src/attention/gating_attention.cpp:47-66, 73-150, 152-157) -- and exist for the shapes and the
-// storage type the fused MFMA kernels do not take (fp32 tensors, head_size != 32, tiny problems).
+// src/attention/gating_attention.cpp:47-66, 73-150, 152-157) -- and exist for what no MFMA kernel
+// takes (fp32 tensors beyond the fp32 kernel's reach, head sizes that are no multiple of 8 or above 64,
+// scratch layouts the reference's kernel would not view as matrices) and as an independent kernel
+// family for the tests.
 // Logits and probabilities stay in fp32 registers; only q/k/v/gate/avg/out are rounded to the
 // storage type, at the points where the reference stores them.
 #include <hip/hip_runtime.h>

@@ -4,8 +4,9 @@
 // tensors (v transposed to [channels, batch * seq_len], the gate with its bias), attention per (batch row, head) with
 // the sigmoid gate applied to the weighted average, output projection -- so this route also leaves the scratch
 // tensors as the reference's kernel does.  The projections run on the strided MFMA GEMM of the pair stack; the
-// attention is the kernel below: MFMA products for q.k and p.v, online softmax in fp32, keys streamed through LDS in
-// chunks of 64, so that the logits of a row never exist and nothing depends on the row's length.
+// attention is the kernel below: MFMA products for q.k and p.v, softmax in fp32 (unshifted in log2 units where a row's
+// sums allow it, with a running maximum where they do not), keys streamed through LDS in chunks of 64, so that the
+// logits of a row never exist and nothing depends on the row's length.
 //
 // Rounding points: q, k, v, gate as bf16 in memory (the reference's), logits
 // x = (q.k * scale + bias[b, key]) + nonbatched_bias[h, query, key] in fp32 with that association
@@ -86,11 +87,11 @@ __device__ __forceinline__ float pair_sums(bf16x8 v, float acc)
 // blocks of 32 MFMA rows.
 //
 // One workgroup = 128 queries of one (batch row, head): wave w owns queries 32 w .. 32 w + 31, keeps their q fragments,
-// running maximum, running sum and the head_size x 32 accumulator of p.v in registers, and walks all keys.  The
+// running sum (and maximum, in the second pass) and the head_size x 32 accumulator of p.v in registers, and walks all keys.  The
 // workgroup stages each chunk of 64 keys once (K in fragment order with the row permutation above, V^T as it lies in
 // the caller's tensor: key-contiguous rows, which is the fragment order of the p.v product; mask bias as fp32, -inf
 // for keys past the end, which is all the handling a ragged length needs), two stages, one barrier per chunk; the
-// pair bias is per (query, key) and comes straight from global memory, requested one chunk ahead.
+// pair bias is per (query, key): each wave fetches its own 32 x 64 tile one chunk ahead (through a private LDS panel).
 //
 // Placement: workgroup ids are dealt round robin over the 8 XCDs; the id is decoded so that each XCD works on groups of
 // 8 batch rows x 8 query blocks of one head at a time.  The 64 workgroups of a group sweep the keys roughly together,
