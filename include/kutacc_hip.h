@@ -270,9 +270,11 @@ kutacc_export int kutacc_hip_residual_add(void *acc, const void *delta, int64_t 
  * around the starting node (ending_node == 0: row i attends over j) or the ending node (ending_node != 0: the same
  * on the transposed pair tensor, result transposed back).  Four device passes on `stream`: LayerNorm + pair-bias
  * projection (one read of pair_act), mask bias, the attention operator, residual update.  bf16, head_size 32,
- * c_z = nheads * 32 in {128, 256}, n_res <= 1024 (the shapes of the MFMA attention kernels; otherwise
- * KUTACC_HIP_EUNSUPPORTED).  `workspace`: device memory, 256-byte aligned, at least
- * kutacc_hip_triangle_attention_workspace(n_res, nheads) bytes; contents unspecified afterwards.
+ * c_z = nheads * 32.  With c_z in {128, 256} and n_res <= 1024 (the shapes of the fused MFMA attention kernels) the
+ * mask bias and the residual update happen inside the operator: three launches.  Any other size runs the chain as
+ * separate passes with the operator on the tiled MFMA route (KUTACC_HIP_PATH_TILED), which needs four more
+ * activation-sized buffers -- the workspace function answers for the size it is asked about.  `workspace`: device memory,
+ * 256-byte aligned, at least kutacc_hip_triangle_attention_workspace(n_res, nheads) bytes; contents unspecified afterwards.
  */
 typedef struct kutacc_hip_triangle_attention_args {
     int64_t n_res;
@@ -385,7 +387,9 @@ kutacc_export int kutacc_hip_layernorm_rows_transposed(const void *x, const floa
  *   column != 0, column-wise: the same operator without pair bias on the msa with its leading axes exchanged, every
  *                residue attending over the sequences; no transposed copy of the msa is made (the LayerNorm reads it
  *                transposed, the output projection adds its result back transposed).
- * bf16; shapes of the MFMA attention kernels (c_m in {128, 256}, attended axis <= 1024), else KUTACC_HIP_EUNSUPPORTED.
+ * bf16.  With c_m in {128, 256} and an attended axis of at most 1024 (the shapes of the fused MFMA attention kernels) mask
+ * bias and residual update happen inside the operator; any other size runs them as passes of their own around the operator
+ * on the tiled MFMA route, with four more activation-sized buffers in the workspace.
  * pair_act [n_res, n_res, c_z], its LayerNorm parameters and bias_w [nheads, c_z] are read by the row-wise form only.
  */
 typedef struct kutacc_hip_msa_attention_args {

@@ -23,11 +23,13 @@ constexpr int64_t HEAD = 32;
 inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 struct Workspace {
-    int64_t z_norm, nb, bias, q, avg, total; // byte offsets
+    int64_t z_norm, nb, bias, q, avg, k, v, gate, out, total; // byte offsets (k .. out: the tiled route only)
 };
 
-// fused_ln: the head kernel normalises the rows of the pair tensor itself, so no normalised copy is kept
-Workspace layout(int64_t n, int64_t heads, bool fused_ln)
+// fused_ln: the head kernel normalises the rows of the pair tensor itself, so no normalised copy is kept.
+// tiled: rows beyond the fused head kernels (more than 1024 residues) -- the operator runs on the tiled MFMA route, which
+// forms k, v and gate in memory, and its result is added to the pair activation by a pass of its own.
+Workspace layout(int64_t n, int64_t heads, bool fused_ln, bool tiled = false)
 {
     const int64_t c = heads * HEAD, act = align256(n * n * c * 2);
     Workspace w;
@@ -36,7 +38,10 @@ Workspace layout(int64_t n, int64_t heads, bool fused_ln)
     w.bias = w.nb + align256(heads * n * n * 2);
     w.q = w.bias + align256(n * n * 2);
     w.avg = w.q + act;
-    w.total = w.avg + act;
+    w.k = w.v = w.gate = w.out = w.total = w.avg + act;
+    if (tiled) {
+        w.v = w.k + act, w.gate = w.v + act, w.out = w.gate + act, w.total = w.out + act;
+    }
     return w;
 }
 // Argument block of the attention call inside the triangle-attention block, on a workspace laid out by layout();
@@ -79,9 +84,37 @@ bool layernorm_policy_allows(int64_t)
     return kutacc_api::block_layernorm_mode() == 1;
 }
 
+// the operator's call with the scratch tensors and the separate result of the tiled route
+kutacc_hip_attention_args_t tiled_call(kutacc_hip_attention_args_t g, char *ws, int64_t k, int64_t v, int64_t gate, int64_t out,
+                                       int64_t bias, int64_t bias_stride_b)
+{
+    const int64_t c = g.nheads * g.head_size, m = g.batch * g.seq_len;
+    g.path = KUTACC_HIP_PATH_TILED;
+    g.bias = ws + bias, g.bias_stride_b = bias_stride_b; // the mask bias as a tensor of its own
+    g.k = ws + k, g.k_stride_b = g.seq_len * c, g.k_stride_s = c, g.k_stride_h = g.head_size;
+    g.gate = ws + gate, g.gate_stride_b = g.seq_len * c, g.gate_stride_s = c, g.gate_stride_h = g.head_size;
+    g.v = ws + v, g.v_stride_h = g.head_size * m, g.v_stride_e = m, g.v_stride_b = g.seq_len;
+    g.out = ws + out, g.out_ld = c;
+    return g;
+}
+
+// true where the fused head kernels do not take the block's attention call (asked with stand-in pointers)
+bool triangle_block_is_tiled(int64_t n, int64_t heads)
+{
+    kutacc_hip_triangle_attention_args_t a;
+    std::memset(&a, 0, sizeof(a));
+    char *fake = reinterpret_cast<char *>(uintptr_t(1) << 20);
+    a.n_res = n, a.nheads = heads, a.dtype = KUTACC_DTYPE_BF16;
+    a.pair_act = fake, a.pair_mask = fake;
+    a.query_w = a.key_w = a.value_w = a.gating_w = a.output_w = fake;
+    a.gating_b = a.output_b = reinterpret_cast<const float *>(fake);
+    const Workspace w = layout(n, heads, false);
+    return !kutacc_launch::fused_attention_supports(triangle_attention_call(&a, fake, w, false));
+}
+
 bool triangle_block_fuses_layernorm(int64_t n, int64_t heads)
 {
-    if (!layernorm_policy_allows(heads * HEAD)) {
+    if (!layernorm_policy_allows(heads * HEAD) || triangle_block_is_tiled(n, heads)) {
         return false;
     }
     kutacc_hip_triangle_attention_args_t a;
@@ -128,7 +161,7 @@ int64_t kutacc_hip_triangle_attention_workspace(int64_t n_res, int64_t nheads)
     if (n_res <= 0 || nheads <= 0 || n_res > 65536 || nheads > 64) {
         return -1;
     }
-    return layout(n_res, nheads, triangle_block_fuses_layernorm(n_res, nheads)).total;
+    return layout(n_res, nheads, triangle_block_fuses_layernorm(n_res, nheads), triangle_block_is_tiled(n_res, nheads)).total;
 }
 
 int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a, void *stream)
@@ -144,8 +177,8 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     // Where the persistent head kernel takes the call, it normalises the rows of the pair tensor itself (LayerNorm is
     // then the first link of the fused chain, and the workspace holds no normalised copy); elsewhere the producer below
     // writes one.
-    const bool fused_ln = triangle_block_fuses_layernorm(n, heads);
-    const Workspace w = layout(n, heads, fused_ln);
+    const bool fused_ln = triangle_block_fuses_layernorm(n, heads), tiled = triangle_block_is_tiled(n, heads);
+    const Workspace w = layout(n, heads, fused_ln, tiled);
     if (a->workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
         return KUTACC_HIP_EINVAL;
     }
@@ -154,6 +187,26 @@ int kutacc_hip_triangle_attention(const kutacc_hip_triangle_attention_args_t *a,
     const int ending = a->ending_node != 0;
 
     const kutacc_hip_attention_args_t g = triangle_attention_call(a, ws, w, fused_ln);
+    if (tiled) {
+        // Rows beyond the fused head kernels: the same chain as separate passes -- LayerNorm + pair bias (read transposed
+        // for the ending node), mask bias, the operator on the tiled MFMA route, residual sum (transposed back).
+        const kutacc_hip_attention_args_t t = tiled_call(g, ws, w.k, w.v, w.gate, w.out, w.bias, n);
+        if (!kutacc_launch::tiled_attention_supports(t)) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        int rc = kutacc_launch::pair_bias(a->pair_act, a->ln_gamma, a->ln_beta, a->bias_w, ws + w.nb, ws + w.z_norm, n, n, c, heads,
+                                          a->ln_eps, KUTACC_DTYPE_BF16, ending, s);
+        if (rc == 0) {
+            rc = kutacc_launch::mask_bias(a->pair_mask, ws + w.bias, n, n, ending, KUTACC_DTYPE_BF16, s);
+        }
+        if (rc == 0) {
+            rc = kutacc_launch::gating_attention_tiled(t, s);
+        }
+        if (rc == 0) {
+            rc = kutacc_launch::residual_add(a->pair_act, ws + w.out, n, n, c, ending, KUTACC_DTYPE_BF16, s);
+        }
+        return rc;
+    }
     if (!kutacc_launch::fused_attention_supports(g)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
@@ -383,11 +436,12 @@ int kutacc_hip_layernorm_rows_transposed(const void *x, const float *gamma, cons
 
 namespace {
 struct MsaWorkspace {
-    int64_t m_norm, nb, bias, q, avg, total;
+    int64_t m_norm, nb, bias, q, avg, k, v, gate, out, total; // (k .. out: the tiled route only)
 };
 
-// fused_ln: the head kernel normalises the msa rows itself, so no normalised copy is kept
-MsaWorkspace msa_layout(int64_t n_seq, int64_t n_res, int64_t heads, bool column, bool fused_ln)
+// fused_ln: the head kernel normalises the msa rows itself, so no normalised copy is kept; tiled: as for the
+// triangle-attention block
+MsaWorkspace msa_layout(int64_t n_seq, int64_t n_res, int64_t heads, bool column, bool fused_ln, bool tiled = false)
 {
     const int64_t act = align256(n_seq * n_res * heads * HEAD * 2);
     MsaWorkspace w;
@@ -396,7 +450,10 @@ MsaWorkspace msa_layout(int64_t n_seq, int64_t n_res, int64_t heads, bool column
     w.bias = w.nb + (column ? 0 : align256(heads * n_res * n_res * 2));
     w.q = w.bias + align256(n_seq * n_res * 2);
     w.avg = w.q + act;
-    w.total = w.avg + act;
+    w.k = w.v = w.gate = w.out = w.total = w.avg + act;
+    if (tiled) {
+        w.v = w.k + act, w.gate = w.v + act, w.out = w.gate + act, w.total = w.out + act;
+    }
     return w;
 }
 // Argument block of the attention call inside the MSA attention block (see triangle_attention_call)
@@ -430,9 +487,22 @@ kutacc_hip_attention_args_t msa_attention_call(const kutacc_hip_msa_attention_ar
     return g;
 }
 
+bool msa_block_is_tiled(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
+{
+    kutacc_hip_msa_attention_args_t a;
+    std::memset(&a, 0, sizeof(a));
+    char *fake = reinterpret_cast<char *>(uintptr_t(1) << 20);
+    a.n_seq = n_seq, a.n_res = n_res, a.nheads = heads, a.dtype = KUTACC_DTYPE_BF16, a.column = column ? 1 : 0;
+    a.msa_act = fake, a.msa_mask = fake;
+    a.query_w = a.key_w = a.value_w = a.gating_w = a.output_w = fake;
+    a.gating_b = a.output_b = reinterpret_cast<const float *>(fake);
+    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column, false);
+    return !kutacc_launch::fused_attention_supports(msa_attention_call(&a, fake, w, false));
+}
+
 bool msa_block_fuses_layernorm(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
 {
-    if (!layernorm_policy_allows(heads * HEAD)) {
+    if (!layernorm_policy_allows(heads * HEAD) || msa_block_is_tiled(n_seq, n_res, heads, column)) {
         return false;
     }
     kutacc_hip_msa_attention_args_t a;
@@ -453,7 +523,9 @@ int64_t kutacc_hip_msa_attention_workspace(int64_t n_seq, int64_t n_res, int64_t
     if (n_seq <= 0 || n_res <= 0 || nheads <= 0 || n_seq > 1 << 20 || n_res > 65536 || nheads > 64) {
         return -1;
     }
-    return msa_layout(n_seq, n_res, nheads, column != 0, msa_block_fuses_layernorm(n_seq, n_res, nheads, column != 0)).total;
+    return msa_layout(n_seq, n_res, nheads, column != 0, msa_block_fuses_layernorm(n_seq, n_res, nheads, column != 0),
+                      msa_block_is_tiled(n_seq, n_res, nheads, column != 0))
+        .total;
 }
 
 int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *stream)
@@ -471,14 +543,39 @@ int kutacc_hip_msa_attention(const kutacc_hip_msa_attention_args_t *a, void *str
     }
     const int64_t n_seq = a->n_seq, n_res = a->n_res, heads = a->nheads, c = heads * HEAD;
     // where the persistent head kernel takes the call it normalises the msa rows itself: no normalised copy, no LayerNorm pass
-    const bool fused_ln = msa_block_fuses_layernorm(n_seq, n_res, heads, column);
-    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column, fused_ln);
+    const bool fused_ln = msa_block_fuses_layernorm(n_seq, n_res, heads, column), tiled = msa_block_is_tiled(n_seq, n_res, heads, column);
+    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column, fused_ln, tiled);
     if (a->workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
         return KUTACC_HIP_EINVAL;
     }
     char *ws = static_cast<char *>(a->workspace);
     hipStream_t s = kutacc_api::stream_or_default(stream);
     const kutacc_hip_attention_args_t g = msa_attention_call(a, ws, w, fused_ln);
+    if (tiled) {
+        // Rows beyond the fused head kernels (more than 1024 keys): LayerNorm (read transposed column-wise), pair bias
+        // (row-wise), mask bias, the operator on the tiled MFMA route, residual sum (transposed back column-wise).
+        const int64_t batch = column ? n_res : n_seq, seq = column ? n_seq : n_res;
+        const kutacc_hip_attention_args_t t = tiled_call(g, ws, w.k, w.v, w.gate, w.out, w.bias, seq);
+        if (!kutacc_launch::tiled_attention_supports(t)) {
+            return KUTACC_HIP_EUNSUPPORTED;
+        }
+        int rc = kutacc_launch::layernorm_rows(a->msa_act, c, a->ln_gamma, a->ln_beta, ws + w.m_norm, c, n_seq * n_res, c, a->ln_eps,
+                                               KUTACC_DTYPE_BF16, s, column ? n_seq : 0);
+        if (rc == 0 && !column) {
+            rc = kutacc_launch::pair_bias(a->pair_act, a->pair_ln_gamma, a->pair_ln_beta, a->bias_w, ws + w.nb, nullptr, n_res, n_res,
+                                          a->c_z, heads, a->ln_eps, KUTACC_DTYPE_BF16, 0, s);
+        }
+        if (rc == 0) {
+            rc = kutacc_launch::mask_bias(a->msa_mask, ws + w.bias, batch, seq, column ? 1 : 0, KUTACC_DTYPE_BF16, s);
+        }
+        if (rc == 0) {
+            rc = kutacc_launch::gating_attention_tiled(t, s);
+        }
+        if (rc == 0) {
+            rc = kutacc_launch::residual_add(a->msa_act, ws + w.out, n_seq, n_res, c, column ? 1 : 0, KUTACC_DTYPE_BF16, s);
+        }
+        return rc;
+    }
     if (!kutacc_launch::fused_attention_supports(g)) {
         return KUTACC_HIP_EUNSUPPORTED;
     }

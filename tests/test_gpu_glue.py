@@ -260,6 +260,35 @@ def test_triangle_attention_block_full_size_sampled_rows(torch_cuda, n):
         helpers.check_close(helpers.to_numpy(sample.contiguous()), want, "bf16", f"block n={n} ending={ending}, sampled rows")
 
 
+def test_triangle_attention_block_beyond_1024_residues(torch_cuda):
+    """1088 residues: past the fused head kernels' longest row, the block runs the same chain as separate passes with the
+    operator on the tiled MFMA route.  Both orientations against the oracle on a sample of attention rows."""
+    torch = torch_cuda
+    n = 1088
+    c = block_case(9100, n, 4)
+    rows = sorted({0, 1, 31, 32, 127, 128, n // 2, n - 65, n - 64, n - 2, n - 1})
+    assert capi.lib().kutacc_hip_triangle_attention_workspace(n, 4) > capi.lib().kutacc_hip_triangle_attention_workspace(1024, 4) * 2
+    for ending in (False, True):
+        res = {}
+        names = profiled_kernels(torch, lambda: res.setdefault("z", run_block(torch, c, ending)))
+        got = res["z"]
+        assert "attention_tiles_kernel" in names and "residual_add_kernel" in names, names
+        assert bool(torch.isfinite(got).all())
+        want = block_oracle_rows(c, ending, rows)
+        sample = got[:, rows].transpose(0, 1) if ending else got[rows]
+        helpers.check_close(helpers.to_numpy(sample.contiguous()), want, "bf16", f"block n={n} ending={ending}, sampled rows")
+
+
+@pytest.mark.parametrize("n,heads", [(72, 3), (100, 5), (45, 1)])
+def test_triangle_attention_block_with_other_channel_counts(torch_cuda, n, heads):
+    """96, 160 and 32 channels (heads of 32): no fused head kernel takes them, the block's tiled route does; whole result
+    against the oracle's composition, both orientations, lengths that are and are not multiples of 8."""
+    for ending in (False, True):
+        c = block_case(9200 + n, n, heads)
+        got = run_block(torch_cuda, c, ending)
+        helpers.check_close(helpers.to_numpy(got), block_oracle(c, ending), "bf16", f"block n={n} heads={heads} ending={ending}")
+
+
 def test_fused_layernorm_drops_the_normalised_copy_from_the_workspace(torch_cuda):
     """With the LayerNorm inside the attention kernel the blocks keep no normalised activation: the workspace is one
     activation smaller wherever the persistent kernel runs (384 residues), and unchanged where it does not (1024)."""
@@ -622,6 +651,27 @@ def test_pair_stack_blocks_replay_from_a_hip_graph(torch_cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert helpers.same_bits(z, want)
+
+
+@pytest.mark.parametrize("column,n_seq,n_res,heads", [(True, 1088, 24, 8), (False, 20, 1040, 8), (False, 24, 56, 3), (True, 40, 24, 5)])
+def test_msa_attention_blocks_on_the_tiled_route(torch_cuda, column, n_seq, n_res, heads):
+    """Attention rows of more than 1024 keys (column-wise over 1088 sequences, row-wise over 1040 residues) and channel
+    counts other than 128 and 256: the block's separate passes with the operator on the tiled MFMA route, whole result
+    against the oracle's composition."""
+    torch = torch_cuda
+    c = msa_case(9300 + n_seq + n_res, n_seq, n_res, heads, 128)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    msa = dev(c["m"])
+    w = {k: dev(c[k]) for k in ("ln_gamma", "ln_beta", "wq", "wk", "wv", "wg", "bg", "wo", "bo")}
+    pair = None if column else {"pair_act": dev(c["z"]), "pair_ln_gamma": dev(c["pair_ln_gamma"]),
+                                "pair_ln_beta": dev(c["pair_ln_beta"]), "bias_w": dev(c["bias_w"])}
+    blk = capi.MsaAttentionBlock(msa, dev(c["mask"]), w, heads, pair)
+    res = {}
+    names = profiled_kernels(torch, lambda: res.setdefault("rc", blk.run()))
+    torch.cuda.synchronize()
+    assert res["rc"] == 0 and "attention_tiles_kernel" in names, (res, names)
+    helpers.check_close(helpers.to_numpy(msa), msa_oracle(c, column), "bf16", f"msa block {n_seq}x{n_res} heads={heads} column={column}")
 
 
 def test_msa_attention_blocks_full_size_sampled_rows(torch_cuda):
