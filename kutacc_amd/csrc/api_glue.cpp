@@ -98,19 +98,15 @@ kutacc_hip_attention_args_t tiled_call(kutacc_hip_attention_args_t g, char *ws, 
     return g;
 }
 
-// true where the fused head kernels do not take the block's attention call (asked with stand-in pointers)
-bool triangle_block_is_tiled(int64_t n, int64_t heads)
+// The sizes the fused head kernels are written for (fused_attention_supports asks the same of the shape, and more of the
+// pointers): blocks of any other size take the tiled route.  By shape alone, so that the workspace functions answer the
+// same with and without a device.
+bool beyond_fused_kernels(int64_t seq_len, int64_t heads)
 {
-    kutacc_hip_triangle_attention_args_t a;
-    std::memset(&a, 0, sizeof(a));
-    char *fake = reinterpret_cast<char *>(uintptr_t(1) << 20);
-    a.n_res = n, a.nheads = heads, a.dtype = KUTACC_DTYPE_BF16;
-    a.pair_act = fake, a.pair_mask = fake;
-    a.query_w = a.key_w = a.value_w = a.gating_w = a.output_w = fake;
-    a.gating_b = a.output_b = reinterpret_cast<const float *>(fake);
-    const Workspace w = layout(n, heads, false);
-    return !kutacc_launch::fused_attention_supports(triangle_attention_call(&a, fake, w, false));
+    const int64_t c = heads * HEAD;
+    return (c != 128 && c != 256) || seq_len > 1024;
 }
+bool triangle_block_is_tiled(int64_t n, int64_t heads) { return beyond_fused_kernels(n, heads); }
 
 bool triangle_block_fuses_layernorm(int64_t n, int64_t heads)
 {
@@ -489,15 +485,7 @@ kutacc_hip_attention_args_t msa_attention_call(const kutacc_hip_msa_attention_ar
 
 bool msa_block_is_tiled(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
 {
-    kutacc_hip_msa_attention_args_t a;
-    std::memset(&a, 0, sizeof(a));
-    char *fake = reinterpret_cast<char *>(uintptr_t(1) << 20);
-    a.n_seq = n_seq, a.n_res = n_res, a.nheads = heads, a.dtype = KUTACC_DTYPE_BF16, a.column = column ? 1 : 0;
-    a.msa_act = fake, a.msa_mask = fake;
-    a.query_w = a.key_w = a.value_w = a.gating_w = a.output_w = fake;
-    a.gating_b = a.output_b = reinterpret_cast<const float *>(fake);
-    const MsaWorkspace w = msa_layout(n_seq, n_res, heads, column, false);
-    return !kutacc_launch::fused_attention_supports(msa_attention_call(&a, fake, w, false));
+    return beyond_fused_kernels(column ? n_seq : n_res, heads);
 }
 
 bool msa_block_fuses_layernorm(int64_t n_seq, int64_t n_res, int64_t heads, bool column)
