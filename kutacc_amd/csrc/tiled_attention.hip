@@ -213,28 +213,30 @@ __global__ __launch_bounds__(256, 2) void attention_tiles_kernel(const TileParam
         }
         reinterpret_cast<float *>(stage + K_SLOTS + V_SLOTS)[tid & (CHUNK - 1)] = bias_keep ? to_f32(bias_raw) * LOG2E : -INFINITY;
     };
-    // Pair bias of the wave's 32 queries for the 64 keys of chunk c: 32 rows x 128 bytes.  Read as whole rows (a load
-    // instruction covers 8 rows x 128 contiguous bytes: 8 cache lines; a lane fetching the 16 bytes of its own query for
-    // its own keys would touch 32 lines per instruction, a quarter of each) and passed through a wave-private LDS panel,
-    // from which each lane takes its query's keys in accumulator order.  Rows past the last query repeat it.
-    uint4 *nb_panel = lds + 2 * STAGE_SLOTS + wave * 256;
-    const bf16_t *nb_head = HAS_NB ? p.nb + (int64_t)h * p.nb_sh : nullptr;
-    auto fetch_nb = [&](int c, auto plain_tag) -> PanelRegs {
+    // Pair bias of this lane's query for the keys of chunk c, in accumulator order: [key block][j] holds keys
+    // 32 kb + 16 j + 8 g .. + 7.  Straight from global memory into registers: a load instruction touches 32 rows, a quarter
+    // of a cache line each, and the other three loads touch the same lines again -- but the LDS is what bounds this kernel
+    // (a wave-private panel filled with whole rows and read back in this order costs 8 KB of LDS traffic per wave and
+    // chunk, a third more than everything else together).
+    struct NbRegs {
+        uint4 v[2][2];
+    };
+    auto fetch_nb = [&](int c, auto plain_tag) -> NbRegs {
         constexpr bool PLAIN = decltype(plain_tag)::value;
-        PanelRegs f = {zero_u4(), zero_u4(), zero_u4(), zero_u4()};
-        if constexpr (HAS_NB) {
-            const int kc0 = c * CHUNK;
-            if constexpr (PLAIN) {
-                return panel_load(nb_head, p.nb_sq, q0 < S ? q0 : S - 1, S - 1, kc0, lane);
-            }
-            const int key = kc0 + 8 * (lane & 7);
-            if (key < S) {
-                uint4 *dst[4] = {&f.r0, &f.r1, &f.r2, &f.r3};
+        NbRegs f;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int row = q0 + 8 * i + (lane >> 3);
-                    const bf16_t *src = nb_head + (int64_t)(row < S ? row : S - 1) * p.nb_sq + key;
-                    *dst[i] = (p.nb_vec && key + 8 <= S) ? *reinterpret_cast<const uint4 *>(src) : load8_checked(src, S - key);
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                f.v[kb][j] = zero_u4();
+                if constexpr (HAS_NB) {
+                    const int key = c * CHUNK + 32 * kb + 16 * j + 8 * g;
+                    if constexpr (PLAIN) {
+                        f.v[kb][j] = *reinterpret_cast<const uint4 *>(nb_row + key);
+                    } else if (key < S) {
+                        f.v[kb][j] = (p.nb_vec && key + 8 <= S) ? *reinterpret_cast<const uint4 *>(nb_row + key)
+                                                                : load8_checked(nb_row + key, S - key);
+                    }
                 }
             }
         }
@@ -256,18 +258,15 @@ __global__ __launch_bounds__(256, 2) void attention_tiles_kernel(const TileParam
             oacc[db] = zero16();
         }
         m_run = -INFINITY, l_run = 0.f;
-        PanelRegs nb_next;
+        NbRegs nb_cur, nb_next;
         // chunks [0, plain) take the PLAIN loads
         const int plain = (p.v_vec && (!HAS_NB || p.nb_vec)) ? S / CHUNK : 0;
         if (plain > 0) {
             fetch(0, std::true_type{});
-            nb_next = fetch_nb(0, std::true_type{});
+            nb_cur = fetch_nb(0, std::true_type{});
         } else {
             fetch(0, std::false_type{});
-            nb_next = fetch_nb(0, std::false_type{});
-        }
-        if constexpr (HAS_NB) {
-            panel_store(nb_panel, lane, nb_next);
+            nb_cur = fetch_nb(0, std::false_type{});
         }
         park(lds);
         __syncthreads();
@@ -296,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiles_kernel(const TileParam
                     for (int j = 0; j < 2; ++j) {
                         const f32x4 b0 = *reinterpret_cast<const f32x4 *>(mask_bias + 32 * kb + 16 * j + 8 * g);
                         const f32x4 b1 = *reinterpret_cast<const f32x4 *>(mask_bias + 32 * kb + 16 * j + 8 * g + 4);
-                        const bf16x8 nbv = as_bf16x8(HAS_NB ? nb_panel[panel_slot(r, 4 * kb + 2 * j + g)] : zero_u4());
+                        const bf16x8 nbv = as_bf16x8(nb_cur.v[kb][j]);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) {
                             float v = fmaf(x[kb][8 * j + e], scale2, e < 4 ? b0[e & 3] : b1[e & 3]);
@@ -346,9 +345,7 @@ __global__ __launch_bounds__(256, 2) void attention_tiles_kernel(const TileParam
             }
             if (more) {
                 park(lds + ((c + 1) & 1) * STAGE_SLOTS); // its last readers passed the barrier that ended the previous chunk
-                if constexpr (HAS_NB) {
-                    panel_store(nb_panel, lane, nb_next); // wave-private, and behind this wave's reads of the chunk just done
-                }
+                nb_cur = nb_next;
             }
             __syncthreads();
         };
@@ -401,7 +398,7 @@ template <int KS, bool HAS_NB>
 hipError_t launch_tiles(const TileParams &p, int64_t blocks, hipStream_t stream)
 {
     constexpr int DB = (KS + 1) / 2;
-    constexpr size_t lds_bytes = (2 * (2 * KS * 64 + DB * 4 * 64 + CHUNK / 4) + (HAS_NB ? 4 * 256 : 0)) * 16;
+    constexpr size_t lds_bytes = 2 * (2 * KS * 64 + DB * 4 * 64 + CHUNK / 4) * 16;
     static_assert(lds_bytes <= 64 * 1024, "two stages fit the LDS a kernel may use without opting in");
     attention_tiles_kernel<KS, HAS_NB><<<dim3((unsigned)blocks), 256, lds_bytes, stream>>>(p);
     return hipGetLastError();
