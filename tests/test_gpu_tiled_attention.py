@@ -78,6 +78,53 @@ def test_rows_longer_than_1024_positions(torch_cuda, B, S, H, d):
     run_and_check(w, capi.PATH_AUTO)
 
 
+@pytest.mark.parametrize("B,S,H,d", [(2048, 2048, 4, 32), (5120, 384, 8, 8)])
+def test_benchmarked_shapes_on_sampled_rows(torch_cuda, B, S, H, d):
+    """The shapes `bench.py --tiled-route` times (triangle attention at 2048 residues, the extra-MSA row attention), drawn
+    on the device: the oracle on a sample of batch rows -- first and last, both sides of the 8-row groups the kernel's
+    placement forms, one fully masked -- and finiteness of every other entry."""
+    import ctypes
+    torch = torch_cuda
+    C = H * d
+    g = torch.Generator(device="cuda").manual_seed(4000 + S)
+    bf = lambda *sh, scale=1.0: (torch.randn(*sh, device="cuda", generator=g) * scale).to(torch.bfloat16)  # noqa: E731
+    x = torch.nn.functional.layer_norm(torch.randn(B, S, C, device="cuda", generator=g), (C,)).to(torch.bfloat16)
+    ws = [bf(C, C, scale=C ** -0.5) for _ in range(5)]
+    bg, bo = torch.ones(C, device="cuda"), torch.randn(C, device="cuda", generator=g) * 0.1
+    keep = torch.rand(B, S, device="cuda", generator=g) >= 0.1
+    keep[:, 0] = True
+    bias = ((~keep).float() * MASK_BIAS).to(torch.bfloat16)
+    rows = sorted({0, 1, 7, 8, 9, B // 2 - 1, B // 2, B - 9, B - 8, B - 2, B - 1})
+    bias[rows[3], :] = MASK_BIAS  # a fully masked row: a uniform average
+    nb = bf(H, S, S)
+    out = torch.empty(B, S, C, device="cuda", dtype=torch.bfloat16)
+    q, k, gate, avg = (torch.empty(B, S, C, device="cuda", dtype=torch.bfloat16) for _ in range(4))
+    v = torch.empty(C, B * S, device="cuda", dtype=torch.bfloat16)
+    a = capi.HipAttentionArgs()
+    a.batch, a.seq_len, a.nheads, a.head_size, a.dtype, a.path = B, S, H, d, capi.K_BF16, capi.PATH_AUTO
+    a.input, a.input_ld = x.data_ptr(), C
+    a.query_w, a.key_w, a.value_w, a.gating_w, a.output_w = (w.data_ptr() for w in ws)
+    a.gating_b, a.output_b = bg.data_ptr(), bo.data_ptr()
+    a.bias, a.bias_stride_b = bias.data_ptr(), S
+    a.nonbatched_bias, a.nb_stride_h, a.nb_stride_q = nb.data_ptr(), S * S, S
+    a.q, a.k, a.v, a.gate, a.avg = q.data_ptr(), k.data_ptr(), v.data_ptr(), gate.data_ptr(), avg.data_ptr()
+    for n in ("q", "k", "gate", "avg"):
+        setattr(a, f"{n}_stride_b", S * C), setattr(a, f"{n}_stride_s", C), setattr(a, f"{n}_stride_h", d)
+    a.v_stride_h, a.v_stride_e, a.v_stride_b = d * B * S, B * S, S
+    a.out, a.out_ld = out.data_ptr(), C
+    print(f"B={B} S={S} H={H} d={d}", flush=True)
+    assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None) == 0
+    torch.cuda.synchronize()
+    assert capi.last_path() == "tiled_mfma"
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(avg).all())
+    from oracle import oracle
+    num = lambda t: helpers.to_numpy(t)  # noqa: E731
+    ref_out, ref_avg = oracle.gating_attention_f32(num(x[rows]), *(num(w) for w in ws[:4]), num(bg), num(ws[4]), num(bo),
+                                                   num(bias[rows]), num(nb), H, return_avg=True)
+    helpers.check_close(num(avg[rows]), ref_avg, "bf16", f"gated average, sampled rows of B={B} S={S}")
+    helpers.check_close(num(out[rows]), ref_out, "bf16", f"out, sampled rows of B={B} S={S}")
+
+
 def test_without_pair_bias_and_with_fully_masked_rows(torch_cuda):
     w = draw_workload(5, 4, 300, 8, 8, pair_bias=False)
     w.bias[1, :] = round_to_bf16(np.full(w.S, MASK_BIAS, dtype=np.float32))  # every key of row 1 masked: a uniform average
