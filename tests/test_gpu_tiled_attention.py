@@ -183,6 +183,32 @@ def test_leaves_q_k_v_gate_as_the_reference_does(torch_cuda):
     helpers.check_close(helpers.to_numpy(scratch["v"]), oracle.from_bf16_bits(ref["v"]), "bf16", "v")
 
 
+def test_replays_from_a_hip_graph(torch_cuda):
+    """The route's seven launches (five products, the attention, nothing that allocates, clears memory or synchronises)
+    captured into a HIP graph on a side stream and replayed three times, with eager work between the replays (the results
+    and the scratch tensors overwritten); every replay reproduces the eager result bit for bit."""
+    import ctypes
+    torch = torch_cuda
+    w = draw_workload(21, 5, 200, 8, 8)
+    ten, scratch = helpers.to_device(w)
+    a = helpers.hip_args(w, ten, scratch, capi.PATH_TILED)
+    assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), None) == 0  # eager: also takes first-call set-up out of the capture
+    torch.cuda.synchronize()
+    want_out, want_avg = ten["out"].clone(), scratch["avg"].clone()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert capi.lib().kutacc_hip_gating_attention(ctypes.byref(a), torch.cuda.current_stream().cuda_stream) == 0
+    for _ in range(3):
+        ten["out"].fill_(7.0)
+        for t in scratch.values():
+            t.fill_(-3.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert helpers.same_bits(ten["out"], want_out) and helpers.same_bits(scratch["avg"], want_avg)
+
+
 def test_unsupported_layouts_fall_back_to_the_generic_kernels(torch_cuda):
     """A head size that is no multiple of 8 is not this route's: the automatic choice takes the scalar kernels, the forced
     routes refuse."""
