@@ -91,7 +91,7 @@ __device__ __forceinline__ float pair_sums(bf16x8 v, float acc)
 // workgroup stages each chunk of 64 keys once (K in fragment order with the row permutation above, V^T as it lies in
 // the caller's tensor: key-contiguous rows, which is the fragment order of the p.v product; mask bias as fp32, -inf
 // for keys past the end, which is all the handling a ragged length needs), two stages, one barrier per chunk; the
-// pair bias is per (query, key): each wave fetches its own 32 x 64 tile one chunk ahead (through a private LDS panel).
+// pair bias is per (query, key): each lane fetches its own query's keys into registers, one chunk ahead.
 //
 // Placement: workgroup ids are dealt round robin over the 8 XCDs; the id is decoded so that each XCD works on groups of
 // 8 batch rows x 8 query blocks of one head at a time.  The 64 workgroups of a group sweep the keys roughly together,
@@ -215,9 +215,8 @@ __global__ __launch_bounds__(256, 2) void attention_tiles_kernel(const TileParam
     };
     // Pair bias of this lane's query for the keys of chunk c, in accumulator order: [key block][j] holds keys
     // 32 kb + 16 j + 8 g .. + 7.  Straight from global memory into registers: a load instruction touches 32 rows, a quarter
-    // of a cache line each, and the other three loads touch the same lines again -- but the LDS is what bounds this kernel
-    // (a wave-private panel filled with whole rows and read back in this order costs 8 KB of LDS traffic per wave and
-    // chunk, a third more than everything else together).
+    // of a cache line each, and the other three loads touch the same lines again.  (Whole 128-byte rows through a
+    // wave-private LDS panel, read back in this order, measured the same and cost 8 KB of LDS traffic per wave and chunk.)
     struct NbRegs {
         uint4 v[2][2];
     };
