@@ -1609,7 +1609,9 @@ __global__ __launch_bounds__(64) void pair_bias_tiles_kernel(const bf16_t *__res
 //                     lane's accumulator row stands for; one more MFMA per tile adds them (WITH_MASK only)
 //   nbc             : fp32 pair-bias tiles of this head and query block, offset by the lane: tile t, piece a at
 //                     nbc[(4 t + a) * 64]; nullptr without a pair bias
-template <bool HAS_NB, bool WITH_MASK>
+//   MFMA_SUMS       : the row sums on the matrix pipe (one 16x16x32 MFMA per 16 keys and row) instead of four dot products
+//                     on the vector ALU; costs ten more registers, which the 256-channel kernel (two waves per SIMD) has
+template <bool HAS_NB, bool WITH_MASK, bool MFMA_SUMS>
 __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 *lds_vA, const uint4 *lds_kB, const uint4 *lds_vB,
                                                const uint32_t *mwA, const uint32_t *mwB, const f32x4 *nbc, bf16x8 qA0, bf16x8 qA1,
                                                bf16x8 qB0, bf16x8 qB1, int NB, int lane, f32x16 &oA_out,
@@ -1659,6 +1661,15 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     v0 = vA[0], v1 = vA[64];
     f32x16 oA = zero16(), oB = zero16();
     float lsumA = 0.f, lsumB = 0.f; // this lane's share of the row sums; the two halves of the wave are added at the end
+    // MFMA_SUMS: the probability fragment of a k-step (lane q + 32 g: query q, keys 8 g .. 8 g + 7) read as the B operand
+    // of a 16x16x32 product is column q % 16, k-group q / 16 + 2 g.  With A = ones in row 0 for k-groups 0 and 2 and in
+    // row 1 for k-groups 1 and 3 (lanes 0 and 32, 17 and 49 of the operand; zero elsewhere), row 0 of the result sums
+    // the 16 keys for queries 0 .. 15 and row 1 for queries 16 .. 31: lane q % 16, register q / 16.
+    f32x4 sumsA = {0.f, 0.f, 0.f, 0.f}, sumsB = {0.f, 0.f, 0.f, 0.f};
+    const bool ones_lane = lane == 0 || lane == 32 || lane == 17 || lane == 49;
+    const uint32_t ones_word = ones_lane ? 0x3f803f80u : 0u;
+    const uint4 ones_rows4 = {ones_word, ones_word, ones_word, ones_word};
+    const bf16x8 ones_rows = as_bf16x8(ones_rows4);
     bf16x2 one2;
     one2[0] = (bf16_t)1.0f, one2[1] = (bf16_t)1.0f;
     // Probabilities -> bf16 by truncation: one byte permute per pair of values where the rounding conversion is a slower
@@ -1674,7 +1685,11 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     };
     // row sums on the vector ALU, two probabilities per dot2: with two rows in flight the row-sum MFMAs of
     // attend_block_l2 (a selector fragment and an accumulator per row) cost more registers than the loop has
-    auto rowsum = [&](float &lsum, bf16x8 pv) {
+    auto rowsum = [&](float &lsum, f32x4 &sums, bf16x8 pv) {
+        if constexpr (MFMA_SUMS) {
+            sums = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones_rows, pv, sums, 0, 0, 0);
+            return;
+        }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             bf16x2 a;
@@ -1695,8 +1710,8 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     // that reads it: the compiler then writes xn to registers of its own (D != C) instead of computing it in place in
     // C's registers, which rotated the roles of the register blocks from one iteration to the next and cost 40 copies
     // per iteration, behind a wait for every load in flight.
-    auto half_step = [&](f32x16 &xc, f32x16 &xn, const f32x16 &C, bf16x8 q0, bf16x8 q1, f32x16 &o, float &lsum, const uint4 *knext,
-                         const uint32_t *mw_next, int t_next) {
+    auto half_step = [&](f32x16 &xc, f32x16 &xn, const f32x16 &C, bf16x8 q0, bf16x8 q1, f32x16 &o, float &lsum, f32x4 &sums,
+                         const uint4 *knext, const uint32_t *mw_next, int t_next) {
         bf16x8 p0, p1;
         const bf16x8 mnext = mask_fragment(mw_next, t_next); // requested first, used by the last MFMA of the step
         exp4(xc, 0);
@@ -1710,12 +1725,12 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
         if constexpr (WITH_MASK) {
             xn = mfma(mnext, onesf, xn);
         }
-        rowsum(lsum, p0);
+        rowsum(lsum, sums, p0);
         k0 = knext[0], k1 = knext[64];
         exp4(xc, 12);
         p1 = pack_trunc(xc, 8);
         o = mfma(as_bf16x8(v1), p1, o);
-        rowsum(lsum, p1);
+        rowsum(lsum, sums, p1);
     };
     for (int pair = 0; pair < npairs; ++pair) {
         if (turn >= 0) {
@@ -1724,27 +1739,34 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
         const int t0 = 2 * pair, t1 = t0 + 1;
         const int tn = pair + 1 < npairs ? t0 + 2 : t0; // next pair's first tile, clamped
         // (A, t0) finished; logits of (B, t0) from C0
-        half_step(xa, xb, C0, qB0, qB1, oA, lsumA, kA + t1 * 128, mwB, t0);
+        half_step(xa, xb, C0, qB0, qB1, oA, lsumA, sumsA, kA + t1 * 128, mwB, t0);
         v0 = vB[t0 * 128], v1 = vB[t0 * 128 + 64];
         fence(); // the loads stay behind the last reader of the registers they fill
         C0 = loadC(clampt(t0 + 2));
         fence();
         // (B, t0) finished; logits of (A, t1) from C1
-        half_step(xb, xa, C1, qA0, qA1, oB, lsumB, kB + t1 * 128, mwA, t1);
+        half_step(xb, xa, C1, qA0, qA1, oB, lsumB, sumsB, kB + t1 * 128, mwA, t1);
         v0 = vA[t1 * 128], v1 = vA[t1 * 128 + 64];
         // (A, t1) finished; logits of (B, t1) from C1
-        half_step(xa, xb, C1, qB0, qB1, oA, lsumA, kA + tn * 128, mwB, t1);
+        half_step(xa, xb, C1, qB0, qB1, oA, lsumA, sumsA, kA + tn * 128, mwB, t1);
         v0 = vB[t1 * 128], v1 = vB[t1 * 128 + 64];
         fence();
         C1 = loadC(clampt(t1 + 2));
         fence();
         // (B, t1) finished; logits of (A, tn) from C0
-        half_step(xb, xa, C0, qA0, qA1, oB, lsumB, kB + tn * 128, mwA, tn);
+        half_step(xb, xa, C0, qA0, qA1, oB, lsumB, sumsB, kB + tn * 128, mwA, tn);
         v0 = vA[tn * 128], v1 = vA[tn * 128 + 64];
     }
     __builtin_amdgcn_s_setprio(0);
     oA_out = oA, oB_out = oB;
-    lA_out = half_swap_sum(lsumA), lB_out = half_swap_sum(lsumB);
+    if constexpr (MFMA_SUMS) {
+        const int src = lane & 15, upper = (lane >> 4) & 1;
+        const float a0 = __shfl(sumsA[0], src, 64), a1 = __shfl(sumsA[1], src, 64);
+        const float b0 = __shfl(sumsB[0], src, 64), b1 = __shfl(sumsB[1], src, 64);
+        lA_out = upper ? a1 : a0, lB_out = upper ? b1 : b0;
+    } else {
+        lA_out = half_swap_sum(lsumA), lB_out = half_swap_sum(lsumB);
+    }
 }
 
 // The repeat of one row's block after an overflow or underflow of the unshifted exponentials, with the pair bias as fp32
@@ -1815,6 +1837,9 @@ template <int C, bool HAS_NB>
 __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_pair_kernel(FusedParams p)
 {
     constexpr int CK = C / 16;
+    // the row sums on the matrix pipe where the registers are there: with 256 channels (two waves per SIMD) always, with
+    // 128 (three) in the loop without mask products only -- the masked loop spills with them
+    constexpr bool PAIR_MFMA_SUMS = C == 256;
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1998,9 +2023,9 @@ __global__ __launch_bounds__(64 * max_waves(C, 1)) void persistent_pair_kernel(F
         f32x16 oA, oB;
         float lA, lB;
         if ((flagsA | flagsB) == 0u) {
-            attend_pair_l2<HAS_NB, false>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, fair_turn);
+            attend_pair_l2<HAS_NB, false, true>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, fair_turn);
         } else {
-            attend_pair_l2<HAS_NB, true>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, fair_turn);
+            attend_pair_l2<HAS_NB, true, PAIR_MFMA_SUMS>(kA, vA, kB, vB, mwA, mwB, nbc, qA0, qA1, qB0, qB1, NT, lane_a, oA, lA, oB, lB, fair_turn);
         }
         // some probability overflowed or a whole row underflowed: repeat that row shifted by its true row maxima
         if (__any(!(lA > 1e-30f && lA < 1e30f))) {
