@@ -1661,15 +1661,10 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     v0 = vA[0], v1 = vA[64];
     f32x16 oA = zero16(), oB = zero16();
     float lsumA = 0.f, lsumB = 0.f; // this lane's share of the row sums; the two halves of the wave are added at the end
-    // MFMA_SUMS: the probability fragment of a k-step (lane q + 32 g: query q, keys 8 g .. 8 g + 7) read as the B operand
-    // of a 16x16x32 product is column q % 16, k-group q / 16 + 2 g.  With A = ones in row 0 for k-groups 0 and 2 and in
-    // row 1 for k-groups 1 and 3 (lanes 0 and 32, 17 and 49 of the operand; zero elsewhere), row 0 of the result sums
-    // the 16 keys for queries 0 .. 15 and row 1 for queries 16 .. 31: lane q % 16, register q / 16.
+    // MFMA_SUMS: as in attend_block_l2 -- rowsum_selector's A operand sums the keys of each query in a 16x16x32 product
+    // fed with the probability fragment; the sums of queries n and n + 16 end up in lane n, registers 0 and 1
     f32x4 sumsA = {0.f, 0.f, 0.f, 0.f}, sumsB = {0.f, 0.f, 0.f, 0.f};
-    const bool ones_lane = lane == 0 || lane == 32 || lane == 17 || lane == 49;
-    const uint32_t ones_word = ones_lane ? 0x3f803f80u : 0u;
-    const uint4 ones_rows4 = {ones_word, ones_word, ones_word, ones_word};
-    const bf16x8 ones_rows = as_bf16x8(ones_rows4);
+    const bf16x8 ones_rows = rowsum_selector(lane);
     bf16x2 one2;
     one2[0] = (bf16_t)1.0f, one2[1] = (bf16_t)1.0f;
     // Probabilities -> bf16 by truncation: one byte permute per pair of values where the rounding conversion is a slower
@@ -1760,10 +1755,7 @@ __device__ __forceinline__ void attend_pair_l2(const uint4 *lds_kA, const uint4 
     __builtin_amdgcn_s_setprio(0);
     oA_out = oA, oB_out = oB;
     if constexpr (MFMA_SUMS) {
-        const int src = lane & 15, upper = (lane >> 4) & 1;
-        const float a0 = __shfl(sumsA[0], src, 64), a1 = __shfl(sumsA[1], src, 64);
-        const float b0 = __shfl(sumsB[0], src, 64), b1 = __shfl(sumsB[1], src, 64);
-        lA_out = upper ? a1 : a0, lB_out = upper ? b1 : b0;
+        lA_out = rowsum_fetch(sumsA, lane), lB_out = rowsum_fetch(sumsB, lane);
     } else {
         lA_out = half_swap_sum(lsumA), lB_out = half_swap_sum(lsumB);
     }
