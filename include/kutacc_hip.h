@@ -451,10 +451,11 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *   "row_pairs" "0": never the attention kernel that walks two batch rows per step (128 channels up to 384 positions,
  *               256 channels up to 256);
  *               "1": wherever it can run; anything else (default): where every workgroup has at least two batch rows
- *   "gemm_tile" "128" / "256" / "192": the batched products of kutacc_af2_triangle_multiplication_equation always on
- *               128 x 128 tiles / on 256 x 256 tiles wherever the shape has whole ones / on 192 x 192 tiles wherever it
- *               has; anything else (default): 256 x 256 where every CU gets at least four tiles, else 192 x 192 where
- *               every CU gets at least two, else 128 x 128
+ *   "gemm_tile" "128" / "256" / "192" / "direct": the batched products of kutacc_af2_triangle_multiplication_equation
+ *               always on 128 x 128 tiles / on 256 x 256 tiles staged through registers wherever the shape has whole
+ *               ones / on 192 x 192 tiles wherever it has / on 256 x 256 tiles whose operands are loaded straight into
+ *               the LDS wherever it has (and k is at least 96); anything else (default): the direct 256 x 256 tiles
+ *               where every CU gets at least two, else 192 x 192 where every CU gets at least two, else 128 x 128
  *   "layernorm" "fused": kutacc_hip_triangle_attention and kutacc_hip_msa_attention let the attention kernel normalise its
  *               input rows itself where it can (sequence lengths of the persistent kernel), which drops the normalised
  *               copy from the workspace and costs 8-15 % of the block's time; "separate" or "auto" (default): the

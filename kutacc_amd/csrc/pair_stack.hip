@@ -661,6 +661,221 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams 
     }
 }
 
+// The 256 x 256 tiles with the operands loaded straight into the LDS (global_load_lds_dwordx4: a wave's 64 lanes
+// write 1 KB of consecutive LDS, each from its own global address), no registers and no LDS store instructions on the
+// way.  The stage is 32 k deep (32 KB: A's 256 rows, then B's), four of them form a ring and a stage is requested three
+// stages ahead of its MFMAs: a wave asks for its eight 1 KB units of stage t + 3 among the MFMAs of stage t, waits at the
+// end of stage t until its units of stage t + 2 have landed (at most the eight youngest loads still in flight) and
+// meets the others at the barrier; after it every wave may read stage t + 2 and overwrite stage t - 1.
+//
+// K-major operand: a unit is 16 rows x 64 bytes, lane l -> row l / 4, 16-byte slot l % 4, and the lane fetches the
+// chunk that the slot holds after the swizzle (chunk ^ direct_swizzle(row)), under which the fragment reads (lane ->
+// its own row, chunk 2 s + g) are free of bank conflicts.  M-major operand: a unit is 4 k x 128 m (256 bytes a row),
+// rows as they lie in memory with the 16-byte slots of row k XOR-ed with 4 (k & 3): the layout the transposing reads
+// of the other kernels expect, with 32 rows per sub-tile.
+constexpr int DIRECT_KSTEP = 32;
+constexpr int DIRECT_STAGE_SLOTS = 2048;
+constexpr int DIRECT_RING = 4;
+constexpr int DIRECT_STRIP_LD = 72; // bf16 per row of a wave's output strip: 64 columns and 16 bytes of padding
+constexpr size_t DIRECT_STRIP_BYTES = 32 * DIRECT_STRIP_LD * 2;
+constexpr size_t DIRECT_GEMM_LDS = DIRECT_RING * DIRECT_STAGE_SLOTS * 16 + 4 * DIRECT_STRIP_BYTES;
+
+// 64-byte rows: rows two apart start in the same banks (32 banks of 4 bytes), so the eight rows that eight consecutive
+// lanes read take four different slots per parity
+__device__ __forceinline__ int direct_swizzle(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+
+// The sixteen MFMAs of a quarter, blocks (i, j) in the order in which the fragments a0 b0 a1 b1 ... arrive.
+__device__ constexpr int DIRECT_MI[16] = {0, 1, 0, 1, 2, 2, 0, 1, 2, 3, 3, 3, 0, 1, 2, 3};
+__device__ constexpr int DIRECT_MJ[16] = {0, 0, 1, 1, 0, 1, 2, 2, 2, 0, 1, 2, 3, 3, 3, 3};
+
+template <bool MMAJOR>
+__global__ __launch_bounds__(256, 1) void pair_gemm_direct_kernel(const GemmParams p, const int64_t total_tiles)
+{
+    typedef const __attribute__((address_space(1))) void *global_ptr;
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, g = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    const int64_t tiles_per_batch = (int64_t)p.MT * p.NT;
+    auto place = [&](int64_t index) -> TilePlace { // the walk of pair_gemm_big_kernel: a contiguous run of tiles per XCD
+        uint32_t v = (uint32_t)(index < total_tiles ? index : total_tiles - 1);
+        const uint32_t per = (uint32_t)total_tiles / 8;
+        if (v < per * 8) {
+            v = (v % 8) * per + v / 8;
+        }
+        const int batch = (int)(v / (uint32_t)tiles_per_batch), t = (int)(v % (uint32_t)tiles_per_batch);
+        int mt, nt;
+        if (p.MT <= p.NT) {
+            mt = t % p.MT, nt = t / p.MT;
+        } else {
+            nt = t % p.NT, mt = t / p.NT;
+        }
+        return TilePlace{batch, mt * BIG_TILE, nt * BIG_TILE};
+    };
+
+    // Waves 0 and 1 bring A, waves 2 and 3 B: unit u = 8 (wave & 1) + i of the operand's sixteen per stage.  An address
+    // is a wave-uniform pointer (tile, stage, unit) plus a 32-bit byte offset per lane that never changes.
+    const bool brings_a = wave < 2;
+    const int64_t ld = brings_a ? (MMAJOR ? p.a_sk : p.a_sm) : (MMAJOR ? p.b_sk : p.b_sn);
+    // byte offsets of this lane's 16 bytes of unit i from the stage's first element of the operand: the unit's place
+    // in the stage and the lane's in the unit; they never change, so a request costs its own instruction, the LDS
+    // address in M0 and nothing else (with one wave per SIMD every instruction issued comes out of the MFMAs' time)
+    uint32_t unit_bytes[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int u = (wave & 1) * 8 + i;
+        if constexpr (MMAJOR) {
+            unit_bytes[i] = (uint32_t)((((lane >> 4) + 4 * (u & 7)) * ld + 8 * ((lane & 15) ^ (4 * (lane >> 4))) + 128 * (u >> 3)) * 2);
+        } else {
+            const int row = lane >> 2;
+            unit_bytes[i] = (uint32_t)(((16 * u + row) * ld + 8 * ((lane & 3) ^ direct_swizzle(row))) * 2);
+        }
+    }
+    const int64_t stage_pitch = MMAJOR ? DIRECT_KSTEP * ld * 2 : DIRECT_KSTEP * 2; // bytes from one stage's elements to the next's
+    auto operand_of = [&](const TilePlace &tp) -> const char * { // element (first row of the tile, k = 0) of this wave's operand
+        if (brings_a) {
+            const bf16_t *a = p.a + (int64_t)tp.batch * p.a_sb;
+            return reinterpret_cast<const char *>(MMAJOR ? a + tp.m0 : a + (int64_t)tp.m0 * ld);
+        }
+        const bf16_t *b = p.b + (int64_t)tp.batch * p.b_sb;
+        return reinterpret_cast<const char *>(MMAJOR ? b + tp.n0 : b + (int64_t)tp.n0 * ld);
+    };
+    // The load is written out: as a builtin the compiler takes every LDS read behind it for a possible reader of its
+    // data and waits for all loads in flight first.  Nothing the compiler generates depends on these loads; the waits
+    // for them are the explicit ones at the end of a stage.  `from`: the stage's first element of the operand; `to`:
+    // LDS byte address of this wave's first unit in the stage.
+    auto request = [&](const char *from, uint32_t to, int i) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(to + i * 1024u), "v"(unit_bytes[i]), "s"(from) : "memory");
+    };
+    const uint32_t ring_bytes = (uint32_t)(uintptr_t)(lds_ptr)lds + (brings_a ? 0u : DIRECT_STAGE_SLOTS * 8u) + (wave & 1) * 8192u;
+
+    f32x16 acc[4][4];
+    int mm_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mm_off[i] = mm_fragment_offset(i, lane);
+    }
+    const int frag_slot[2] = {r * 4 + (g ^ direct_swizzle(r)), r * 4 + ((2 + g) ^ direct_swizzle(r))};
+    bf16x8 af[2][4], bq[2][4];
+    // fragment n of a quarter's eight, in the order a0 b0 a1 b1 ...
+    auto fragment = [&](int set, const uint4 *stage, int s, int n) {
+        const int i = n >> 1;
+        const int ba = wm * 4 + i, bb = wn * 4 + i; // 32-row blocks of the operands' 256 rows
+        if (!(n & 1)) {
+            if constexpr (MMAJOR) {
+                af[set][i] = mm_fragment((const lds_char *)(stage + (ba >> 2) * 512), mm_off[ba & 3], s);
+            } else {
+                af[set][i] = as_bf16x8(stage[ba * 128 + frag_slot[s]]);
+            }
+        } else {
+            if constexpr (MMAJOR) {
+                bq[set][i] = mm_fragment((const lds_char *)(stage + DIRECT_STAGE_SLOTS / 2 + (bb >> 2) * 512), mm_off[bb & 3], s);
+            } else {
+                bq[set][i] = as_bf16x8(stage[DIRECT_STAGE_SLOTS / 2 + bb * 128 + frag_slot[s]]);
+            }
+        }
+    };
+    // One quarter in a fixed order: per pair of MFMAs on `set` one fragment for the other set (quarter s_next of
+    // `stage`) in front, and behind the pair's first MFMA what `issue` requests for pair n.  `fresh`: a tile's first
+    // quarter, which touches every block once, starts the sums (a zero operand costs nothing; clearing 256 accumulator
+    // registers is 512 instructions a tile).
+    auto quarter = [&](int set, const uint4 *stage, int s_next, auto issue, auto fresh) {
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            fragment(set ^ 1, stage, s_next, n);
+            acc[DIRECT_MI[2 * n]][DIRECT_MJ[2 * n]] =
+                mfma(bq[set][DIRECT_MJ[2 * n]], af[set][DIRECT_MI[2 * n]], decltype(fresh)::value ? zero16() : acc[DIRECT_MI[2 * n]][DIRECT_MJ[2 * n]]);
+            issue(n);
+            acc[DIRECT_MI[2 * n + 1]][DIRECT_MJ[2 * n + 1]] = mfma(bq[set][DIRECT_MJ[2 * n + 1]], af[set][DIRECT_MI[2 * n + 1]],
+                                                                 decltype(fresh)::value ? zero16() : acc[DIRECT_MI[2 * n + 1]][DIRECT_MJ[2 * n + 1]]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto ring_step = [](int slot, int d) { return slot + d >= DIRECT_RING ? slot + d - DIRECT_RING : slot + d; };
+
+    const int KT = p.K / DIRECT_KSTEP; // at least three (the launcher sees to it)
+    int64_t v = blockIdx.x;
+    TilePlace cur = place(v);
+    const char *cur_operand = operand_of(cur), *next_operand = cur_operand;
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            request(cur_operand + t * stage_pitch, ring_bytes + t * DIRECT_STAGE_SLOTS * 16u, i);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 8; ++n) {
+        fragment(0, lds, 0, n);
+    }
+    int slot = 0; // of the ring, where the current stage lies
+    for (; v < total_tiles; v += gridDim.x) {
+        const TilePlace next = place(v + gridDim.x);
+        next_operand = operand_of(next);
+        auto stage = [&](int kt, auto fresh) {
+            const bool over = kt + 3 >= KT; // the requests go on to the next tile
+            const char *from = (over ? next_operand : cur_operand) + (over ? kt + 3 - KT : kt + 3) * stage_pitch;
+            const uint32_t to = ring_bytes + ring_step(slot, 3) * DIRECT_STAGE_SLOTS * 16u;
+            quarter(0, lds + slot * DIRECT_STAGE_SLOTS, 1, [&](int n) {
+                if (n & 1) {
+                    request(from, to, n >> 1);
+                }
+            }, fresh);
+            quarter(1, lds + ring_step(slot, 1) * DIRECT_STAGE_SLOTS, 0, [&](int n) {
+                if (n & 1) {
+                    request(from, to, 4 + (n >> 1));
+                }
+            }, std::false_type{});
+            // this wave's units of the stage after next have landed when at most the eight requests of this stage are
+            // in flight; behind the barrier every wave's have, and every wave has left the stage before this one
+            asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+            slot = ring_step(slot, 1);
+        };
+        stage(0, std::true_type{});
+        for (int kt = 1; kt < KT; ++kt) {
+            stage(kt, std::false_type{});
+        }
+
+        // Each wave rounds its block to bf16 through a strip of its own (32 rows x 64 columns) behind the ring and
+        // writes whole 128-byte pieces of rows; a wave's LDS accesses complete in order, so the strip needs no barrier.
+        bf16_t *ct = reinterpret_cast<bf16_t *>(reinterpret_cast<char *>(lds + DIRECT_RING * DIRECT_STAGE_SLOTS) + wave * DIRECT_STRIP_BYTES);
+        bf16_t *c = p.c + (int64_t)cur.batch * p.c_sb;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int jh = 0; jh < 2; ++jh) {
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        bf16x4 ov;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            ov[e] = (bf16_t)acc[i][2 * jh + jj][4 * q + e];
+                        }
+                        *reinterpret_cast<bf16x4 *>(ct + r * DIRECT_STRIP_LD + 32 * jj + 8 * q + 4 * g) = ov;
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int piece = lane + 64 * e;
+                    const int row = piece >> 3, chunk = piece & 7;
+                    const int64_t gm = cur.m0 + 128 * wm + 32 * i + row, gn = cur.n0 + 128 * wn + 64 * jh + chunk * 8;
+                    *reinterpret_cast<uint4 *>(c + gm * p.c_sm + gn) = *reinterpret_cast<const uint4 *>(ct + row * DIRECT_STRIP_LD + chunk * 8);
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        cur = next;
+        cur_operand = next_operand;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the requests for a tile past the last one: let them land before the LDS is given back
+}
+
 // Transition with the hidden layer kept on chip: out = relu(x . W1^T + b1) . W2^T + b2 for row tiles of x
 // (reference src/attention/transition.cpp:31-38 runs two GEMMs through a [rows, c_i] intermediate; with
 // c_i = 4 c_o that intermediate is four fifths of the HBM traffic).  A wave owns RB blocks of 32 rows, whose
@@ -1252,10 +1467,32 @@ hipError_t launch_big_tiles(const GemmParams &p, int64_t blocks, hipStream_t str
     return hipGetLastError();
 }
 
-// 0: the 256 x 256 tiles where every CU gets at least four of them (measured at 128 channels: 0.36 of the MFMA peak
-// against 0.31 at 1024 x 1024, 0.31 against 0.29 at 768 x 768, no gain at 512 x 512), else the 192 x 192 tiles where
-// every CU gets at least two (384 x 384: 24.6 us against 25.8-26.6; 576 x 576: 74-78 against 79-86; 192 x 192 loses),
-// else the 128 x 128 tiles; 1: 256 x 256 wherever the shape has whole ones; 3: 192 x 192 wherever it has; 2: neither
+template <bool MM>
+hipError_t launch_direct_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
+{
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&pair_gemm_direct_kernel<MM>), DIRECT_GEMM_LDS, configured)) {
+        return e;
+    }
+    int device = 0, cus = 0;
+    if (hipError_t e = hipGetDevice(&device)) {
+        return e;
+    }
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device)) {
+        return e;
+    }
+    const int64_t grid = blocks < cus ? blocks : (cus >= 8 ? cus / 8 * 8 : cus);
+    pair_gemm_direct_kernel<MM><<<dim3((unsigned)grid), 256, DIRECT_GEMM_LDS, stream>>>(p, blocks);
+    return hipGetLastError();
+}
+
+// 0: the 256 x 256 tiles with operands loaded straight into the LDS where every CU gets at least two of them (measured
+// at 128 channels, outgoing / incoming, against the next best form: 512 x 512 46 / 44 us against 49-56 / 58; 768 x 768
+// 150 / 134 against 154 / 158; 1024 x 1024 281-289 / 270 against 308 / 322; 256 x 256, one tile per two CUs, loses:
+// 14.3 against 12.4), else the 192 x 192 tiles where every CU gets at least two (384 x 384: 24.6 us against 25.8-26.6;
+// 576 x 576: 74-78 against 79-86; 192 x 192 loses), else the 128 x 128 tiles; 4: the direct 256 x 256 tiles wherever the
+// shape has whole ones; 1: the 256 x 256 tiles staged through registers wherever it has; 3: 192 x 192 likewise; 2: none
+// of them
 std::atomic<int> g_big_tile_mode{0};
 constexpr int64_t BIG_TILE_MIN_WORKGROUPS = 1024;
 
@@ -1370,7 +1607,7 @@ int transition_block_fused(void *act, const float *ln_gamma, const float *ln_bet
 int pair_gemm_tuning(const char *name, const char *value)
 {
     if (!std::strcmp(name, "gemm_tile")) { // "256": wherever the shape allows the large tiles, "128": never, anything else: the default rule
-        g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : (value && !std::strcmp(value, "192") ? 3 : 0)));
+        g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : (value && !std::strcmp(value, "192") ? 3 : (value && !std::strcmp(value, "direct") ? 4 : 0))));
         return 0;
     }
     return KUTACC_HIP_EINVAL;
@@ -1470,6 +1707,15 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
     const int tile_mode = g_big_tile_mode.load();
     if (!gated && am == bm && g.bias_axis == 0 && !g.relu && g.k % KSTEP == 0 && (am ? g.a_stride_k : g.a_stride_m) < (1 << 26) &&
         (bm ? g.b_stride_k : g.b_stride_n) < (1 << 26) && tile_mode != 2) {
+        // (the direct kernel's lane offsets span the tile's 256 rows: pitches below 2^22 elements keep them in 32 bits)
+        if ((tile_mode == 4 || tile_mode == 0) && (am ? g.a_stride_k : g.a_stride_m) < (1 << 22) && (bm ? g.b_stride_k : g.b_stride_n) < (1 << 22) &&
+            g.m % BIG_TILE == 0 && g.n % BIG_TILE == 0 && g.k >= 3 * DIRECT_KSTEP && g.m / BIG_TILE * (g.n / BIG_TILE) * p.batches <= INT32_MAX &&
+            (tile_mode == 4 || g.m / BIG_TILE * (g.n / BIG_TILE) * p.batches >= BIG_TILE_MIN_WORKGROUPS / 2)) {
+            p.MT = (int)(g.m / BIG_TILE), p.NT = (int)(g.n / BIG_TILE);
+            const int64_t big_blocks = (int64_t)p.MT * p.NT * p.batches;
+            kutacc_prof::KernelTimer t(am ? "pair_gemm_direct_kernel<m-major>" : "pair_gemm_direct_kernel", flops, stream);
+            return kutacc_hip_status(am ? launch_direct_tiles<true>(p, big_blocks, stream) : launch_direct_tiles<false>(p, big_blocks, stream));
+        }
         // 256 x 256 tiles where every CU gets at least four; else 192 x 192 where every CU gets at least two
         for (const int side : {BIG_TILE, 192}) {
             const bool forced = tile_mode == (side == BIG_TILE ? 1 : 3);

@@ -143,21 +143,26 @@ def first_profiled_kernel(torch, fn):
 
 
 @pytest.mark.parametrize("mmajor", [False, True], ids=["k-major", "m-major"])
-@pytest.mark.parametrize("side", [256, 192])
-@pytest.mark.parametrize("units", [(2, 1, 1, 64), (1, 2, 1, 192), (3, 1, 3, 320), (9, 1, 1, 128), (300, 1, 1, 64)])
-def test_gemm_large_tiles(torch_cuda, gemm_tile, units, side, mmajor):
-    """The 256 x 256 tiles (128 x 128 per wave) and the 192 x 192 ones (96 x 96 per wave) against the float64 product
-    and, bit for bit, against the 128 x 128 tiles, which add the same products in the same order: one and several
-    k-steps, an odd number of them (the kernel takes them in pairs), several tiles per batch, and more tiles than the
-    chip has CUs (a workgroup then walks several, its operand pipeline running across the tile boundary)."""
+@pytest.mark.parametrize("tile", ["256", "192", "direct"])
+@pytest.mark.parametrize("units", [(2, 1, 1, 64), (1, 2, 1, 192), (3, 1, 3, 320), (9, 1, 1, 128), (300, 1, 1, 64), (40, 2, 2, 512)])
+def test_gemm_large_tiles(torch_cuda, gemm_tile, units, tile, mmajor):
+    """The 256 x 256 tiles (128 x 128 per wave; staged through registers, and loaded straight into the LDS) and the
+    192 x 192 ones (96 x 96 per wave) against the float64 product and, bit for bit, against the 128 x 128 tiles, which
+    add the same products in the same order: one and several k-steps, an odd number of them (the register-staged kernels
+    take them in pairs), several tiles per batch, and more tiles than the chip has CUs (a workgroup then walks several,
+    its operand pipeline running across the tile boundary).  The direct tiles need three stages of 32 k: the one-step
+    cases run with 128 there."""
     nb, mt, nt, K = units
+    side = 192 if tile == "192" else 256
+    if tile == "direct":
+        K = max(K, 128)
     M, N = mt * side, nt * side
     shape = (nb, M, N, K)
     rng = np.random.Generator(np.random.PCG64(300 + M + N + K))
     A, B = draw(rng, nb, M, K), draw(rng, nb, N, K, scale=1 / math.sqrt(K))
-    gemm_tile(str(side))
+    gemm_tile(tile)
     name = first_profiled_kernel(torch_cuda, lambda: run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED))
-    assert name.startswith("pair_gemm_big_kernel"), name
+    assert name.startswith("pair_gemm_direct_kernel" if tile == "direct" else "pair_gemm_big_kernel"), name
     got = run_gemm(torch_cuda, A, B, a_mmajor=mmajor, b_mmajor=mmajor, path=capi.PATH_FUSED, c_pad=8)
     ref = gemm_ref(A, B)
     helpers.assert_within(got, ref, GEMM_TOL(ref), f"large tiles {shape}")
@@ -166,12 +171,12 @@ def test_gemm_large_tiles(torch_cuda, gemm_tile, units, side, mmajor):
     assert np.array_equal(got, small)
 
 
-@pytest.mark.parametrize("n", [384, 576, 768, 1024])
+@pytest.mark.parametrize("n", [384, 512, 576, 768, 1024])
 def test_equation_at_384_residues_and_more_takes_the_large_tiles(torch_cuda, n):
-    """128 channels of 768 x 768 (nine 256 x 256 tiles per channel, more than four per CU, which is where the default
-    rule switches to them) and of 1024 x 1024 (eight tiles per workgroup); of 384 x 384 and 576 x 576, whose sides are
-    whole 192 x 192 tiles (two and four and a half per CU).  Sampled channels against the oracle; the incoming form
-    equals the outgoing one on transposed operands bit for bit."""
+    """128 channels of 512 x 512, 768 x 768 and 1024 x 1024 (whole 256 x 256 tiles, two, four and a half and eight per
+    CU: the default rule gives them to the kernel that loads its operands straight into the LDS); of 384 x 384 and
+    576 x 576, whose sides are whole 192 x 192 tiles (two and four and a half per CU).  Sampled channels against the
+    oracle; the incoming form equals the outgoing one on transposed operands bit for bit."""
     from oracle import oracle
     torch = torch_cuda
     c_i = 128
@@ -180,8 +185,10 @@ def test_equation_at_384_residues_and_more_takes_the_large_tiles(torch_cuda, n):
     right = (torch.randn(c_i, n, n, device="cuda", generator=g) * n ** -0.5).to(torch.bfloat16)
     for incoming in (False, True):
         name = first_profiled_kernel(torch, lambda: equation(torch, left, right, n, incoming))
-        form = ("m-major" if incoming else "") + (", " if incoming and n < 768 else "") + ("192" if n < 768 else "")
-        assert name == "pair_gemm_big_kernel" + (f"<{form}>" if form else ""), name
+        if n % 256 == 0:
+            assert name == "pair_gemm_direct_kernel" + ("<m-major>" if incoming else ""), name
+        else:
+            assert name == "pair_gemm_big_kernel<" + ("m-major, " if incoming else "") + "192>", name
     out_c = equation(torch, left, right, n, False)
     in_c = equation(torch, left, right, n, True)
     chans = [0, 63, 127]
