@@ -22,6 +22,12 @@
 //
 // Shapes the MFMA kernel does not take (k, n or a leading dimension not a multiple of 8, pointers not
 // 16-byte aligned) run on a scalar kernel with the same epilogues.
+//
+// The batched product of the triangle equation, where its sides are whole large tiles and there are enough of them,
+// runs on persistent kernels with 256 x 256 (or 192 x 192) tiles per workgroup: pair_gemm_direct_kernel, whose
+// operands go straight from global memory into the LDS, and pair_gemm_big_kernel, which stages them through
+// registers.  The transition keeps its hidden layer on chip (transition_fused_kernel); the gated projection of large
+// pair tensors streams the activation once (gated_projection_kernel).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -1606,7 +1612,7 @@ int transition_block_fused(void *act, const float *ln_gamma, const float *ln_bet
 
 int pair_gemm_tuning(const char *name, const char *value)
 {
-    if (!std::strcmp(name, "gemm_tile")) { // "256": wherever the shape allows the large tiles, "128": never, anything else: the default rule
+    if (!std::strcmp(name, "gemm_tile")) { // "128", "256", "192", "direct": see g_big_tile_mode; anything else: the default rule
         g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : (value && !std::strcmp(value, "192") ? 3 : (value && !std::strcmp(value, "direct") ? 4 : 0))));
         return 0;
     }
