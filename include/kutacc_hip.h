@@ -456,6 +456,11 @@ kutacc_export int kutacc_hip_profile_read(int index, char *name, int name_len, d
  *               ones / on 192 x 192 tiles wherever it has / on 256 x 256 tiles whose operands are loaded straight into
  *               the LDS wherever it has (and k is at least 96); anything else (default): the direct 256 x 256 tiles
  *               where every CU gets at least two, else 192 x 192 where every CU gets at least two, else 128 x 128
+ *   "gated_projection" "streaming" / "tiled": the gated projections of kutacc_af2_triangle_multiplication_calc_proj and
+ *               of kutacc_hip_triangle_multiplication at 128 channels on the kernel that gives every wave its own positions
+ *               and keeps the weights in the LDS / on the tiled kernel of the general products; "blocks" or anything else
+ *               (default): on the kernel that keeps a wave's weights in registers and shares the activation through
+ *               the LDS
  *   "layernorm" "fused": kutacc_hip_triangle_attention and kutacc_hip_msa_attention let the attention kernel normalise its
  *               input rows itself where it can (sequence lengths of the persistent kernel), which drops the normalised
  *               copy from the workspace and costs 8-15 % of the block's time; "separate" or "auto" (default): the

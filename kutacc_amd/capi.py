@@ -316,7 +316,7 @@ def set_blocking(blocking: bool) -> None:
 
 def set_tuning(name: str, value: str | None) -> int:
     """kutacc_hip_set_tuning: the hooks include/kutacc_hip.h lists ("plan", "fragments", "debug", "row_pairs",
-    "gemm_tile", "layernorm", "scratch", "pointer_checks"); None = the default of that hook."""
+    "gemm_tile", "gated_projection", "layernorm", "scratch", "pointer_checks"); None = the default of that hook."""
     return lib().kutacc_hip_set_tuning(name.encode(), None if value is None else value.encode())
 
 

@@ -26,8 +26,9 @@
 // The batched product of the triangle equation, where its sides are whole large tiles and there are enough of them,
 // runs on persistent kernels with 256 x 256 (or 192 x 192) tiles per workgroup: pair_gemm_direct_kernel, whose
 // operands go straight from global memory into the LDS, and pair_gemm_big_kernel, which stages them through
-// registers.  The transition keeps its hidden layer on chip (transition_fused_kernel); the gated projection of large
-// pair tensors streams the activation once (gated_projection_kernel).
+// registers.  The transition keeps its hidden layer on chip (transition_fused_kernel); the gated projections of 128
+// channels have kernels of their own that read the activation once (gated_projection_blocks_kernel, and
+// gated_projection_kernel behind a tuning switch).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -1355,6 +1356,197 @@ __global__ __launch_bounds__(256 * SIDES, 2 / SIDES) void gated_projection_kerne
     }
 }
 
+// The gated projection with the weights in registers and the activation shared through the LDS.  In the kernel above
+// every wave multiplies its own positions by all four weight matrices, whose fragments it reads from the LDS for every
+// step: 128 KB of LDS reads per wave and step of 64 positions, and whole steps as the unit of work (at 384 x 384
+// positions a CU has nine steps for eight waves).  Here a workgroup takes the steps one after the other and a wave owns
+// 32 output channels of one side: its two 32 x 128 weight blocks (projection and gate) stay in 64 registers, and per
+// step it reads the 64 x 128 activation (16 KB, loaded once per workgroup straight into the LDS, a ring of stages
+// requested RING - 1 steps ahead) and the mask (128 bytes, each wave's own copy), multiplies, gates and writes 32
+// channels x 128 bytes.  Eight equal shares of every step, an eighth of the LDS reads.  Same arithmetic in the same
+// order as the kernel above: the results are bit-identical.
+template <int SIDES>
+__global__ __launch_bounds__(256 * SIDES, 2 / SIDES) void gated_projection_blocks_kernel(const bf16_t *__restrict__ x, GatedSide s0, GatedSide s1,
+                                                                                        const bf16_t *__restrict__ mask, int64_t out_ld,
+                                                                                        int64_t n_pos, int steps_per_group)
+{
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    constexpr int C = 128, CK = C / 16, WAVES = 4 * SIDES, RING = SIDES == 2 ? 4 : 3, UNITS = 16 / WAVES;
+    constexpr int STAGE_SLOTS = 1024; // 64 positions x 256 bytes
+    constexpr int WAVE_SLOTS = 256 + RING * 16; // a panel for the way out, and RING mask rows of 256 bytes
+    extern __shared__ uint4 lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rv = lane & 31, gv = lane >> 5;
+    const GatedSide &sd = (SIDES == 2 && wave >= 4) ? s1 : s0;
+    const int cb = wave & 3; // this wave's 32 channels
+    uint4 *panel = lds + RING * STAGE_SLOTS + wave * WAVE_SLOTS;
+    const uint4 *mask_rows = panel + 256;
+
+    const int64_t total_steps = (n_pos + 63) / 64;
+    const int64_t first = (int64_t)blockIdx.x * steps_per_group;
+    const int64_t stop = first + steps_per_group < total_steps ? first + steps_per_group : total_steps;
+    if (first >= stop) {
+        return;
+    }
+
+    // A stage holds its 64 rows of 256 bytes with the 16-byte slots of row r XOR-ed with r % 8 (the fragment reads, lane
+    // -> its own row, then hit eight different bank groups per eight lanes).  A request is a unit of four rows: lane l
+    // writes slot l % 16 of row l / 16 and fetches the chunk that belongs there.  Units past the last position fetch the
+    // last four positions again (their results are never stored), so every wave issues the same number of requests,
+    // which the waits below count.
+    uint32_t lane_bytes[2]; // for even and odd units
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+        lane_bytes[par] = (uint32_t)((lane >> 4) * 256 + (((lane & 15) ^ ((4 * par + (lane >> 4)) & 7)) * 16));
+    }
+    const uint32_t x_lds = (uint32_t)(uintptr_t)(lds_ptr)lds, mask_lds = (uint32_t)(uintptr_t)(lds_ptr)mask_rows;
+    auto request = [&](int64_t step, int slot) {
+#pragma unroll
+        for (int i = 0; i < UNITS; ++i) {
+            const int u = wave * UNITS + i;
+            int64_t pos = step * 64 + 4 * u;
+            pos = pos + 4 <= n_pos ? pos : n_pos - 4;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(x_lds + slot * (STAGE_SLOTS * 16u) + u * 1024u),
+                         "v"(lane_bytes[i & 1]), "s"(x + pos * C)
+                         : "memory");
+        }
+        // the mask of the step's positions, two per lane (lanes 32-63 repeat lanes 0-31); past the end: the last two
+        const uint32_t last_pair = (uint32_t)(n_pos - step * 64 - 2) * 2u;
+        const uint32_t mine = 4u * (uint32_t)(lane & 31);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(mask_lds + slot * 256u), "v"(mine < last_pair ? mine : last_pair),
+                     "s"(mask + step * 64)
+                     : "memory");
+    };
+    auto ring = [](int slot) { return slot >= RING ? slot - RING : slot; };
+
+    // requests are issued RING - 1 steps ahead; a step that lies past this workgroup's last one fetches the last one again
+#pragma unroll
+    for (int d = 0; d < RING - 1; ++d) {
+        request(first + d < stop ? first + d : stop - 1, d);
+    }
+    bf16x8 wp[CK], wg[CK];
+#pragma unroll
+    for (int ks = 0; ks < CK; ++ks) {
+        wp[ks] = *reinterpret_cast<const bf16x8 *>(sd.wp + (int64_t)(cb * 32 + rv) * C + ks * 16 + gv * 8);
+        wg[ks] = *reinterpret_cast<const bf16x8 *>(sd.wg + (int64_t)(cb * 32 + rv) * C + ks * 16 + gv * 8);
+    }
+    float pbias = sd.bp[cb * 32 + rv], gneg = -LOG2E * sd.bg[cb * 32 + rv];
+    // The weights are asked for behind the first requests and waited for here, before the loop: the compiler does not
+    // know of the requests, and a wait it places for one of its own loads waits for every request issued before that
+    // load -- once, here, that is one memory round trip for both; inside the loop it would stall every step.
+#pragma unroll
+    for (int ks = 0; ks < CK; ++ks) {
+        asm volatile("" : "+v"(wp[ks]), "+v"(wg[ks]));
+    }
+    asm volatile("" : "+v"(pbias), "+v"(gneg));
+
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    int slot = 0;
+    for (int64_t step = first; step < stop; ++step) {
+        {
+            const int64_t ahead = step + RING - 1;
+            request(ahead < stop ? ahead : stop - 1, ring(slot + RING - 1));
+        }
+        const uint4 *stage = lds + slot * STAGE_SLOTS;
+        const char *mrow = reinterpret_cast<const char *>(mask_rows + slot * 16);
+        const int64_t base = step * 64;
+        bf16x8 af[2][CK];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+                af[rb][ks] = as_bf16x8(stage[(rb * 32 + rv) * 16 + ((2 * ks + gv) ^ (rv & 7))]);
+            }
+        }
+        // projection first, rounded to bf16 and parked as packed pairs, then the gate: half the accumulators live
+        bf16x8 pp[2][2];
+        {
+            f32x16 pa[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                pa[rb] = zero16();
+            }
+#pragma unroll
+            for (int ks = 0; ks < CK; ++ks) {
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    pa[rb] = mfma(af[rb][ks], wp[ks], pa[rb]);
+                }
+            }
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    pa[rb][v] += pbias;
+                }
+                pp[rb][0] = pack8(pa[rb], 0), pp[rb][1] = pack8(pa[rb], 8);
+            }
+        }
+        f32x16 ga[2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+            ga[rb] = zero16();
+        }
+#pragma unroll
+        for (int ks = 0; ks < CK; ++ks) {
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                ga[rb] = mfma(af[rb][ks], wg[ks], ga[rb]);
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const bf16x4 mk = *reinterpret_cast<const bf16x4 *>(mrow + 2 * (rb * 32 + 8 * a + 4 * gv)); // the lane's four consecutive positions
+                bf16x4 ov;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float pv = to_f32(pp[rb][a >> 1][4 * (a & 1) + c]) * to_f32(mk[c]);
+                    // sigmoid(gate + bias) = 1 / (1 + 2^-(gate*log2e + bias*log2e)); the gate stays in fp32
+                    const float e = __builtin_amdgcn_exp2f(fmaf(ga[rb][4 * a + c], -LOG2E, gneg));
+                    ov[c] = (bf16_t)(pv * __builtin_amdgcn_rcpf(1.0f + e));
+                }
+                *(reinterpret_cast<bf16x4 *>(panel + panel_slot(rv, rb * 4 + a)) + gv) = ov;
+            }
+        }
+        {
+            // 32 channels x eight 16-byte pieces of 8 positions; the pieces past the last position repeat the last valid
+            // one (same data to the same address), so that the stores, too, are the same number in every step
+            const int64_t left = n_pos - base;
+            const int valid = left >= 64 ? 8 : (int)(left >> 3);
+            const int piece = (lane & 7) < valid ? (lane & 7) : valid - 1;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ch = 8 * i + (lane >> 3);
+                const uint4 v = panel[panel_slot(ch, piece)];
+                *reinterpret_cast<uint4 *>(sd.out + (int64_t)(cb * 32 + ch) * out_ld + base + piece * 8) = v;
+            }
+        }
+        // The next step's stage has landed when nothing older than what this wave has issued since its request is in
+        // flight: the requests of the steps after it (UNITS + 1 each) and four stores per step gone by.  Behind the
+        // barrier every wave's part of it has, and every wave has left this step's stage.
+        const int64_t gone = step - first;
+        if constexpr (RING == 4) {
+            if (gone == 0) {
+                asm volatile("s_waitcnt vmcnt(10)\n\ts_barrier" ::: "memory");
+            } else if (gone == 1) {
+                asm volatile("s_waitcnt vmcnt(14)\n\ts_barrier" ::: "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+            }
+        } else {
+            if (gone == 0) {
+                asm volatile("s_waitcnt vmcnt(9)\n\ts_barrier" ::: "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(13)\n\ts_barrier" ::: "memory");
+            }
+        }
+        slot = ring(slot + 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // requests repeated past the last step: let them land before the LDS is given back
+}
+
 // Any strides, any sizes: one thread per element of C, same epilogues and rounding points.
 __global__ __launch_bounds__(256) void pair_gemm_scalar_kernel(const GemmParams p)
 {
@@ -1451,7 +1643,6 @@ hipError_t launch_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
     pair_gemm_kernel<AM, BM, G><<<dim3((unsigned)blocks), 256, GEMM_LDS, stream>>>(p);
     return hipGetLastError();
 }
-constexpr int64_t GATED_STREAMING_MIN_POSITIONS = 512 * 512;
 
 template <bool MM, int BW>
 hipError_t launch_big_tiles(const GemmParams &p, int64_t blocks, hipStream_t stream)
@@ -1502,6 +1693,10 @@ hipError_t launch_direct_tiles(const GemmParams &p, int64_t blocks, hipStream_t 
 std::atomic<int> g_big_tile_mode{0};
 constexpr int64_t BIG_TILE_MIN_WORKGROUPS = 1024;
 
+// which kernel takes a gated projection that gated_projection_fits(): 0 (default) and 1: the one with the weights in
+// registers ("blocks"); 2: the streaming kernel; 3: the tiled kernel
+std::atomic<int> g_gated_mode{0};
+
 // the dedicated kernel of the gated projection: 128 -> 128 channels, dense operands, positions in whole 16-byte runs
 bool gated_projection_fits(const kutacc_hip_gemm_args_t &g)
 {
@@ -1536,6 +1731,32 @@ hipError_t launch_gated_projection(const kutacc_hip_gemm_args_t &g, const kutacc
     }
     gated_projection_kernel<SIDES><<<dim3((unsigned)gx), 64 * WAVES, lds_bytes, stream>>>(
         (const bf16_t *)g.b, s0, s1, (const bf16_t *)g.mask, g.c_stride_m, g.n, (int)ppw);
+    return hipGetLastError();
+}
+
+template <int SIDES>
+hipError_t launch_gated_projection_blocks(const kutacc_hip_gemm_args_t &g, const kutacc_hip_gemm_args_t *second, hipStream_t stream)
+{
+    constexpr int WAVES = 4 * SIDES, RING = SIDES == 2 ? 4 : 3;
+    constexpr size_t lds_bytes = (size_t)(RING * 1024 + WAVES * (256 + RING * 16)) * 16;
+    static size_t configured[KUTACC_DEVICE_SLOTS] = {};
+    static int cu_table[KUTACC_DEVICE_SLOTS] = {};
+    if (const hipError_t e = kutacc_opt_in_lds(reinterpret_cast<const void *>(&gated_projection_blocks_kernel<SIDES>), lds_bytes, configured)) {
+        return e;
+    }
+    const int cus = kutacc_device_attribute(hipDeviceAttributeMultiprocessorCount, 256, cu_table);
+    // eight resident waves per CU (two workgroups of four, or one of eight); every workgroup an equal run of steps
+    const int64_t steps = (g.n + 63) / 64;
+    const int64_t cap = (int64_t)cus * (2 / SIDES);
+    const int64_t groups = steps < cap ? steps : cap;
+    const int64_t per_group = (steps + groups - 1) / groups;
+    const GatedSide s0 = {(const bf16_t *)g.a, (const bf16_t *)g.a_gate, g.bias, g.bias_gate, (bf16_t *)g.c};
+    GatedSide s1 = s0;
+    if (SIDES == 2) {
+        s1 = GatedSide{(const bf16_t *)second->a, (const bf16_t *)second->a_gate, second->bias, second->bias_gate, (bf16_t *)second->c};
+    }
+    gated_projection_blocks_kernel<SIDES><<<dim3((unsigned)((steps + per_group - 1) / per_group)), 64 * WAVES, lds_bytes, stream>>>(
+        (const bf16_t *)g.b, s0, s1, (const bf16_t *)g.mask, g.c_stride_m, g.n, (int)per_group);
     return hipGetLastError();
 }
 
@@ -1616,6 +1837,10 @@ int pair_gemm_tuning(const char *name, const char *value)
         g_big_tile_mode.store(value && !std::strcmp(value, "256") ? 1 : (value && !std::strcmp(value, "128") ? 2 : (value && !std::strcmp(value, "192") ? 3 : (value && !std::strcmp(value, "direct") ? 4 : 0))));
         return 0;
     }
+    if (!std::strcmp(name, "gated_projection")) { // "blocks", "streaming", "tiled": see g_gated_mode; anything else: the default rule
+        g_gated_mode.store(value && !std::strcmp(value, "blocks") ? 1 : (value && !std::strcmp(value, "streaming") ? 2 : (value && !std::strcmp(value, "tiled") ? 3 : 0)));
+        return 0;
+    }
     return KUTACC_HIP_EINVAL;
 }
 
@@ -1656,9 +1881,10 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
     } else if (g.path == KUTACC_HIP_PATH_FUSED && !mfma_ok) {
         return KUTACC_HIP_EUNSUPPORTED;
     }
-    // The streaming kernel pays a 64 KB weight load per workgroup and works in steps of 64 positions per wave: it
-    // wins once every wave has several steps (measured: 141 us against 225 us at 1024 x 1024 positions, but 36 us
-    // against 31 us at 384 x 384), so small pair tensors stay on the tiled kernel.
+    // Gated projections of 128 channels on dense operands have kernels of their own (gated_projection_fits): by default
+    // the one with the weights in registers, at every size (one side, us, against the tiled kernel up to 384 x 384
+    // positions and the streaming kernel beyond: 256 x 256 12.7 against 14.2; 384 x 384 23-25 against 28; 512 x 512 30.5
+    // against 39.7; 768 x 768 61 against 91; 1024 x 1024 143 against 144-147).
     if (second != nullptr) {
         // a second gated projection of the same B and mask (other weights, biases and result) rides along as batch 1 of
         // the tiled kernel, so that the tile of B both need comes from HBM once; any other route: the caller runs the two
@@ -1671,26 +1897,35 @@ int pair_gemm(const kutacc_hip_gemm_args_t &g, hipStream_t stream, const kutacc_
                           (g.bias_axis == 0 || (h.bias && h.bias_gate)) &&
                           (g.bias_axis != 1 || (kutacc_hip_aligned16(h.bias) && kutacc_hip_aligned16(h.bias_gate))) && kutacc_hip_aligned16(h.a) &&
                           kutacc_hip_aligned16(h.a_gate) && kutacc_hip_aligned16(h.c);
-        const bool streaming = gated && gated_projection_fits(g) && gated_projection_fits(h) && g.n <= INT32_MAX / 2 &&
-                               g.n >= GATED_STREAMING_MIN_POSITIONS;
+        const int gated_mode = g_gated_mode.load();
+        const bool dedicated = gated && gated_mode != 3 && gated_projection_fits(g) && gated_projection_fits(h) && g.n <= INT32_MAX / 2;
         if (!same || !gated || g.path == KUTACC_HIP_PATH_GENERIC) {
             return KUTACC_HIP_EUNSUPPORTED;
         }
-        if (streaming) { // large pair tensors: both sides in one pass of the streaming kernel over the activation
-            kutacc_prof::KernelTimer t("gated_projection_kernel<2>", 8.0 * (double)g.m * (double)g.n * (double)g.k, stream);
-            return kutacc_hip_status(launch_gated_projection<2>(g, second, stream));
+        if (dedicated) { // both sides in one pass over the activation
+            if (gated_mode == 2) {
+                kutacc_prof::KernelTimer t("gated_projection_kernel<2>", 8.0 * (double)g.m * (double)g.n * (double)g.k, stream);
+                return kutacc_hip_status(launch_gated_projection<2>(g, second, stream));
+            }
+            kutacc_prof::KernelTimer t("gated_projection_blocks_kernel<2>", 8.0 * (double)g.m * (double)g.n * (double)g.k, stream);
+            return kutacc_hip_status(launch_gated_projection_blocks<2>(g, second, stream));
         }
-        if (!mfma_ok || (gated_projection_fits(g) && g.n >= GATED_STREAMING_MIN_POSITIONS)) {
+        // (one that fits a dedicated kernel by itself: the caller runs the two separately)
+        if (!mfma_ok || (gated_mode != 3 && gated_projection_fits(g))) {
             return KUTACC_HIP_EUNSUPPORTED;
         }
         p.a_alt = (const bf16_t *)h.a, p.a_gate_alt = (const bf16_t *)h.a_gate, p.bias_alt = h.bias, p.bias_gate_alt = h.bias_gate;
         p.c_alt = (bf16_t *)h.c;
         p.batches = 2;
     }
-    if (g.path != KUTACC_HIP_PATH_GENERIC && gated && gated_projection_fits(g) && g.n <= INT32_MAX / 2 &&
-        g.n >= GATED_STREAMING_MIN_POSITIONS) {
-        kutacc_prof::KernelTimer t("gated_projection_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);
-        return kutacc_hip_status(launch_gated_projection<1>(g, nullptr, stream));
+    if (g.path != KUTACC_HIP_PATH_GENERIC && gated && second == nullptr && g_gated_mode.load() != 3 && gated_projection_fits(g) &&
+        g.n <= INT32_MAX / 2) {
+        if (g_gated_mode.load() == 2) {
+            kutacc_prof::KernelTimer t("gated_projection_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);
+            return kutacc_hip_status(launch_gated_projection<1>(g, nullptr, stream));
+        }
+        kutacc_prof::KernelTimer t("gated_projection_blocks_kernel", 4.0 * (double)g.m * (double)g.n * (double)g.k, stream);
+        return kutacc_hip_status(launch_gated_projection_blocks<1>(g, nullptr, stream));
     }
     // rows of 128 or 256 features against a dense weight matrix: the attention's output-projection kernel keeps
     // the weight slab in LDS and streams the rows, which suits these HBM-bound shapes better than square tiles

@@ -411,11 +411,46 @@ def test_triangle_multiplication_block_seeded_sweep(torch_cuda, index, n):
     helpers.check_close(helpers.to_numpy(pair), tm_block_oracle(c, incoming), "bf16", f"TM block sweep {index}: n={n} incoming={incoming}")
 
 
+@pytest.mark.parametrize("n", [48, 72, 384])
+def test_triangle_multiplication_block_on_each_gated_projection_kernel(torch_cuda, n):
+    """The block's two gated projections go out in one launch.  Its default kernel (weights in registers, both sides in
+    one pass over the activation) must give the block's result bit for bit as the streaming kernel does, and within the
+    rounding of the intermediates as the tiled kernel does."""
+    torch = torch_cuda
+    case = tm_block_case(900 + n, n, 128, 128)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(  # noqa: E731
+        device="cuda", dtype=torch.bfloat16 if a.ndim >= 2 else torch.float32)
+    w = {k: dev(v) for k, v in case.items() if k not in ("z", "mask")}
+    want = {None: "gated_projection_blocks_kernel<2>", "streaming": "gated_projection_kernel<2>", "tiled": "pair_gemm_kernel<gated>"}
+    res = {}
+    for mode in want:
+        assert capi.set_tuning("gated_projection", mode) == 0
+        try:
+            pair = dev(case["z"])
+            capi.lib().kutacc_hip_profile_enable(1)
+            assert capi.TriangleMultiplicationBlock(pair, dev(case["mask"]), w, False).run() == 0
+            torch.cuda.synchronize()
+            names = []
+            for i in range(16):
+                name = ctypes.create_string_buffer(96)
+                ms, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+                if capi.lib().kutacc_hip_profile_read(i, name, 96, ctypes.byref(ms), ctypes.byref(cnt), ctypes.byref(fl)) != 0:
+                    break
+                names.append(name.value.decode())
+        finally:
+            capi.lib().kutacc_hip_profile_enable(0)
+            capi.set_tuning("gated_projection", None)
+        assert want[mode] in names, (mode, names)
+        res[mode] = pair
+    assert helpers.same_bits(res[None], res["streaming"])
+    tiled = helpers.to_numpy(res["tiled"])
+    helpers.assert_within(helpers.to_numpy(res[None]), tiled, 4e-2 + 2e-2 * np.abs(tiled), "weights in registers vs tiled kernel")
+
+
 @pytest.mark.parametrize("incoming", [False, True], ids=["outgoing", "incoming"])
 @pytest.mark.parametrize("n", [384, 512, 768])  # 768: the equation on the 256 x 256 tiles
 def test_triangle_multiplication_block_full_size(torch_cuda, incoming, n):
-    """384 residues, 128 channels, the real shape, and 512, from where on the gated projections run on the streaming
-    kernel (both sides in one pass).  The oracle follows a sample of output positions (i, j) through the
+    """384 residues, 128 channels, the real shape, 512 and 768 (both gated projections in one pass over the activation).  The oracle follows a sample of output positions (i, j) through the
     whole block: their centre needs the left projections of row i and the right projections of row j (columns for the
     incoming form), which the oracle computes for just those rows."""
     from oracle import oracle

@@ -478,12 +478,65 @@ def test_triangle_multiplication_full_size_properties(torch_cuda):
     assert helpers.same_bits(swapped, in_c)
 
 
-def test_gated_projection_streaming_kernel(torch_cuda):
-    """Large pair tensors take the weight-resident streaming kernel of the gated projection (channel-first output in
-    128-byte runs).  512 x 512 positions plus a ragged tail of 40; the oracle checks a sample of positions and the
-    ends of the range, and the tiled kernel on the same operands must agree within one bf16 rounding."""
+def gated_projection_once(torch, t, c, n_pos, ld_out, mode, ld_w=None):
+    """One gated projection [c, n_pos] = f(x [n_pos, c]) through kutacc_hip_gemm under kutacc_hip_set_tuning("gated_projection",
+    mode); returns the name of the kernel that ran and the result (allocated with row pitch ld_out, filled with -3)."""
+    ld_w = ld_w or c
+    assert capi.set_tuning("gated_projection", mode) == 0
+    try:
+        out = torch.full((c, ld_out), -3.0, dtype=torch.bfloat16, device="cuda")
+        g = capi.HipGemmArgs()
+        g.m, g.n, g.k, g.batches, g.dtype, g.path = c, n_pos, c, 1, capi.K_BF16, capi.PATH_FUSED
+        g.a, g.a_gate, g.a_stride_m, g.a_stride_k = t["pw"].data_ptr(), t["gw"].data_ptr(), ld_w, 1
+        g.b, g.b_stride_n, g.b_stride_k = t["x"].data_ptr(), c, 1
+        g.c, g.c_stride_m = out.data_ptr(), ld_out
+        g.bias, g.bias_gate, g.bias_axis, g.mask = t["pb"].data_ptr(), t["gb"].data_ptr(), 2, t["mask"].data_ptr()
+        name = first_profiled_kernel(torch, lambda: capi.lib().kutacc_hip_gemm(ctypes.byref(g), None))
+        assert not capi.error_flag()
+        return name, out
+    finally:
+        capi.set_tuning("gated_projection", None)
+
+
+@pytest.mark.parametrize("n_pos,pad", [(8, 0), (72, 8), (64 * 3 + 8, 0), (384 * 384, 0), (512 * 512 + 40, 24), (64 * 700, 0)])
+def test_gated_projection_with_weights_in_registers(torch_cuda, n_pos, pad):
+    """The default kernel of the gated projection at 128 channels: a wave keeps the weights of its 32 output channels in
+    registers, the workgroup shares the activation through the LDS (loaded straight into it, a ring of stages requested
+    ahead).  One step, a ragged last step, fewer steps than the ring is deep, more steps than workgroups, a padded
+    output pitch (the padding stays untouched): bit for bit against the streaming kernel, which does the same arithmetic
+    in the same order, and a sample of positions against the oracle."""
     from oracle import oracle
     torch = torch_cuda
+    c = 128
+    rng = np.random.Generator(np.random.PCG64(900 + n_pos))
+    x = draw(rng, n_pos, c)
+    mask = (rng.random(n_pos) > 0.15).astype(np.float32)
+    pw, gw = draw(rng, c, c, scale=1 / math.sqrt(c)), draw(rng, c, c, scale=1 / math.sqrt(c))
+    pb, gb = (rng.standard_normal(c) * 0.5).astype(np.float32), (rng.standard_normal(c) * 0.5).astype(np.float32)
+    t = dict(x=dev(torch, x), mask=dev(torch, mask), pw=dev(torch, pw), gw=dev(torch, gw), pb=dev(torch, pb, torch.float32),
+             gb=dev(torch, gb, torch.float32))
+    name, got = gated_projection_once(torch, t, c, n_pos, n_pos + pad, None)
+    assert name == "gated_projection_blocks_kernel", name
+    name, other = gated_projection_once(torch, t, c, n_pos, n_pos + pad, "streaming")
+    assert name == "gated_projection_kernel", name
+    assert helpers.same_bits(got, other)
+    if pad:
+        assert bool((got[:, n_pos:] == -3.0).all())
+    sample = np.unique(np.concatenate([np.arange(0, min(96, n_pos)), np.arange(max(0, n_pos - 96), n_pos),
+                                       rng.choice(n_pos, size=min(n_pos, 512), replace=False)]))
+    ref = oracle.tm_calc_proj_f32(x[sample][None], mask[sample][None], pw, pb, gw, gb)[:, 0]
+    helpers.check_close(helpers.to_numpy(got[:, torch.from_numpy(sample).cuda()]), ref, "bf16", "gated projection, weights in registers")
+    assert bool((got[:, :n_pos][:, t["mask"] == 0] == 0).all())
+
+
+def test_gated_projection_streaming_kernel(torch_cuda):
+    """The weight-resident streaming kernel of the gated projection (every wave its own positions, the weights in the
+    LDS; behind kutacc_hip_set_tuning("gated_projection", "streaming")).  512 x 512 positions plus a ragged tail of 40; the
+    oracle checks a sample of positions and the ends of the range, and the tiled kernel on the same operands must agree
+    within one bf16 rounding."""
+    from oracle import oracle
+    torch = torch_cuda
+    capi.set_tuning("gated_projection", "streaming")
     n_pos, c = 512 * 512 + 40, 128
     rng = np.random.Generator(np.random.PCG64(900))
     x = draw(rng, n_pos, c)
@@ -512,6 +565,7 @@ def test_gated_projection_streaming_kernel(torch_cuda):
         assert capi.lib().kutacc_hip_profile_read(0, name, 96, ctypes.byref(ms), ctypes.byref(cnt), ctypes.byref(fl)) == 0
         capi.lib().kutacc_hip_profile_enable(0)
         outs.append((name.value.decode(), out))
+    capi.set_tuning("gated_projection", None)
     assert outs[0][0] == "gated_projection_kernel" and outs[1][0] == "pair_gemm_kernel<gated>", [o[0] for o in outs]
     sample = np.concatenate([np.arange(0, 96), np.arange(n_pos - 96, n_pos),
                              rng.choice(n_pos, size=2048, replace=False)])
