@@ -255,12 +255,18 @@ int kutacc_hip_gated_residual_projection(const void *a, int64_t a_ld, const void
                                                         kutacc_api::stream_or_default(stream));
 }
 
+// The channel-first intermediates of the block (projections and centre: one n x n plane per channel) keep their planes
+// 17 cache lines further apart than the positions need.  At 1024 residues a plane is exactly 2 MB, every step of the
+// kernels that write or read them touches the same offset of all 128 planes, and addresses 2 MB apart fall on the same
+// memory channel: one gated projection at 1024 x 1024 positions 145-151 us dense, 119-127 us padded.
+constexpr int64_t TM_PLANE_PAD = 1088;
+
 int64_t kutacc_hip_triangle_multiplication_workspace(int64_t n_res, int64_t c_z, int64_t c_i)
 {
     if (n_res <= 0 || c_z <= 0 || c_i <= 0 || n_res > 65536 || c_z > 4096 || c_i > 4096) {
         return -1;
     }
-    return 4 * align256(n_res * n_res * (c_z > c_i ? c_z : c_i) * 2);
+    return 4 * align256((n_res * n_res + TM_PLANE_PAD) * (c_z > c_i ? c_z : c_i) * 2);
 }
 
 int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_args_t *a, void *stream)
@@ -276,7 +282,7 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
         (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
         return KUTACC_HIP_EINVAL;
     }
-    const int64_t n = a->n_res, cz = a->c_z, ci = a->c_i, rows = n * n, buf = need / 4;
+    const int64_t n = a->n_res, cz = a->c_z, ci = a->c_i, rows = n * n, buf = need / 4, plane = rows + TM_PLANE_PAD;
     char *ws = static_cast<char *>(a->workspace);
     void *act = ws, *left = ws + buf, *right = ws + 2 * buf, *center_cf = ws + 3 * buf;
     void *center = left, *gate = right, *out = center_cf; // each is free again by the time its second tenant arrives
@@ -296,7 +302,7 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
             g[side].a = side ? a->right_proj_w : a->left_proj_w, g[side].a_gate = side ? a->right_gate_w : a->left_gate_w;
             g[side].a_stride_m = cz, g[side].a_stride_k = 1;
             g[side].b = act, g[side].b_stride_n = cz, g[side].b_stride_k = 1;
-            g[side].c = side ? right : left, g[side].c_stride_m = rows;
+            g[side].c = side ? right : left, g[side].c_stride_m = plane;
             g[side].bias = side ? a->right_proj_b : a->left_proj_b, g[side].bias_gate = side ? a->right_gate_b : a->left_gate_b;
             g[side].bias_axis = 2, g[side].mask = a->pair_mask;
         }
@@ -319,7 +325,7 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
         } else {
             g.a = right, g.a_stride_m = 1, g.a_stride_k = n, g.b = left, g.b_stride_n = 1, g.b_stride_k = n;
         }
-        g.a_stride_batch = g.b_stride_batch = g.c_stride_batch = rows;
+        g.a_stride_batch = g.b_stride_batch = g.c_stride_batch = plane;
         g.c = center_cf, g.c_stride_m = n;
         rc = kutacc_launch::pair_gemm(g, s);
     }
@@ -331,7 +337,7 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
                              kutacc_hip_aligned16(a->ln_center_beta);
     // 4. center_layer_norm, channel-first in, channel-last out
     if (rc == 0 && !norm_inside) {
-        rc = kutacc_launch::layernorm_channel_first(center_cf, rows, a->ln_center_gamma, a->ln_center_beta, center, ci, ci, rows,
+        rc = kutacc_launch::layernorm_channel_first(center_cf, plane, a->ln_center_gamma, a->ln_center_beta, center, ci, ci, rows,
                                                     a->ln_eps, KUTACC_DTYPE_BF16, s);
     }
     // 5. gate from the normalised input
@@ -349,7 +355,7 @@ int kutacc_hip_triangle_multiplication(const kutacc_hip_triangle_multiplication_
     // 6. output projection of the normalised centre, times sigmoid(gate), added to the pair activation: one kernel
     //    when the shape allows, else projection, gating and residual as three passes
     if (rc == 0 && norm_inside) {
-        rc = kutacc_launch::row_projection_projected_gate_residual(center_cf, rows, a->output_w, a->output_b, act, cz,
+        rc = kutacc_launch::row_projection_projected_gate_residual(center_cf, plane, a->output_w, a->output_b, act, cz,
                                                                    a->gating_w, a->gating_b, a->pair_act, cz, rows, s,
                                                                    a->ln_center_gamma, a->ln_center_beta, a->ln_eps);
     } else if (rc == 0 && gate_inside) {
