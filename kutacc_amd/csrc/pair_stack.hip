@@ -698,7 +698,6 @@ __device__ constexpr int DIRECT_MJ[16] = {0, 0, 1, 1, 0, 1, 2, 2, 2, 0, 1, 2, 3,
 template <bool MMAJOR>
 __global__ __launch_bounds__(256, 1) void pair_gemm_direct_kernel(const GemmParams p, const int64_t total_tiles)
 {
-    typedef const __attribute__((address_space(1))) void *global_ptr;
     typedef __attribute__((address_space(3))) void *lds_ptr;
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1223,7 +1222,6 @@ __global__ __launch_bounds__(256 * SIDES, 2 / SIDES) void gated_projection_kerne
     constexpr int C = 128, CK = C / 16, WAVES = 4 * SIDES, THREADS = 64 * WAVES;
     extern __shared__ uint4 lds[]; // [SIDES][2 matrices][4 channel blocks][CK][64 lanes], then one panel per wave
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 31, g = lane >> 5;
     uint4 *panel = lds + SIDES * 2 * 4 * CK * 64 + wave * 256;
     const int64_t start = ((int64_t)blockIdx.x * WAVES + wave) * pos_per_wave;
     const int64_t stop = start + pos_per_wave < n_pos ? start + pos_per_wave : n_pos;
