@@ -370,6 +370,29 @@ struct TilePlace {
     int batch, m0, n0;
 };
 
+// Where tile `index` of a persistent workgroup's walk lies (tiles of `side` x `side`).  Workgroup ids are dealt round
+// robin over the 8 XCDs, and id + gridDim.x lands on the same XCD when the grid is a multiple of 8: each XCD gets a
+// contiguous run of tiles, so that neighbours in the walk (which share an operand tile) share an L2; within a batch the
+// dimension with fewer tiles runs fastest.  An index past the last tile gives the last one: a valid address, never used.
+// (The launchers keep the number of tiles within 32 bits: 64-bit divisions cost a few thousand clocks per tile.)
+__device__ __forceinline__ TilePlace walk_place(const GemmParams &p, int64_t total_tiles, int64_t index, int side)
+{
+    uint32_t v = (uint32_t)(index < total_tiles ? index : total_tiles - 1);
+    const uint32_t per = (uint32_t)total_tiles / 8;
+    if (v < per * 8) {
+        v = (v % 8) * per + v / 8;
+    }
+    const uint32_t tiles_per_batch = (uint32_t)p.MT * (uint32_t)p.NT;
+    const int batch = (int)(v / tiles_per_batch), t = (int)(v % tiles_per_batch);
+    int mt, nt;
+    if (p.MT <= p.NT) {
+        mt = t % p.MT, nt = t / p.MT;
+    } else {
+        nt = t % p.NT, mt = t / p.NT;
+    }
+    return TilePlace{batch, mt * side, nt * side};
+}
+
 // The order of one quarter (k-step of 16) of pair_gemm_big_kernel's k-loop, as scheduling-group barriers, whose sizes
 // must be integer constants: NMFMA MFMAs in pairs, with this quarter's LDS reads, global loads or LDS stores dealt
 // evenly between them.
@@ -427,26 +450,7 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_big_kernel(const GemmParams 
     const int r = lane & 31, g = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    // Workgroup ids are dealt round robin over the 8 XCDs, and id + gridDim.x lands on the same XCD when the grid is a
-    // multiple of 8: each XCD gets a contiguous run of tiles, so that neighbours in the walk (which share an operand
-    // tile) share an L2.
-    const int64_t tiles_per_batch = (int64_t)p.MT * p.NT;
-    auto place = [&](int64_t index) -> TilePlace {
-        // (the launcher keeps the number of tiles within 32 bits: 64-bit divisions cost a few thousand clocks per tile)
-        uint32_t v = (uint32_t)(index < total_tiles ? index : total_tiles - 1); // past the last tile: a valid address, never used
-        const uint32_t per = (uint32_t)total_tiles / 8;
-        if (v < per * 8) {
-            v = (v % 8) * per + v / 8;
-        }
-        const int batch = (int)(v / (uint32_t)tiles_per_batch), t = (int)(v % (uint32_t)tiles_per_batch);
-        int mt, nt;
-        if (p.MT <= p.NT) {
-            mt = t % p.MT, nt = t / p.MT;
-        } else {
-            nt = t % p.NT, mt = t / p.NT;
-        }
-        return TilePlace{batch, mt * TILE_SIDE, nt * TILE_SIDE};
-    };
+    auto place = [&](int64_t index) -> TilePlace { return walk_place(p, total_tiles, index, TILE_SIDE); };
 
     // The pieces this wave stages: piece e = wave * BW + i of the step's 4 BW; pieces 0 .. 2 BW - 1 belong to A, the rest
     // to B.  M, N and K are whole tiles and steps here, so an address is a wave-uniform pointer (tile, k-step, piece:
@@ -704,22 +708,7 @@ __global__ __launch_bounds__(256, 1) void pair_gemm_direct_kernel(const GemmPara
     const int r = lane & 31, g = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    const int64_t tiles_per_batch = (int64_t)p.MT * p.NT;
-    auto place = [&](int64_t index) -> TilePlace { // the walk of pair_gemm_big_kernel: a contiguous run of tiles per XCD
-        uint32_t v = (uint32_t)(index < total_tiles ? index : total_tiles - 1);
-        const uint32_t per = (uint32_t)total_tiles / 8;
-        if (v < per * 8) {
-            v = (v % 8) * per + v / 8;
-        }
-        const int batch = (int)(v / (uint32_t)tiles_per_batch), t = (int)(v % (uint32_t)tiles_per_batch);
-        int mt, nt;
-        if (p.MT <= p.NT) {
-            mt = t % p.MT, nt = t / p.MT;
-        } else {
-            nt = t % p.NT, mt = t / p.NT;
-        }
-        return TilePlace{batch, mt * BIG_TILE, nt * BIG_TILE};
-    };
+    auto place = [&](int64_t index) -> TilePlace { return walk_place(p, total_tiles, index, BIG_TILE); };
 
     // Waves 0 and 1 bring A, waves 2 and 3 B: unit u = 8 (wave & 1) + i of the operand's sixteen per stage.  An address
     // is a wave-uniform pointer (tile, stage, unit) plus a 32-bit byte offset per lane that never changes.
