@@ -536,7 +536,6 @@ def test_gated_projection_streaming_kernel(torch_cuda):
     within one bf16 rounding."""
     from oracle import oracle
     torch = torch_cuda
-    capi.set_tuning("gated_projection", "streaming")
     n_pos, c = 512 * 512 + 40, 128
     rng = np.random.Generator(np.random.PCG64(900))
     x = draw(rng, n_pos, c)
@@ -545,27 +544,11 @@ def test_gated_projection_streaming_kernel(torch_cuda):
     pb, gb = (rng.standard_normal(c) * 0.5).astype(np.float32), (rng.standard_normal(c) * 0.5).astype(np.float32)
     t = dict(x=dev(torch, x), mask=dev(torch, mask), pw=dev(torch, pw), gw=dev(torch, gw), pb=dev(torch, pb, torch.float32),
              gb=dev(torch, gb, torch.float32))
-    # weights with a padded leading dimension are outside the streaming kernel's shapes: the same product on the tiled kernel
+    # weights with a padded leading dimension are outside the dedicated kernels' shapes: the same product on the tiled kernel
     pad_w = lambda w: torch.nn.functional.pad(w, (0, 8)).contiguous()  # noqa: E731
-    outs = []
-    for wp_t, wg_t, ld_w in ((t["pw"], t["gw"], c), (pad_w(t["pw"]), pad_w(t["gw"]), c + 8)):
-        out = torch.full((c, n_pos), -3.0, dtype=torch.bfloat16, device="cuda")
-        g = capi.HipGemmArgs()
-        g.m, g.n, g.k, g.batches, g.dtype, g.path = c, n_pos, c, 1, capi.K_BF16, capi.PATH_FUSED
-        g.a, g.a_gate, g.a_stride_m, g.a_stride_k = wp_t.data_ptr(), wg_t.data_ptr(), ld_w, 1
-        g.b, g.b_stride_n, g.b_stride_k = t["x"].data_ptr(), c, 1
-        g.c, g.c_stride_m = out.data_ptr(), n_pos
-        g.bias, g.bias_gate, g.bias_axis, g.mask = t["pb"].data_ptr(), t["gb"].data_ptr(), 2, t["mask"].data_ptr()
-        capi.lib().kutacc_hip_profile_enable(1)
-        rc = capi.lib().kutacc_hip_gemm(ctypes.byref(g), None)
-        torch.cuda.synchronize()
-        assert rc == 0, rc
-        name = ctypes.create_string_buffer(96)
-        ms, cnt, fl = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
-        assert capi.lib().kutacc_hip_profile_read(0, name, 96, ctypes.byref(ms), ctypes.byref(cnt), ctypes.byref(fl)) == 0
-        capi.lib().kutacc_hip_profile_enable(0)
-        outs.append((name.value.decode(), out))
-    capi.set_tuning("gated_projection", None)
+    padded = dict(t, pw=pad_w(t["pw"]), gw=pad_w(t["gw"]))
+    outs = [gated_projection_once(torch, t, c, n_pos, n_pos, "streaming"),
+            gated_projection_once(torch, padded, c, n_pos, n_pos, "streaming", ld_w=c + 8)]
     assert outs[0][0] == "gated_projection_kernel" and outs[1][0] == "pair_gemm_kernel<gated>", [o[0] for o in outs]
     sample = np.concatenate([np.arange(0, 96), np.arange(n_pos - 96, n_pos),
                              rng.choice(n_pos, size=2048, replace=False)])
